@@ -1,0 +1,205 @@
+/*
+ * vui_amd.h - C ABI of the MI355X (gfx950) decode-step library for Vui.
+ *
+ * The reference has no native boundary for this path: its "operator API" is the Python
+ * surface of src/vui/model.py and src/vui/engine.py, whose GPU arithmetic is delegated to
+ * torch/cuBLAS, flash_attn_with_kvcache and torch.cuda.CUDAGraph.  Each entry point below
+ * names the reference call it stands in for.  All pointers marked "device" are HIP device
+ * pointers; the library never allocates, frees or synchronises: buffers (weights, KV caches,
+ * workspace, outputs) are owned by the caller, work is enqueued on the given stream, and
+ * every call may be recorded into a HIP graph.
+ *
+ * Return value: 0 on success, a negative VUI_E* code on failure; vui_last_error() returns a
+ * human-readable description of the last failure on the calling thread.
+ */
+#ifndef VUI_AMD_H
+#define VUI_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VUI_OK 0
+#define VUI_EINVAL (-22)  /* bad argument / unsupported shape */
+#define VUI_EHIP (-5)     /* a HIP runtime call failed */
+#define VUI_ENOMEM (-12)  /* workspace too small */
+
+#define VUI_DTYPE_BF16 0
+#define VUI_DTYPE_F32 1
+
+#define VUI_MAX_LAYERS 64
+#define VUI_MAX_RQ_LAYERS 16
+#define VUI_MAX_BATCH 16
+
+typedef void* vui_stream_t; /* hipStream_t */
+
+/* Architecture numbers; mirrors VuiConfig (src/vui/config.py:16-52) as consumed by
+ * Vui.__init__ (src/vui/model.py:1061-1136). */
+typedef struct vui_config {
+  int32_t dtype;          /* VUI_DTYPE_*: element type of weights, activations and KV caches */
+  int32_t d_model, n_layers, n_heads, n_kv_heads, head_dim, ffn;
+  int32_t n_quantizers, codebook_size;
+  int32_t rq_dim, rq_layers, rq_heads, rq_ffn;
+  int32_t rope_dim;       /* leading features of each head that are rotated (<= head_dim, even) */
+  int32_t max_seqlen;     /* S of the KV caches and of the RoPE table */
+  int32_t n_slots;        /* KV cache slots (reference: max_rows + 1, engine.py:380-387) */
+  int32_t window;         /* sliding window of every layer, 0 = full attention (model.py:256) */
+  float norm_eps;         /* backbone RMSNorm eps (model.py:391) */
+  float rq_norm_eps;      /* RQ RMSNorm eps (model.py:287) */
+  int32_t int8_backbone;  /* 1: backbone linears are int8 weight-only with per-row scales */
+} vui_config;
+
+/* One backbone block (src/vui/model.py:300-340).  nn.Linear layout (out, in), row-major. */
+typedef struct vui_layer_weights {
+  const void* attn_norm;  /* (d) */
+  const void* wqkv;       /* ((H+2KV)*hd, d)   dtype, or int8 when int8_backbone */
+  const void* wo;         /* (d, d) */
+  const void* mlp_norm;   /* (d) */
+  const void* w1;         /* (ffn, d) */
+  const void* w3;         /* (ffn, d) */
+  const void* w2;         /* (d, ffn) */
+  /* per-output-row scales (dtype elements) when int8_backbone, else NULL */
+  const void *s_qkv, *s_o, *s_1, *s_3, *s_2;
+} vui_layer_weights;
+
+/* One RQ block (src/vui/model.py:577-597). */
+typedef struct vui_rq_layer_weights {
+  const void *attn_norm, *wqkv, *wo, *mlp_norm, *w1, *w3, *w2;
+} vui_rq_layer_weights;
+
+typedef struct vui_weights {
+  const void* audio_emb;    /* (Q*CS, d)   model.py:552-563 */
+  const void* final_norm;   /* (d)         decoder.norm */
+  const void* codec_head;   /* (CS, d)     model.py:1083 */
+  const void* eos_w;        /* (1, d)      model.py:1099 */
+  const void* eos_b;        /* (1) */
+  const float* rope_table;  /* (max_seqlen, rope_dim, 2) fp32 cos/sin, rope.py:60-77 */
+  vui_layer_weights layers[VUI_MAX_LAYERS];
+  const void* rq_backbone_proj; /* (R, d) or NULL when R == d (nn.Identity, model.py:653-657) */
+  const void* rq_code_emb;      /* ((Q-1)*CS, R) */
+  const void* rq_pos_emb;       /* (Q, R) */
+  const void* rq_head_w;        /* (Q-1, CS, R) */
+  const void* rq_norm;          /* (R) */
+  vui_rq_layer_weights rq_layers[VUI_MAX_RQ_LAYERS];
+} vui_weights;
+
+typedef struct vui_ctx vui_ctx;
+
+const char* vui_last_error(void);
+int vui_version(void);
+
+/* Bytes of device workspace a context needs for up to max_batch rows. */
+int64_t vui_workspace_bytes(const vui_config* cfg, int max_batch);
+/* Bytes of ONE of the two (K or V) backbone caches: layers * slots * S * KV * hd elements.
+ * Layout (layers, slots, S, KV, hd); layer l's (slots, S, KV, hd) slab is what the reference
+ * calls flash_kv_caches[l].k_cache (model.py:71-99, 473-495). */
+int64_t vui_kv_bytes(const vui_config* cfg);
+
+/* Host-side object holding the configuration and the device pointers.  The workspace must
+ * stay valid and must not be shared with another context that runs concurrently.
+ * Stands in for Vui.setup_decode_graph's static buffers (model.py:1228-1246) and
+ * RQTransformer.setup_cuda_graph_kv's (model.py:841-858). */
+int vui_ctx_create(const vui_config* cfg, const vui_weights* w, void* workspace, int64_t workspace_bytes,
+                   int max_batch, vui_ctx** out);
+void vui_ctx_destroy(vui_ctx* ctx);
+/* One-time device-side initialisation of the workspace (zeroes counters).  Enqueued on stream. */
+int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream);
+
+/* One backbone decode step for B rows (B <= max_batch).
+ *   Engine._backbone_decode_body / _backbone_decode_body_b  (engine.py:434-449, 485-502)
+ *   Vui._decode_step_inner                                  (model.py:1280-1287)
+ * Exactly one of codes_in / emb_in is non-NULL:
+ *   codes_in  device (B, Q) int64: the previous frame, zero-padded to Q (engine.py:473-479)
+ *   emb_in    device (B, d) dtype: a ready embedding (text/speaker token; prefill, engine.py:674-694)
+ * slot_idx   device (B) int32 row -> KV slot, or NULL for the identity map
+ * seq_lens   device (n_slots) int32: position at which each slot's new K/V row is written;
+ *            after the step seq_lens[slot] += 1 for the B rows' slots (seq_inc == NULL), or
+ *            seq_lens[s] += seq_inc[s] for every slot (engine.py:502)
+ * k_cache/v_cache  device, layout above
+ * hidden_out (B, d), cb0_out (B, CS), eos_out (B, 1): dtype, device; any may be NULL to skip
+ * n_splits   key-range splits per (row, head) in attention, fixed per captured graph (>=1) */
+int vui_backbone_step(vui_ctx* ctx, const int64_t* codes_in, const void* emb_in, const int32_t* slot_idx,
+                      int32_t* seq_lens, const int32_t* seq_inc, int B, void* k_cache, void* v_cache,
+                      void* hidden_out, void* cb0_out, void* eos_out, int n_splits, vui_stream_t stream);
+
+/* Sampling parameters shared by the two samplers.  The uniform for (row b, codebook c) of
+ * frame f is Philox4x32-10(key = seed, counter = (f, b, c, 0)); *frame_ctr is read on the
+ * device, so a captured graph can be replayed with a new frame number. */
+typedef struct vui_sample_params {
+  float temperature;      /* <= 0 means greedy */
+  int32_t top_k;          /* 1 = greedy (lowest index of the maximum), <= 0 = no truncation */
+  uint64_t seed;
+  const int32_t* frame_ctr; /* device (1) int32 frame number, or NULL for frame 0 */
+} vui_sample_params;
+
+/* Code-0 sampler with repetition penalty for B rows:
+ *   Engine._rep_apply / _sample_cb0 / _rep_push  (engine.py:571-590, 855-863, 1451-1466)
+ * logits (B, CS) dtype device; rep_counts (B, CS) fp32 device or NULL; rep_hist (B, window)
+ * int32 and rep_pos (B, 2) int32 {head, filled} device ring state or NULL (no window);
+ * code0_out (B) int64 device. */
+int vui_sample_cb0(vui_ctx* ctx, const void* logits, float* rep_counts, int32_t* rep_hist, int32_t* rep_pos,
+                   float penalty, int window, const vui_sample_params* sp, int64_t* code0_out, int B,
+                   vui_stream_t stream);
+
+/* RQ depth head: all remaining codebooks of one frame for B rows.
+ *   RQTransformer._generate_graph_body_kv / generate_cuda_graph_kv  (model.py:908-1016)
+ * hidden (B, d) dtype, code0 (B) int64, logit_bias (Q-1, CS) fp32 or NULL, n_q = Q' in [2, Q];
+ * codes_out (B, codes_stride) int64: columns [0, Q') written, columns [Q', codes_stride)
+ * zeroed when zero_pad != 0 (the padding the next backbone step expects). */
+int vui_rq_generate(vui_ctx* ctx, const void* hidden, const int64_t* code0, const float* logit_bias,
+                    int n_q, const vui_sample_params* sp, int64_t* codes_out, int codes_stride, int zero_pad,
+                    int B, vui_stream_t stream);
+
+/* The whole per-frame step: backbone step on codes_io, code-0 sampling, RQ head; the new frame
+ * is written back to codes_io (zero-padded to Q) so the call can be repeated or replayed.
+ *   Engine._stream_row / _render_rows loop body (engine.py:1450-1485, 1011-1044)
+ * frames_out: optional device (max_frames, B, Q) int64 log; the frame goes to row *frame_ctr.
+ * eos_prob_out fp32 device, may be NULL: sigmoid(eos logit) (engine.py:1468-1471); (B) values, or,
+ *   when frames_out is given, a (max_frames, B) log whose row *frame_ctr is written.
+ * frame_ctr (device int32) is incremented at the end of the step. */
+int vui_frame_step(vui_ctx* ctx, int64_t* codes_io, const int32_t* slot_idx, int32_t* seq_lens,
+                   const int32_t* seq_inc, int B, void* k_cache, void* v_cache, float* rep_counts,
+                   int32_t* rep_hist, int32_t* rep_pos, float penalty, int window,
+                   const vui_sample_params* sp_cb0, const vui_sample_params* sp_rq, const float* logit_bias,
+                   int n_q, void* hidden_out, void* cb0_out, float* eos_prob_out, int64_t* frames_out,
+                   int max_frames, int32_t* frame_ctr, int n_splits, vui_stream_t stream);
+
+/* HIP graph helpers (stand in for torch.cuda.CUDAGraph capture/replay, model.py:873-876,
+ * 1254-1256; engine.py:465-468).  begin/end bracket any sequence of the calls above issued
+ * on `stream`; the returned handle is replayed with vui_graph_launch. */
+typedef struct vui_graph vui_graph;
+int vui_graph_begin(vui_stream_t stream);
+int vui_graph_end(vui_stream_t stream, vui_graph** out);
+int vui_graph_launch(vui_graph* g, vui_stream_t stream);
+void vui_graph_destroy(vui_graph* g);
+
+/* ---- single kernels, for micro-benchmarks and unit parity tests ---- */
+
+/* y = [rmsnorm_w(x)] W^T for B rows.  x (B, K), W (N, K), y (B, N); norm_w (K) or NULL.
+ * RMSNorm.forward + nn.Linear (model.py:286-297, 158, 220).  w_int8 != 0: W is int8 with
+ * `scales` (N) dtype. */
+int vui_rmsnorm_gemv(int dtype, const void* x, const void* norm_w, float eps, const void* W, const void* scales,
+                     int w_int8, void* y, int B, int N, int K, vui_stream_t stream);
+/* In-place interleaved rotation of x (B, n_heads, head_dim) at positions pos (B) int32.
+ * apply_rotary_emb (rope.py:23-57). */
+int vui_rope(int dtype, void* x, const float* rope_table, const int32_t* pos, int B, int n_heads, int head_dim,
+             int rope_dim, vui_stream_t stream);
+/* Decode attention for B rows over caches (slots, S, KV, hd): appends k_new/v_new (B, KV, hd)
+ * at seq_lens[slot] (when non-NULL), then out (B, H, hd) = softmax(q K^T / sqrt(hd)) V over
+ * positions 0..seq_lens[slot].  flash_attn_with_kvcache (model.py:247-257).
+ * scratch: device, vui_attn_scratch_bytes(B, H, hd, n_splits) bytes, zero-initialised once. */
+int64_t vui_attn_scratch_bytes(int B, int H, int hd, int n_splits);
+int vui_decode_attn(int dtype, const void* q, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
+                    const int32_t* seq_lens, const int32_t* slot_idx, void* out, int B, int H, int KV, int hd,
+                    int S, int window, int n_splits, void* scratch, vui_stream_t stream);
+/* One draw per row from logits (B, CS) fp32 with the RQ-head rule (model.py:955-962). */
+int vui_sample_logits(const float* logits, const float* bias, int CS, const vui_sample_params* sp, int codebook,
+                      int64_t* out, int B, vui_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VUI_AMD_H */

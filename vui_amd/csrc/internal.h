@@ -1,0 +1,136 @@
+// Internal launcher interface between the kernel translation units and the C ABI layer.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/vui_amd.h"
+
+// epilogues of the fused GEMV
+enum {
+  EPI_STORE = 0,   // y = rnd(acc)
+  EPI_RESID = 1,   // y = rnd(resid + rnd(acc))
+  EPI_SWIGLU = 2,  // y = rnd(rnd(silu(rnd(acc1))) * rnd(acc3))   (two weight matrices)
+  EPI_QKV = 3,     // split into q | k | v, rotate q and k, append k and v to the KV cache
+  EPI_ADDVEC = 4,  // y = rnd(rnd(acc) + vec[n])
+  EPI_RQ_QKV = 5,  // split into q | k | v without rotation, k/v into the depth-head cache
+};
+
+struct GemvArgs {
+  int dtype;      // VUI_DTYPE_*
+  int w_int8;     // weights are int8 with per-row scales
+  const void* x;  // (B, K)
+  const void* norm_w;  // (K) or nullptr: no RMSNorm prologue
+  float eps;
+  const void* W;   // (N, K)
+  const void* W2;  // second matrix for EPI_SWIGLU
+  const void* sc;  // (N) scales for int8
+  const void* sc2;
+  void* y;         // (B, ldy)
+  int ldy;
+  const void* resid;  // (B, ldy) for EPI_RESID (may alias y)
+  const void* vec;    // (N) for EPI_ADDVEC
+  int B, N, K;
+  int epi;
+  // EPI_QKV / EPI_RQ_QKV
+  const float* rope;  // (S, rope_dim, 2)
+  int rope_dim, hd, nq, nkv;  // nq = H*hd, nkv = KV*hd
+  void* kc;           // layer slab (slots, S, KV, hd)  | depth-head (B, Q, R)
+  void* vc;
+  const int32_t* seq_lens;
+  const int32_t* slot_idx;
+  int S;       // cache length (positions)
+  int rq_pos;  // EPI_RQ_QKV: position written
+  // optional extra output row with bias (the eos head), plus the position update it carries
+  const void* Wx;  // (1, K)
+  const void* bx;  // (1)
+  void* yx;        // (B, 1)
+  void* hid_out;   // (B, K): the staged (normalised) activations, written by the extra block
+  int32_t* upd_seq_lens;       // if set: after the step seq_lens are advanced by the extra block
+  const int32_t* upd_seq_inc;  // (n_slots) or nullptr (+1 for the B rows' slots)
+  int n_slots;
+};
+
+int launch_gemv(const GemvArgs& a, hipStream_t st);
+
+struct AttnArgs {
+  int dtype;
+  const void* q;  // (B, H*hd), already rotated
+  const void* kc; // (slots, S, KV, hd) with the new row already appended
+  const void* vc;
+  const int32_t* seq_lens;  // position of the newest key per slot
+  const int32_t* slot_idx;
+  void* out;  // (B, H*hd)
+  int B, H, KV, hd, S, window, n_splits;
+  float* part;        // (B, H, n_splits, hd + 2) fp32
+  uint32_t* counter;  // (B*H), zero between launches
+};
+int launch_decode_attn(const AttnArgs& a, hipStream_t st);
+int launch_kv_append(int dtype, const void* k_new, const void* v_new, void* kc, void* vc, const int32_t* seq_lens,
+                     const int32_t* slot_idx, int B, int KV, int hd, int S, hipStream_t st);
+
+int launch_embed(int dtype, const int64_t* codes, const void* table, void* x, int B, int Q, int CS, int d,
+                 hipStream_t st);
+int launch_copy_rows(int dtype, const void* src, void* dst, int64_t n, hipStream_t st);
+int launch_rope(int dtype, void* x, const float* table, const int32_t* pos, int B, int nh, int hd, int rope_dim,
+                hipStream_t st);
+
+struct RqAttnArgs {
+  int dtype;
+  const void* q;   // (B, R)
+  const void* kc;  // (B, Q, R)
+  const void* vc;
+  void* out;  // (B, R)
+  int B, heads, hd, Q, pos;
+};
+int launch_rq_attn(const RqAttnArgs& a, hipStream_t st);
+
+struct SampleArgs {
+  int dtype;           // element type of logits (VUI_DTYPE_F32 allowed for the raw entry point)
+  const void* logits;  // (B, CS)
+  const float* bias;   // (CS) fp32 or nullptr
+  float* rep_counts;   // (B, CS) or nullptr
+  int32_t* rep_hist;   // (B, window) or nullptr
+  int32_t* rep_pos;    // (B, 2) {head, filled}
+  float penalty;
+  int window;
+  float temperature;
+  int top_k;
+  uint64_t seed;
+  const int32_t* frame_ctr;
+  int codebook;  // Philox counter word 2
+  int CS, B;
+  int64_t* out;  // out[b * out_stride + out_col]
+  int out_stride, out_col;
+  // optional: build the depth head's next input token  x[b] = rnd(emb[code + emb_off] + pos_vec)
+  const void* tok_emb;  // (rows, R)
+  const void* tok_pos;  // (R)
+  void* tok_out;        // (B, R)
+  int64_t tok_emb_off;
+  int R;
+  // optional: eos probability = sigmoid(eos_logit[b])
+  const void* eos_logit;  // (B) dtype
+  float* eos_prob;        // (B)
+  // optional zero padding of out[b, pad_from..pad_to)
+  int pad_from, pad_to;
+};
+int launch_sample(const SampleArgs& a, hipStream_t st);
+
+// x[b] = rnd(emb[code[b] + off] + pos_vec); optionally codes_out[b*stride] = code[b]
+int launch_rq_token(int dtype, const int64_t* code, int64_t off, const void* emb, const void* pos_vec, void* x,
+                    int B, int R, int64_t* codes_out, int stride, int CS, hipStream_t st);
+// frames_out[*ctr] = codes (B*Q) if ctr < max_frames; *ctr += 1
+// and eos_out[(frames_out ? *ctr : 0) * B + b] = eos_in[b]
+int launch_frame_finish(const int64_t* codes, int64_t* frames_out, int n, int max_frames, int32_t* ctr,
+                        const float* eos_in, float* eos_out, int B, hipStream_t st);
+int launch_add_rows(int dtype, const void* a, const void* vec, void* out, int B, int R, hipStream_t st);
+int launch_fill_u32(uint32_t* p, uint32_t v, int64_t n, hipStream_t st);
+
+void vui_set_error(const char* fmt, ...);
+#define HIP_TRY(expr)                                                                  \
+  do {                                                                                 \
+    hipError_t _e = (expr);                                                            \
+    if (_e != hipSuccess) {                                                            \
+      vui_set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, __LINE__); \
+      return VUI_EHIP;                                                                 \
+    }                                                                                  \
+  } while (0)

@@ -1,0 +1,328 @@
+// Small kernels around the GEMVs: embedding gather-sum, stand-alone RoPE, the fused
+// temperature / top-k / repetition-penalty sampler with a counter-based generator, the depth
+// head's token builder and the per-frame bookkeeping.
+#include "common.h"
+#include "internal.h"
+
+// ---- audio embedding: x[b] = rnd(sum_q table[codes[b,q] + q*CS])   (model.py:559-563) ----
+template <typename T>
+__global__ void embed_kernel(const int64_t* codes, const T* table, T* x, int Q, int CS, int d) {
+  const int b = blockIdx.y;
+  const int k = blockIdx.x * blockDim.x + threadIdx.x;
+  if (k >= d) return;
+  float s = 0.f;
+  for (int q = 0; q < Q; ++q) {
+    int64_t c = codes[(size_t)b * Q + q];
+    c = c < 0 ? 0 : (c >= CS ? CS - 1 : c);
+    s += El<T>::ld(table + ((size_t)(c + (int64_t)q * CS)) * d + k);
+  }
+  El<T>::st(x + (size_t)b * d + k, s);
+}
+
+int launch_embed(int dtype, const int64_t* codes, const void* table, void* x, int B, int Q, int CS, int d,
+                 hipStream_t st) {
+  dim3 grid((d + 255) / 256, B);
+  if (dtype == VUI_DTYPE_F32)
+    hipLaunchKernelGGL(embed_kernel<float>, grid, dim3(256), 0, st, codes, (const float*)table, (float*)x, Q, CS, d);
+  else
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, dim3(256), 0, st, codes, (const bf16_t*)table, (bf16_t*)x, Q, CS, d);
+  HIP_TRY(hipGetLastError());
+  return VUI_OK;
+}
+
+__global__ void copy_bytes_kernel(const uint8_t* src, uint8_t* dst, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = src[i];
+}
+int launch_copy_rows(int dtype, const void* src, void* dst, int64_t n, hipStream_t st) {
+  const int64_t bytes = n * (dtype == VUI_DTYPE_F32 ? 4 : 2);
+  hipLaunchKernelGGL(copy_bytes_kernel, dim3((unsigned)((bytes + 255) / 256)), dim3(256), 0, st, (const uint8_t*)src,
+                     (uint8_t*)dst, bytes);
+  HIP_TRY(hipGetLastError());
+  return VUI_OK;
+}
+
+__global__ void fill_u32_kernel(uint32_t* p, uint32_t v, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+int launch_fill_u32(uint32_t* p, uint32_t v, int64_t n, hipStream_t st) {
+  hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, p, v, n);
+  HIP_TRY(hipGetLastError());
+  return VUI_OK;
+}
+
+// ---- stand-alone interleaved RoPE (rope.py:16-57), in place on (B, nh, hd) ----
+template <typename T>
+__global__ void rope_kernel(T* x, const float* table, const int32_t* pos, int nh, int hd, int rope_dim) {
+  const int b = blockIdx.x;
+  const int p = pos[b];
+  for (int i = threadIdx.x; i < nh * (rope_dim / 2); i += blockDim.x) {
+    const int h = i / (rope_dim / 2), j = i % (rope_dim / 2);
+    T* px = x + ((size_t)b * nh + h) * hd + 2 * j;
+    const float x0 = El<T>::ld(px), x1 = El<T>::ld(px + 1);
+    const float* f0 = table + ((size_t)p * rope_dim + 2 * j) * 2;
+    const float* f1 = f0 + 2;
+    El<T>::st(px, rope_mix(x0, f0[0], -x1, f0[1]));
+    El<T>::st(px + 1, rope_mix(x1, f1[0], x0, f1[1]));
+  }
+}
+int launch_rope(int dtype, void* x, const float* table, const int32_t* pos, int B, int nh, int hd, int rope_dim,
+                hipStream_t st) {
+  if ((rope_dim & 1) || rope_dim > hd) { vui_set_error("rope: bad rope_dim %d", rope_dim); return VUI_EINVAL; }
+  if (dtype == VUI_DTYPE_F32)
+    hipLaunchKernelGGL(rope_kernel<float>, dim3(B), dim3(256), 0, st, (float*)x, table, pos, nh, hd, rope_dim);
+  else
+    hipLaunchKernelGGL(rope_kernel<bf16_t>, dim3(B), dim3(256), 0, st, (bf16_t*)x, table, pos, nh, hd, rope_dim);
+  HIP_TRY(hipGetLastError());
+  return VUI_OK;
+}
+
+// ---- Philox4x32-10 (Salmon et al. 2011) ----
+__device__ __forceinline__ uint32_t philox_u32(uint64_t seed, uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3) {
+  uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+    const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    c1 = (uint32_t)p1; c3 = (uint32_t)p0; c0 = n0; c2 = n2;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  return c0;
+}
+
+__device__ __forceinline__ uint32_t float_key(float f) {  // order-preserving map to uint32
+  const uint32_t u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// ---- sampler: one 256-thread workgroup per row ----
+// RQ rule (model.py:955-962): l = (logit + bias) / T; drop l < k-th largest; softmax; draw.
+// code-0 rule (engine.py:571-576, 855-863): penalise by penalty^count; softmax(l / T); keep the
+// top-k probabilities; renormalise; draw.  Both reduce to: keep {l >= k-th largest l},
+// weights exp(l - max), inverse CDF in index order with one uniform.
+#define SAMP_THREADS 256
+#define SAMP_MAX_E 32  // elements per thread -> CS <= 8192
+
+template <typename T, int EMAX>
+__global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const SampleArgs p) {
+  __shared__ float sred[SAMP_THREADS / WAVE];
+  __shared__ int ired[SAMP_THREADS / WAVE];
+  __shared__ float wsum[SAMP_THREADS / WAVE];
+  __shared__ int s_pick;
+  const int b = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int CS = p.CS;
+  const int E = (CS + SAMP_THREADS - 1) / SAMP_THREADS;  // contiguous elements per thread
+  const T* lg = (const T*)p.logits + (size_t)b * CS;
+  const bool greedy = (p.top_k == 1) || !(p.temperature > 0.f);
+  const float invT_div = greedy ? 1.0f : p.temperature;
+
+  float l[EMAX];
+#pragma unroll
+  for (int e = 0; e < EMAX; ++e) {
+    l[e] = -INFINITY;
+    const int j = tid * E + e;
+    if (e < E && j < CS) {
+      float v = El<T>::ld(lg + j);
+      if (p.bias) v += p.bias[j];
+      if (p.rep_counts && p.penalty > 1.0f) {
+        const float f = powf(p.penalty, p.rep_counts[(size_t)b * CS + j]);
+        v = (v > 0.f) ? v / f : v * f;
+      }
+      l[e] = v / invT_div;
+    }
+  }
+
+  // maximum and its lowest index
+  float m = -INFINITY; int mi = 0x7fffffff;
+#pragma unroll
+  for (int e = 0; e < EMAX; ++e)
+    if (e < E && l[e] > m) { m = l[e]; mi = tid * E + e; }
+  {
+    float wm = wave_max(m);
+    int cand = (m == wm) ? mi : 0x7fffffff;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) cand = min(cand, __shfl_xor(cand, o, WAVE));
+    if (lane == 0) { sred[wave] = wm; ired[wave] = cand; }
+  }
+  __syncthreads();
+  float M = sred[0]; int Mi = ired[0];
+#pragma unroll
+  for (int w = 1; w < SAMP_THREADS / WAVE; ++w) {
+    if (sred[w] > M) { M = sred[w]; Mi = ired[w]; }
+    else if (sred[w] == M) Mi = min(Mi, ired[w]);
+  }
+  __syncthreads();
+
+  int pick = Mi;
+  if (!greedy) {
+    // key of the k-th largest value, built bit by bit
+    uint32_t thr = 0u;
+    if (p.top_k > 0 && p.top_k < CS) {
+      uint32_t key[EMAX];
+#pragma unroll
+      for (int e = 0; e < EMAX; ++e) key[e] = (e < E && tid * E + e < CS) ? float_key(l[e]) : 0u;
+      for (int bit = 31; bit >= 0; --bit) {
+        const uint32_t cand = thr | (1u << bit);
+        int c = 0;
+#pragma unroll
+        for (int e = 0; e < EMAX; ++e)
+          if (e < E) c += (key[e] >= cand);
+        c = wave_sum_i(c);
+        if (lane == 0) ired[wave] = c;
+        __syncthreads();
+        int tot = 0;
+#pragma unroll
+        for (int w = 0; w < SAMP_THREADS / WAVE; ++w) tot += ired[w];
+        if (tot >= p.top_k) thr = cand;
+        __syncthreads();
+      }
+    }
+    // weights, their total, and the inverse CDF in index order
+    float wloc = 0.f;
+    float pw[EMAX];
+#pragma unroll
+    for (int e = 0; e < EMAX; ++e) {
+      pw[e] = 0.f;
+      if (e < E && tid * E + e < CS && float_key(l[e]) >= thr) pw[e] = expf(l[e] - M);
+      wloc += pw[e];
+    }
+    // inclusive scan of wloc over threads: within the wave, then across waves
+    float incl = wloc;
+#pragma unroll
+    for (int o = 1; o < WAVE; o <<= 1) {
+      const float t = __shfl_up(incl, o, WAVE);
+      if (lane >= o) incl += t;
+    }
+    if (lane == WAVE - 1) wsum[wave] = incl;
+    if (tid == 0) s_pick = -1;
+    __syncthreads();
+    float base = 0.f, total = 0.f;
+#pragma unroll
+    for (int w = 0; w < SAMP_THREADS / WAVE; ++w) { if (w < wave) base += wsum[w]; total += wsum[w]; }
+    const uint32_t frame = p.frame_ctr ? (uint32_t)p.frame_ctr[0] : 0u;
+    const uint32_t rnd = philox_u32(p.seed, frame, (uint32_t)b, (uint32_t)p.codebook, 0u);
+    const float u = (float)(rnd >> 8) * (1.0f / 16777216.0f);
+    const float target = u * total;
+    const float before = base + incl - wloc;  // sum of everything ahead of this thread
+    if (target >= before && target < before + wloc) {
+      float run = before; int j = -1;
+#pragma unroll
+      for (int e = 0; e < EMAX; ++e) {
+        if (e < E && j < 0) { run += pw[e]; if (pw[e] > 0.f && run > target) j = tid * E + e; }
+      }
+      if (j < 0) {  // rounding at the thread's upper edge: take its last kept element
+#pragma unroll
+        for (int e = 0; e < EMAX; ++e) if (e < E && pw[e] > 0.f) j = tid * E + e;
+      }
+      if (j >= 0) atomicMax(&s_pick, j);
+    }
+    __syncthreads();
+    pick = (s_pick >= 0) ? s_pick : Mi;
+  }
+
+  if (tid == 0) {
+    p.out[(size_t)b * p.out_stride + p.out_col] = (int64_t)pick;
+    if (p.rep_counts && p.penalty > 1.0f) {
+      float* cnt = p.rep_counts + (size_t)b * CS;
+      if (p.window > 0 && p.rep_hist) {
+        int head = p.rep_pos[b * 2], filled = p.rep_pos[b * 2 + 1];
+        int32_t* hist = p.rep_hist + (size_t)b * p.window;
+        if (filled == p.window) cnt[hist[head]] -= 1.0f;
+        hist[head] = pick;
+        head = (head + 1) % p.window;
+        if (filled < p.window) ++filled;
+        p.rep_pos[b * 2] = head; p.rep_pos[b * 2 + 1] = filled;
+      }
+      cnt[pick] += 1.0f;
+    }
+    if (p.eos_prob) {
+      const float z = El<T>::ld((const T*)p.eos_logit + b);
+      p.eos_prob[b] = 1.0f / (1.0f + expf(-z));
+    }
+  }
+  for (int j = p.pad_from + tid; j < p.pad_to; j += SAMP_THREADS) p.out[(size_t)b * p.out_stride + j] = 0;
+  if (p.tok_out) {
+    const T* e = (const T*)p.tok_emb + ((size_t)pick + p.tok_emb_off) * p.R;
+    for (int k = tid; k < p.R; k += SAMP_THREADS)
+      El<T>::st((T*)p.tok_out + (size_t)b * p.R + k, El<T>::ld(e + k) + El<T>::ld((const T*)p.tok_pos + k));
+  }
+}
+
+int launch_sample(const SampleArgs& a, hipStream_t st) {
+  if (a.CS < 1 || a.CS > SAMP_THREADS * SAMP_MAX_E) {
+    vui_set_error("sample: codebook_size %d out of range (max %d)", a.CS, SAMP_THREADS * SAMP_MAX_E);
+    return VUI_EINVAL;
+  }
+  const bool small = a.CS <= SAMP_THREADS * 8;
+  if (a.dtype == VUI_DTYPE_F32) {
+    if (small) hipLaunchKernelGGL((sample_kernel<float, 8>), dim3(a.B), dim3(SAMP_THREADS), 0, st, a);
+    else hipLaunchKernelGGL((sample_kernel<float, SAMP_MAX_E>), dim3(a.B), dim3(SAMP_THREADS), 0, st, a);
+  } else {
+    if (small) hipLaunchKernelGGL((sample_kernel<bf16_t, 8>), dim3(a.B), dim3(SAMP_THREADS), 0, st, a);
+    else hipLaunchKernelGGL((sample_kernel<bf16_t, SAMP_MAX_E>), dim3(a.B), dim3(SAMP_THREADS), 0, st, a);
+  }
+  HIP_TRY(hipGetLastError());
+  return VUI_OK;
+}
+
+// ---- depth head token from a code: x[b] = rnd(emb[code + off] + pos_vec)   (model.py:922-925, 967-970) ----
+template <typename T>
+__global__ void rq_token_kernel(const int64_t* code, int64_t off, const T* emb, const T* pos_vec, T* x, int R,
+                                int64_t* codes_out, int stride, int CS) {
+  const int b = blockIdx.x;
+  int64_t c = code[b];
+  c = c < 0 ? 0 : (c >= CS ? CS - 1 : c);
+  const T* e = emb + (size_t)(c + off) * R;
+  for (int k = threadIdx.x; k < R; k += blockDim.x)
+    El<T>::st(x + (size_t)b * R + k, El<T>::ld(e + k) + El<T>::ld(pos_vec + k));
+  if (codes_out && threadIdx.x == 0) codes_out[(size_t)b * stride] = c;
+}
+int launch_rq_token(int dtype, const int64_t* code, int64_t off, const void* emb, const void* pos_vec, void* x,
+                    int B, int R, int64_t* codes_out, int stride, int CS, hipStream_t st) {
+  if (dtype == VUI_DTYPE_F32)
+    hipLaunchKernelGGL(rq_token_kernel<float>, dim3(B), dim3(256), 0, st, code, off, (const float*)emb,
+                       (const float*)pos_vec, (float*)x, R, codes_out, stride, CS);
+  else
+    hipLaunchKernelGGL(rq_token_kernel<bf16_t>, dim3(B), dim3(256), 0, st, code, off, (const bf16_t*)emb,
+                       (const bf16_t*)pos_vec, (bf16_t*)x, R, codes_out, stride, CS);
+  HIP_TRY(hipGetLastError());
+  return VUI_OK;
+}
+
+// out[b] = rnd(rnd(a[b]) + vec)   (depth head token 0 when backbone_proj is the identity)
+template <typename T>
+__global__ void add_rows_kernel(const T* a, const T* vec, T* out, int R) {
+  const int b = blockIdx.x;
+  for (int k = threadIdx.x; k < R; k += blockDim.x)
+    El<T>::st(out + (size_t)b * R + k, El<T>::ld(a + (size_t)b * R + k) + El<T>::ld(vec + k));
+}
+int launch_add_rows(int dtype, const void* a, const void* vec, void* out, int B, int R, hipStream_t st) {
+  if (dtype == VUI_DTYPE_F32)
+    hipLaunchKernelGGL(add_rows_kernel<float>, dim3(B), dim3(256), 0, st, (const float*)a, (const float*)vec, (float*)out, R);
+  else
+    hipLaunchKernelGGL(add_rows_kernel<bf16_t>, dim3(B), dim3(256), 0, st, (const bf16_t*)a, (const bf16_t*)vec, (bf16_t*)out, R);
+  HIP_TRY(hipGetLastError());
+  return VUI_OK;
+}
+
+__global__ void frame_finish_kernel(const int64_t* codes, int64_t* frames_out, int n, int max_frames, int32_t* ctr,
+                                    const float* eos_in, float* eos_out, int B) {
+  const int f = ctr[0];
+  const bool in_range = f >= 0 && f < max_frames;
+  if (frames_out && in_range)
+    for (int i = threadIdx.x; i < n; i += blockDim.x) frames_out[(size_t)f * n + i] = codes[i];
+  if (eos_out && (in_range || !frames_out))
+    for (int b = threadIdx.x; b < B; b += blockDim.x) eos_out[(frames_out ? (size_t)f * B : 0) + b] = eos_in[b];
+  __syncthreads();
+  if (threadIdx.x == 0) ctr[0] = f + 1;
+}
+int launch_frame_finish(const int64_t* codes, int64_t* frames_out, int n, int max_frames, int32_t* ctr,
+                        const float* eos_in, float* eos_out, int B, hipStream_t st) {
+  hipLaunchKernelGGL(frame_finish_kernel, dim3(1), dim3(256), 0, st, codes, frames_out, n, max_frames, ctr, eos_in,
+                     eos_out, B);
+  HIP_TRY(hipGetLastError());
+  return VUI_OK;
+}

@@ -1,0 +1,377 @@
+"""Decode-loop driver over the native step.  Mirrors the decode-step surface of the
+reference's Engine (src/vui/engine.py): rows/slots over one shared KV cache with a padding
+slot, graph-captured batched and bucketed backbone steps, code-0 sampling with the rolling
+repetition penalty, the depth-head call, and -- new here -- the whole frame as ONE graph.
+
+Text handling, the codec/vocoder and the serving layers are outside this package: prompts
+enter as embeddings or token ids.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+import torch
+from torch import Tensor
+
+from . import _lib
+from .model import MAX_BATCH, Graph, Vui, make_sample_params
+
+FRAME_RATE = 12.5  # codec frames per second (src/vui/qwen_codec.py:27-30)
+
+
+@dataclass(frozen=True)
+class GenConfig:
+    """Sampling + generation settings; the fields the decode step reads, with the reference's
+    defaults (src/vui/engine.py:60-86)."""
+
+    temperature: float = 0.9
+    top_k: int | None = 100
+    top_p: float | None = None
+    rep_penalty: float = 1.1
+    rep_window: int = 24
+    eos_threshold: float = 0.45
+    min_secs: float = 0.5
+    max_turn_secs: float = 15.0
+    max_secs: float = 30.0
+    n_codebooks: int = 0  # 0 = all Q quantizers
+    rq_top_k: int = 100  # the reference bakes top_k=100 into the RQ graphs (engine.py:393-397)
+    seed: int = 0
+
+
+def _make_buckets(max_bs: int) -> list[int]:
+    """src/vui/engine.py:134-142."""
+    buckets, b = [], 1
+    while b < max_bs:
+        buckets.append(b)
+        b *= 2
+    if not buckets or buckets[-1] != max_bs:
+        buckets.append(max_bs)
+    return buckets
+
+
+def _get_bucket(batch_size: int, buckets: list[int]) -> int:
+    for b in buckets:
+        if batch_size <= b:
+            return b
+    return buckets[-1]
+
+
+class Row:
+    """One conversation slot of the shared KV cache (src/vui/engine.py:157-270)."""
+
+    def __init__(self, engine: "Engine", idx: int):
+        self._engine = engine
+        self._idx = idx
+        self._prompt_offset = 0
+        self._closed = False
+        self._slot = torch.tensor([idx], dtype=torch.int32, device=engine.device)
+
+    @property
+    def idx(self) -> int:
+        return self._idx
+
+    @property
+    def offset(self) -> int:
+        return int(self._engine.seq_lens[self._idx].item())
+
+    def prefill_emb(self, emb: Tensor) -> Tensor:
+        """Write a (1, T, d) embedding block at the row's offset; returns the final-norm output
+        (1, T, d).  Engine._prefill_emb, src/vui/engine.py:674-694."""
+        return self._engine._prefill_emb(self, emb)
+
+    def mark_prompt(self) -> int:
+        self._prompt_offset = self.offset
+        return self._prompt_offset
+
+    def rewind(self) -> int:
+        return self._engine._rewind_row(self, self._prompt_offset)
+
+    def reset(self) -> int:
+        return self._engine._rewind_row(self, 0)
+
+    def close(self) -> None:
+        if not self._closed:
+            self._engine._release_row(self)
+            self._closed = True
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+
+class Engine:
+    """Streaming (B=1) and batched (B=N) decode over one flash-style KV cache."""
+
+    def __init__(self, name: str | None = None, *, model: Vui | None = None, codec=None, max_rows: int = 1,
+                 max_seq: int | None = None):
+        if model is None:
+            if name is None:
+                raise ValueError("pass model= or a local checkpoint path")
+            model = Vui.from_pretrained_inf(name)
+        if max_rows < 1 or max_rows > MAX_BATCH:
+            raise ValueError(f"max_rows must be in [1, {MAX_BATCH}]")
+        self.model = model
+        self.codec = codec
+        self.max_rows = max_rows
+        self.device = model.device
+        self.dtype = model.dtype
+        cfg = model.config.model
+        self.Q, self.CS, self.D = cfg.n_quantizers, cfg.codebook_size, cfg.d_model
+        trained = model.decoder.max_seqlen
+        self.max_seq = max_seq or trained
+        if self.max_seq > trained:
+            raise ValueError(f"max_seq={self.max_seq} exceeds trained ceiling {trained}")
+        self._cond_bias = model._cond_bias
+        self._setup_graphs()
+        self._setup_rep_state()
+        self._free: set[int] = set(range(max_rows))
+        self._rows: dict[int, Row] = {}
+        self._frame_graphs: dict = {}
+
+    # ------------------------------------------------------------------ setup
+    def _setup_graphs(self) -> None:
+        """src/vui/engine.py:375-432.  KV cache of max_rows + 1 slots (the last one is the write-only
+        target of bucket padding rows), static in/out buffers, batched and bucketed step graphs."""
+        model, dev, dt = self.model, self.device, self.dtype
+        model.decoder.allocate_flash_kv_cache(self.max_rows + 1, dev, dt, max_seqlen=self.max_seq)
+        self.seq_lens = model.decoder.flash_kv_caches[0].seq_lens
+        self._pad_slot = self.max_rows
+        self._buckets = _make_buckets(self.max_rows)
+        rq_batch_sizes = tuple(sorted(set(self._buckets) | {1, self.max_rows}))
+        model.rq_transformer.setup_cuda_graph_kv(dev, dt, top_k=100, batch_sizes=rq_batch_sizes)
+        self._zero_rq_bias = torch.zeros(self.Q - 1, self.CS, device=dev, dtype=torch.float32)
+        N = self.max_rows
+        self._g_codes_in = torch.zeros(N, self.Q, device=dev, dtype=torch.long)
+        self._g_hidden_out = torch.zeros(N, self.D, device=dev, dtype=dt)
+        self._g_cb0_out = torch.zeros(N, self.CS, device=dev, dtype=dt)
+        self._g_eos_out = torch.zeros(N, 1, device=dev, dtype=dt)
+        self._decode_graph = None
+        B_max = self._buckets[-1]
+        self._gc_codes_in = torch.zeros(B_max, self.Q, device=dev, dtype=torch.long)
+        self._gc_hidden_out = torch.zeros(B_max, self.D, device=dev, dtype=dt)
+        self._gc_cb0_out = torch.zeros(B_max, self.CS, device=dev, dtype=dt)
+        self._gc_eos_out = torch.zeros(B_max, 1, device=dev, dtype=dt)
+        self._g_slot_idx = torch.full((B_max,), self._pad_slot, device=dev, dtype=torch.int32)
+        self._g_seq_inc = torch.zeros(self.max_rows + 1, device=dev, dtype=torch.int32)
+        self._bucketed_graphs: dict[int, Graph] = {}
+        # fused frame state
+        self._frame_ctr = torch.zeros(1, dtype=torch.int32, device=dev)
+        self._code0 = torch.zeros(N, dtype=torch.long, device=dev)
+
+    def _splits(self, B: int) -> int:
+        return self.model.decoder.default_splits(B)
+
+    def _backbone_decode_body(self, stream: int) -> None:
+        """One decode step across all max_rows slots (src/vui/engine.py:434-449)."""
+        B = self.max_rows
+        self.model.decoder._step(codes=self._g_codes_in, emb=None, slot_idx=None, seq_inc=None, B=B,
+                                 hidden_out=self._g_hidden_out, cb0_out=self._g_cb0_out, eos_out=self._g_eos_out,
+                                 n_splits=self._splits(B), stream=stream)
+
+    def _capture(self, body) -> Graph:
+        """Warm once and capture; warm-up and capture advance seq_lens, so it is restored
+        (src/vui/engine.py:451-471)."""
+        saved = self.seq_lens.clone()
+        g = Graph(self.model, body, warmup=1)
+        torch.cuda.current_stream().synchronize()
+        self.seq_lens.copy_(saved)
+        return g
+
+    def _decode_step(self) -> tuple[Tensor, Tensor, Tensor]:
+        """Replay the batched backbone graph; returns views of the static (hidden, cb0, eos)
+        buffers (src/vui/engine.py:850-853)."""
+        if self._decode_graph is None:
+            self._decode_graph = self._capture(self._backbone_decode_body)
+        self._decode_graph.replay()
+        return self._g_hidden_out, self._g_cb0_out, self._g_eos_out
+
+    def _set_codes_in(self, row_idx: int, codes: Tensor) -> None:
+        """src/vui/engine.py:473-479: frames shorter than Q are zero-padded."""
+        Q_out = codes.shape[0]
+        if Q_out < self.Q:
+            self._g_codes_in[row_idx].zero_()
+            self._g_codes_in[row_idx, :Q_out] = codes
+        else:
+            self._g_codes_in[row_idx] = codes
+
+    def _backbone_decode_body_b(self, B: int, stream: int) -> None:
+        """Step for B rows with slot indirection (src/vui/engine.py:485-502)."""
+        self.model.decoder._step(codes=self._gc_codes_in, emb=None, slot_idx=self._g_slot_idx,
+                                 seq_inc=self._g_seq_inc, B=B, hidden_out=self._gc_hidden_out,
+                                 cb0_out=self._gc_cb0_out, eos_out=self._gc_eos_out, n_splits=self._splits(B),
+                                 stream=stream)
+
+    def _bucketed_decode_step(self, B_active: int) -> tuple[Tensor, Tensor, Tensor]:
+        """src/vui/engine.py:525-534: pad the active rows up to the bucket with rows that write to the
+        padding slot, replay that bucket's graph."""
+        B_bucket = _get_bucket(B_active, self._buckets)
+        self._g_slot_idx[B_active:B_bucket].fill_(self._pad_slot)
+        g = self._bucketed_graphs.get(B_bucket)
+        if g is None:
+            saved_idx, saved_inc = self._g_slot_idx.clone(), self._g_seq_inc.clone()
+            self._g_slot_idx[:B_bucket].fill_(self._pad_slot)
+            self._g_seq_inc.zero_()
+            g = self._capture(lambda st: self._backbone_decode_body_b(B_bucket, st))
+            self._g_slot_idx.copy_(saved_idx)
+            self._g_seq_inc.copy_(saved_inc)
+            self._bucketed_graphs[B_bucket] = g
+        g.replay()
+        return self._gc_hidden_out[:B_active], self._gc_cb0_out[:B_active], self._gc_eos_out[:B_active]
+
+    # ------------------------------------------------------------------ repetition penalty
+    def _setup_rep_state(self) -> None:
+        """Device-resident rolling counts (src/vui/engine.py:540-553); the ring position lives on the
+        device too so that the sampler can run inside a captured graph."""
+        N = self.max_rows
+        self._rep_counts = torch.zeros(N, self.CS, device=self.device, dtype=torch.float32)
+        self._rep_history: Tensor | None = None
+        self._rep_pos = torch.zeros(N, 2, device=self.device, dtype=torch.int32)
+        self._rep_window_cur = 0
+
+    def _rep_reset(self, penalty: float, window: int) -> None:
+        """src/vui/engine.py:555-569."""
+        self._rep_counts.zero_()
+        self._rep_pos.zero_()
+        if penalty <= 1.0:
+            return
+        if window > 0 and (self._rep_history is None or self._rep_window_cur != window):
+            self._rep_history = torch.zeros(self.max_rows, window, device=self.device, dtype=torch.int32)
+            self._rep_window_cur = window
+            self._frame_graphs = {}
+        elif window > 0:
+            self._rep_history.zero_()
+
+    def _sample_cb0(self, logits: Tensor, cfg: GenConfig, *, top_k: int | None = -1, frame_ctr: Tensor | None = None,
+                    out: Tensor | None = None) -> Tensor:
+        """Penalise (when cfg.rep_penalty > 1), sample and push: the three steps of
+        src/vui/engine.py:571-590 and 855-863 in one kernel.  (N, CS) -> (N,)."""
+        B = logits.shape[0]
+        nat = self.model._native
+        k = cfg.top_k if top_k == -1 else top_k
+        sp = make_sample_params(cfg.temperature, k, cfg.seed, frame_ctr if frame_ctr is not None else self._frame_ctr)
+        out = out if out is not None else torch.empty(B, dtype=torch.long, device=self.device)
+        use_rep = cfg.rep_penalty > 1.0
+        win = cfg.rep_window if (use_rep and self._rep_history is not None) else 0
+        _lib.check(nat.lib.vui_sample_cb0(
+            nat.handle, logits.contiguous().data_ptr(), self._rep_counts.data_ptr() if use_rep else None,
+            _lib.ptr(self._rep_history) if win else None, self._rep_pos.data_ptr() if win else None,
+            float(cfg.rep_penalty), win, C.byref(sp), out.data_ptr(), B, torch.cuda.current_stream().cuda_stream),
+            "vui_sample_cb0")
+        return out
+
+    # ------------------------------------------------------------------ rows
+    def new_row(self) -> Row:
+        if not self._free:
+            raise RuntimeError(f"No free rows (max_rows={self.max_rows} all in use)")
+        idx = min(self._free)
+        self._free.remove(idx)
+        row = Row(self, idx)
+        self._rows[idx] = row
+        self.seq_lens[idx] = 0
+        return row
+
+    def _release_row(self, row: Row) -> None:
+        self._rows.pop(row.idx, None)
+        self._free.add(row.idx)
+
+    def reset(self) -> None:
+        for row in list(self._rows.values()):
+            row.close()
+        self.seq_lens.zero_()
+
+    def _rewind_row(self, row: Row, offset: int) -> int:
+        """KV rewind = overwrite one int32; K/V beyond it are never cleared (engine.py:651-654)."""
+        self.seq_lens[row.idx] = offset
+        return offset
+
+    def _prefill_emb(self, row: Row, emb: Tensor) -> Tensor:
+        T = emb.shape[1]
+        if row.offset + T > self.max_seq:
+            raise ValueError(f"prefill of {T} positions at offset {row.offset} exceeds max_seq={self.max_seq}")
+        pos = torch.arange(row.offset, row.offset + T, device=self.device)
+        return self.model.decoder.forward_flash(emb.to(self.dtype), pos, slot_idx=row._slot)
+
+    def set_conditioning(self, *, sq_scores=None, wps_score: float = 0.0) -> None:
+        self.model.set_cond_bias(sq_scores=sq_scores, wps_score=wps_score)
+        self._cond_bias = self.model._cond_bias
+
+    # ------------------------------------------------------------------ fused frame loop
+    def _frame_graph(self, B: int, cfg: GenConfig, slot_idx: Tensor | None, max_frames: int):
+        """One HIP graph holding a whole frame: backbone step on the previous frame, code-0
+        sampling with repetition penalty, the depth head, frame log, counters."""
+        nq = cfg.n_codebooks if cfg.n_codebooks > 0 else self.Q
+        key = (B, nq, cfg.temperature, cfg.top_k, cfg.rq_top_k, cfg.rep_penalty, cfg.rep_window, cfg.seed,
+               None if slot_idx is None else tuple(slot_idx.tolist()), max_frames)
+        hit = self._frame_graphs.get(key)
+        if hit is not None:
+            return hit
+        nat = self.model._native
+        dec = self.model.decoder
+        frames = torch.zeros(max_frames, B, self.Q, dtype=torch.long, device=self.device)
+        eos = torch.zeros(max_frames, B, dtype=torch.float32, device=self.device)
+        sp0 = make_sample_params(cfg.temperature, cfg.top_k, cfg.seed, self._frame_ctr)
+        sp1 = make_sample_params(cfg.temperature, cfg.rq_top_k if cfg.top_k != 1 else 1, cfg.seed, self._frame_ctr)
+        use_rep = cfg.rep_penalty > 1.0
+        win = cfg.rep_window if (use_rep and self._rep_history is not None) else 0
+        codes_io = self._gc_codes_in if slot_idx is not None else self._g_codes_in
+        ns = self._splits(B)
+
+        def body(st):
+            _lib.check(nat.lib.vui_frame_step(
+                nat.handle, codes_io.data_ptr(), _lib.ptr(slot_idx), self.seq_lens.data_ptr(), None, B,
+                dec._k.data_ptr(), dec._v.data_ptr(), self._rep_counts.data_ptr() if use_rep else None,
+                _lib.ptr(self._rep_history) if win else None, self._rep_pos.data_ptr() if win else None,
+                float(cfg.rep_penalty), win, C.byref(sp0), C.byref(sp1), None, nq, self._g_hidden_out.data_ptr(),
+                self._g_cb0_out.data_ptr(), eos.data_ptr(), frames.data_ptr(), max_frames,
+                self._frame_ctr.data_ptr(), ns, st), "vui_frame_step")
+
+        # captured without a warm-up run: the step mutates seq_lens, the rep state and the counter
+        g = Graph(self.model, body, warmup=0)
+        entry = (g, frames, eos, (sp0, sp1, slot_idx))
+        self._frame_graphs[key] = entry
+        return entry
+
+    @torch.inference_mode()
+    def generate(self, rows: list[Row], first_hidden: Tensor, n_frames: int, cfg: GenConfig = GenConfig(),
+                 *, sync_every: int = 0) -> tuple[Tensor, Tensor]:
+        """Generate n_frames codec frames for the given rows, starting from the final-norm hidden
+        of each row's last prefill position (B, d).
+
+        Frame 0 follows src/vui/engine.py:1414-1433 (code 0 from codec_head(hidden), sampled without
+        top-k unless greedy; depth head; feed back); frames 1.. replay the one-graph frame step
+        (engine.py:1450-1485).  Returns (frames (n_frames, B, Q') int64, eos_prob (n_frames, B) fp32;
+        row 0 of eos_prob is 0).  EOS is reported, not acted on: the caller truncates."""
+        B = len(rows)
+        nq = cfg.n_codebooks if cfg.n_codebooks > 0 else self.Q
+        identity = [r.idx for r in rows] == list(range(B))
+        slot_idx = None if identity else torch.tensor([r.idx for r in rows], dtype=torch.int32, device=self.device)
+        codes_io = self._g_codes_in if identity else self._gc_codes_in
+        self._rep_reset(cfg.rep_penalty, cfg.rep_window)
+        self._frame_ctr.zero_()
+        # frame 0
+        cb0 = self.model.codec_head(first_hidden.to(self.dtype))
+        k0 = 1 if cfg.top_k == 1 else 0
+        code0 = self._sample_cb0(cb0, cfg, top_k=k0)
+        rq = self.model.rq_transformer
+        rq.seed = cfg.seed
+        sp1 = make_sample_params(cfg.temperature, cfg.rq_top_k if cfg.top_k != 1 else 1, cfg.seed, self._frame_ctr)
+        nat = self.model._native
+        _lib.check(nat.lib.vui_rq_generate(nat.handle, first_hidden.to(self.dtype).contiguous().data_ptr(),
+                                           code0.data_ptr(), None, nq, C.byref(sp1), codes_io.data_ptr(), self.Q, 1, B,
+                                           torch.cuda.current_stream().cuda_stream), "vui_rq_generate")
+        first = codes_io[:B, :nq].clone()
+        self._frame_ctr.fill_(1)
+        if n_frames <= 1:
+            return first[None], torch.zeros(1, B, device=self.device)
+        g, frames, eos, _ = self._frame_graph(B, cfg, slot_idx, max(n_frames, 1))
+        # the capture above ran nothing, state is as left by frame 0
+        frames[0, :, :nq] = first
+        for f in range(1, n_frames):
+            g.replay()
+            if sync_every and f % sync_every == 0:
+                torch.cuda.current_stream().synchronize()
+        torch.cuda.current_stream().synchronize()
+        return frames[:n_frames, :, :nq].clone(), eos[:n_frames].clone()
