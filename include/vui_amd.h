@@ -108,6 +108,20 @@ void vui_ctx_destroy(vui_ctx* ctx);
 /* One-time device-side initialisation of the workspace (zeroes counters).  Enqueued on stream. */
 int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream);
 
+/* The batch-1 bf16 calls below run as one persistent kernel ("fused") when the device can keep
+ * one workgroup per compute unit resident and the dimensions fit; otherwise, and for B > 1, fp32
+ * or int8 weights, as a sequence of kernels.  vui_ctx_fused(ctx, enable): enable = 1/0 switches the
+ * fused form on/off, -1 only queries; returns 1 when the fused form will be used, else 0 (then
+ * vui_last_error() says why it is unavailable).  No counterpart in the reference. */
+int vui_ctx_fused(vui_ctx* ctx, int enable);
+/* Synchronous health check: VUI_EHIP if a fused launch gave up waiting for another workgroup. */
+int vui_ctx_status(vui_ctx* ctx);
+
+/* Profiling aid: fused launches made after this call let workgroup `workgroup` write up to `cap`
+ * words (100 MHz clock << 8 | phase tag) into the device buffer buf (cap + 1 words, the last one
+ * receives the count); buf = NULL switches it off.  No counterpart in the reference. */
+int vui_debug_phase_clock(vui_ctx* ctx, uint64_t* buf, int cap, int workgroup);
+
 /* One backbone decode step for B rows (B <= max_batch).
  *   Engine._backbone_decode_body / _backbone_decode_body_b  (engine.py:434-449, 485-502)
  *   Vui._decode_step_inner                                  (model.py:1280-1287)

@@ -1,0 +1,187 @@
+"""Engine-level behaviour on the GPU: the one-graph frame loop against the oracle and against the
+step-by-step composition, batched/bucketed steps with slot indirection, int8 weights at batch 16."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import vui_oracle as O
+from tests.util import TINY_SD, make_model, rel_err, tiny_dims
+
+pytestmark = pytest.mark.gpu
+BF, F32 = torch.bfloat16, torch.float32
+
+
+def _engine(d, sd, dt, max_rows=1, S=None, int8=False):
+    from vui_amd.engine import Engine
+
+    m = make_model(d, sd, dt, int8=int8, max_seqlen=S or d.max_seqlen)
+    return m, Engine(model=m, max_rows=max_rows, max_seq=S or d.max_seqlen)
+
+
+@pytest.mark.parametrize("dt,fused", [(F32, 0), (BF, 0), (BF, 1)])
+def test_frame_loop_greedy_matches_oracle_tiny(dt, fused):
+    """Prefill + 10 greedy frames at reduced dims: token-exact against the oracle in fp32; in bf16 the
+    frames agree until the first near-tie, and the two GPU forms agree with each other exactly."""
+    from vui_amd.engine import GenConfig
+
+    d = tiny_dims(2)
+    sd = O.synthetic_state_dict(d, **TINY_SD)
+    m, eng = _engine(d, sd, dt)
+    assert m._native.fused(fused) == bool(fused and dt == BF)
+    ids = torch.tensor([3, 11, 42, 7, 19])
+    row = eng.new_row()
+    h = row.prefill_emb(m.token_emb(ids.cuda()[None]))[:, -1]
+    frames, eos = eng.generate([row], h, 10, GenConfig(temperature=1.0, top_k=1, rep_penalty=1.0))
+    m._native.status()
+    o = O.OracleModel(d, sd, dt)
+    ho = o.prefill(o.embed_text(ids))[-1:]
+    col = {}
+    ref = o.generate_frames(ho, 10, top_k=1, temperature=1.0, collect=col)[:, 0]
+    if dt == F32:
+        np.testing.assert_array_equal(frames[:, 0].cpu().numpy(), ref.numpy())
+        eos_ref = torch.sigmoid(torch.stack(col["eos"])[1:, 0, 0])
+        np.testing.assert_allclose(eos[1:, 0].cpu().numpy(), eos_ref.numpy(), rtol=1e-4, atol=1e-5)
+    else:
+        same = (frames[:, 0].cpu() == ref).all(dim=1)
+        assert bool(same[0]) and int(same.sum()) >= 5, same
+    assert int(eng.seq_lens[0]) == 5 + 9
+
+
+def test_frame_graph_equals_stepwise_composition():
+    """The fused frame graph reproduces decode_step + code-0 sampling + depth head called one by one
+    (same seeds): sampled tokens, rolling repetition counts and positions, over 12 frames."""
+    from vui_amd.engine import GenConfig
+
+    d = tiny_dims(2)
+    sd = O.synthetic_state_dict(d, **TINY_SD)
+    cfg = GenConfig(temperature=0.9, top_k=10, rq_top_k=10, rep_penalty=1.3, rep_window=4, seed=11)
+    ids = torch.tensor([1, 2, 3])
+    out = {}
+    for fused in (0, 1):
+        m, eng = _engine(d, sd, BF)
+        m._native.fused(fused)
+        row = eng.new_row()
+        h = row.prefill_emb(m.token_emb(ids.cuda()[None]))[:, -1]
+        frames, eos = eng.generate([row], h, 12, cfg)
+        m._native.status()
+        out[fused] = (frames.cpu(), eos.cpu(), eng._rep_counts.cpu().clone(), eng._rep_pos.cpu().clone())
+    assert torch.equal(out[0][0], out[1][0])
+    np.testing.assert_allclose(out[0][1].numpy(), out[1][1].numpy(), rtol=0, atol=0)
+    assert torch.equal(out[0][2], out[1][2]) and torch.equal(out[0][3], out[1][3])
+    # ring-buffer invariant: counts == histogram of the last `window` code-0 values (engine.py:930-934)
+    frames, _, counts, pos = out[1]
+    last = frames[-4:, 0, 0]
+    hist = torch.bincount(last, minlength=d.codebook_size).float()
+    assert torch.equal(counts[0], hist)
+    assert pos[0].tolist() == [12 % 4, 4]
+
+
+def test_sampled_frames_follow_oracle_distribution_tiny():
+    """Sampling (T=0.9, top-k 8): code 0 of frame 1 over 2000 seeds against the oracle's analytic kept
+    distribution (chi-square); every drawn code lies in the kept set."""
+    from vui_amd.engine import GenConfig
+
+    d = tiny_dims(2)
+    sd = O.synthetic_state_dict(d, **TINY_SD)
+    m, eng = _engine(d, sd, F32)
+    ids = torch.tensor([5, 6, 7])
+    row = eng.new_row()
+    h = row.prefill_emb(m.token_emb(ids.cuda()[None]))[:, -1]
+    row.mark_prompt()
+    o = O.OracleModel(d, sd, F32)
+    ho = o.prefill(o.embed_text(ids))[-1:]
+    cb0, _ = o.heads(ho)
+    w = O.cb0_probs(cb0[0], 0.9, 0)  # frame 0 draws code 0 without top-k (engine.py:1416-1424)
+    hist = np.zeros(d.codebook_size)
+    for seed in range(2000):
+        row.rewind()
+        frames, _ = eng.generate([row], h, 1, GenConfig(temperature=0.9, top_k=8, rep_penalty=1.0, seed=seed))
+        hist[int(frames[0, 0, 0])] += 1
+    exp = w / w.sum() * hist.sum()
+    keep = exp > 5
+    chi2 = (((hist - exp) ** 2)[keep] / exp[keep]).sum()
+    dof = int(keep.sum()) - 1
+    assert chi2 < dof + 5 * (2 * dof) ** 0.5, (chi2, dof)
+
+
+def test_batched_and_bucketed_steps():
+    """_decode_step over all rows and _bucketed_decode_step with slot indirection and a padding slot
+    (engine.py:434-534) give each row the same result as stepping it alone."""
+    d = tiny_dims(2)
+    sd = O.synthetic_state_dict(d, **TINY_SD)
+    m, eng = _engine(d, sd, BF, max_rows=4)
+    g = torch.Generator().manual_seed(2)
+    rows = [eng.new_row() for _ in range(4)]
+    for i, r in enumerate(rows):  # ragged prompts
+        ids = torch.randint(0, d.vocab_size, (2 + i,), generator=g).cuda()
+        r.prefill_emb(m.token_emb(ids[None]))
+    base = eng.seq_lens.clone()
+    assert base.tolist()[:4] == [2, 3, 4, 5]
+    codes = torch.randint(0, d.codebook_size, (4, d.n_quantizers), generator=g).cuda()
+    # all rows at once (short frame: zero padded, engine.py:473-479)
+    for i in range(4):
+        eng._set_codes_in(i, codes[i, :3])
+    hid, cb0, eos = eng._decode_step()
+    ref_h, ref_c = hid.clone(), cb0.clone()
+    assert eng.seq_lens.tolist() == [3, 4, 5, 6, 0]
+    # rows 3 and 1 only, through the bucket of 2 with slot indirection
+    eng.seq_lens.copy_(base)
+    eng._gc_codes_in.zero_()
+    eng._gc_codes_in[0, :3] = codes[3, :3]
+    eng._gc_codes_in[1, :3] = codes[1, :3]
+    eng._g_slot_idx[:2] = torch.tensor([3, 1], dtype=torch.int32)
+    eng._g_seq_inc.zero_()
+    eng._g_seq_inc[3] = 1
+    eng._g_seq_inc[1] = 1
+    h2, c2, e2 = eng._bucketed_decode_step(2)
+    assert torch.equal(h2[0], ref_h[3]) and torch.equal(h2[1], ref_h[1])
+    assert torch.equal(c2[0], ref_c[3]) and torch.equal(c2[1], ref_c[1])
+    assert eng.seq_lens.tolist() == [2, 4, 4, 6, 0]
+    # three active rows in the bucket of 4: the padding row writes to the padding slot only
+    eng.seq_lens.copy_(base)
+    eng._gc_codes_in.zero_()
+    for j, r in enumerate((0, 2, 3)):
+        eng._gc_codes_in[j, :3] = codes[r, :3]
+    eng._g_slot_idx[:3] = torch.tensor([0, 2, 3], dtype=torch.int32)
+    eng._g_seq_inc.zero_()
+    eng._g_seq_inc[[0, 2, 3]] = 1
+    h3, c3, _ = eng._bucketed_decode_step(3)
+    for j, r in enumerate((0, 2, 3)):
+        assert torch.equal(h3[j], ref_h[r]) and torch.equal(c3[j], ref_c[r])
+    assert eng.seq_lens.tolist() == [3, 3, 5, 6, 0]
+    with pytest.raises(RuntimeError, match="No free rows"):
+        eng.new_row()
+
+
+def test_int8_batch16_ragged_vs_oracle():
+    """BASELINE config 5 at full dims: 16 streams, ragged cache lengths in [128, 2048], backbone linears
+    as weight-only int8 (per-row scales): logits against the oracle evaluating the same int8 weights
+    (dequantise-then-matmul), tolerance 2^-5 * max|logit|."""
+    S = 2112
+    d = O.Dims()
+    sd = O.synthetic_state_dict(d, seed=0)
+    m = make_model(d, sd, BF, int8=True, max_seqlen=S)
+    B = 16
+    m.decoder.allocate_flash_kv_cache(B, m.device, BF, max_seqlen=S)
+    g = torch.Generator().manual_seed(0)
+    lens = torch.randint(128, 2049, (B,), generator=g)
+    check = [0, 7, 15]  # rows verified against the CPU oracle (each costs a full CPU step)
+    kc = O.rnd(0.5 * torch.randn(d.n_layers, B, S, d.n_kv_heads, d.head_dim, generator=g), BF)
+    vc = O.rnd(0.5 * torch.randn(d.n_layers, B, S, d.n_kv_heads, d.head_dim, generator=g), BF)
+    m.decoder._k.copy_(kc.to(BF))
+    m.decoder._v.copy_(vc.to(BF))
+    m.decoder.flash_kv_caches[0].seq_lens.copy_(lens.to(torch.int32))
+    codes = torch.randint(0, d.codebook_size, (B, d.n_quantizers), generator=g)
+    hid = torch.empty(B, d.d_model, dtype=BF, device="cuda")
+    cb0 = torch.empty(B, d.codebook_size, dtype=BF, device="cuda")
+    m.decoder._step(codes=codes.cuda(), emb=None, slot_idx=None, seq_inc=None, B=B, hidden_out=hid, cb0_out=cb0,
+                    eos_out=None, n_splits=4, stream=torch.cuda.current_stream().cuda_stream)
+    assert m.decoder.flash_kv_caches[0].seq_lens.cpu().tolist() == (lens + 1).tolist()
+    o = O.OracleModel(d, sd, BF, n_slots=1, max_seqlen=S, int8=True)
+    for b in check:
+        o.k_cache[:, 0] = kc[:, b]
+        o.v_cache[:, 0] = vc[:, b]
+        o.seq_lens[0] = int(lens[b])
+        h_ref, cb_ref, _ = o.decode_step(codes[b:b + 1])
+        assert rel_err(cb0[b:b + 1], cb_ref) <= 2.0 ** -5, (b, rel_err(cb0[b:b + 1], cb_ref))
+        assert rel_err(hid[b:b + 1], h_ref) <= 2.0 ** -5

@@ -121,8 +121,10 @@ def test_config1_greedy_grid_fp32():
 BF16_TOL = 2.0 ** -5  # stated bf16 tolerance: 8 bf16 ulps of the largest logit
 
 
-def test_nano_backbone_bf16_vs_oracle():
-    """One decode step at Vui Nano dims in bf16 at several cache lengths.
+@pytest.mark.parametrize("fused", [0, 1])
+def test_nano_backbone_bf16_vs_oracle(fused):
+    """One decode step at Vui Nano dims in bf16 at several cache lengths, as a sequence of kernels
+    (fused=0) and as the one persistent kernel (fused=1).
 
     With an empty cache the native step equals the oracle's bf16 regime bit for bit (same
     roundings, same per-row summation).  With a filled cache the attention sums run in another
@@ -135,6 +137,7 @@ def test_nano_backbone_bf16_vs_oracle():
     d, sd, m, o = _nano_models(BF, S=S)
     of = O.OracleModel(d, {k: O.rnd(v, BF) for k, v in sd.items()}, F32, max_seqlen=S)
     m.decoder.allocate_flash_kv_cache(1, m.device, BF, max_seqlen=S)
+    assert m._native.fused(fused) == bool(fused), "the fused kernel must be available on an MI355X"
     g = torch.Generator().manual_seed(3)
     for L in (0, 255, 1023):
         kc = O.rnd(torch.randn(d.n_layers, 1, S, d.n_kv_heads, d.head_dim, generator=g), BF)
@@ -155,7 +158,7 @@ def test_nano_backbone_bf16_vs_oracle():
         m.decoder._step(codes=codes.cuda(), emb=None, slot_idx=None, seq_inc=None, B=1, hidden_out=hid,
                         cb0_out=cb0, eos_out=eos, n_splits=32, stream=torch.cuda.current_stream().cuda_stream)
         assert int(m.decoder.flash_kv_caches[0].seq_lens[0]) == L + 1
-        if L == 0:
+        if L == 0 and not fused:
             assert torch.equal(cb0.float().cpu(), cb_ref) and torch.equal(hid.float().cpu(), h_ref)
             assert torch.equal(eos.float().cpu(), eos_ref)
         assert rel_err(cb0, cb_ref) <= BF16_TOL, (L, rel_err(cb0, cb_ref))
@@ -166,15 +169,22 @@ def test_nano_backbone_bf16_vs_oracle():
             assert int(cb0[0].float().argmax()) == int(cb_ref[0].argmax())
 
 
-def test_nano_rq_bf16_vs_oracle():
-    """Depth head at Vui Nano dims in bf16: teacher-forced logits within tolerance and greedy
-    tokens equal wherever the oracle's top-2 margin exceeds it."""
+@pytest.mark.parametrize("fused", [0, 1])
+def test_nano_rq_bf16_vs_oracle(fused):
+    """Depth head at Vui Nano dims in bf16: greedy tokens equal wherever the oracle's top-2 margin
+    exceeds the tolerance (batch of 4 through the kernel sequence; row by row through the fused kernel)."""
     d, sd, m, o = _nano_models(BF)
+    assert m._native.fused(fused) == bool(fused)
     g = torch.Generator().manual_seed(4)
     hidden = O.rnd(torch.randn(4, d.d_model, generator=g), BF)
     code0 = torch.randint(0, d.codebook_size, (4,), generator=g)
     ref, logits = o.rq_generate(hidden, code0, 1.0, 1, return_logits=True)
-    got = m.rq_transformer.generate(hidden.to(BF).cuda(), code0.cuda(), temperature=1.0, top_k=1).cpu()
+    hd_, c0_ = hidden.to(BF).cuda(), code0.cuda()
+    if fused:
+        got = torch.cat([m.rq_transformer.generate(hd_[b:b + 1], c0_[b:b + 1], temperature=1.0, top_k=1) for b in range(4)]).cpu()
+        m._native.status()
+    else:
+        got = m.rq_transformer.generate(hd_, c0_, temperature=1.0, top_k=1).cpu()
     tol = BF16_TOL
     for b in range(4):
         for i in range(d.n_quantizers - 1):

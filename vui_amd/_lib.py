@@ -59,6 +59,9 @@ SIGNATURES = {
     "vui_ctx_create": (_I, [C.POINTER(VuiConfigC), C.POINTER(WeightsC), _P, _L, _I, C.POINTER(_P)]),
     "vui_ctx_destroy": (None, [_P]),
     "vui_ctx_init": (_I, [_P, _P]),
+    "vui_ctx_fused": (_I, [_P, _I]),
+    "vui_ctx_status": (_I, [_P]),
+    "vui_debug_phase_clock": (_I, [_P, _P, _I, _I]),
     "vui_backbone_step": (_I, [_P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _P]),
     "vui_sample_cb0": (_I, [_P, _P, _P, _P, _P, _F, _I, C.POINTER(SampleParamsC), _P, _I, _P]),
     "vui_rq_generate": (_I, [_P, _P, _P, _P, _I, C.POINTER(SampleParamsC), _P, _I, _I, _I, _P]),

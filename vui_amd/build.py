@@ -9,7 +9,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libvui_amd.so")
-SOURCES = ["gemv.hip", "attn.hip", "misc.hip", "api.hip"]
+SOURCES = ["gemv.hip", "attn.hip", "misc.hip", "frame.hip", "api.hip"]
 FLAGS = [
     "-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
     # packed-fp32 instructions are kept out of every code object of this library
@@ -27,12 +27,13 @@ def _hipcc() -> str:
 def build(verbose: bool = True) -> str:
     """Compiles every translation unit and links the shared library.  Always recompiles."""
     hipcc = _hipcc()
+    extra = os.environ.get("VUI_EXTRA_HIPCC_FLAGS", "").split()
     objdir = os.path.join(CSRC, "build")
     os.makedirs(objdir, exist_ok=True)
 
     def one(src: str) -> str:
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        cmd = [hipcc, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed on {src}:\n{r.stdout}\n{r.stderr}")
@@ -42,7 +43,7 @@ def build(verbose: bool = True) -> str:
                 print("\n".join(lines), file=sys.stderr)
         return obj
 
-    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as ex:
+    with ThreadPoolExecutor(max_workers=min(5, len(SOURCES))) as ex:
         objs = list(ex.map(one, SOURCES))
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)

@@ -31,7 +31,20 @@ struct vui_ctx {
   void *rx, *rq_q, *rq_att, *rq_h, *rq_kc, *rq_vc, *rq_logits;
   int64_t* code0;
   float* eos_prob;
+  // fused frame kernel
+  uint64_t* ll;
+  size_t ll_words;
+  vui_weights* wdev;
+  uint32_t* ctl;  // [0] epoch, [1] arrive, [2] err
+  int fused_ok, fused_on, nwg, ns;
+  size_t lds_bytes;
+  char fused_why[96];
+  uint64_t* prof;
+  int prof_cap, prof_wg;
 };
+
+#define FUSED_NWG 256
+#define FUSED_NS 32
 
 struct Carve {
   size_t off = 0;
@@ -87,6 +100,9 @@ static size_t carve(const vui_config* c, int Bm, vui_ctx* x) {
   TAKE(rq_logits, void*, (size_t)Bm * c->codebook_size * e);
   TAKE(code0, int64_t*, Bm * 8);
   TAKE(eos_prob, float*, Bm * 4);
+  TAKE(ll, uint64_t*, frame_ll_words(*c, FUSED_NS) * 8);
+  TAKE(wdev, vui_weights*, sizeof(vui_weights));
+  TAKE(ctl, uint32_t*, 256);
 #undef TAKE
   return cv.off;
 }
@@ -136,6 +152,8 @@ int vui_ctx_create(const vui_config* cfg, const vui_weights* w, void* workspace,
   c->max_batch = max_batch;
   c->esz = cfg->dtype == VUI_DTYPE_F32 ? 4 : 2;
   c->base = (char*)workspace;
+  c->fused_ok = 0; c->fused_on = 1; c->fused_why[0] = 0;
+  c->prof = nullptr; c->prof_cap = 0; c->prof_wg = 0;
   carve(cfg, max_batch, c);
   *out = c;
   return VUI_OK;
@@ -145,8 +163,63 @@ void vui_ctx_destroy(vui_ctx* ctx) { delete ctx; }
 
 int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream) {
   if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
-  return launch_fill_u32(ctx->counter, 0u, (int64_t)ctx->max_batch * ctx->cfg.n_heads, (hipStream_t)stream);
+  hipStream_t st = (hipStream_t)stream;
+  int rc = launch_fill_u32(ctx->counter, 0u, (int64_t)ctx->max_batch * ctx->cfg.n_heads, st);
+  if (rc) return rc;
+  // fused frame kernel: exchange words and control words start at zero (epoch 0 = "never written")
+  ctx->ll_words = frame_ll_words(ctx->cfg, FUSED_NS);
+  if ((rc = launch_fill_u32((uint32_t*)ctx->ll, 0u, (int64_t)ctx->ll_words * 2, st))) return rc;
+  if ((rc = launch_fill_u32(ctx->ctl, 0u, 64, st))) return rc;
+  HIP_TRY(hipMemcpyAsync(ctx->wdev, &ctx->w, sizeof(vui_weights), hipMemcpyHostToDevice, st));
+  HIP_TRY(hipStreamSynchronize(st));
+  ctx->fused_ok = 0;
+  ctx->fused_why[0] = 0;
+  ctx->ns = FUSED_NS;
+  ctx->lds_bytes = frame_lds_bytes(ctx->cfg);
+  int n_cu = 0;
+  ctx->nwg = FUSED_NWG;
+  if (frame_supported(ctx->cfg, ctx->nwg, ctx->ns, ctx->fused_why, sizeof(ctx->fused_why))) {
+    const int cap = frame_max_resident(ctx->lds_bytes, &n_cu);
+    if (cap < 0) return cap;
+    if (cap >= ctx->nwg) ctx->fused_ok = 1;
+    else snprintf(ctx->fused_why, sizeof(ctx->fused_why), "only %d workgroups can be resident (%d CUs), %d needed", cap, n_cu, ctx->nwg);
+  }
+  return VUI_OK;
 }
+
+int vui_ctx_fused(vui_ctx* ctx, int enable) {
+  if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
+  if (enable >= 0) ctx->fused_on = enable ? 1 : 0;
+  if (!ctx->fused_ok && ctx->fused_why[0]) vui_set_error("fused frame kernel unavailable: %s", ctx->fused_why);
+  return (ctx->fused_ok && ctx->fused_on) ? 1 : 0;
+}
+
+int vui_debug_phase_clock(vui_ctx* ctx, uint64_t* buf, int cap, int workgroup) {
+  if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
+  ctx->prof = buf; ctx->prof_cap = buf ? cap : 0; ctx->prof_wg = workgroup;
+  return VUI_OK;
+}
+
+int vui_ctx_status(vui_ctx* ctx) {
+  if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
+  uint32_t h[4] = {0, 0, 0, 0};
+  HIP_TRY(hipMemcpy(h, ctx->ctl, sizeof(h), hipMemcpyDeviceToHost));
+  if (h[2]) { vui_set_error("fused frame kernel: an exchange wait timed out (epoch %u)", h[0]); return VUI_EHIP; }
+  return VUI_OK;
+}
+
+static void fused_base(vui_ctx* ctx, FrameArgs& a) {
+  const vui_config& c = ctx->cfg;
+  memset(&a, 0, sizeof(a));
+  a.d = c.d_model; a.L = c.n_layers; a.H = c.n_heads; a.KV = c.n_kv_heads; a.hd = c.head_dim; a.F = c.ffn;
+  a.Q = c.n_quantizers; a.CS = c.codebook_size; a.R = c.rq_dim; a.rqL = c.rq_layers; a.rqH = c.rq_heads; a.rqF = c.rq_ffn;
+  a.rope_dim = c.rope_dim; a.S = c.max_seqlen; a.window = c.window; a.eps = c.norm_eps; a.rq_eps = c.rq_norm_eps;
+  a.w = ctx->wdev; a.n_slots = c.n_slots;
+  a.ll = ctx->ll; a.epoch = ctx->ctl; a.arrive = ctx->ctl + 1; a.err = ctx->ctl + 2;
+  a.prof = ctx->prof; a.prof_cap = ctx->prof_cap; a.prof_wg = ctx->prof_wg;
+  a.ns = ctx->ns; a.lds_kv_off = (int)(ctx->lds_bytes - (size_t)c.rq_layers * c.n_quantizers * 2 * c.rq_dim * 2);
+}
+static bool use_fused(vui_ctx* ctx, int B) { return ctx->fused_ok && ctx->fused_on && B == 1; }
 
 static int check_batch(vui_ctx* ctx, int B, int n_splits) {
   if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
@@ -164,6 +237,17 @@ int vui_backbone_step(vui_ctx* ctx, const int64_t* codes_in, const void* emb_in,
   if (!seq_lens || !k_cache || !v_cache) { vui_set_error("seq_lens and the KV caches are required"); return VUI_EINVAL; }
   const vui_config& c = ctx->cfg;
   hipStream_t st = (hipStream_t)stream;
+  if (use_fused(ctx, B)) {
+    FrameArgs a;
+    fused_base(ctx, a);
+    a.mode = FR_BACKBONE;
+    a.codes_in = codes_in; a.emb_in = (const uint16_t*)emb_in; a.slot_idx = slot_idx; a.seq_lens = seq_lens; a.seq_inc = seq_inc;
+    a.kc = (uint16_t*)k_cache; a.vc = (uint16_t*)v_cache;
+    a.hidden_out = (uint16_t*)(hidden_out ? hidden_out : ctx->hidden);
+    a.cb0_out = (uint16_t*)(cb0_out ? cb0_out : ctx->cb0);
+    a.eos_out = (uint16_t*)(eos_out ? eos_out : ctx->eos);
+    return launch_frame(a, ctx->nwg, ctx->lds_bytes, st);
+  }
   const int d = c.d_model, H = c.n_heads, KV = c.n_kv_heads, hd = c.head_dim;
   if (codes_in) rc = launch_embed(c.dtype, codes_in, ctx->w.audio_emb, ctx->x, B, c.n_quantizers, c.codebook_size, d, st);
   else rc = launch_copy_rows(c.dtype, emb_in, ctx->x, (int64_t)B * d, st);
@@ -292,6 +376,15 @@ int vui_rq_generate(vui_ctx* ctx, const void* hidden, const int64_t* code0, cons
   if (!hidden || !code0 || !sp || !codes_out) { vui_set_error("NULL argument"); return VUI_EINVAL; }
   if (n_q < 2 || n_q > c.n_quantizers || codes_stride < n_q) { vui_set_error("n_q=%d outside [2,%d] or stride %d too small", n_q, c.n_quantizers, codes_stride); return VUI_EINVAL; }
   hipStream_t st = (hipStream_t)stream;
+  if (use_fused(ctx, B)) {
+    FrameArgs a;
+    fused_base(ctx, a);
+    a.mode = FR_RQ;
+    a.rq_hidden = (const uint16_t*)hidden; a.rq_code0 = code0; a.logit_bias = logit_bias; a.n_q = n_q;
+    a.temp1 = sp->temperature; a.topk1 = sp->top_k; a.seed1 = sp->seed; a.frame_ctr1 = sp->frame_ctr;
+    a.codes_out = codes_out; a.codes_stride = codes_stride; a.zero_pad = zero_pad;
+    return launch_frame(a, ctx->nwg, ctx->lds_bytes, st);
+  }
   const int R = c.rq_dim, CS = c.codebook_size;
   const char* pos_emb = (const char*)ctx->w.rq_pos_emb;
   const size_t rowb = (size_t)R * ctx->esz;
@@ -346,6 +439,24 @@ int vui_frame_step(vui_ctx* ctx, int64_t* codes_io, const int32_t* slot_idx, int
   hipStream_t st = (hipStream_t)stream;
   void* hid = hidden_out ? hidden_out : ctx->hidden;
   void* cb0 = cb0_out ? cb0_out : ctx->cb0;
+  if (window > 0 && rep_counts && penalty > 1.0f && (!rep_hist || !rep_pos)) { vui_set_error("a repetition window needs rep_hist and rep_pos"); return VUI_EINVAL; }
+  if (n_q < 2 || n_q > c.n_quantizers) { vui_set_error("n_q=%d outside [2,%d]", n_q, c.n_quantizers); return VUI_EINVAL; }
+  if (use_fused(ctx, B)) {
+    if (!seq_lens || !k_cache || !v_cache) { vui_set_error("seq_lens and the KV caches are required"); return VUI_EINVAL; }
+    FrameArgs a;
+    fused_base(ctx, a);
+    a.mode = FR_BACKBONE | FR_CB0 | FR_RQ | FR_FINISH;
+    a.codes_in = codes_io; a.slot_idx = slot_idx; a.seq_lens = seq_lens; a.seq_inc = seq_inc;
+    a.kc = (uint16_t*)k_cache; a.vc = (uint16_t*)v_cache;
+    a.hidden_out = (uint16_t*)hid; a.cb0_out = (uint16_t*)cb0; a.eos_out = (uint16_t*)ctx->eos;
+    a.rep_counts = rep_counts; a.rep_hist = rep_hist; a.rep_pos = rep_pos; a.penalty = penalty; a.rep_window = window;
+    a.temp0 = sp_cb0->temperature; a.topk0 = sp_cb0->top_k; a.seed0 = sp_cb0->seed; a.frame_ctr0 = sp_cb0->frame_ctr;
+    a.temp1 = sp_rq->temperature; a.topk1 = sp_rq->top_k; a.seed1 = sp_rq->seed; a.frame_ctr1 = sp_rq->frame_ctr;
+    a.code0_out = ctx->code0; a.logit_bias = logit_bias; a.n_q = n_q;
+    a.codes_out = codes_io; a.codes_stride = c.n_quantizers; a.zero_pad = 1;
+    a.frames_out = frames_out; a.eos_prob_out = eos_prob_out; a.max_frames = max_frames; a.frame_ctr = frame_ctr;
+    return launch_frame(a, ctx->nwg, ctx->lds_bytes, st);
+  }
   if ((rc = vui_backbone_step(ctx, codes_io, nullptr, slot_idx, seq_lens, seq_inc, B, k_cache, v_cache, hid, cb0,
                               ctx->eos, n_splits, stream)))
     return rc;

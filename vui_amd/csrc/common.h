@@ -63,26 +63,60 @@ __device__ __forceinline__ void ld8_i8(const int8_t* p, float* o) {
   o[6] = (float)(int8_t)((r.y >> 16) & 0xff); o[7] = (float)(int8_t)(r.y >> 24);
 }
 
+// ---- wave64 reductions on the DPP data path (no LDS crossbar traffic) ----
+// Within a row of 16 lanes: quad xor-1, quad xor-2, half-row mirror, row mirror leave the row
+// total in every lane of the row; the four row totals are then read as scalars and added.
+#define DPP_QUAD_XOR1 0xB1   // quad_perm [1,0,3,2]
+#define DPP_QUAD_XOR2 0x4E   // quad_perm [2,3,0,1]
+#define DPP_ROW_HALF_MIRROR 0x141
+#define DPP_ROW_MIRROR 0x140
+
+template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template <int CTRL> __device__ __forceinline__ int dpp_i(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
+__device__ __forceinline__ float lane_f(float v, int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l)); }
+
+// sum within aligned groups of 16 lanes (every lane of the group gets it)
+__device__ __forceinline__ float group16_sum(float v) {
+  v += dpp_f<DPP_QUAD_XOR1>(v);
+  v += dpp_f<DPP_QUAD_XOR2>(v);
+  v += dpp_f<DPP_ROW_HALF_MIRROR>(v);
+  v += dpp_f<DPP_ROW_MIRROR>(v);
+  return v;
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  v = group16_sum(v);
+  return (lane_f(v, 0) + lane_f(v, 16)) + (lane_f(v, 32) + lane_f(v, 48));
+}
+__device__ __forceinline__ float group16_max(float v) {
+  v = fmaxf(v, dpp_f<DPP_QUAD_XOR1>(v));
+  v = fmaxf(v, dpp_f<DPP_QUAD_XOR2>(v));
+  v = fmaxf(v, dpp_f<DPP_ROW_HALF_MIRROR>(v));
+  v = fmaxf(v, dpp_f<DPP_ROW_MIRROR>(v));
   return v;
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
-  return v;
+  v = group16_max(v);
+  return fmaxf(fmaxf(lane_f(v, 0), lane_f(v, 16)), fmaxf(lane_f(v, 32), lane_f(v, 48)));
 }
 __device__ __forceinline__ int wave_sum_i(int v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
-  return v;
+  v += dpp_i<DPP_QUAD_XOR1>(v);
+  v += dpp_i<DPP_QUAD_XOR2>(v);
+  v += dpp_i<DPP_ROW_HALF_MIRROR>(v);
+  v += dpp_i<DPP_ROW_MIRROR>(v);
+  return (__builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16)) +
+         (__builtin_amdgcn_readlane(v, 32) + __builtin_amdgcn_readlane(v, 48));
 }
-// sum within aligned groups of 16 lanes
-__device__ __forceinline__ float group16_sum(float v) {
-#pragma unroll
-  for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
-  return v;
+__device__ __forceinline__ int wave_min_i(int v) {
+  v = min(v, dpp_i<DPP_QUAD_XOR1>(v));
+  v = min(v, dpp_i<DPP_QUAD_XOR2>(v));
+  v = min(v, dpp_i<DPP_ROW_HALF_MIRROR>(v));
+  v = min(v, dpp_i<DPP_ROW_MIRROR>(v));
+  return min(min(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16)),
+             min(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
 }
 
 // a*c + b*s with both products rounded before the add (the reference multiplies and adds as

@@ -1,0 +1,1035 @@
+// The whole per-frame step of one stream as ONE persistent kernel (batch 1, bf16).
+//
+// On this GPU a dependent kernel boundary costs 4-5 us (every boundary writes back and
+// invalidates the eight per-XCD L2s) and a frame is a chain of ~400 dependent small GEMVs, so
+// the chain is run inside one resident grid instead: one workgroup per CU, every workgroup
+// walks the same phase list, owns a fixed slice of each weight matrix and keeps the residual
+// stream redundantly in LDS.  Between phases the workgroups exchange the small activation
+// vectors through "flag-in-data" words: an 8-byte word = 4 bytes of payload (two bf16 or one
+// fp32) + the 4-byte launch epoch, written and polled with device-scope relaxed atomics, which
+// bypass the non-coherent L2s.  A consumer that sees the current epoch has the data: no barrier,
+// no cache flush.  Weight loads of a phase are issued before its poll, so HBM latency overlaps
+// the wait.  Every phase has its own word buffer, so nothing is reused within a launch.
+//
+// Arithmetic and rounding points are those of the per-kernel path (gemv.hip / attn.hip /
+// sample.h), i.e. of the reference: src/vui/model.py:204-258, 282-297, 359-375 (backbone block),
+// :908-986 (depth head), src/vui/engine.py:434-449, 571-590, 855-863, 1450-1485 (frame loop).
+#include "common.h"
+#include "internal.h"
+#include "sample.h"
+#include <stdio.h>
+
+#define FR_THREADS 256
+#define SPIN_LIMIT (1 << 21)
+
+__device__ __forceinline__ uint64_t ll_ld(const uint64_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void ll_st(uint64_t* p, uint32_t payload, uint32_t epoch) {
+  __hip_atomic_store(p, ((uint64_t)epoch << 32) | payload, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t pack2(float a, float b) { return (uint32_t)f2bf(a) | ((uint32_t)f2bf(b) << 16); }
+
+struct Ctl {
+  uint32_t epoch;
+  uint32_t* err;
+  int dead;
+};
+
+// Wait until words [0, n) of buf carry the current epoch; sink(i, payload) once per word.
+// Threads take words tid, tid+256, ...  A thread that exceeds the spin limit raises the error
+// word and stops waiting for the rest of the launch, so every wave always reaches the end.
+template <typename F>
+__device__ __forceinline__ void ll_poll(const uint64_t* buf, int n, Ctl& c, F&& sink) {
+  for (int base = 0; base < n; base += FR_THREADS * 4) {
+    int idx[4];
+    bool ok[4];
+    uint64_t v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { idx[i] = base + (int)threadIdx.x + FR_THREADS * i; ok[i] = idx[i] >= n; }
+    int spins = 0;
+    while (true) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) if (!ok[i]) v[i] = ll_ld(buf + idx[i]);
+      bool all = true;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (!ok[i]) {
+          if ((uint32_t)(v[i] >> 32) == c.epoch || c.dead) { ok[i] = true; sink(idx[i], (uint32_t)v[i]); }
+          else all = false;
+        }
+      if (all) break;
+      if (++spins > SPIN_LIMIT) {
+        c.dead = 1;
+        __hip_atomic_store(c.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+  }
+}
+
+// ---- per-workgroup slice of a GEMV: adjacent row pairs, dealt round-robin over workgroups ----
+struct Plan {
+  int np;      // row pairs of this workgroup
+  int KS;      // waves sharing one pair along K (1, 2 or 4)
+  int kpart;   // this wave's K part
+  int nslots;  // pairs this wave works on (<= 2)
+  int gp[2];   // their global pair indices
+  int c0, c1;  // this wave's 8-element chunk range of K
+};
+
+// row pairs of workgroup wg when pairs are dealt round-robin (the one division per phase type)
+__device__ __forceinline__ int pairs_of(int npairs, int wg, int nwg) {
+  return (npairs > wg) ? (npairs - wg + nwg - 1) / nwg : 0;
+}
+// the rest of the plan costs a few shifts, so it is rebuilt at each use instead of being kept live
+__device__ __forceinline__ Plan plan_of(int np, int K, int wg, int nwg, int wave) {
+  Plan p;
+  p.np = np;
+  p.KS = np >= 3 ? 1 : (np == 2 ? 2 : (np == 1 ? 4 : 1));
+  const int nch = K >> 3;
+  if (p.KS == 1) {
+    p.kpart = 0;
+    p.nslots = (wave < np ? 1 : 0) + (wave + 4 < np ? 1 : 0);
+    p.gp[0] = wg + wave * nwg;
+    p.gp[1] = wg + (wave + 4) * nwg;
+    p.c0 = 0; p.c1 = nch;
+  } else {
+    const int sh = p.KS == 2 ? 1 : 2;
+    const int li = wave >> sh;
+    p.kpart = wave & (p.KS - 1);
+    p.nslots = 1;
+    p.gp[0] = wg + li * nwg;
+    p.gp[1] = p.gp[0];
+    const int per = (nch + p.KS - 1) >> sh;
+    p.c0 = p.kpart * per;
+    p.c1 = min(nch, p.c0 + per);
+  }
+  return p;
+}
+__device__ __forceinline__ Plan make_plan(int npairs, int K, int wg, int nwg, int wave) {
+  return plan_of(pairs_of(npairs, wg, nwg), K, wg, nwg, wave);
+}
+
+template <int MAXC, bool DUAL>
+struct WRegs {
+  uint4 a[2][2][MAXC];
+  uint4 b[DUAL ? 2 : 1][DUAL ? 2 : 1][DUAL ? MAXC : 1];
+};
+
+__device__ __forceinline__ void cvt8(const uint4& r, float* o) {
+  o[0] = __uint_as_float(r.x << 16); o[1] = __uint_as_float(r.x & 0xffff0000u);
+  o[2] = __uint_as_float(r.y << 16); o[3] = __uint_as_float(r.y & 0xffff0000u);
+  o[4] = __uint_as_float(r.z << 16); o[5] = __uint_as_float(r.z & 0xffff0000u);
+  o[6] = __uint_as_float(r.w << 16); o[7] = __uint_as_float(r.w & 0xffff0000u);
+}
+
+template <int MAXC, bool DUAL>
+__device__ __forceinline__ void gemv_prefetch(const bf16_t* W, const bf16_t* W2, int K, const Plan& p,
+                                              WRegs<MAXC, DUAL>& r) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int rr = 0; rr < 2; ++rr)
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int c = p.c0 + lane + WAVE * i;
+        const bool on = s < p.nslots && c < p.c1;
+        const size_t off = ((size_t)(2 * p.gp[s] + rr)) * K + (size_t)c * 8;
+        r.a[s][rr][i] = on ? *reinterpret_cast<const uint4*>(W + off) : make_uint4(0, 0, 0, 0);
+        if (DUAL) r.b[s][rr][i] = on ? *reinterpret_cast<const uint4*>(W2 + off) : make_uint4(0, 0, 0, 0);
+      }
+}
+
+// xs: K staged activations in LDS (fp32).  red: 4 x 4 floats of LDS.  epi(gp, v0, v1, u0, u1) is
+// called by one lane per finished pair with the fp32 dot products of rows 2gp, 2gp+1 (u*: second matrix).
+template <int MAXC, bool DUAL, typename Epi>
+__device__ __forceinline__ void gemv_compute(const float* xs, const Plan& p, const WRegs<MAXC, DUAL>& r, float* red,
+                                             Epi&& epi) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float res[2][4];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    if (s < p.nslots) {
+#pragma unroll
+      for (int i = 0; i < MAXC; ++i) {
+        const int c = p.c0 + lane + WAVE * i;
+        if (c < p.c1) {
+          const float4 xa = *reinterpret_cast<const float4*>(xs + c * 8);
+          const float4 xb = *reinterpret_cast<const float4*>(xs + c * 8 + 4);
+          const float xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+#pragma unroll
+          for (int rr = 0; rr < 2; ++rr) {
+            float w[8];
+            cvt8(r.a[s][rr][i], w);
+            float t = acc[rr];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) t = fmaf(w[e], xv[e], t);
+            acc[rr] = t;
+            if (DUAL) {
+              cvt8(r.b[s][rr][i], w);
+              float t2 = acc[2 + rr];
+#pragma unroll
+              for (int e = 0; e < 8; ++e) t2 = fmaf(w[e], xv[e], t2);
+              acc[2 + rr] = t2;
+            }
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < (DUAL ? 4 : 2); ++j) res[s][j] = (s < p.nslots) ? wave_sum(acc[j]) : 0.f;
+    if (!DUAL) res[s][2] = res[s][3] = 0.f;
+  }
+  if (p.KS > 1) {  // uniform over the workgroup
+    if (lane == 0) { red[wave * 4 + 0] = res[0][0]; red[wave * 4 + 1] = res[0][1]; red[wave * 4 + 2] = res[0][2]; red[wave * 4 + 3] = res[0][3]; }
+    __syncthreads();
+    if (p.kpart == 0 && lane == 0) {
+      float t[4] = {0.f, 0.f, 0.f, 0.f};
+      for (int k = 0; k < p.KS; ++k)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) t[j] += red[(wave + k) * 4 + j];
+      epi(p.gp[0], t[0], t[1], t[2], t[3]);
+    }
+  } else if (lane == 0) {
+    if (p.nslots > 0) epi(p.gp[0], res[0][0], res[0][1], res[0][2], res[0][3]);
+    if (p.nslots > 1) epi(p.gp[1], res[1][0], res[1][1], res[1][2], res[1][3]);
+  }
+}
+
+// norm weights of a thread's features (k = tid, tid+256, ...), fetched ahead of the wait
+struct NormW { float w[4]; };
+__device__ __forceinline__ NormW load_normw(const bf16_t* nw, int K) {
+  NormW r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int k = (int)threadIdx.x + FR_THREADS * i;
+    r.w[i] = k < K ? bf2f(nw[k]) : 0.f;
+  }
+  return r;
+}
+// two-rounding RMSNorm of src[0..K) (LDS, K <= 1024) into dst (LDS); every wave derives the same scale
+__device__ __forceinline__ void stage_norm(const float* src, const NormW& nw, float eps, int K, float* dst) {
+  const int lane = threadIdx.x & 63;
+  float ss = 0.f;
+  for (int k = lane; k < K; k += WAVE) { const float v = src[k]; ss += v * v; }
+  ss = wave_sum(ss);
+  const float r = 1.0f / sqrtf(ss / (float)K + eps);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int k = (int)threadIdx.x + FR_THREADS * i;
+    if (k < K) {
+      const float v = bf2f(f2bf(src[k] * r));
+      dst[k] = bf2f(f2bf(v * nw.w[i]));
+    }
+  }
+}
+
+// Exchange helpers: wait for a vector of bf16 pairs and put it into LDS.  Both carry the
+// workgroup barriers that separate them from earlier readers and later users of dst.
+__device__ __forceinline__ void poll_set(float* dst, const uint64_t* buf, int nwords, Ctl& c) {
+  __syncthreads();
+  ll_poll(buf, nwords, c, [&](int i, uint32_t v) {
+    dst[2 * i] = bf2f((bf16_t)(v & 0xffff)); dst[2 * i + 1] = bf2f((bf16_t)(v >> 16)); });
+  __syncthreads();
+}
+// dst = rnd(dst + incoming): the residual add (src/vui/model.py:367, 374)
+__device__ __forceinline__ void poll_add(float* dst, const uint64_t* buf, int nwords, Ctl& c) {
+  __syncthreads();
+  ll_poll(buf, nwords, c, [&](int i, uint32_t v) {
+    dst[2 * i] = bf2f(f2bf(dst[2 * i] + bf2f((bf16_t)(v & 0xffff))));
+    dst[2 * i + 1] = bf2f(f2bf(dst[2 * i + 1] + bf2f((bf16_t)(v >> 16)))); });
+  __syncthreads();
+}
+
+// fixed LDS carve-up (bytes)
+#define LDS_XRES 0                       // 1024 floats: residual stream
+#define LDS_XN (LDS_XRES + 4096)         // 2048 floats: staged GEMV input / attention scratch
+#define LDS_LG (LDS_XN + 8192)           // 2048 floats: logits
+#define LDS_SC (LDS_LG + 8192)           // 1024 floats: attention scores of one split
+#define LDS_QKV (LDS_SC + 4096)          // 3 x 128 floats: q, new k, new v of one head
+#define LDS_RED (LDS_QKV + 1536)         // 64 floats
+#define LDS_MISC (LDS_RED + 256)         // 64 ints: sampled codes of the frame
+#define LDS_SAMP (LDS_MISC + 256)        // SampleShared
+#define LDS_FIXED (LDS_SAMP + 192)
+
+// optional per-phase timestamps (100 MHz wall clock) written by one workgroup, for profiling
+#define TS(id)                                                                                    \
+  do {                                                                                            \
+    if (a.prof && wg == a.prof_wg && tid == 0 && nts < a.prof_cap) a.prof[nts++] = (wall_clock64() << 8) | (uint64_t)(id); \
+  } while (0)
+
+struct LayerP { const bf16_t *attn_norm, *wqkv, *wo, *mlp_norm, *w1, *w3, *w2; };
+
+// wait for up to 3 scattered words per thread (nullptr = none); returns payloads
+__device__ __forceinline__ void poll3(const uint64_t* p0, const uint64_t* p1, const uint64_t* p2, Ctl& c, uint32_t& r0,
+                                      uint32_t& r1, uint32_t& r2) {
+  bool k0 = p0 == nullptr, k1 = p1 == nullptr, k2 = p2 == nullptr;
+  uint64_t v0 = 0, v1 = 0, v2 = 0;
+  int spins = 0;
+  while (true) {
+    if (!k0) v0 = ll_ld(p0);
+    if (!k1) v1 = ll_ld(p1);
+    if (!k2) v2 = ll_ld(p2);
+    if (!k0 && ((uint32_t)(v0 >> 32) == c.epoch || c.dead)) k0 = true;
+    if (!k1 && ((uint32_t)(v1 >> 32) == c.epoch || c.dead)) k1 = true;
+    if (!k2 && ((uint32_t)(v2 >> 32) == c.epoch || c.dead)) k2 = true;
+    if (k0 && k1 && k2) break;
+    if (++spins > SPIN_LIMIT) { c.dead = 1; __hip_atomic_store(c.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+    __builtin_amdgcn_s_sleep(1);
+  }
+  r0 = (uint32_t)v0; r1 = (uint32_t)v1; r2 = (uint32_t)v2;
+}
+
+__global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* xres = (float*)(smem + LDS_XRES);
+  float* xn = (float*)(smem + LDS_XN);
+  float* lg = (float*)(smem + LDS_LG);
+  float* sc = (float*)(smem + LDS_SC);
+  float* qh = (float*)(smem + LDS_QKV);
+  float* red = (float*)(smem + LDS_RED);
+  int* codes_l = (int*)(smem + LDS_MISC);
+  SampleShared& ssh = *(SampleShared*)(smem + LDS_SAMP);
+  LayerP* lp = (LayerP*)(smem + LDS_FIXED);          // backbone layers, then depth-head layers
+  bf16_t* rqkv = (bf16_t*)(smem + a.lds_kv_off);
+
+  const int wg = blockIdx.x, nwg = gridDim.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  Ctl c;
+  c.epoch = __hip_atomic_load(a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+  c.err = a.err;
+  c.dead = 0;
+  const uint32_t ep = c.epoch;
+  uint64_t* llp = a.ll;
+  const vui_weights& W = *a.w;
+  const int d = a.d;
+  int code0 = 0;
+  float eos_logit = 0.f;
+  const uint32_t frame0 = a.frame_ctr0 ? (uint32_t)a.frame_ctr0[0] : 0u;
+  const uint32_t frame1 = a.frame_ctr1 ? (uint32_t)a.frame_ctr1[0] : 0u;
+  int slot = 0, pos = 0;
+  int nts = 0;
+  TS(0);
+
+  // weight pointer tables into LDS (one pass, so no phase waits on a pointer load later)
+  for (int i = tid; i < a.L + a.rqL; i += FR_THREADS) {
+    LayerP t;
+    if (i < a.L) {
+      const vui_layer_weights& s = W.layers[i];
+      t.attn_norm = (const bf16_t*)s.attn_norm; t.wqkv = (const bf16_t*)s.wqkv; t.wo = (const bf16_t*)s.wo;
+      t.mlp_norm = (const bf16_t*)s.mlp_norm; t.w1 = (const bf16_t*)s.w1; t.w3 = (const bf16_t*)s.w3; t.w2 = (const bf16_t*)s.w2;
+    } else {
+      const vui_rq_layer_weights& s = W.rq_layers[i - a.L];
+      t.attn_norm = (const bf16_t*)s.attn_norm; t.wqkv = (const bf16_t*)s.wqkv; t.wo = (const bf16_t*)s.wo;
+      t.mlp_norm = (const bf16_t*)s.mlp_norm; t.w1 = (const bf16_t*)s.w1; t.w3 = (const bf16_t*)s.w3; t.w2 = (const bf16_t*)s.w2;
+    }
+    lp[i] = t;
+  }
+  const bf16_t* g_final_norm = (const bf16_t*)W.final_norm;
+  const bf16_t* g_codec_head = (const bf16_t*)W.codec_head;
+  const bf16_t* g_eos_w = (const bf16_t*)W.eos_w;
+  const bf16_t* g_eos_b = (const bf16_t*)W.eos_b;
+  const float* g_rope = W.rope_table;
+  const bf16_t* g_rq_proj = (const bf16_t*)W.rq_backbone_proj;
+  const bf16_t* g_rq_emb = (const bf16_t*)W.rq_code_emb;
+  const bf16_t* pos_emb = (const bf16_t*)W.rq_pos_emb;
+  const bf16_t* g_rq_head = (const bf16_t*)W.rq_head_w;
+  const bf16_t* g_rq_norm = (const bf16_t*)W.rq_norm;
+  // the epoch has been read (the fence waits for it) before this workgroup reports its arrival
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  if (tid == 0) __hip_atomic_fetch_add(a.arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+  if (a.mode & FR_BACKBONE) {
+    slot = a.slot_idx ? a.slot_idx[0] : 0;
+    pos = a.seq_lens[slot];
+    if (pos < 0) pos = 0;
+    if (pos >= a.S) pos = a.S - 1;
+    // input embedding, redundantly in every workgroup (all row loads of a feature in flight together)
+    if (a.codes_in) {
+      const bf16_t* table = (const bf16_t*)W.audio_emb;
+      for (int k = tid; k < d; k += FR_THREADS) {
+        float s = 0.f;
+        for (int q0 = 0; q0 < a.Q; q0 += 16) {
+          bf16_t r[16];
+#pragma unroll
+          for (int q = 0; q < 16; ++q) {
+            r[q] = 0;
+            if (q0 + q < a.Q) {
+              int64_t cc = a.codes_in[q0 + q];
+              cc = cc < 0 ? 0 : (cc >= a.CS ? a.CS - 1 : cc);
+              r[q] = table[(size_t)(cc + (int64_t)(q0 + q) * a.CS) * d + k];
+            }
+          }
+#pragma unroll
+          for (int q = 0; q < 16; ++q) if (q0 + q < a.Q) s += bf2f(r[q]);
+        }
+        xres[k] = bf2f(f2bf(s));
+      }
+    } else {
+      for (int k = tid; k < d; k += FR_THREADS) xres[k] = bf2f(a.emb_in[k]);
+    }
+    __syncthreads();
+
+    const int nq = a.H * a.hd, nkv = a.KV * a.hd, hd = a.hd;
+    const int np_qkv = (nq + 2 * nkv) / 2;
+    const int n_qkv = pairs_of(np_qkv, wg, nwg), n_o = pairs_of(d / 2, wg, nwg), n_sw = pairs_of(a.F / 2, wg, nwg);
+    const Plan P_qkv = plan_of(n_qkv, d, wg, nwg, wave);
+    // QKV epilogue constants of this wave's pairs: region, index in region, rotation factors
+    int q_region[2], q_m[2];
+    float4 q_rot[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int n = 2 * P_qkv.gp[s];
+      int region, m;
+      if (n < nq) { region = 0; m = n; }
+      else if (n < nq + nkv) { region = 1; m = n - nq; }
+      else { region = 2; m = n - nq - nkv; }
+      const int dd = m % hd;
+      q_region[s] = region; q_m[s] = m;
+      q_rot[s] = make_float4(1.f, 0.f, 1.f, 0.f);
+      if (s < P_qkv.nslots && region != 2 && dd < a.rope_dim)
+        q_rot[s] = *reinterpret_cast<const float4*>(g_rope + ((size_t)pos * a.rope_dim + dd) * 2);
+      else q_region[s] |= 4;  // no rotation
+    }
+    const uint64_t* ybuf = nullptr;  // previous layer's MLP output, still to be added to xres
+    // attention split geometry (identical in every workgroup)
+    const int len = pos + 1;
+    const int start = (a.window > 0) ? max(0, len - 1 - a.window) : 0;
+    const int nkeys = len - start;
+    const int NS = a.ns;
+    int ns_eff = (nkeys + 31) / 32;
+    ns_eff = max(1, min(ns_eff, NS));
+    int chunk = (nkeys + ns_eff - 1) / ns_eff;
+    chunk = (chunk + 15) / 16 * 16;
+    const size_t slab = (size_t)a.n_slots * a.S * nkv;
+    const int att_h = wg % a.H, att_s = wg / a.H;
+    const bool att_on = att_s < ns_eff && wg < a.H * NS;
+    const int att_lo = start + att_s * chunk, att_hi = min(att_lo + chunk, len);
+    const int kvh = att_h / (a.H / a.KV);
+    const int cpd = (hd + 15) / 16;
+    const bool mrg_on = wg < a.H * cpd;
+
+    for (int l = 0; l < a.L; ++l) {
+      const LayerP Lw = lp[l];
+      bf16_t* kcl = a.kc + slab * l;
+      bf16_t* vcl = a.vc + slab * l;
+      // ---- QKV + RoPE + cache append ----
+      WRegs<2, false> wr;
+      const Plan P_qkv = plan_of(n_qkv, d, wg, nwg, wave);
+      gemv_prefetch<2, false>(Lw.wqkv, nullptr, d, P_qkv, wr);
+      const NormW nw1 = load_normw(Lw.attn_norm, d);
+      TS(1);
+      if (ybuf) poll_add(xres, ybuf, d / 2, c);
+      TS(2);
+      stage_norm(xres, nw1, a.eps, d, xn);
+      __syncthreads();
+      TS(3);
+      uint64_t* qkvbuf = llp;
+      llp += np_qkv;
+      gemv_compute<2, false>(xn, P_qkv, wr, red, [&](int gp, float v0, float v1, float, float) {
+        const bool s0 = (gp == P_qkv.gp[0]);
+        float o0 = bf2f(f2bf(v0)), o1 = bf2f(f2bf(v1));
+        const int rg = s0 ? q_region[0] : q_region[1];
+        const int region = rg & 3, m = s0 ? q_m[0] : q_m[1];
+        if (!(rg & 4)) {
+          const float4 f = s0 ? q_rot[0] : q_rot[1];
+          const float r0 = rope_mix(o0, f.x, -o1, f.y);
+          const float r1 = rope_mix(o1, f.z, o0, f.w);
+          o0 = r0; o1 = r1;
+        }
+        const uint32_t pk = pack2(o0, o1);
+        ll_st(qkvbuf + gp, pk, ep);
+        if (region == 1) *reinterpret_cast<uint32_t*>(kcl + ((size_t)slot * a.S + pos) * nkv + m) = pk;
+        if (region == 2) *reinterpret_cast<uint32_t*>(vcl + ((size_t)slot * a.S + pos) * nkv + m) = pk;
+      });
+      TS(4);
+
+      // ---- attention: workgroup (h, s) handles keys [lo, hi) of head h ----
+      uint64_t* part = llp;
+      llp += (size_t)a.H * NS * (hd + 2);
+      if (att_on) {
+        const int h = att_h, lo = att_lo, hi = att_hi;
+        const bool has_new = (pos >= lo && pos < hi);
+        const int grp = lane >> 4, l16 = lane & 15, g = wave * 4 + grp;
+        const bool act = l16 * 8 < hd;
+        const size_t rowstride = (size_t)nkv;
+        const bf16_t* kbase = kcl + ((size_t)slot * a.S) * rowstride + kvh * hd + l16 * 8;
+        const bf16_t* vbase = vcl + ((size_t)slot * a.S) * rowstride + kvh * hd + l16 * 8;
+        // the first four keys/values of this lane group are fetched before q is waited for
+        uint4 kreg[4], vreg[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int j = lo + g + 16 * i;
+          const bool on = act && j < hi && j != pos;
+          kreg[i] = on ? *reinterpret_cast<const uint4*>(kbase + (size_t)j * rowstride) : make_uint4(0, 0, 0, 0);
+          vreg[i] = on ? *reinterpret_cast<const uint4*>(vbase + (size_t)j * rowstride) : make_uint4(0, 0, 0, 0);
+        }
+        const int hw = hd / 2;
+        __syncthreads();
+        {
+          const uint64_t* p0 = (tid < hw) ? qkvbuf + (att_h * hd) / 2 + tid : nullptr;
+          const uint64_t* p1 = (has_new && tid < hw) ? qkvbuf + (nq + kvh * hd) / 2 + tid : nullptr;
+          const uint64_t* p2 = (has_new && tid < hw) ? qkvbuf + (nq + nkv + kvh * hd) / 2 + tid : nullptr;
+          uint32_t r0, r1, r2;
+          poll3(p0, p1, p2, c, r0, r1, r2);
+          if (tid < hw) {
+            qh[2 * tid] = bf2f((bf16_t)(r0 & 0xffff)); qh[2 * tid + 1] = bf2f((bf16_t)(r0 >> 16));
+            if (has_new) {
+              qh[128 + 2 * tid] = bf2f((bf16_t)(r1 & 0xffff)); qh[128 + 2 * tid + 1] = bf2f((bf16_t)(r1 >> 16));
+              qh[256 + 2 * tid] = bf2f((bf16_t)(r2 & 0xffff)); qh[256 + 2 * tid + 1] = bf2f((bf16_t)(r2 >> 16));
+            }
+          }
+        }
+        __syncthreads();
+        const float scale = 1.0f / sqrtf((float)hd);
+        float q8[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) q8[e] = act ? qh[l16 * 8 + e] : 0.f;
+        float mloc = -INFINITY;
+        {
+          int i = 0;
+          for (int j = lo + g; j < hi; j += 16, ++i) {
+            float k8[8];
+            float dsum = 0.f;
+            if (act) {
+              if (j == pos) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) k8[e] = qh[128 + l16 * 8 + e];
+              } else if (i < 4) {
+                cvt8(i == 0 ? kreg[0] : (i == 1 ? kreg[1] : (i == 2 ? kreg[2] : kreg[3])), k8);
+              } else {
+                El<bf16_t>::ld8(kbase + (size_t)j * rowstride, k8);
+              }
+#pragma unroll
+              for (int e = 0; e < 8; ++e) dsum = fmaf(q8[e], k8[e], dsum);
+            }
+            dsum = group16_sum(dsum) * scale;
+            if (l16 == 0) sc[j - lo] = dsum;
+            mloc = fmaxf(mloc, dsum);
+          }
+        }
+        if (l16 == 0) red[g] = mloc;
+        __syncthreads();
+        float M = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) M = fmaxf(M, red[i]);
+        float acc[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+        float lsum = 0.f;
+        {
+          int i = 0;
+          for (int j = lo + g; j < hi; j += 16, ++i) {
+            const float pw = expf(sc[j - lo] - M);
+            lsum += pw;
+            if (act) {
+              float v8[8];
+              if (j == pos) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v8[e] = qh[256 + l16 * 8 + e];
+              } else if (i < 4) {
+                cvt8(i == 0 ? vreg[0] : (i == 1 ? vreg[1] : (i == 2 ? vreg[2] : vreg[3])), v8);
+              } else {
+                El<bf16_t>::ld8(vbase + (size_t)j * rowstride, v8);
+              }
+#pragma unroll
+              for (int e = 0; e < 8; ++e) acc[e] = fmaf(pw, v8[e], acc[e]);
+            }
+          }
+        }
+        __syncthreads();  // maxima in red and QKV's xn fully read before they are reused
+        float* accs = xn;  // 16 x 128 floats
+        if (act) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) accs[g * 128 + l16 * 8 + e] = acc[e];
+        }
+        if (l16 == 0) red[16 + g] = lsum;
+        __syncthreads();
+        uint64_t* po = part + ((size_t)h * NS + att_s) * (hd + 2);
+        if (tid < hd) {
+          float t = 0.f;
+#pragma unroll
+          for (int gg = 0; gg < 16; ++gg) t += accs[gg * 128 + tid];
+          ll_st(po + 2 + tid, __float_as_uint(t), ep);
+        }
+        if (tid == 0) {
+          float t = 0.f;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) t += red[16 + i];
+          ll_st(po, __float_as_uint(M), ep);
+          ll_st(po + 1, __float_as_uint(t), ep);
+        }
+      }
+      TS(5);
+      // ---- merge the splits: workgroup (h, 16-feature chunk); one wait for everything ----
+      uint64_t* attbuf = llp;
+      llp += d / 2;
+      if (mrg_on) {
+        const int h = wg / cpd, cc = wg % cpd;
+        const uint64_t* pb = part + (size_t)h * NS * (hd + 2);
+        float* ml = sc;         // 2 * ns_eff floats
+        float* part_lds = lg;   // ns_eff x 16 raw accumulators
+        __syncthreads();
+        {
+          // thread items: it = tid and tid + 256 -> (split, feature); threads < 2*ns_eff also fetch max/sum
+          const int it0 = tid, it1 = tid + FR_THREADS;
+          const int nitem = ns_eff * 16;
+          const int dim0 = cc * 16 + (it0 & 15), dim1 = cc * 16 + (it1 & 15);
+          const uint64_t* p0 = (it0 < nitem && dim0 < hd) ? pb + (size_t)(it0 >> 4) * (hd + 2) + 2 + dim0 : nullptr;
+          const uint64_t* p1 = (it1 < nitem && dim1 < hd) ? pb + (size_t)(it1 >> 4) * (hd + 2) + 2 + dim1 : nullptr;
+          const uint64_t* p2 = (tid < 2 * ns_eff) ? pb + (size_t)(tid >> 1) * (hd + 2) + (tid & 1) : nullptr;
+          uint32_t r0, r1, r2;
+          poll3(p0, p1, p2, c, r0, r1, r2);
+          if (it0 < nitem) part_lds[it0] = p0 ? __uint_as_float(r0) : 0.f;
+          if (it1 < nitem) part_lds[it1] = p1 ? __uint_as_float(r1) : 0.f;
+          if (tid < 2 * ns_eff) ml[tid] = __uint_as_float(r2);
+        }
+        __syncthreads();
+        if (tid < 16) {
+          float Mx = -INFINITY;
+          for (int s = 0; s < ns_eff; ++s) Mx = fmaxf(Mx, ml[2 * s]);
+          float Lt = 0.f, o = 0.f;
+          for (int s = 0; s < ns_eff; ++s) {
+            const float w = expf(ml[2 * s] - Mx);
+            Lt = fmaf(w, ml[2 * s + 1], Lt);
+            o = fmaf(w, part_lds[s * 16 + tid], o);
+          }
+          const float val = o / Lt;
+          const float nb = dpp_f<DPP_QUAD_XOR1>(val);  // neighbour feature
+          const int d0 = cc * 16 + tid;
+          if (!(tid & 1) && d0 < hd) ll_st(attbuf + (h * hd + d0) / 2, pack2(val, nb), ep);
+        }
+      }
+      TS(6);
+      // ---- out_proj ----
+      uint64_t* obuf = llp;
+      llp += d / 2;
+      {
+        WRegs<2, false> w2;
+        const Plan P_o = plan_of(n_o, d, wg, nwg, wave);
+        gemv_prefetch<2, false>(Lw.wo, nullptr, d, P_o, w2);
+        poll_set(xn, attbuf, d / 2, c);
+        TS(7);
+        gemv_compute<2, false>(xn, P_o, w2, red, [&](int gp, float v0, float v1, float, float) {
+          ll_st(obuf + gp, pack2(v0, v1), ep); });
+      }
+      TS(8);
+      // ---- SwiGLU ----
+      uint64_t* hbuf = llp;
+      llp += a.F / 2;
+      {
+        WRegs<2, true> w3;
+        const Plan P_sw = plan_of(n_sw, d, wg, nwg, wave);
+        gemv_prefetch<2, true>(Lw.w1, Lw.w3, d, P_sw, w3);
+        const NormW nw2 = load_normw(Lw.mlp_norm, d);
+        poll_add(xres, obuf, d / 2, c);
+        TS(9);
+        stage_norm(xres, nw2, a.eps, d, xn);
+        __syncthreads();
+        TS(10);
+        gemv_compute<2, true>(xn, P_sw, w3, red, [&](int gp, float v0, float v1, float u0, float u1) {
+          const float a0 = bf2f(f2bf(v0)), a1 = bf2f(f2bf(v1)), c0 = bf2f(f2bf(u0)), c1 = bf2f(f2bf(u1));
+          const float s0 = bf2f(f2bf(a0 / (1.0f + expf(-a0)))), s1 = bf2f(f2bf(a1 / (1.0f + expf(-a1))));
+          ll_st(hbuf + gp, pack2(s0 * c0, s1 * c1), ep);
+        });
+      }
+      TS(11);
+      // ---- W2 ----
+      uint64_t* yb = llp;
+      llp += d / 2;
+      {
+        WRegs<4, false> w4;
+        const Plan P_w2 = plan_of(n_o, a.F, wg, nwg, wave);
+        gemv_prefetch<4, false>(Lw.w2, nullptr, a.F, P_w2, w4);
+        poll_set(xn, hbuf, a.F / 2, c);
+        TS(12);
+        gemv_compute<4, false>(xn, P_w2, w4, red, [&](int gp, float v0, float v1, float, float) {
+          ll_st(yb + gp, pack2(v0, v1), ep); });
+      }
+      ybuf = yb;
+      TS(13);
+    }
+    // ---- final norm, codec head, eos head ----
+    {
+      const Plan p = make_plan(a.CS / 2, d, wg, nwg, wave);
+      WRegs<2, false> wr;
+      gemv_prefetch<2, false>(g_codec_head, nullptr, d, p, wr);
+      const NormW nwf = load_normw(g_final_norm, d);
+      float eosw[16];  // this lane's eos-head weights (k = lane, lane+64, ...), d <= 1024
+#pragma unroll
+      for (int i = 0; i < 16; ++i) { const int k = lane + WAVE * i; eosw[i] = k < d ? bf2f(g_eos_w[k]) : 0.f; }
+      const float eosb = bf2f(*g_eos_b);
+      poll_add(xres, ybuf, d / 2, c);
+      stage_norm(xres, nwf, a.eps, d, xn);
+      __syncthreads();
+      uint64_t* lgbuf = llp;
+      llp += a.CS / 2;
+      gemv_compute<2, false>(xn, p, wr, red, [&](int gp, float v0, float v1, float, float) {
+        const uint32_t pk = pack2(v0, v1);
+        ll_st(lgbuf + gp, pk, ep);
+        if (a.cb0_out) *reinterpret_cast<uint32_t*>(a.cb0_out + 2 * gp) = pk;
+      });
+      // eos logit: every workgroup (it is a 1 x d dot product), outputs by workgroup 0
+      {
+        float t = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { const int k = lane + WAVE * i; if (k < d) t += xn[k] * eosw[i]; }
+        t = wave_sum(t);
+        eos_logit = bf2f(f2bf(t + eosb));
+      }
+      if (wg == 0) {
+        if (a.hidden_out) for (int k = tid; k < d; k += FR_THREADS) a.hidden_out[k] = f2bf(xn[k]);
+        if (a.eos_out && tid == 0) a.eos_out[0] = f2bf(eos_logit);
+      }
+      if (a.mode & FR_CB0) {
+        const int E = (a.CS + FR_THREADS - 1) / FR_THREADS;
+        poll_set(lg, lgbuf, a.CS / 2, c);
+        const bool greedy = (a.topk0 == 1) || !(a.temp0 > 0.f);
+        const float div = greedy ? 1.0f : a.temp0;
+        const float* counts = (a.rep_counts && a.penalty > 1.0f) ? a.rep_counts : nullptr;
+        float lv[8];
+        uint32_t key[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          lv[e] = -INFINITY;
+          key[e] = 0u;
+          const int j = tid * E + e;
+          if (e < E && j < a.CS) {
+            lv[e] = sample_value(lg[j], nullptr, j, counts, a.penalty, div);
+            key[e] = float_key(counts ? lv[e] : lg[j]);
+          }
+        }
+        TS(20);
+        code0 = block_sample<8>(lv, key, counts ? 0 : 16, a.CS, E, greedy, a.topk0, a.seed0, frame0, 0u, 0u, ssh);
+        TS(21);
+      }
+    }
+  }
+
+  // ------------------------------------------------------------------ depth head
+  if (a.mode & FR_RQ) {
+    const int R = a.R, CS = a.CS, Q = a.Q;
+    const int rhd = R / a.rqH;
+    if (!(a.mode & FR_BACKBONE)) {
+      for (int k = tid; k < d; k += FR_THREADS) xn[k] = bf2f(a.rq_hidden[k]);
+      __syncthreads();
+    }
+    if (!(a.mode & FR_CB0)) {
+      int64_t cc = a.rq_code0[0];
+      code0 = (int)(cc < 0 ? 0 : (cc >= CS ? CS - 1 : cc));
+    }
+    if (tid == 0) codes_l[0] = code0;
+    const int m_qkv = pairs_of(3 * R / 2, wg, nwg), m_o = pairs_of(R / 2, wg, nwg), m_sw = pairs_of(a.rqF / 2, wg, nwg),
+              m_hd = pairs_of(CS / 2, wg, nwg);
+    const NormW nw_rq = load_normw(g_rq_norm, R);
+    // attention lane layout: QP key slots x PP feature parts per wave
+    const int QP = Q <= 16 ? 16 : (Q <= 32 ? 32 : 64), PP = 64 / QP;
+    const int fpp = rhd / PP;  // features per part
+    // token 0: projected hidden + pos_emb[0]
+    if (g_rq_proj) {
+      const Plan p = make_plan(R / 2, d, wg, nwg, wave);
+      WRegs<2, false> wr;
+      gemv_prefetch<2, false>(g_rq_proj, nullptr, d, p, wr);
+      // only pairs this wave really owns are inside pos_emb[0, R)
+      const uint32_t pe0 = p.nslots > 0 ? *reinterpret_cast<const uint32_t*>(pos_emb + 2 * p.gp[0]) : 0u;
+      const uint32_t pe1 = p.nslots > 1 ? *reinterpret_cast<const uint32_t*>(pos_emb + 2 * p.gp[1]) : 0u;
+      uint64_t* tb = llp;
+      llp += R / 2;
+      gemv_compute<2, false>(xn, p, wr, red, [&](int gp, float v0, float v1, float, float) {
+        const uint32_t pe = (gp == p.gp[0]) ? pe0 : pe1;
+        const float o0 = bf2f(f2bf(v0)) + __uint_as_float(pe << 16), o1 = bf2f(f2bf(v1)) + __uint_as_float(pe & 0xffff0000u);
+        ll_st(tb + gp, pack2(o0, o1), ep);
+      });
+      poll_set(xres, tb, R / 2, c);
+    } else {
+      __syncthreads();
+      for (int k = tid; k < R; k += FR_THREADS) xres[k] = bf2f(f2bf(xn[k] + bf2f(pos_emb[k])));
+      __syncthreads();
+    }
+
+    int prev_code = code0;
+    for (int t = 0; t < a.n_q; ++t) {
+      if (t >= 1) {
+        const bf16_t* e = g_rq_emb + ((size_t)prev_code + (size_t)(t - 1) * CS) * R;
+        __syncthreads();
+        for (int k = tid; k < R; k += FR_THREADS) xres[k] = bf2f(f2bf(bf2f(e[k]) + bf2f(pos_emb[(size_t)t * R + k])));
+        __syncthreads();
+      }
+      const uint64_t* ybuf = nullptr;
+      for (int l = 0; l < a.rqL; ++l) {
+        const LayerP Lw = lp[a.L + l];
+        bf16_t* kst = rqkv + ((size_t)l * Q + t) * 2 * R;  // [k (R) | v (R)] of this layer and position
+        // ---- A: QKV ----
+        uint64_t* qkvb = llp;
+        llp += 3 * R / 2;
+        {
+          TS(30);
+          WRegs<2, false> wr;
+          const Plan R_qkv = plan_of(m_qkv, R, wg, nwg, wave);
+          gemv_prefetch<2, false>(Lw.wqkv, nullptr, R, R_qkv, wr);
+          const NormW nw1 = load_normw(Lw.attn_norm, R);
+          if (ybuf) poll_add(xres, ybuf, R / 2, c);
+          TS(31);
+          stage_norm(xres, nw1, a.rq_eps, R, xn);
+          __syncthreads();
+          gemv_compute<2, false>(xn, R_qkv, wr, red, [&](int gp, float v0, float v1, float, float) {
+            ll_st(qkvb + gp, pack2(v0, v1), ep); });
+        }
+        const bool kv_only = (t == 0 && l == a.rqL - 1);  // position 0 only feeds later keys/values
+        // ---- B: attention (redundantly in every workgroup) + out_proj ----
+        uint64_t* ob = llp;
+        if (!kv_only) llp += R / 2;
+        {
+          WRegs<2, false> wr;
+          const Plan R_o = plan_of(m_o, R, wg, nwg, wave);
+          if (!kv_only) gemv_prefetch<2, false>(Lw.wo, nullptr, R, R_o, wr);
+          __syncthreads();  // xn (A's input) fully consumed before q overwrites it
+          ll_poll(qkvb, 3 * R / 2, c, [&](int i, uint32_t v) {
+            const int n = 2 * i;
+            if (n < R) { xn[n] = bf2f((bf16_t)(v & 0xffff)); xn[n + 1] = bf2f((bf16_t)(v >> 16)); }
+            else *reinterpret_cast<uint32_t*>(kst + (n - R)) = v;
+          });
+          __syncthreads();
+          if (kv_only) break;
+          TS(32);
+          const int nk = t + 1;
+          const int kj = lane / PP, part = lane % PP;
+          for (int hh = wave; hh < a.rqH; hh += 4) {
+            const float scale = 1.0f / sqrtf((float)rhd);
+            // lane (key kj, part): partial dot over fpp features
+            float dsum = 0.f;
+            if (kj < nk) {
+              const bf16_t* kp = rqkv + ((size_t)l * Q + kj) * 2 * R + hh * rhd + part * fpp;
+              const float* qp = xn + hh * rhd + part * fpp;
+              if (!(fpp & 7)) {
+                for (int i = 0; i < fpp; i += 8) {
+                  const uint4 kk = *reinterpret_cast<const uint4*>(kp + i);
+                  const float4 qa = *reinterpret_cast<const float4*>(qp + i);
+                  const float4 qb = *reinterpret_cast<const float4*>(qp + i + 4);
+                  float k8[8];
+                  cvt8(kk, k8);
+                  dsum = fmaf(qa.x, k8[0], dsum); dsum = fmaf(qa.y, k8[1], dsum);
+                  dsum = fmaf(qa.z, k8[2], dsum); dsum = fmaf(qa.w, k8[3], dsum);
+                  dsum = fmaf(qb.x, k8[4], dsum); dsum = fmaf(qb.y, k8[5], dsum);
+                  dsum = fmaf(qb.z, k8[6], dsum); dsum = fmaf(qb.w, k8[7], dsum);
+                }
+              } else if (!(fpp & 1)) {
+                for (int i = 0; i < fpp; i += 2) {
+                  const uint32_t kk = *reinterpret_cast<const uint32_t*>(kp + i);
+                  dsum = fmaf(qp[i], __uint_as_float(kk << 16), dsum);
+                  dsum = fmaf(qp[i + 1], __uint_as_float(kk & 0xffff0000u), dsum);
+                }
+              } else {
+                for (int i = 0; i < fpp; ++i) dsum = fmaf(qp[i], bf2f(kp[i]), dsum);
+              }
+            }
+            if (PP >= 2) dsum += dpp_f<DPP_QUAD_XOR1>(dsum);
+            if (PP >= 4) dsum += dpp_f<DPP_QUAD_XOR2>(dsum);
+            const float sco = (kj < nk) ? dsum * scale : -INFINITY;
+            const float M = wave_max(sco);
+            const float pw = (kj < nk) ? expf(sco - M) : 0.f;
+            const float Ls = wave_sum(part == 0 ? pw : 0.f);
+            // lane = feature: weighted sum of the values
+            float o0 = 0.f, o1 = 0.f;
+            const bf16_t* vb = rqkv + ((size_t)l * Q) * 2 * R + R + hh * rhd;
+            for (int j = 0; j < nk; ++j) {
+              const float pj = lane_f(pw, j * PP);
+              if (lane < rhd) o0 = fmaf(pj, bf2f(vb[(size_t)j * 2 * R + lane]), o0);
+              if (lane + WAVE < rhd) o1 = fmaf(pj, bf2f(vb[(size_t)j * 2 * R + lane + WAVE]), o1);
+            }
+            if (lane < rhd) xn[R + hh * rhd + lane] = bf2f(f2bf(o0 / Ls));
+            if (lane + WAVE < rhd) xn[R + hh * rhd + lane + WAVE] = bf2f(f2bf(o1 / Ls));
+          }
+          __syncthreads();
+          TS(33);
+          gemv_compute<2, false>(xn + R, R_o, wr, red, [&](int gp, float v0, float v1, float, float) {
+            ll_st(ob + gp, pack2(v0, v1), ep); });
+        }
+        TS(34);
+        // ---- C: SwiGLU ----
+        uint64_t* hb = llp;
+        llp += a.rqF / 2;
+        {
+          WRegs<2, true> wr;
+          const Plan R_sw = plan_of(m_sw, R, wg, nwg, wave);
+          gemv_prefetch<2, true>(Lw.w1, Lw.w3, R, R_sw, wr);
+          const NormW nw2 = load_normw(Lw.mlp_norm, R);
+          poll_add(xres, ob, R / 2, c);
+          TS(35);
+          stage_norm(xres, nw2, a.rq_eps, R, xn);
+          __syncthreads();
+          gemv_compute<2, true>(xn, R_sw, wr, red, [&](int gp, float v0, float v1, float u0, float u1) {
+            const float a0 = bf2f(f2bf(v0)), a1 = bf2f(f2bf(v1)), c0 = bf2f(f2bf(u0)), c1 = bf2f(f2bf(u1));
+            const float s0 = bf2f(f2bf(a0 / (1.0f + expf(-a0)))), s1 = bf2f(f2bf(a1 / (1.0f + expf(-a1))));
+            ll_st(hb + gp, pack2(s0 * c0, s1 * c1), ep);
+          });
+        }
+        TS(36);
+        // ---- D: W2 ----
+        uint64_t* yb = llp;
+        llp += R / 2;
+        {
+          WRegs<4, false> wr;
+          const Plan R_w2 = plan_of(m_o, a.rqF, wg, nwg, wave);
+          gemv_prefetch<4, false>(Lw.w2, nullptr, a.rqF, R_w2, wr);
+          poll_set(xn, hb, a.rqF / 2, c);
+          TS(37);
+          gemv_compute<4, false>(xn, R_w2, wr, red, [&](int gp, float v0, float v1, float, float) {
+            ll_st(yb + gp, pack2(v0, v1), ep); });
+        }
+        ybuf = yb;
+      }
+      if (t >= 1) {
+        // ---- head t-1: logits of codebook t, then the draw in every workgroup ----
+        WRegs<2, false> wr;
+        const Plan R_hd = plan_of(m_hd, R, wg, nwg, wave);
+        gemv_prefetch<2, false>(g_rq_head + (size_t)(t - 1) * CS * R, nullptr, R, R_hd, wr);
+        TS(40);
+        poll_add(xres, ybuf, R / 2, c);
+        TS(41);
+        stage_norm(xres, nw_rq, a.rq_eps, R, xn);
+        __syncthreads();
+        uint64_t* lgbuf = llp;
+        llp += CS / 2;
+        gemv_compute<2, false>(xn, R_hd, wr, red, [&](int gp, float v0, float v1, float, float) {
+          ll_st(lgbuf + gp, pack2(v0, v1), ep); });
+        TS(42);
+        poll_set(lg, lgbuf, CS / 2, c);
+        TS(43);
+        const int E = (CS + FR_THREADS - 1) / FR_THREADS;
+        const bool greedy = (a.topk1 == 1) || !(a.temp1 > 0.f);
+        const float div = greedy ? 1.0f : a.temp1;
+        const float* bias = a.logit_bias ? a.logit_bias + (size_t)(t - 1) * CS : nullptr;
+        float lv[8];
+        uint32_t key[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          lv[e] = -INFINITY;
+          key[e] = 0u;
+          const int j = tid * E + e;
+          if (e < E && j < CS) {
+            lv[e] = sample_value(lg[j], bias, j, nullptr, 1.0f, div);
+            key[e] = float_key(bias ? lv[e] : lg[j]);
+          }
+        }
+        prev_code = block_sample<8>(lv, key, bias ? 0 : 16, CS, E, greedy, a.topk1, a.seed1, frame1, 0u, (uint32_t)t, ssh);
+        TS(44);
+#ifdef VUI_SAMPLE_CLOCK
+        if (a.prof && wg == a.prof_wg && tid == 0)
+          for (int k = 0; k < 6; ++k) if (nts < a.prof_cap) a.prof[nts++] = (ssh.ts[k] << 8) | (uint64_t)(60 + k);
+#endif
+        if (tid == 0) codes_l[t] = prev_code;
+      }
+    }
+  }
+
+  // ------------------------------------------------------------------ bookkeeping by workgroup 0
+  __syncthreads();
+  TS(50);
+  if (a.prof && wg == a.prof_wg && tid == 0) a.prof[a.prof_cap] = (uint64_t)nts;
+  if (wg == 0) {
+    if ((a.mode & FR_CB0) && tid == 0) {
+      if (a.code0_out) a.code0_out[0] = code0;
+      if (a.rep_counts && a.penalty > 1.0f) rep_push(a.rep_counts, a.rep_hist, a.rep_pos, a.rep_window, code0);
+    }
+    if (a.mode & FR_RQ) {
+      for (int t = tid; t < a.codes_stride; t += FR_THREADS) {
+        if (t < a.n_q) a.codes_out[t] = codes_l[t];
+        else if (a.zero_pad) a.codes_out[t] = 0;
+      }
+    }
+    if (a.mode & FR_BACKBONE) {
+      if (a.seq_inc) { for (int s = tid; s < a.n_slots; s += FR_THREADS) a.seq_lens[s] += a.seq_inc[s]; }
+      else if (tid == 0) a.seq_lens[slot] += 1;
+    }
+    if (a.mode & FR_FINISH) {
+      const int f = a.frame_ctr[0];
+      const bool in_range = f >= 0 && f < a.max_frames;
+      if (a.frames_out && in_range)
+        for (int t = tid; t < a.Q; t += FR_THREADS) a.frames_out[(size_t)f * a.Q + t] = (t < a.n_q) ? codes_l[t] : 0;
+      if (a.eos_prob_out && tid == 0 && (in_range || !a.frames_out))
+        a.eos_prob_out[a.frames_out ? f : 0] = 1.0f / (1.0f + expf(-eos_logit));
+      __syncthreads();
+      if (tid == 0) a.frame_ctr[0] = f + 1;
+    }
+    if (tid == 0) {
+      // every workgroup has read the epoch before it may change
+      int spins = 0;
+      while (__hip_atomic_load(a.arrive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (uint32_t)nwg && ++spins < SPIN_LIMIT)
+        __builtin_amdgcn_s_sleep(1);
+      __hip_atomic_store(a.arrive, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(a.epoch, ep, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// host side
+size_t frame_ll_words(const vui_config& c, int ns) {
+  const size_t d = c.d_model, hd = c.head_dim;
+  size_t per_layer = (size_t)(c.n_heads + 2 * c.n_kv_heads) * hd / 2 + (size_t)c.n_heads * ns * (hd + 2) + d / 2 + d / 2 +
+                     c.ffn / 2 + d / 2;
+  size_t total = per_layer * c.n_layers + c.codebook_size / 2;
+  const size_t R = c.rq_dim;
+  size_t rq_layer = 3 * R / 2 + R / 2 + c.rq_ffn / 2 + R / 2;
+  total += R / 2 + (size_t)c.n_quantizers * (rq_layer * c.rq_layers + c.codebook_size / 2);
+  return total + 64;
+}
+
+static size_t frame_ptr_bytes(const vui_config& c) {
+  return (((size_t)(c.n_layers + c.rq_layers) * sizeof(LayerP)) + 15) & ~(size_t)15;
+}
+size_t frame_lds_bytes(const vui_config& c) {
+  return (size_t)LDS_FIXED + frame_ptr_bytes(c) + (size_t)c.rq_layers * c.n_quantizers * 2 * c.rq_dim * 2;
+}
+
+bool frame_supported(const vui_config& c, int nwg, int ns, char* why, size_t why_len) {
+  const char* r = nullptr;
+  if (c.dtype != VUI_DTYPE_BF16) r = "bf16 only";
+  else if (c.int8_backbone) r = "int8 weights use the per-kernel path";
+  else if (c.d_model > 1024 || c.ffn > 2048 || c.rq_dim > 1024 || c.rq_ffn > 2048) r = "vector longer than the LDS staging area";
+  else if (c.codebook_size > 2048 || (c.codebook_size & 1)) r = "codebook_size > 2048";
+  else if (c.n_quantizers > 64) r = "too many codebooks";
+  else if ((c.head_dim & 7) || c.head_dim > 128) r = "head_dim";
+  else if ((c.rq_dim / c.rq_heads) % 4 || c.rq_dim / c.rq_heads > 128) r = "depth-head head_dim must be a multiple of 4, at most 128";
+  else if (frame_lds_bytes(c) > 160 * 1024) r = "depth-head keys/values do not fit in LDS";
+  else if (c.rq_layers < 1) r = "no depth head";
+  else {
+    const int np_max = (c.n_heads + 2 * c.n_kv_heads) * c.head_dim / 2;
+    int m = np_max;
+    if (c.ffn / 2 > m) m = c.ffn / 2;
+    if (c.codebook_size / 2 > m) m = c.codebook_size / 2;
+    if (3 * c.rq_dim / 2 > m) m = 3 * c.rq_dim / 2;
+    if (c.rq_ffn / 2 > m) m = c.rq_ffn / 2;
+    if (m > 8 * nwg) r = "too few workgroups for the widest matrix";
+    if ((c.max_seqlen + ns - 1) / ns + 16 > 1024) r = "key split longer than the LDS score buffer";
+    if (nwg < c.n_heads * ns || nwg < c.n_heads * ((c.head_dim + 15) / 16)) r = "too few workgroups for the attention split";
+  }
+  if (r && why) snprintf(why, why_len, "%s", r);
+  return r == nullptr;
+}
+
+int frame_max_resident(size_t lds_bytes, int* n_cu) {
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  hipDeviceProp_t prop;
+  HIP_TRY(hipGetDeviceProperties(&prop, dev));
+  // the attribute is per kernel, not per context: never lower it for another, larger context
+  static size_t lds_attr = 0;
+  if (lds_bytes > lds_attr) {
+    HIP_TRY(hipFuncSetAttribute((const void*)frame_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    lds_attr = lds_bytes;
+  }
+  int occ = 0;
+  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, frame_kernel, FR_THREADS, lds_bytes));
+  if (n_cu) *n_cu = prop.multiProcessorCount;
+  return occ * prop.multiProcessorCount;
+}
+
+int launch_frame(const FrameArgs& a, int nwg, size_t lds_bytes, hipStream_t st) {
+  hipLaunchKernelGGL(frame_kernel, dim3(nwg), dim3(FR_THREADS), lds_bytes, st, a);
+  HIP_TRY(hipGetLastError());
+  return VUI_OK;
+}

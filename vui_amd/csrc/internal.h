@@ -125,6 +125,64 @@ int launch_frame_finish(const int64_t* codes, int64_t* frames_out, int n, int ma
 int launch_add_rows(int dtype, const void* a, const void* vec, void* out, int B, int R, hipStream_t st);
 int launch_fill_u32(uint32_t* p, uint32_t v, int64_t n, hipStream_t st);
 
+// ---- fused frame kernel (frame.hip) ----
+struct FrameArgs {
+  int d, L, H, KV, hd, F, Q, CS, R, rqL, rqH, rqF, rope_dim, S, window;
+  float eps, rq_eps;
+  const vui_weights* w;  // device copy
+  // backbone
+  const int64_t* codes_in;
+  const uint16_t* emb_in;
+  const int32_t* slot_idx;
+  int32_t* seq_lens;
+  const int32_t* seq_inc;
+  int n_slots;
+  uint16_t *kc, *vc;
+  uint16_t *hidden_out, *cb0_out, *eos_out;
+  // code-0 sampling
+  float* rep_counts;
+  int32_t* rep_hist;
+  int32_t* rep_pos;
+  float penalty;
+  int rep_window;
+  float temp0; int topk0;
+  float temp1; int topk1;
+  uint64_t seed0, seed1;
+  const int32_t* frame_ctr0;
+  const int32_t* frame_ctr1;
+  int64_t* code0_out;
+  // depth head
+  const uint16_t* rq_hidden;
+  const int64_t* rq_code0;
+  const float* logit_bias;
+  int n_q;
+  int64_t* codes_out;
+  int codes_stride, zero_pad;
+  // frame bookkeeping
+  int64_t* frames_out;
+  float* eos_prob_out;
+  int max_frames;
+  int32_t* frame_ctr;
+  // exchange
+  uint64_t* ll;
+  uint32_t* epoch;
+  uint32_t* arrive;
+  uint32_t* err;
+  int ns;    // attention key splits per head
+  int mode;  // FR_* bits
+  int lds_kv_off;  // byte offset of the depth-head K/V store in LDS
+  uint64_t* prof;  // optional (prof_cap + 1) words: (clock << 8 | tag) per phase point, count in the last word
+  int prof_cap, prof_wg;
+};
+
+enum { FR_BACKBONE = 1, FR_CB0 = 2, FR_RQ = 4, FR_FINISH = 8 };
+
+size_t frame_ll_words(const vui_config& c, int ns);
+size_t frame_lds_bytes(const vui_config& c);
+bool frame_supported(const vui_config& c, int nwg, int ns, char* why, size_t why_len);
+int frame_max_resident(size_t lds_bytes, int* n_cu);
+int launch_frame(const FrameArgs& a, int nwg, size_t lds_bytes, hipStream_t st);
+
 void vui_set_error(const char* fmt, ...);
 #define HIP_TRY(expr)                                                                  \
   do {                                                                                 \

@@ -3,6 +3,7 @@
 // head's token builder and the per-frame bookkeeping.
 #include "common.h"
 #include "internal.h"
+#include "sample.h"
 
 // ---- audio embedding: x[b] = rnd(sum_q table[codes[b,q] + q*CS])   (model.py:559-563) ----
 template <typename T>
@@ -78,166 +79,42 @@ int launch_rope(int dtype, void* x, const float* table, const int32_t* pos, int 
   return VUI_OK;
 }
 
-// ---- Philox4x32-10 (Salmon et al. 2011) ----
-__device__ __forceinline__ uint32_t philox_u32(uint64_t seed, uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3) {
-  uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
-#pragma unroll
-  for (int r = 0; r < 10; ++r) {
-    const uint64_t p0 = (uint64_t)0xD2511F53u * c0;
-    const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
-    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
-    const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
-    c1 = (uint32_t)p1; c3 = (uint32_t)p0; c0 = n0; c2 = n2;
-    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
-  }
-  return c0;
-}
-
-__device__ __forceinline__ uint32_t float_key(float f) {  // order-preserving map to uint32
-  const uint32_t u = __float_as_uint(f);
-  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-}
-
-// ---- sampler: one 256-thread workgroup per row ----
-// RQ rule (model.py:955-962): l = (logit + bias) / T; drop l < k-th largest; softmax; draw.
-// code-0 rule (engine.py:571-576, 855-863): penalise by penalty^count; softmax(l / T); keep the
-// top-k probabilities; renormalise; draw.  Both reduce to: keep {l >= k-th largest l},
-// weights exp(l - max), inverse CDF in index order with one uniform.
-#define SAMP_THREADS 256
-#define SAMP_MAX_E 32  // elements per thread -> CS <= 8192
-
+// ---- sampler: one 256-thread workgroup per row (see sample.h) ----
 template <typename T, int EMAX>
 __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const SampleArgs p) {
-  __shared__ float sred[SAMP_THREADS / WAVE];
-  __shared__ int ired[SAMP_THREADS / WAVE];
-  __shared__ float wsum[SAMP_THREADS / WAVE];
-  __shared__ int s_pick;
-  const int b = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  __shared__ SampleShared sh;
+  const int b = blockIdx.x, tid = threadIdx.x;
   const int CS = p.CS;
   const int E = (CS + SAMP_THREADS - 1) / SAMP_THREADS;  // contiguous elements per thread
   const T* lg = (const T*)p.logits + (size_t)b * CS;
   const bool greedy = (p.top_k == 1) || !(p.temperature > 0.f);
-  const float invT_div = greedy ? 1.0f : p.temperature;
+  const float div = greedy ? 1.0f : p.temperature;
+  const float* counts = (p.rep_counts && p.penalty > 1.0f) ? p.rep_counts + (size_t)b * CS : nullptr;
 
+  // untouched bf16 logits order the elements with 16-bit keys; bias or penalty need all 32 bits
+  const bool raw_keys = sizeof(T) == 2 && !p.bias && !counts;
   float l[EMAX];
+  uint32_t key[EMAX];
 #pragma unroll
   for (int e = 0; e < EMAX; ++e) {
     l[e] = -INFINITY;
+    key[e] = 0u;
     const int j = tid * E + e;
     if (e < E && j < CS) {
-      float v = El<T>::ld(lg + j);
-      if (p.bias) v += p.bias[j];
-      if (p.rep_counts && p.penalty > 1.0f) {
-        const float f = powf(p.penalty, p.rep_counts[(size_t)b * CS + j]);
-        v = (v > 0.f) ? v / f : v * f;
-      }
-      l[e] = v / invT_div;
+      const float raw = El<T>::ld(lg + j);
+      l[e] = sample_value(raw, p.bias, j, counts, p.penalty, div);
+      key[e] = float_key(raw_keys ? raw : l[e]);
     }
   }
-
-  // maximum and its lowest index
-  float m = -INFINITY; int mi = 0x7fffffff;
-#pragma unroll
-  for (int e = 0; e < EMAX; ++e)
-    if (e < E && l[e] > m) { m = l[e]; mi = tid * E + e; }
-  {
-    float wm = wave_max(m);
-    int cand = (m == wm) ? mi : 0x7fffffff;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) cand = min(cand, __shfl_xor(cand, o, WAVE));
-    if (lane == 0) { sred[wave] = wm; ired[wave] = cand; }
-  }
-  __syncthreads();
-  float M = sred[0]; int Mi = ired[0];
-#pragma unroll
-  for (int w = 1; w < SAMP_THREADS / WAVE; ++w) {
-    if (sred[w] > M) { M = sred[w]; Mi = ired[w]; }
-    else if (sred[w] == M) Mi = min(Mi, ired[w]);
-  }
-  __syncthreads();
-
-  int pick = Mi;
-  if (!greedy) {
-    // key of the k-th largest value, built bit by bit
-    uint32_t thr = 0u;
-    if (p.top_k > 0 && p.top_k < CS) {
-      uint32_t key[EMAX];
-#pragma unroll
-      for (int e = 0; e < EMAX; ++e) key[e] = (e < E && tid * E + e < CS) ? float_key(l[e]) : 0u;
-      for (int bit = 31; bit >= 0; --bit) {
-        const uint32_t cand = thr | (1u << bit);
-        int c = 0;
-#pragma unroll
-        for (int e = 0; e < EMAX; ++e)
-          if (e < E) c += (key[e] >= cand);
-        c = wave_sum_i(c);
-        if (lane == 0) ired[wave] = c;
-        __syncthreads();
-        int tot = 0;
-#pragma unroll
-        for (int w = 0; w < SAMP_THREADS / WAVE; ++w) tot += ired[w];
-        if (tot >= p.top_k) thr = cand;
-        __syncthreads();
-      }
-    }
-    // weights, their total, and the inverse CDF in index order
-    float wloc = 0.f;
-    float pw[EMAX];
-#pragma unroll
-    for (int e = 0; e < EMAX; ++e) {
-      pw[e] = 0.f;
-      if (e < E && tid * E + e < CS && float_key(l[e]) >= thr) pw[e] = expf(l[e] - M);
-      wloc += pw[e];
-    }
-    // inclusive scan of wloc over threads: within the wave, then across waves
-    float incl = wloc;
-#pragma unroll
-    for (int o = 1; o < WAVE; o <<= 1) {
-      const float t = __shfl_up(incl, o, WAVE);
-      if (lane >= o) incl += t;
-    }
-    if (lane == WAVE - 1) wsum[wave] = incl;
-    if (tid == 0) s_pick = -1;
-    __syncthreads();
-    float base = 0.f, total = 0.f;
-#pragma unroll
-    for (int w = 0; w < SAMP_THREADS / WAVE; ++w) { if (w < wave) base += wsum[w]; total += wsum[w]; }
-    const uint32_t frame = p.frame_ctr ? (uint32_t)p.frame_ctr[0] : 0u;
-    const uint32_t rnd = philox_u32(p.seed, frame, (uint32_t)b, (uint32_t)p.codebook, 0u);
-    const float u = (float)(rnd >> 8) * (1.0f / 16777216.0f);
-    const float target = u * total;
-    const float before = base + incl - wloc;  // sum of everything ahead of this thread
-    if (target >= before && target < before + wloc) {
-      float run = before; int j = -1;
-#pragma unroll
-      for (int e = 0; e < EMAX; ++e) {
-        if (e < E && j < 0) { run += pw[e]; if (pw[e] > 0.f && run > target) j = tid * E + e; }
-      }
-      if (j < 0) {  // rounding at the thread's upper edge: take its last kept element
-#pragma unroll
-        for (int e = 0; e < EMAX; ++e) if (e < E && pw[e] > 0.f) j = tid * E + e;
-      }
-      if (j >= 0) atomicMax(&s_pick, j);
-    }
-    __syncthreads();
-    pick = (s_pick >= 0) ? s_pick : Mi;
-  }
+  const uint32_t frame = p.frame_ctr ? (uint32_t)p.frame_ctr[0] : 0u;
+  const int pick = block_sample<EMAX>(l, key, raw_keys ? 16 : 0, CS, E, greedy, p.top_k, p.seed, frame, (uint32_t)b,
+                                      (uint32_t)p.codebook, sh);
 
   if (tid == 0) {
     p.out[(size_t)b * p.out_stride + p.out_col] = (int64_t)pick;
-    if (p.rep_counts && p.penalty > 1.0f) {
-      float* cnt = p.rep_counts + (size_t)b * CS;
-      if (p.window > 0 && p.rep_hist) {
-        int head = p.rep_pos[b * 2], filled = p.rep_pos[b * 2 + 1];
-        int32_t* hist = p.rep_hist + (size_t)b * p.window;
-        if (filled == p.window) cnt[hist[head]] -= 1.0f;
-        hist[head] = pick;
-        head = (head + 1) % p.window;
-        if (filled < p.window) ++filled;
-        p.rep_pos[b * 2] = head; p.rep_pos[b * 2 + 1] = filled;
-      }
-      cnt[pick] += 1.0f;
-    }
+    if (counts)
+      rep_push(p.rep_counts + (size_t)b * CS, p.rep_hist ? p.rep_hist + (size_t)b * p.window : nullptr,
+               p.rep_pos ? p.rep_pos + b * 2 : nullptr, p.window, pick);
     if (p.eos_prob) {
       const float z = El<T>::ld((const T*)p.eos_logit + b);
       p.eos_prob[b] = 1.0f / (1.0f + expf(-z));

@@ -1,0 +1,187 @@
+// Block-wide sampler shared by the stand-alone sampling kernel and the fused frame kernel.
+#pragma once
+#include "common.h"
+
+// ---- Philox4x32-10 (Salmon et al. 2011) ----
+__device__ __forceinline__ uint32_t philox_u32(uint64_t seed, uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3) {
+  uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+    const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    c1 = (uint32_t)p1; c3 = (uint32_t)p0; c0 = n0; c2 = n2;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  return c0;
+}
+
+__device__ __forceinline__ uint32_t float_key(float f) {  // order-preserving map to uint32
+  const uint32_t u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+#define SAMP_THREADS 256
+#define SAMP_MAX_E 32  // elements per thread -> CS <= 8192
+
+struct SampleShared {
+  float sred[SAMP_THREADS / WAVE];
+  int ired[SAMP_THREADS / WAVE];
+  float wsum[SAMP_THREADS / WAVE];
+  int cnt[2][3 * SAMP_THREADS / WAVE];
+  int pick;
+#ifdef VUI_SAMPLE_CLOCK
+  unsigned long long ts[8];
+#endif
+};
+#ifdef VUI_SAMPLE_CLOCK
+#define SAMP_TS(k) do { if (threadIdx.x == 0) sh.ts[k] = wall_clock64(); } while (0)
+#else
+#define SAMP_TS(k) do { } while (0)
+#endif
+
+// One draw from the values l[e] (element index tid*E + e, -inf beyond CS) held by a 256-thread
+// block.  RQ rule (src/vui/model.py:955-962): drop l < k-th largest, softmax, draw.  code-0 rule
+// (src/vui/engine.py:855-863): softmax, keep the top-k probabilities, renormalise, draw.  Both
+// are: keep {l >= k-th largest l}, weights exp(l - max), inverse CDF in index order with one
+// uniform.  greedy: the lowest index of the maximum.  Every thread returns the same pick.
+//
+// key[e] orders the elements for the top-k cut (any order-preserving image of l[e]); bits below
+// low_bit are known to carry no information (16 when the keys come from bf16 values), so the
+// search for the k-th largest key, two bits per barrier, only walks bits 31..low_bit and stops
+// as soon as exactly top_k keys lie above the candidate.
+template <int EMAX>
+__device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32_t (&key)[EMAX], int low_bit, int CS,
+                                            int E, bool greedy, int top_k, uint64_t seed, uint32_t frame,
+                                            uint32_t row, uint32_t codebook, SampleShared& sh) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  SAMP_TS(0);
+  float m = -INFINITY; int mi = 0x7fffffff;
+#pragma unroll
+  for (int e = 0; e < EMAX; ++e)
+    if (e < E && l[e] > m) { m = l[e]; mi = tid * E + e; }
+  {
+    const float wm = wave_max(m);
+    const int cand = wave_min_i((m == wm) ? mi : 0x7fffffff);
+    if (lane == 0) { sh.sred[wave] = wm; sh.ired[wave] = cand; }
+  }
+  __syncthreads();
+  float M = sh.sred[0]; int Mi = sh.ired[0];
+#pragma unroll
+  for (int w = 1; w < SAMP_THREADS / WAVE; ++w) {
+    if (sh.sred[w] > M) { M = sh.sred[w]; Mi = sh.ired[w]; }
+    else if (sh.sred[w] == M) Mi = min(Mi, sh.ired[w]);
+  }
+  __syncthreads();
+  if (greedy) return Mi;
+  SAMP_TS(1);
+
+  // key of the k-th largest value, two bits per step
+  uint32_t thr = 0u;
+  if (top_k > 0 && top_k < CS) {
+    int it = 0;
+    for (int bit = 30; bit >= low_bit; bit -= 2, ++it) {
+      const uint32_t c1 = thr | (1u << bit), c2 = thr | (2u << bit), c3 = thr | (3u << bit);
+      // per-lane counts on the vector ALU (three 10-bit fields), one packed wave reduction
+      int pk = 0;
+#pragma unroll
+      for (int e = 0; e < EMAX; ++e)
+        if (e < E) pk += (key[e] >= c1 ? 1 : 0) + (key[e] >= c2 ? (1 << 10) : 0) + (key[e] >= c3 ? (1 << 20) : 0);
+      pk = wave_sum_i(pk);  // per field at most 64 * EMAX <= 1023 when EMAX <= 15; wider EMAX uses two sums
+      int n1 = pk & 1023, n2 = (pk >> 10) & 1023, n3 = (pk >> 20) & 1023;
+      if (EMAX > 15) {
+        int q1 = 0, q2 = 0, q3 = 0;
+#pragma unroll
+        for (int e = 0; e < EMAX; ++e)
+          if (e < E) { q1 += key[e] >= c1; q2 += key[e] >= c2; q3 += key[e] >= c3; }
+        n1 = wave_sum_i(q1); n2 = wave_sum_i(q2); n3 = wave_sum_i(q3);
+      }
+      int* buf = sh.cnt[it & 1];
+      if (lane == 0) { buf[wave * 3] = n1; buf[wave * 3 + 1] = n2; buf[wave * 3 + 2] = n3; }
+      __syncthreads();
+      int t1 = 0, t2 = 0, t3 = 0;
+#pragma unroll
+      for (int w = 0; w < SAMP_THREADS / WAVE; ++w) { t1 += buf[w * 3]; t2 += buf[w * 3 + 1]; t3 += buf[w * 3 + 2]; }
+      int tsel = CS;
+      if (t3 >= top_k) { thr = c3; tsel = t3; }
+      else if (t2 >= top_k) { thr = c2; tsel = t2; }
+      else if (t1 >= top_k) { thr = c1; tsel = t1; }
+      if (tsel == top_k) break;  // exactly k keys are >= thr: the kept set is final
+    }
+  }
+  SAMP_TS(2);
+  // weights, their total, and the inverse CDF in index order
+  float wloc = 0.f;
+  float pw[EMAX];
+#pragma unroll
+  for (int e = 0; e < EMAX; ++e) {
+    pw[e] = 0.f;
+    if (e < E && tid * E + e < CS && key[e] >= thr) pw[e] = expf(l[e] - M);
+    wloc += pw[e];
+  }
+  // inclusive scan over the wave: shifts inside each row of 16 lanes, then the row totals
+  float incl = wloc;
+  incl += dpp_f<0x111>(incl);  // row_shr:1, lanes shifted in from outside the row read 0
+  incl += dpp_f<0x112>(incl);  // row_shr:2
+  incl += dpp_f<0x114>(incl);  // row_shr:4
+  incl += dpp_f<0x118>(incl);  // row_shr:8
+  {
+    const float t0 = lane_f(incl, 15), t1 = lane_f(incl, 31), t2 = lane_f(incl, 47);
+    const int row = lane >> 4;
+    incl += (row >= 1 ? t0 : 0.f) + (row >= 2 ? t1 : 0.f) + (row >= 3 ? t2 : 0.f);
+  }
+  SAMP_TS(3);
+  if (lane == WAVE - 1) sh.wsum[wave] = incl;
+  if (tid == 0) sh.pick = -1;
+  __syncthreads();
+  float base = 0.f, total = 0.f;
+#pragma unroll
+  for (int w = 0; w < SAMP_THREADS / WAVE; ++w) { if (w < wave) base += sh.wsum[w]; total += sh.wsum[w]; }
+  SAMP_TS(4);
+  const uint32_t rnd = philox_u32(seed, frame, row, codebook, 0u);
+  const float u = (float)(rnd >> 8) * (1.0f / 16777216.0f);
+  const float target = u * total;
+  const float before = base + incl - wloc;  // sum of everything ahead of this thread
+  if (target >= before && target < before + wloc) {
+    float run = before; int j = -1;
+#pragma unroll
+    for (int e = 0; e < EMAX; ++e) {
+      if (e < E && j < 0) { run += pw[e]; if (pw[e] > 0.f && run > target) j = tid * E + e; }
+    }
+    if (j < 0) {  // rounding at the thread's upper edge: take its last kept element
+#pragma unroll
+      for (int e = 0; e < EMAX; ++e) if (e < E && pw[e] > 0.f) j = tid * E + e;
+    }
+    if (j >= 0) atomicMax(&sh.pick, j);
+  }
+  __syncthreads();
+  const int pick = (sh.pick >= 0) ? sh.pick : Mi;
+  SAMP_TS(5);
+  __syncthreads();
+  return pick;
+}
+
+// penalised, biased, temperature-scaled value of one logit
+__device__ __forceinline__ float sample_value(float v, const float* bias, int j, const float* counts, float penalty,
+                                              float div) {
+  if (bias) v += bias[j];
+  if (counts && penalty > 1.0f) {
+    const float f = powf(penalty, counts[j]);
+    v = (v > 0.f) ? v / f : v * f;
+  }
+  return v / div;
+}
+
+// rolling repetition state of one row (src/vui/engine.py:578-590); one thread
+__device__ __forceinline__ void rep_push(float* cnt, int32_t* hist, int32_t* pos2, int window, int pick) {
+  if (window > 0 && hist) {
+    int head = pos2[0], filled = pos2[1];
+    if (filled == window) cnt[hist[head]] -= 1.0f;
+    hist[head] = pick;
+    head = (head + 1) % window;
+    if (filled < window) ++filled;
+    pos2[0] = head; pos2[1] = filled;
+  }
+  cnt[pick] += 1.0f;
+}

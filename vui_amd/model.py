@@ -168,6 +168,13 @@ class _Native:
         self.lib = lib
         _lib.check(lib.vui_ctx_init(h, torch.cuda.current_stream().cuda_stream), "vui_ctx_init")
 
+    def fused(self, enable: int = -1) -> bool:
+        """Query (-1) or switch (1/0) the one-kernel form of the batch-1 bf16 calls."""
+        return bool(self.lib.vui_ctx_fused(self.handle, enable))
+
+    def status(self) -> None:
+        _lib.check(self.lib.vui_ctx_status(self.handle), "vui_ctx_status")
+
     def __del__(self):
         try:
             if getattr(self, "handle", None):
