@@ -97,34 +97,97 @@ def gpu_bench(args):
                    "preset": args.preset, "kv_len": [L_start, L_end], "sampling": "T=0.9 top-k=100 rep=1.1/24",
                    "setup_s": round(setup_s, 1)},
         "frame_bytes": {k: int(v) for k, v in fb.items()},
-        "frame_hbm_frac": round(fb["frame"] / (ms_per * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "fused": bool(model._native.fused(-1)),
     }
     return out, (model, eng, d, sd)
 
 
-def kernel_roofline(model, eng):
-    """Live timing of the dominant kernel: the backbone decode step (all 22 layers + heads) replayed
-    as a graph at a fixed KV length, HIP events on the launching stream."""
+# HBM traffic of one frame_kernel launch on the default workload, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (KiB per dispatch) scaled by what the same counters read for a plain copy of known size;
+# see profiles/frame_kernel_e2e_b1.txt.  None until measured.
+MEASURED_TRAFFIC_BYTES = 518_986_473  # at cache length 596..651 (algorithmic 414.6 MB there): 1.25 x
+
+
+def kernel_roofline(out, fb):
+    """The dominant kernel is frame_kernel: one launch per codec frame holds the whole step, so its
+    average duration is the timed region's HIP-event time per replay (same stream), and its
+    algorithmic bytes are those of one frame at the run's mean cache length."""
+    us = out["ms_per_step"] * 1e3
+    ach = fb["frame"] / (us * 1e-6) / 1e9
+    return {"bound": "hbm", "kernel": "frame_kernel (backbone step + code-0 sampling + depth head, one launch per frame)",
+            "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES, "us_per_launch": round(us, 2), "algorithmic_bytes": int(fb["frame"])}
+
+
+def suite(model, eng, d, sd):
+    """Extra lines for the other benchmark configs: backbone step at KV 256/1024/4096, depth head alone,
+    16 int8 streams with ragged caches."""
     import torch
 
+    from tests.util import dims_to_config
+    from vui_amd.engine import Engine, GenConfig
+    from vui_amd.model import Vui
+
+    lines = []
     m = model.config.model
-    n = 200
-    L0 = 1024 - n // 2
-    eng._decode_step()  # captures on first use
-    eng.seq_lens[0] = L0
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(n):  # the cache length walks from 924 to 1124: 1024 on average
-        eng._decode_graph.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    us = e0.elapsed_time(e1) * 1e3 / n
-    b = frame_bytes(m, L0 + n / 2)["backbone"]
-    ach = b / (us * 1e-6) / 1e9
-    return {"bound": "hbm", "kernel": "backbone decode step (graph of fused RMSNorm+GEMV / attention kernels), KV len 1024",
-            "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
-            "traffic": None, "us_per_launch": round(us, 2), "algorithmic_bytes": int(b)}
+
+    def timed(fn, n):
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / n
+
+    # config 2: backbone decode step, B=1, N(0,1) cache at three lengths (the walk over 200 steps is centred on L)
+    model2 = Vui(dims_to_config(d, 4608), sd, device="cuda", dtype=torch.bfloat16)
+    eng2 = Engine(model=model2, max_rows=1, max_seq=4608)
+    model2.decoder._k.normal_()
+    model2.decoder._v.normal_()
+    eng2._decode_step()
+    for L in (256, 1024, 4096):
+        n = 200
+        eng2.seq_lens[0] = L - n // 2
+        us = timed(eng2._decode_graph.replay, n)
+        b = frame_bytes(m, L)["backbone"]
+        lines.append({"config": "backbone_step_b1", "kv_len": L, "us_per_step": round(us, 2), "us_per_layer": round(us / m.n_layers, 2),
+                      "algorithmic_bytes": int(b), "achieved_GBs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4)})
+    # config 3: depth head alone, 1000 frames, T=0.8 top-k 50
+    rq = model2.rq_transformer
+    rq.setup_cuda_graph_kv(model2.device, torch.bfloat16, top_k=50, batch_sizes=(1,))
+    g = torch.Generator().manual_seed(0)
+    hid = torch.randn(1, m.d_model, generator=g).to(torch.bfloat16).cuda()
+    c0 = torch.randint(0, m.codebook_size, (1,), generator=g).cuda()
+    rq.generate_cuda_graph_kv(hid, c0, 0.8)
+    gr = rq._gkv_graphs[(1, m.n_quantizers, 0.8)]
+    us = timed(gr.replay, 1000)
+    b = frame_bytes(m, 0)["rq_unique"]
+    lines.append({"config": "rq_head_b1", "frames": 1000, "us_per_frame": round(us, 2), "unique_bytes": int(b),
+                  "achieved_GBs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4)})
+    del eng2, model2
+    # config 5: 16 streams, int8 backbone weights, ragged caches U[128, 2048]
+    S = 2048 + 256
+    model5 = Vui(dims_to_config(d, S), sd, device="cuda", dtype=torch.bfloat16, int8=True)
+    eng5 = Engine(model=model5, max_rows=16, max_seq=S)
+    model5.decoder._k.normal_()
+    model5.decoder._v.normal_()
+    lens = torch.randint(128, 2049, (16,), generator=g)
+    rows = [eng5.new_row() for _ in range(16)]
+    eng5.seq_lens[:16] = lens.to(torch.int32).cuda()
+    hid16 = torch.randn(16, m.d_model, generator=g).to(torch.bfloat16).cuda()
+    n = 100
+    eng5.generate(rows, hid16, 1, GenConfig())
+    gr5, _, _, _ = eng5._frame_graph(16, GenConfig(), None, n + 1)
+    eng5.seq_lens[:16] = lens.to(torch.int32).cuda()
+    us = timed(gr5.replay, n)
+    kv_bytes = float((lens.float() + n / 2 + 1).sum()) * 2 * m.kv_heads * m.head_dim * 2 * m.n_layers
+    wbytes = frame_bytes(m, 0, 1)["backbone"] - (m.n_quantizers * m.d_model + 2 * m.kv_heads * m.head_dim * 2 * m.n_layers)
+    lines.append({"config": "e2e_b16_int8_ragged", "us_per_frame_step": round(us, 1), "aggregate_frames_per_s": round(16e6 / us, 1),
+                  "kv_bytes": int(kv_bytes), "int8_weight_bytes": int(wbytes),
+                  "achieved_GBs": round((kv_bytes + wbytes) / us / 1e3, 1)})
+    return lines
 
 
 def cpu_baseline(d, sd, n_frames: int = 12, n_ctx: int = 96):
@@ -158,6 +221,9 @@ def main():
     ap.add_argument("--preset", default="A", choices=["A", "B"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--suite", action="store_true", help="also print one JSON line per further benchmark config")
+    ap.add_argument("--calib", action="store_true",
+                    help="end with three plain 512 MiB device copies (reference points for hardware counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (streams are independent); "
@@ -165,10 +231,21 @@ def main():
         sys.exit(2)
     out, (model, eng, d, sd) = gpu_bench(args)
     if not args.no_roofline:
-        out["roofline"] = kernel_roofline(model, eng)
+        out["roofline"] = kernel_roofline(out, out["frame_bytes"])
+    extra = suite(model, eng, d, sd) if args.suite else []
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(d, sd)
+    if args.calib:
+        import torch
+
+        src = torch.empty(512 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
     print(json.dumps(out))
+    for ln in extra:
+        print(json.dumps(ln))
 
 
 if __name__ == "__main__":
