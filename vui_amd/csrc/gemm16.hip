@@ -1,0 +1,187 @@
+// Skinny GEMM for 9..16 activation rows on the matrix cores: y (B, N) = x (B, K) W^T (N, K).
+//
+// One workgroup owns 16 consecutive output features; its four waves split K in steps of 64 and
+// each issues v_mfma_f32_16x16x32_bf16 with A = a 16 x 32 weight tile (lane i: feature i % 16,
+// eight consecutive k) and B = the activations (lane i: row i % 16, the same k), so the 16 x 16
+// fp32 accumulator holds all rows of 16 features.  Each lane reads 32 contiguous weight bytes per
+// step (two MFMAs), i.e. a full 128-byte line per feature; the k order inside a step is permuted the
+// same way for A and B, which a dot product does not see.  int8 weights are widened to bf16 in
+// registers (exact) and scaled per feature in the epilogue.  Activations are staged in LDS as bf16
+// after the two-rounding RMSNorm (src/vui/model.py:286-297); row stride K + 8 keeps the 16 rows of a
+// B-operand read on distinct banks.
+#include "common.h"
+#include "gemv_epi.h"
+#include "internal.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+#define G16_THREADS 256
+#define G16_MAXS 8  // K steps (of 64) per wave held in registers: K <= 2048
+
+union U128 { uint4 u; bf16x8 v; };
+
+__device__ __forceinline__ bf16x8 as_bf16x8(const uint4& x) { U128 t; t.u = x; return t.v; }
+
+// 8 int8 (two dwords) -> 8 bf16, exact
+__device__ __forceinline__ uint4 i8x8_to_bf16(uint32_t lo, uint32_t hi) {
+  auto cv = [](uint32_t w, int sh) -> uint32_t {
+    const float f = (float)(int8_t)((w >> sh) & 0xff);
+    return __float_as_uint(f) >> 16;
+  };
+  uint4 r;
+  r.x = cv(lo, 0) | (cv(lo, 8) << 16);
+  r.y = cv(lo, 16) | (cv(lo, 24) << 16);
+  r.z = cv(hi, 0) | (cv(hi, 8) << 16);
+  r.w = cv(hi, 16) | (cv(hi, 24) << 16);
+  return r;
+}
+
+template <typename WT> struct W16;
+template <> struct W16<bf16_t> {
+  struct Raw { uint4 lo, hi; };
+  static __device__ __forceinline__ Raw load(const bf16_t* p) {
+    Raw r; r.lo = *reinterpret_cast<const uint4*>(p); r.hi = *reinterpret_cast<const uint4*>(p + 8); return r;
+  }
+  static __device__ __forceinline__ Raw zero() { Raw r; r.lo = make_uint4(0, 0, 0, 0); r.hi = r.lo; return r; }
+  static __device__ __forceinline__ void split(const Raw& r, uint4& a, uint4& b) { a = r.lo; b = r.hi; }
+};
+template <> struct W16<int8_t> {
+  typedef uint4 Raw;  // 16 int8
+  static __device__ __forceinline__ Raw load(const int8_t* p) { return *reinterpret_cast<const uint4*>(p); }
+  static __device__ __forceinline__ Raw zero() { return make_uint4(0, 0, 0, 0); }
+  static __device__ __forceinline__ void split(const Raw& r, uint4& a, uint4& b) {
+    a = i8x8_to_bf16(r.x, r.y); b = i8x8_to_bf16(r.z, r.w);
+  }
+};
+
+template <typename WT, bool DUAL>
+__global__ __launch_bounds__(G16_THREADS) void gemm16_kernel(const GemvArgs p) {
+  extern __shared__ __align__(16) unsigned char smem16[];
+  const int K = p.K, KP = K + 8;
+  bf16_t* xs = (bf16_t*)smem16;                       // 16 x KP
+  float* red = (float*)(smem16 + (size_t)16 * KP * 2);  // 4 waves x 64 lanes x (4 | 8)
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int f16 = lane & 15, kg = lane >> 4;
+  const int n0 = (int)blockIdx.x * 16;
+  const int row = min(n0 + f16, p.N - 1);
+  const int nsteps = (K + 63) >> 6;
+
+  // this wave's weight tiles: steps wave, wave + 4, ...
+  typename W16<WT>::Raw wr[G16_MAXS], wr2[DUAL ? G16_MAXS : 1];
+  const WT* wrow = (const WT*)p.W + (size_t)row * K;
+  const WT* wrow2 = DUAL ? (const WT*)p.W2 + (size_t)row * K : nullptr;
+#pragma unroll
+  for (int i = 0; i < G16_MAXS; ++i) {
+    const int k = (wave + 4 * i) * 64 + kg * 16;
+    const bool on = (wave + 4 * i) < nsteps && k < K;  // K is a multiple of 16 here
+    wr[i] = on ? W16<WT>::load(wrow + k) : W16<WT>::zero();
+    if (DUAL) wr2[i] = on ? W16<WT>::load(wrow2 + k) : W16<WT>::zero();
+  }
+
+  // activations -> LDS (bf16), rows >= B are zero
+  {
+    const bf16_t* x = (const bf16_t*)p.x;
+    const bf16_t* nw = (const bf16_t*)p.norm_w;
+    for (int b = wave; b < 16; b += 4) {
+      bf16_t* dst = xs + (size_t)b * KP;
+      if (b >= p.B) { for (int k = lane; k < K; k += WAVE) dst[k] = 0; continue; }
+      const bf16_t* xr = x + (size_t)b * K;
+      if (nw) {
+        float ss = 0.f;
+        for (int k = lane; k < K; k += WAVE) { const float v = bf2f(xr[k]); ss += v * v; }
+        ss = wave_sum(ss);
+        const float r = 1.0f / sqrtf(ss / (float)K + p.eps);
+        for (int k = lane; k < K; k += WAVE) {
+          const float v = bf2f(f2bf(bf2f(xr[k]) * r));
+          dst[k] = f2bf(v * bf2f(nw[k]));
+        }
+      } else {
+        for (int k = lane; k < K; k += WAVE) dst[k] = xr[k];
+      }
+    }
+  }
+  __syncthreads();
+
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < G16_MAXS; ++i) {
+    const int step = wave + 4 * i;
+    if (step < nsteps) {
+      const int k = step * 64 + kg * 16;
+      if (k < K) {
+        const bf16_t* xp = xs + (size_t)f16 * KP + k;
+        const uint4 b_lo = *reinterpret_cast<const uint4*>(xp);
+        const uint4 b_hi = *reinterpret_cast<const uint4*>(xp + 8);
+        uint4 a_lo, a_hi;
+        W16<WT>::split(wr[i], a_lo, a_hi);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_lo), as_bf16x8(b_lo), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_hi), as_bf16x8(b_hi), acc, 0, 0, 0);
+        if (DUAL) {
+          W16<WT>::split(wr2[i], a_lo, a_hi);
+          acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_lo), as_bf16x8(b_lo), acc2, 0, 0, 0);
+          acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_hi), as_bf16x8(b_hi), acc2, 0, 0, 0);
+        }
+      }
+    }
+  }
+  // add the four K parts in a fixed order
+  const int per = DUAL ? 8 : 4;
+  float* mine = red + ((size_t)wave * 64 + lane) * per;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) { mine[r] = acc[r]; if (DUAL) mine[4 + r] = acc2[r]; }
+  __syncthreads();
+  if (wave != 0) return;
+  float v[4], v2[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    v[r] = 0.f; v2[r] = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      v[r] += red[((size_t)w * 64 + lane) * per + r];
+      if (DUAL) v2[r] += red[((size_t)w * 64 + lane) * per + 4 + r];
+    }
+  }
+  // lane holds features n0 + 4 * kg + r (r = 0..3) of activation row f16
+  const int b = f16;
+  if (b >= p.B) return;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int n = n0 + 4 * kg + r;
+    if (n < p.N) {
+      float a = v[r], ap = v[r ^ 1], a2 = v2[r];
+      if (p.w_int8) {
+        a *= bf2f(((const bf16_t*)p.sc)[n]);
+        ap *= bf2f(((const bf16_t*)p.sc)[min(n ^ 1, p.N - 1)]);
+        if (DUAL) a2 *= bf2f(((const bf16_t*)p.sc2)[n]);
+      }
+      epilogue<bf16_t>(p, n, b, a, ap, a2);
+    }
+  }
+}
+
+static size_t g16_lds(int K, bool dual) { return (size_t)16 * (K + 8) * 2 + (size_t)4 * 64 * (dual ? 8 : 4) * 4; }
+
+template <typename WT, bool DUAL>
+static int launch_g16(const GemvArgs& a, hipStream_t st) {
+  static size_t attr = 0;
+  const size_t lds = g16_lds(a.K, DUAL);
+  if (lds > 64 * 1024 && lds > attr) {
+    HIP_TRY(hipFuncSetAttribute((const void*)gemm16_kernel<WT, DUAL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr = lds;
+  }
+  hipLaunchKernelGGL((gemm16_kernel<WT, DUAL>), dim3((a.N + 15) / 16), dim3(G16_THREADS), lds, st, a);
+  HIP_TRY(hipGetLastError());
+  return VUI_OK;
+}
+
+bool gemm16_supported(const GemvArgs& a) {
+  return a.dtype == VUI_DTYPE_BF16 && a.B > 8 && a.B <= 16 && (a.K % 16) == 0 && a.K <= G16_MAXS * 4 * 64 &&
+         g16_lds(a.K, a.epi == EPI_SWIGLU) <= 150 * 1024;
+}
+
+int launch_gemm16(const GemvArgs& a, hipStream_t st) {
+  const bool dual = a.epi == EPI_SWIGLU;
+  if (a.w_int8) return dual ? launch_g16<int8_t, true>(a, st) : launch_g16<int8_t, false>(a, st);
+  return dual ? launch_g16<bf16_t, true>(a, st) : launch_g16<bf16_t, false>(a, st);
+}

@@ -51,6 +51,9 @@ struct GemvArgs {
 };
 
 int launch_gemv(const GemvArgs& a, hipStream_t st);
+// 16-row MFMA form of the same operation (gemm16.hip); the extra row / position update of `a` is not handled there
+bool gemm16_supported(const GemvArgs& a);
+int launch_gemm16(const GemvArgs& a, hipStream_t st);
 
 struct AttnArgs {
   int dtype;
