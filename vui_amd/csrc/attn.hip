@@ -52,19 +52,29 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attn_kernel(const AttnArgs
   const T* kbase = (const T*)p.kc + ((size_t)slot * p.S) * rowstride + kvh * hd + l16 * 8;
   const T* vbase = (const T*)p.vc + ((size_t)slot * p.S) * rowstride + kvh * hd + l16 * 8;
 
-  // pass 1: scores
+  // pass 1: scores (four keys per lane group in flight)
   float mloc = -INFINITY;
-  for (int j = lo + g; j < hi; j += ATT_KEYS_PER_ITER) {
-    float k8[8];
-    float d = 0.f;
-    if (act) {
-      El<T>::ld8(kbase + (size_t)j * rowstride, k8);
+  for (int j0 = lo + g; j0 < hi; j0 += 4 * ATT_KEYS_PER_ITER) {
+    float k8[4][8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) d = fmaf(q8[e], k8[e], d);
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + u * ATT_KEYS_PER_ITER;
+      if (act && j < hi) El<T>::ld8(kbase + (size_t)j * rowstride, k8[u]);
     }
-    d = group16_sum(d) * scale;
-    if (l16 == 0) sc[j - lo] = d;
-    mloc = fmaxf(mloc, d);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + u * ATT_KEYS_PER_ITER;
+      if (j < hi) {
+        float d = 0.f;
+        if (act) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) d = fmaf(q8[e], k8[u][e], d);
+        }
+        d = group16_sum(d) * scale;
+        if (l16 == 0) sc[j - lo] = d;
+        mloc = fmaxf(mloc, d);
+      }
+    }
   }
   if (l16 == 0) red[g] = mloc;
   __syncthreads();
@@ -77,14 +87,24 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attn_kernel(const AttnArgs
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
   float l = 0.f;
-  for (int j = lo + g; j < hi; j += ATT_KEYS_PER_ITER) {
-    const float pw = expf(sc[j - lo] - M);
-    l += pw;
-    if (act) {
-      float v8[8];
-      El<T>::ld8(vbase + (size_t)j * rowstride, v8);
+  for (int j0 = lo + g; j0 < hi; j0 += 4 * ATT_KEYS_PER_ITER) {
+    float v8[4][8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] = fmaf(pw, v8[e], acc[e]);
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + u * ATT_KEYS_PER_ITER;
+      if (act && j < hi) El<T>::ld8(vbase + (size_t)j * rowstride, v8[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + u * ATT_KEYS_PER_ITER;
+      if (j < hi) {
+        const float pw = expf(sc[j - lo] - M);
+        l += pw;
+        if (act) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[e] = fmaf(pw, v8[u][e], acc[e]);
+        }
+      }
     }
   }
   if (act) {

@@ -21,6 +21,13 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
 union U128 { uint4 u; bf16x8 v; };
 
+__device__ __forceinline__ void cvt8u(const uint4& r, float* o) {
+  o[0] = __uint_as_float(r.x << 16); o[1] = __uint_as_float(r.x & 0xffff0000u);
+  o[2] = __uint_as_float(r.y << 16); o[3] = __uint_as_float(r.y & 0xffff0000u);
+  o[4] = __uint_as_float(r.z << 16); o[5] = __uint_as_float(r.z & 0xffff0000u);
+  o[6] = __uint_as_float(r.w << 16); o[7] = __uint_as_float(r.w & 0xffff0000u);
+}
+
 __device__ __forceinline__ bf16x8 as_bf16x8(const uint4& x) { U128 t; t.u = x; return t.v; }
 
 // 8 int8 (two dwords) -> 8 bf16, exact
@@ -79,25 +86,58 @@ __global__ __launch_bounds__(G16_THREADS) void gemm16_kernel(const GemvArgs p) {
     if (DUAL) wr2[i] = on ? W16<WT>::load(wrow2 + k) : W16<WT>::zero();
   }
 
-  // activations -> LDS (bf16), rows >= B are zero
+  // activations -> LDS (bf16), rows >= B are zero.  A wave stages rows wave, wave+4, ...: all their
+  // 16-byte chunks (and the norm weights) are requested first, then normalised and written.
   {
     const bf16_t* x = (const bf16_t*)p.x;
     const bf16_t* nw = (const bf16_t*)p.norm_w;
-    for (int b = wave; b < 16; b += 4) {
+    const int nch = K >> 3;  // 8-element chunks per row (K is a multiple of 16)
+    uint4 xr[4][4], wn[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = lane + WAVE * i;
+      wn[i] = (nw && c < nch) ? *reinterpret_cast<const uint4*>(nw + c * 8) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int b = wave + 4 * j;
+        xr[j][i] = (b < p.B && c < nch) ? *reinterpret_cast<const uint4*>(x + (size_t)b * K + c * 8) : make_uint4(0, 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int b = wave + 4 * j;
       bf16_t* dst = xs + (size_t)b * KP;
-      if (b >= p.B) { for (int k = lane; k < K; k += WAVE) dst[k] = 0; continue; }
-      const bf16_t* xr = x + (size_t)b * K;
+      float r = 1.f;
       if (nw) {
         float ss = 0.f;
-        for (int k = lane; k < K; k += WAVE) { const float v = bf2f(xr[k]); ss += v * v; }
-        ss = wave_sum(ss);
-        const float r = 1.0f / sqrtf(ss / (float)K + p.eps);
-        for (int k = lane; k < K; k += WAVE) {
-          const float v = bf2f(f2bf(bf2f(xr[k]) * r));
-          dst[k] = f2bf(v * bf2f(nw[k]));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float v8[8];
+          cvt8u(xr[j][i], v8);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) ss = fmaf(v8[e], v8[e], ss);
         }
-      } else {
-        for (int k = lane; k < K; k += WAVE) dst[k] = xr[k];
+        ss = wave_sum(ss);
+        r = 1.0f / sqrtf(ss / (float)K + p.eps);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = lane + WAVE * i;
+        if (c < nch) {
+          uint4 o = xr[j][i];
+          if (nw) {
+            float v8[8], w8[8], y8[8];
+            cvt8u(xr[j][i], v8);
+            cvt8u(wn[i], w8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) y8[e] = bf2f(f2bf(v8[e] * r)) * w8[e];
+            o.x = (uint32_t)f2bf(y8[0]) | ((uint32_t)f2bf(y8[1]) << 16);
+            o.y = (uint32_t)f2bf(y8[2]) | ((uint32_t)f2bf(y8[3]) << 16);
+            o.z = (uint32_t)f2bf(y8[4]) | ((uint32_t)f2bf(y8[5]) << 16);
+            o.w = (uint32_t)f2bf(y8[6]) | ((uint32_t)f2bf(y8[7]) << 16);
+          }
+          *reinterpret_cast<uint4*>(dst + c * 8) = o;
+        }
       }
     }
   }

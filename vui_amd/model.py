@@ -283,7 +283,7 @@ class Decoder:
     def default_splits(self, B: int) -> int:
         """Key-range splits per (row, head) so that B*H*splits workgroups roughly fill 256 CUs."""
         H = self._model.config.model.n_heads
-        return max(1, min(32, 512 // max(1, B * H)))
+        return max(1, min(32, 1024 // max(1, B * H)))
 
     def forward_flash(self, x: Tensor, positions: Tensor, per_sample_positions: bool = False,
                       slot_idx: Tensor | None = None) -> Tensor:
