@@ -218,3 +218,48 @@ def test_sampler_histogram(lib):
     chi2 = (((hist - exp) ** 2)[keep] / exp[keep]).sum()
     dof = keep.sum() - 1
     assert chi2 < dof + 5 * (2 * dof) ** 0.5, (chi2, dof)
+
+
+@pytest.mark.parametrize("CS,top_k", [(2048, 100), (2048, 1000), (32, 5), (1000, 37)])
+def test_sampler_16bit_key_search_equals_32bit(lib, CS, top_k):
+    """bf16 logits take the two-round 8-bit histogram search for the k-th largest key; with a
+    repetition state attached (all counts zero, so values are unchanged) the same logits take the
+    generic 32-bit search.  Same (seed, frame) -> same picks, and the picks lie in the oracle's kept set."""
+    from vui_amd import _lib
+
+    B = 16
+    g = torch.Generator().manual_seed(CS * 7 + top_k)
+    lg = (torch.randn(B, CS, generator=g) * 2).to(BF)
+    lg[2, :CS // 2] = lg[2, 0]  # heavy ties around the cut
+    cfgc = _lib.VuiConfigC()
+    cfgc.dtype, cfgc.d_model, cfgc.n_layers, cfgc.n_heads, cfgc.n_kv_heads, cfgc.head_dim, cfgc.ffn = 0, 64, 1, 4, 4, 16, 64
+    cfgc.n_quantizers, cfgc.codebook_size, cfgc.rq_dim, cfgc.rq_layers, cfgc.rq_heads, cfgc.rq_ffn = 4, CS, 64, 0, 1, 8
+    cfgc.rope_dim, cfgc.max_seqlen, cfgc.n_slots, cfgc.norm_eps, cfgc.rq_norm_eps = 16, 16, 1, 1e-5, 1e-6
+    n = lib.vui_workspace_bytes(C.byref(cfgc), 16)
+    assert n > 0, _lib.last_error()
+    ws = torch.zeros(n + 256, dtype=torch.uint8, device="cuda")
+    dummy = torch.zeros(64, dtype=torch.float32, device="cuda")
+    w = _lib.WeightsC()
+    for f in ("audio_emb", "final_norm", "codec_head", "eos_w", "eos_b", "rope_table"):
+        setattr(w, f, dummy.data_ptr())
+    for f in ("attn_norm", "wqkv", "wo", "mlp_norm", "w1", "w3", "w2"):
+        setattr(w.layers[0], f, dummy.data_ptr())
+    h = C.c_void_p()
+    _lib.check(lib.vui_ctx_create(C.byref(cfgc), C.byref(w), (ws.data_ptr() + 255) & ~255, n, 16, C.byref(h)), "ctx")
+    ld = lg.cuda()
+    counts = torch.zeros(B, CS, dtype=torch.float32, device="cuda")
+    for frame in range(20):
+        ctr = torch.tensor([frame], dtype=torch.int32, device="cuda")
+        sp = _lib.SampleParamsC()
+        sp.temperature, sp.top_k, sp.seed, sp.frame_ctr = 0.9, top_k, 99, ctr.data_ptr()
+        a = torch.empty(B, dtype=torch.long, device="cuda")
+        b = torch.empty(B, dtype=torch.long, device="cuda")
+        _lib.check(lib.vui_sample_cb0(h, ld.data_ptr(), None, None, None, 1.0, 0, C.byref(sp), a.data_ptr(), B, stream()), "a")
+        counts.zero_()
+        _lib.check(lib.vui_sample_cb0(h, ld.data_ptr(), counts.data_ptr(), None, None, 1.0001, 0, C.byref(sp), b.data_ptr(), B,
+                                      stream()), "b")
+        assert torch.equal(a, b), frame
+        for r in range(B):
+            kept = O.cb0_probs(lg[r].float(), 0.9, top_k)
+            assert kept[int(a[r])] > 0
+    lib.vui_ctx_destroy(h)

@@ -253,7 +253,7 @@ __device__ __forceinline__ void poll_add(float* dst, const uint64_t* buf, int nw
 #define LDS_RED (LDS_QKV + 1536)         // 64 floats
 #define LDS_MISC (LDS_RED + 256)         // 64 ints: sampled codes of the frame
 #define LDS_SAMP (LDS_MISC + 256)        // SampleShared
-#define LDS_FIXED (LDS_SAMP + 192)
+#define LDS_FIXED (LDS_SAMP + 1280)
 
 // optional per-phase timestamps (100 MHz wall clock) written by one workgroup, for profiling
 #define TS(id)                                                                                    \

@@ -31,6 +31,8 @@ struct SampleShared {
   float wsum[SAMP_THREADS / WAVE];
   int cnt[2][3 * SAMP_THREADS / WAVE];
   int pick;
+  int hist[256];   // 8-bit digit histogram of the 16-bit key search
+  int sel[2];      // chosen digit, count of keys above it
 #ifdef VUI_SAMPLE_CLOCK
   unsigned long long ts[8];
 #endif
@@ -77,9 +79,50 @@ __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32
   if (greedy) return Mi;
   SAMP_TS(1);
 
-  // key of the k-th largest value, two bits per step
+  // key of the k-th largest value
   uint32_t thr = 0u;
-  if (top_k > 0 && top_k < CS) {
+  if (top_k > 0 && top_k < CS && low_bit == 16) {
+    // 16-bit keys: two rounds of an 8-bit digit histogram in LDS (high byte, then low byte among the
+    // keys that share the chosen high byte); the digit is the largest one whose suffix count reaches k
+    int need = top_k;
+#pragma unroll
+    for (int round = 0; round < 2; ++round) {
+      const int shift = round == 0 ? 24 : 16;
+      sh.hist[tid] = 0;  // SAMP_THREADS == 256 bins
+      __syncthreads();
+#pragma unroll
+      for (int e = 0; e < EMAX; ++e)
+        if (e < E && tid * E + e < CS && (round == 0 || (key[e] >> 24) == (thr >> 24)))
+          atomicAdd(&sh.hist[(key[e] >> shift) & 255], 1);
+      __syncthreads();
+      // suffix sums over the 256 bins: thread t owns bin t; S(t) = sum of bins >= t
+      const int mine = sh.hist[tid];
+      // reverse inclusive scan: row_shl shifts (a lane reads from higher lanes of its row; lanes shifted in
+      // from outside read 0), then the totals of the higher rows
+      int v = mine;
+      v += dpp_i<0x101>(v);  // row_shl:1
+      v += dpp_i<0x102>(v);  // row_shl:2
+      v += dpp_i<0x104>(v);  // row_shl:4
+      v += dpp_i<0x108>(v);  // row_shl:8
+      {
+        const int t3 = __builtin_amdgcn_readlane(v, 48), t2 = __builtin_amdgcn_readlane(v, 32), t1 = __builtin_amdgcn_readlane(v, 16);
+        const int row = lane >> 4;
+        v += (row <= 2 ? t3 : 0) + (row <= 1 ? t2 : 0) + (row <= 0 ? t1 : 0);
+      }
+      if (lane == 0) sh.cnt[0][wave] = v;  // wave total
+      __syncthreads();
+      int above = 0;  // keys in higher waves' bins
+#pragma unroll
+      for (int w = 0; w < SAMP_THREADS / WAVE; ++w) if (w > wave) above += sh.cnt[0][w];
+      const int suffix = v + above;          // keys with digit >= tid
+      const int suffix_next = suffix - mine; // keys with digit > tid
+      if (suffix >= need && suffix_next < need) { sh.sel[0] = tid; sh.sel[1] = suffix_next; }
+      __syncthreads();
+      thr |= (uint32_t)sh.sel[0] << shift;
+      need -= sh.sel[1];
+      __syncthreads();
+    }
+  } else if (top_k > 0 && top_k < CS) {
     int it = 0;
     for (int bit = 30; bit >= low_bit; bit -= 2, ++it) {
       const uint32_t c1 = thr | (1u << bit), c2 = thr | (2u << bit), c3 = thr | (3u << bit);
@@ -88,7 +131,7 @@ __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32
 #pragma unroll
       for (int e = 0; e < EMAX; ++e)
         if (e < E) pk += (key[e] >= c1 ? 1 : 0) + (key[e] >= c2 ? (1 << 10) : 0) + (key[e] >= c3 ? (1 << 20) : 0);
-      pk = wave_sum_i(pk);  // per field at most 64 * EMAX <= 1023 when EMAX <= 15; wider EMAX uses two sums
+      pk = wave_sum_i(pk);  // per field at most 64 * EMAX <= 1023 when EMAX <= 15; wider EMAX uses three sums
       int n1 = pk & 1023, n2 = (pk >> 10) & 1023, n3 = (pk >> 20) & 1023;
       if (EMAX > 15) {
         int q1 = 0, q2 = 0, q3 = 0;
