@@ -9,12 +9,15 @@ typedef uint16_t bf16_t;  // raw bfloat16 bits
 
 __device__ __forceinline__ float bf2f(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
 
-// round-to-nearest-even, NaN kept quiet (same result as torch's float -> bfloat16)
-__device__ __forceinline__ bf16_t f2bf(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
+// round-to-nearest-even, NaN kept quiet (same result as torch's float -> bfloat16): gfx950 converts in
+// hardware (v_cvt_pk_bf16_f32), bit-identical to the integer formula on every fp32 input
+__device__ __forceinline__ bf16_t f2bf(float f) { return __builtin_bit_cast(bf16_t, (__bf16)f); }
+// two values -> one packed word (low half = a)
+__device__ __forceinline__ uint32_t f2bf2(float a, float b) {
+  typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
+  typedef float f2_t __attribute__((ext_vector_type(2)));
+  const f2_t v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf2_t));
 }
 
 template <typename T> struct El;
@@ -32,10 +35,10 @@ template <> struct El<bf16_t> {
   }
   static __device__ __forceinline__ void st8(bf16_t* p, const float* v) {
     uint4 r;
-    r.x = (uint32_t)f2bf(v[0]) | ((uint32_t)f2bf(v[1]) << 16);
-    r.y = (uint32_t)f2bf(v[2]) | ((uint32_t)f2bf(v[3]) << 16);
-    r.z = (uint32_t)f2bf(v[4]) | ((uint32_t)f2bf(v[5]) << 16);
-    r.w = (uint32_t)f2bf(v[6]) | ((uint32_t)f2bf(v[7]) << 16);
+    r.x = f2bf2(v[0], v[1]);
+    r.y = f2bf2(v[2], v[3]);
+    r.z = f2bf2(v[4], v[5]);
+    r.w = f2bf2(v[6], v[7]);
     *reinterpret_cast<uint4*>(p) = r;
   }
 };

@@ -28,7 +28,7 @@ __device__ __forceinline__ uint64_t ll_ld(const uint64_t* p) {
 __device__ __forceinline__ void ll_st(uint64_t* p, uint32_t payload, uint32_t epoch) {
   __hip_atomic_store(p, ((uint64_t)epoch << 32) | payload, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ uint32_t pack2(float a, float b) { return (uint32_t)f2bf(a) | ((uint32_t)f2bf(b) << 16); }
+__device__ __forceinline__ uint32_t pack2(float a, float b) { return f2bf2(a, b); }
 
 struct Ctl {
   uint32_t epoch;
@@ -210,20 +210,30 @@ __device__ __forceinline__ NormW load_normw(const bf16_t* nw, int K) {
   }
   return r;
 }
-// two-rounding RMSNorm of src[0..K) (LDS, K <= 1024) into dst (LDS); every wave derives the same scale
+// two-rounding RMSNorm of src[0..K) into dst (both LDS; src holds 1024 floats, K <= 1024, K % 4 == 0);
+// every wave derives the same scale.  Straight-line: all LDS reads are issued before any use.
 __device__ __forceinline__ void stage_norm(const float* src, const NormW& nw, float eps, int K, float* dst) {
   const int lane = threadIdx.x & 63;
+  float4 q[4];
+  float own[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) q[i] = *reinterpret_cast<const float4*>(src + 4 * lane + 256 * i);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) own[i] = src[(int)threadIdx.x + FR_THREADS * i];
   float ss = 0.f;
-  for (int k = lane; k < K; k += WAVE) { const float v = src[k]; ss += v * v; }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float t = (q[i].x * q[i].x + q[i].y * q[i].y) + (q[i].z * q[i].z + q[i].w * q[i].w);
+    ss += (4 * lane + 256 * i < K) ? t : 0.f;
+  }
   ss = wave_sum(ss);
   const float r = 1.0f / sqrtf(ss / (float)K + eps);
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int k = (int)threadIdx.x + FR_THREADS * i;
-    if (k < K) {
-      const float v = bf2f(f2bf(src[k] * r));
-      dst[k] = bf2f(f2bf(v * nw.w[i]));
-    }
+    const float v = bf2f(f2bf(own[i] * r));
+    const float o = bf2f(f2bf(v * nw.w[i]));
+    if (k < K) dst[k] = o;
   }
 }
 
@@ -859,7 +869,9 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           poll_add(xres, ob, R / 2, c);
           TS(35);
           stage_norm(xres, nw2, a.rq_eps, R, xn);
+          TS(70);
           __syncthreads();
+          TS(71);
           gemv_compute<2, true>(xn, R_sw, wr, red, [&](int gp, float v0, float v1, float u0, float u1) {
             const float a0 = bf2f(f2bf(v0)), a1 = bf2f(f2bf(v1)), c0 = bf2f(f2bf(u0)), c1 = bf2f(f2bf(u1));
             const float s0 = bf2f(f2bf(a0 / (1.0f + expf(-a0)))), s1 = bf2f(f2bf(a1 / (1.0f + expf(-a1))));
