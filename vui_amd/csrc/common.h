@@ -20,6 +20,20 @@ __device__ __forceinline__ uint32_t f2bf2(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf2_t));
 }
 
+// acc + w.lo*x.lo + w.hi*x.hi on packed bf16 pairs, fp32 accumulate (v_dot2c_f32_bf16)
+__device__ __forceinline__ float dot2_bf(uint32_t w, uint32_t x, float acc) {
+  typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf2_t, w), __builtin_bit_cast(bf2_t, x), acc, false);
+}
+__device__ __forceinline__ float dot8_bf(const uint4& w, const uint4& x, float acc) {
+  acc = dot2_bf(w.x, x.x, acc);
+  acc = dot2_bf(w.y, x.y, acc);
+  acc = dot2_bf(w.z, x.z, acc);
+  return dot2_bf(w.w, x.w, acc);
+}
+__device__ __forceinline__ float bf_lo(uint32_t v) { return __uint_as_float(v << 16); }
+__device__ __forceinline__ float bf_hi(uint32_t v) { return __uint_as_float(v & 0xffff0000u); }
+
 template <typename T> struct El;
 template <> struct El<bf16_t> {
   static __device__ __forceinline__ float ld(const bf16_t* p) { return bf2f(*p); }

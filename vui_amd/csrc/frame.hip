@@ -142,40 +142,30 @@ __device__ __forceinline__ void gemv_prefetch(const bf16_t* W, const bf16_t* W2,
       }
 }
 
-// xs: K staged activations in LDS (fp32).  red: 4 x 4 floats of LDS.  epi(gp, v0, v1, u0, u1) is
-// called by one lane per finished pair with the fp32 dot products of rows 2gp, 2gp+1 (u*: second matrix).
+// xp: K staged activations in LDS as packed bf16 pairs (K/2 words; every activation this kernel
+// multiplies is a bf16 value, so nothing is lost).  red: 4 x 4 floats of LDS.  epi(gp, v0, v1, u0, u1)
+// is called by one lane per finished pair with the fp32 dot products of rows 2gp, 2gp+1 (u*: second matrix).
 template <int MAXC, bool DUAL, typename Epi>
-__device__ __forceinline__ void gemv_compute(const float* xs, const Plan& p, const WRegs<MAXC, DUAL>& r, float* red,
+__device__ __forceinline__ void gemv_compute(const uint32_t* xp, const Plan& p, const WRegs<MAXC, DUAL>& r, float* red,
                                              Epi&& epi) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   float res[2][4];
+  uint4 x[MAXC];
+  if (p.nslots > 0) {
+    // lanes beyond the K range hold zero weights; their reads are clamped to a staged chunk
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) x[i] = *reinterpret_cast<const uint4*>(xp + 4 * min(p.c0 + lane + WAVE * i, p.c1 - 1));
+  }
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     if (s < p.nslots) {
 #pragma unroll
       for (int i = 0; i < MAXC; ++i) {
-        const int c = p.c0 + lane + WAVE * i;
-        if (c < p.c1) {
-          const float4 xa = *reinterpret_cast<const float4*>(xs + c * 8);
-          const float4 xb = *reinterpret_cast<const float4*>(xs + c * 8 + 4);
-          const float xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
 #pragma unroll
-          for (int rr = 0; rr < 2; ++rr) {
-            float w[8];
-            cvt8(r.a[s][rr][i], w);
-            float t = acc[rr];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) t = fmaf(w[e], xv[e], t);
-            acc[rr] = t;
-            if (DUAL) {
-              cvt8(r.b[s][rr][i], w);
-              float t2 = acc[2 + rr];
-#pragma unroll
-              for (int e = 0; e < 8; ++e) t2 = fmaf(w[e], xv[e], t2);
-              acc[2 + rr] = t2;
-            }
-          }
+        for (int rr = 0; rr < 2; ++rr) {
+          acc[rr] = dot8_bf(r.a[s][rr][i], x[i], acc[rr]);
+          if (DUAL) acc[2 + rr] = dot8_bf(r.b[s][rr][i], x[i], acc[2 + rr]);
         }
       }
     }
@@ -199,27 +189,27 @@ __device__ __forceinline__ void gemv_compute(const float* xs, const Plan& p, con
   }
 }
 
-// norm weights of a thread's features (k = tid, tid+256, ...), fetched ahead of the wait
-struct NormW { float w[4]; };
+// norm weights of a thread's feature pairs (pairs tid and tid + 256), fetched ahead of the wait
+struct NormW { uint32_t w[2]; };
 __device__ __forceinline__ NormW load_normw(const bf16_t* nw, int K) {
   NormW r;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int k = (int)threadIdx.x + FR_THREADS * i;
-    r.w[i] = k < K ? bf2f(nw[k]) : 0.f;
+  for (int i = 0; i < 2; ++i) {
+    const int j = (int)threadIdx.x + FR_THREADS * i;
+    r.w[i] = 2 * j < K ? reinterpret_cast<const uint32_t*>(nw)[j] : 0u;
   }
   return r;
 }
-// two-rounding RMSNorm of src[0..K) into dst (both LDS; src holds 1024 floats, K <= 1024, K % 4 == 0);
-// every wave derives the same scale.  Straight-line: all LDS reads are issued before any use.
-__device__ __forceinline__ void stage_norm(const float* src, const NormW& nw, float eps, int K, float* dst) {
+// two-rounding RMSNorm of src[0..K) (LDS, 1024 floats, K <= 1024, K % 4 == 0) into packed bf16 pairs
+// dst[0..K/2); every wave derives the same scale.  Straight-line: all LDS reads are issued before any use.
+__device__ __forceinline__ void stage_norm(const float* src, const NormW& nw, float eps, int K, uint32_t* dst) {
   const int lane = threadIdx.x & 63;
   float4 q[4];
-  float own[4];
+  float2 own[2];
 #pragma unroll
   for (int i = 0; i < 4; ++i) q[i] = *reinterpret_cast<const float4*>(src + 4 * lane + 256 * i);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) own[i] = src[(int)threadIdx.x + FR_THREADS * i];
+  for (int i = 0; i < 2; ++i) own[i] = *reinterpret_cast<const float2*>(src + 2 * ((int)threadIdx.x + FR_THREADS * i));
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -227,30 +217,36 @@ __device__ __forceinline__ void stage_norm(const float* src, const NormW& nw, fl
     ss += (4 * lane + 256 * i < K) ? t : 0.f;
   }
   ss = wave_sum(ss);
-  const float r = 1.0f / sqrtf(ss / (float)K + eps);
+  const float r = __builtin_amdgcn_rsqf(ss * (1.0f / (float)K) + eps);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int k = (int)threadIdx.x + FR_THREADS * i;
-    const float v = bf2f(f2bf(own[i] * r));
-    const float o = bf2f(f2bf(v * nw.w[i]));
-    if (k < K) dst[k] = o;
+  for (int i = 0; i < 2; ++i) {
+    const int j = (int)threadIdx.x + FR_THREADS * i;
+    const uint32_t v = f2bf2(own[i].x * r, own[i].y * r);
+    const uint32_t o = f2bf2(bf_lo(v) * bf_lo(nw.w[i]), bf_hi(v) * bf_hi(nw.w[i]));
+    if (2 * j < K) dst[j] = o;
   }
 }
 
 // Exchange helpers: wait for a vector of bf16 pairs and put it into LDS.  Both carry the
 // workgroup barriers that separate them from earlier readers and later users of dst.
+__device__ __forceinline__ void poll_words(uint32_t* dst, const uint64_t* buf, int nwords, Ctl& c) {
+  __syncthreads();
+  ll_poll(buf, nwords, c, [&](int i, uint32_t v) { dst[i] = v; });
+  __syncthreads();
+}
 __device__ __forceinline__ void poll_set(float* dst, const uint64_t* buf, int nwords, Ctl& c) {
   __syncthreads();
   ll_poll(buf, nwords, c, [&](int i, uint32_t v) {
-    dst[2 * i] = bf2f((bf16_t)(v & 0xffff)); dst[2 * i + 1] = bf2f((bf16_t)(v >> 16)); });
+    *reinterpret_cast<float2*>(dst + 2 * i) = make_float2(bf_lo(v), bf_hi(v)); });
   __syncthreads();
 }
 // dst = rnd(dst + incoming): the residual add (src/vui/model.py:367, 374)
 __device__ __forceinline__ void poll_add(float* dst, const uint64_t* buf, int nwords, Ctl& c) {
   __syncthreads();
   ll_poll(buf, nwords, c, [&](int i, uint32_t v) {
-    dst[2 * i] = bf2f(f2bf(dst[2 * i] + bf2f((bf16_t)(v & 0xffff))));
-    dst[2 * i + 1] = bf2f(f2bf(dst[2 * i + 1] + bf2f((bf16_t)(v >> 16)))); });
+    const float2 o = *reinterpret_cast<const float2*>(dst + 2 * i);
+    const uint32_t pk = f2bf2(o.x + bf_lo(v), o.y + bf_hi(v));
+    *reinterpret_cast<float2*>(dst + 2 * i) = make_float2(bf_lo(pk), bf_hi(pk)); });
   __syncthreads();
 }
 
@@ -297,6 +293,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
   extern __shared__ __align__(16) unsigned char smem[];
   float* xres = (float*)(smem + LDS_XRES);
   float* xn = (float*)(smem + LDS_XN);
+  uint32_t* xp = (uint32_t*)(smem + LDS_XN);  // the same bytes as packed bf16 pairs
   float* lg = (float*)(smem + LDS_LG);
   float* sc = (float*)(smem + LDS_SC);
   float* qh = (float*)(smem + LDS_QKV);
@@ -433,12 +430,12 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       TS(1);
       if (ybuf) poll_add(xres, ybuf, d / 2, c);
       TS(2);
-      stage_norm(xres, nw1, a.eps, d, xn);
+      stage_norm(xres, nw1, a.eps, d, xp);
       __syncthreads();
       TS(3);
       uint64_t* qkvbuf = llp;
       llp += np_qkv;
-      gemv_compute<2, false>(xn, P_qkv, wr, red, [&](int gp, float v0, float v1, float, float) {
+      gemv_compute<2, false>(xp, P_qkv, wr, red, [&](int gp, float v0, float v1, float, float) {
         const bool s0 = (gp == P_qkv.gp[0]);
         float o0 = bf2f(f2bf(v0)), o1 = bf2f(f2bf(v1));
         const int rg = s0 ? q_region[0] : q_region[1];
@@ -620,9 +617,9 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
         WRegs<2, false> w2;
         const Plan P_o = plan_of(n_o, d, wg, nwg, wave);
         gemv_prefetch<2, false>(Lw.wo, nullptr, d, P_o, w2);
-        poll_set(xn, attbuf, d / 2, c);
+        poll_words(xp, attbuf, d / 2, c);
         TS(7);
-        gemv_compute<2, false>(xn, P_o, w2, red, [&](int gp, float v0, float v1, float, float) {
+        gemv_compute<2, false>(xp, P_o, w2, red, [&](int gp, float v0, float v1, float, float) {
           ll_st(obuf + gp, pack2(v0, v1), ep); });
       }
       TS(8);
@@ -636,10 +633,10 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
         const NormW nw2 = load_normw(Lw.mlp_norm, d);
         poll_add(xres, obuf, d / 2, c);
         TS(9);
-        stage_norm(xres, nw2, a.eps, d, xn);
+        stage_norm(xres, nw2, a.eps, d, xp);
         __syncthreads();
         TS(10);
-        gemv_compute<2, true>(xn, P_sw, w3, red, [&](int gp, float v0, float v1, float u0, float u1) {
+        gemv_compute<2, true>(xp, P_sw, w3, red, [&](int gp, float v0, float v1, float u0, float u1) {
           const float a0 = bf2f(f2bf(v0)), a1 = bf2f(f2bf(v1)), c0 = bf2f(f2bf(u0)), c1 = bf2f(f2bf(u1));
           const float s0 = bf2f(f2bf(a0 / (1.0f + expf(-a0)))), s1 = bf2f(f2bf(a1 / (1.0f + expf(-a1))));
           ll_st(hbuf + gp, pack2(s0 * c0, s1 * c1), ep);
@@ -653,9 +650,9 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
         WRegs<4, false> w4;
         const Plan P_w2 = plan_of(n_o, a.F, wg, nwg, wave);
         gemv_prefetch<4, false>(Lw.w2, nullptr, a.F, P_w2, w4);
-        poll_set(xn, hbuf, a.F / 2, c);
+        poll_words(xp, hbuf, a.F / 2, c);
         TS(12);
-        gemv_compute<4, false>(xn, P_w2, w4, red, [&](int gp, float v0, float v1, float, float) {
+        gemv_compute<4, false>(xp, P_w2, w4, red, [&](int gp, float v0, float v1, float, float) {
           ll_st(yb + gp, pack2(v0, v1), ep); });
       }
       ybuf = yb;
@@ -667,16 +664,16 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       WRegs<2, false> wr;
       gemv_prefetch<2, false>(g_codec_head, nullptr, d, p, wr);
       const NormW nwf = load_normw(g_final_norm, d);
-      float eosw[16];  // this lane's eos-head weights (k = lane, lane+64, ...), d <= 1024
+      uint32_t eosw[8];  // this lane's eos-head weight pairs (pair = lane, lane+64, ...), d <= 1024
 #pragma unroll
-      for (int i = 0; i < 16; ++i) { const int k = lane + WAVE * i; eosw[i] = k < d ? bf2f(g_eos_w[k]) : 0.f; }
+      for (int i = 0; i < 8; ++i) { const int j = lane + WAVE * i; eosw[i] = 2 * j < d ? reinterpret_cast<const uint32_t*>(g_eos_w)[j] : 0u; }
       const float eosb = bf2f(*g_eos_b);
       poll_add(xres, ybuf, d / 2, c);
-      stage_norm(xres, nwf, a.eps, d, xn);
+      stage_norm(xres, nwf, a.eps, d, xp);
       __syncthreads();
       uint64_t* lgbuf = llp;
       llp += a.CS / 2;
-      gemv_compute<2, false>(xn, p, wr, red, [&](int gp, float v0, float v1, float, float) {
+      gemv_compute<2, false>(xp, p, wr, red, [&](int gp, float v0, float v1, float, float) {
         const uint32_t pk = pack2(v0, v1);
         ll_st(lgbuf + gp, pk, ep);
         if (a.cb0_out) *reinterpret_cast<uint32_t*>(a.cb0_out + 2 * gp) = pk;
@@ -685,12 +682,12 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       {
         float t = 0.f;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) { const int k = lane + WAVE * i; if (k < d) t += xn[k] * eosw[i]; }
+        for (int i = 0; i < 8; ++i) { const int j = lane + WAVE * i; t = dot2_bf(eosw[i], xp[min(j, d / 2 - 1)], t); }
         t = wave_sum(t);
         eos_logit = bf2f(f2bf(t + eosb));
       }
       if (wg == 0) {
-        if (a.hidden_out) for (int k = tid; k < d; k += FR_THREADS) a.hidden_out[k] = f2bf(xn[k]);
+        if (a.hidden_out) for (int j = tid; j < d / 2; j += FR_THREADS) reinterpret_cast<uint32_t*>(a.hidden_out)[j] = xp[j];
         if (a.eos_out && tid == 0) a.eos_out[0] = f2bf(eos_logit);
       }
       if (a.mode & FR_CB0) {
@@ -723,7 +720,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
     const int R = a.R, CS = a.CS, Q = a.Q;
     const int rhd = R / a.rqH;
     if (!(a.mode & FR_BACKBONE)) {
-      for (int k = tid; k < d; k += FR_THREADS) xn[k] = bf2f(a.rq_hidden[k]);
+      for (int j = tid; j < d / 2; j += FR_THREADS) xp[j] = reinterpret_cast<const uint32_t*>(a.rq_hidden)[j];
       __syncthreads();
     }
     if (!(a.mode & FR_CB0)) {
@@ -735,8 +732,9 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
               m_hd = pairs_of(CS / 2, wg, nwg);
     const NormW nw_rq = load_normw(g_rq_norm, R);
     // attention lane layout: QP key slots x PP feature parts per wave
-    const int QP = Q <= 16 ? 16 : (Q <= 32 ? 32 : 64), PP = 64 / QP;
-    const int fpp = rhd / PP;  // features per part
+    int PP = Q <= 16 ? 4 : (Q <= 32 ? 2 : 1);
+    while (PP > 1 && ((rhd % PP) || ((rhd / PP) & 1))) PP >>= 1;
+    const int fpp = rhd / PP;  // features per part, even
     // token 0: projected hidden + pos_emb[0]
     if (g_rq_proj) {
       const Plan p = make_plan(R / 2, d, wg, nwg, wave);
@@ -747,7 +745,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       const uint32_t pe1 = p.nslots > 1 ? *reinterpret_cast<const uint32_t*>(pos_emb + 2 * p.gp[1]) : 0u;
       uint64_t* tb = llp;
       llp += R / 2;
-      gemv_compute<2, false>(xn, p, wr, red, [&](int gp, float v0, float v1, float, float) {
+      gemv_compute<2, false>(xp, p, wr, red, [&](int gp, float v0, float v1, float, float) {
         const uint32_t pe = (gp == p.gp[0]) ? pe0 : pe1;
         const float o0 = bf2f(f2bf(v0)) + __uint_as_float(pe << 16), o1 = bf2f(f2bf(v1)) + __uint_as_float(pe & 0xffff0000u);
         ll_st(tb + gp, pack2(o0, o1), ep);
@@ -755,7 +753,11 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       poll_set(xres, tb, R / 2, c);
     } else {
       __syncthreads();
-      for (int k = tid; k < R; k += FR_THREADS) xres[k] = bf2f(f2bf(xn[k] + bf2f(pos_emb[k])));
+      for (int j = tid; j < R / 2; j += FR_THREADS) {
+        const uint32_t h2 = xp[j], p2 = reinterpret_cast<const uint32_t*>(pos_emb)[j];
+        const uint32_t pk = f2bf2(bf_lo(h2) + bf_lo(p2), bf_hi(h2) + bf_hi(p2));
+        xres[2 * j] = bf_lo(pk); xres[2 * j + 1] = bf_hi(pk);
+      }
       __syncthreads();
     }
 
@@ -782,9 +784,9 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           const NormW nw1 = load_normw(Lw.attn_norm, R);
           if (ybuf) poll_add(xres, ybuf, R / 2, c);
           TS(31);
-          stage_norm(xres, nw1, a.rq_eps, R, xn);
+          stage_norm(xres, nw1, a.rq_eps, R, xp);
           __syncthreads();
-          gemv_compute<2, false>(xn, R_qkv, wr, red, [&](int gp, float v0, float v1, float, float) {
+          gemv_compute<2, false>(xp, R_qkv, wr, red, [&](int gp, float v0, float v1, float, float) {
             ll_st(qkvb + gp, pack2(v0, v1), ep); });
         }
         const bool kv_only = (t == 0 && l == a.rqL - 1);  // position 0 only feeds later keys/values
@@ -797,42 +799,28 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           if (!kv_only) gemv_prefetch<2, false>(Lw.wo, nullptr, R, R_o, wr);
           __syncthreads();  // xn (A's input) fully consumed before q overwrites it
           ll_poll(qkvb, 3 * R / 2, c, [&](int i, uint32_t v) {
-            const int n = 2 * i;
-            if (n < R) { xn[n] = bf2f((bf16_t)(v & 0xffff)); xn[n + 1] = bf2f((bf16_t)(v >> 16)); }
-            else *reinterpret_cast<uint32_t*>(kst + (n - R)) = v;
+            if (2 * i < R) xp[i] = v;                                             // q, packed
+            else *reinterpret_cast<uint32_t*>(kst + (2 * i - R)) = v;             // new key | value
           });
           __syncthreads();
           if (kv_only) break;
           TS(32);
           const int nk = t + 1;
           const int kj = lane / PP, part = lane % PP;
+          const float scale = 1.0f / sqrtf((float)rhd);
           for (int hh = wave; hh < a.rqH; hh += 4) {
-            const float scale = 1.0f / sqrtf((float)rhd);
-            // lane (key kj, part): partial dot over fpp features
+            // lane (key kj, part): partial dot over fpp features (fpp % 2 == 0)
             float dsum = 0.f;
-            if (kj < nk) {
-              const bf16_t* kp = rqkv + ((size_t)l * Q + kj) * 2 * R + hh * rhd + part * fpp;
-              const float* qp = xn + hh * rhd + part * fpp;
+            {
+              const int kk = min(kj, nk - 1);
+              const uint32_t* kp = reinterpret_cast<const uint32_t*>(rqkv + ((size_t)l * Q + kk) * 2 * R + hh * rhd + part * fpp);
+              const uint32_t* qp = xp + (hh * rhd + part * fpp) / 2;
               if (!(fpp & 7)) {
-                for (int i = 0; i < fpp; i += 8) {
-                  const uint4 kk = *reinterpret_cast<const uint4*>(kp + i);
-                  const float4 qa = *reinterpret_cast<const float4*>(qp + i);
-                  const float4 qb = *reinterpret_cast<const float4*>(qp + i + 4);
-                  float k8[8];
-                  cvt8(kk, k8);
-                  dsum = fmaf(qa.x, k8[0], dsum); dsum = fmaf(qa.y, k8[1], dsum);
-                  dsum = fmaf(qa.z, k8[2], dsum); dsum = fmaf(qa.w, k8[3], dsum);
-                  dsum = fmaf(qb.x, k8[4], dsum); dsum = fmaf(qb.y, k8[5], dsum);
-                  dsum = fmaf(qb.z, k8[6], dsum); dsum = fmaf(qb.w, k8[7], dsum);
-                }
-              } else if (!(fpp & 1)) {
-                for (int i = 0; i < fpp; i += 2) {
-                  const uint32_t kk = *reinterpret_cast<const uint32_t*>(kp + i);
-                  dsum = fmaf(qp[i], __uint_as_float(kk << 16), dsum);
-                  dsum = fmaf(qp[i + 1], __uint_as_float(kk & 0xffff0000u), dsum);
-                }
+#pragma unroll 2
+                for (int i = 0; i < fpp / 2; i += 4)
+                  dsum = dot8_bf(*reinterpret_cast<const uint4*>(kp + i), *reinterpret_cast<const uint4*>(qp + i), dsum);
               } else {
-                for (int i = 0; i < fpp; ++i) dsum = fmaf(qp[i], bf2f(kp[i]), dsum);
+                for (int i = 0; i < fpp / 2; ++i) dsum = dot2_bf(kp[i], qp[i], dsum);
               }
             }
             if (PP >= 2) dsum += dpp_f<DPP_QUAD_XOR1>(dsum);
@@ -844,17 +832,23 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
             // lane = feature: weighted sum of the values
             float o0 = 0.f, o1 = 0.f;
             const bf16_t* vb = rqkv + ((size_t)l * Q) * 2 * R + R + hh * rhd;
+            const int f0 = min(lane, rhd - 1), f1 = min(lane + WAVE, rhd - 1);
             for (int j = 0; j < nk; ++j) {
               const float pj = lane_f(pw, j * PP);
-              if (lane < rhd) o0 = fmaf(pj, bf2f(vb[(size_t)j * 2 * R + lane]), o0);
-              if (lane + WAVE < rhd) o1 = fmaf(pj, bf2f(vb[(size_t)j * 2 * R + lane + WAVE]), o1);
+              o0 = fmaf(pj, bf2f(vb[(size_t)j * 2 * R + f0]), o0);
+              if (rhd > WAVE) o1 = fmaf(pj, bf2f(vb[(size_t)j * 2 * R + f1]), o1);
             }
-            if (lane < rhd) xn[R + hh * rhd + lane] = bf2f(f2bf(o0 / Ls));
-            if (lane + WAVE < rhd) xn[R + hh * rhd + lane + WAVE] = bf2f(f2bf(o1 / Ls));
+            const float inv = 1.0f / Ls;
+            o0 *= inv; o1 *= inv;
+            const float n0 = dpp_f<DPP_QUAD_XOR1>(o0), n1 = dpp_f<DPP_QUAD_XOR1>(o1);  // neighbour features
+            if (!(lane & 1)) {
+              if (lane < rhd) xp[(R + hh * rhd + lane) / 2] = f2bf2(o0, n0);
+              if (lane + WAVE < rhd) xp[(R + hh * rhd + lane + WAVE) / 2] = f2bf2(o1, n1);
+            }
           }
           __syncthreads();
           TS(33);
-          gemv_compute<2, false>(xn + R, R_o, wr, red, [&](int gp, float v0, float v1, float, float) {
+          gemv_compute<2, false>(xp + R / 2, R_o, wr, red, [&](int gp, float v0, float v1, float, float) {
             ll_st(ob + gp, pack2(v0, v1), ep); });
         }
         TS(34);
@@ -868,11 +862,11 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           const NormW nw2 = load_normw(Lw.mlp_norm, R);
           poll_add(xres, ob, R / 2, c);
           TS(35);
-          stage_norm(xres, nw2, a.rq_eps, R, xn);
+          stage_norm(xres, nw2, a.rq_eps, R, xp);
           TS(70);
           __syncthreads();
           TS(71);
-          gemv_compute<2, true>(xn, R_sw, wr, red, [&](int gp, float v0, float v1, float u0, float u1) {
+          gemv_compute<2, true>(xp, R_sw, wr, red, [&](int gp, float v0, float v1, float u0, float u1) {
             const float a0 = bf2f(f2bf(v0)), a1 = bf2f(f2bf(v1)), c0 = bf2f(f2bf(u0)), c1 = bf2f(f2bf(u1));
             const float s0 = bf2f(f2bf(a0 / (1.0f + expf(-a0)))), s1 = bf2f(f2bf(a1 / (1.0f + expf(-a1))));
             ll_st(hb + gp, pack2(s0 * c0, s1 * c1), ep);
@@ -886,9 +880,9 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           WRegs<4, false> wr;
           const Plan R_w2 = plan_of(m_o, a.rqF, wg, nwg, wave);
           gemv_prefetch<4, false>(Lw.w2, nullptr, a.rqF, R_w2, wr);
-          poll_set(xn, hb, a.rqF / 2, c);
+          poll_words(xp, hb, a.rqF / 2, c);
           TS(37);
-          gemv_compute<4, false>(xn, R_w2, wr, red, [&](int gp, float v0, float v1, float, float) {
+          gemv_compute<4, false>(xp, R_w2, wr, red, [&](int gp, float v0, float v1, float, float) {
             ll_st(yb + gp, pack2(v0, v1), ep); });
         }
         ybuf = yb;
@@ -901,11 +895,11 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
         TS(40);
         poll_add(xres, ybuf, R / 2, c);
         TS(41);
-        stage_norm(xres, nw_rq, a.rq_eps, R, xn);
+        stage_norm(xres, nw_rq, a.rq_eps, R, xp);
         __syncthreads();
         uint64_t* lgbuf = llp;
         llp += CS / 2;
-        gemv_compute<2, false>(xn, R_hd, wr, red, [&](int gp, float v0, float v1, float, float) {
+        gemv_compute<2, false>(xp, R_hd, wr, red, [&](int gp, float v0, float v1, float, float) {
           ll_st(lgbuf + gp, pack2(v0, v1), ep); });
         TS(42);
         poll_set(lg, lgbuf, CS / 2, c);
@@ -1005,7 +999,8 @@ bool frame_supported(const vui_config& c, int nwg, int ns, char* why, size_t why
   else if (c.codebook_size > 2048 || (c.codebook_size & 1)) r = "codebook_size > 2048";
   else if (c.n_quantizers > 64) r = "too many codebooks";
   else if ((c.head_dim & 7) || c.head_dim > 128) r = "head_dim";
-  else if ((c.rq_dim / c.rq_heads) % 4 || c.rq_dim / c.rq_heads > 128) r = "depth-head head_dim must be a multiple of 4, at most 128";
+  else if ((c.rq_dim / c.rq_heads) % 2 || c.rq_dim / c.rq_heads > 128) r = "depth-head head_dim must be even, at most 128";
+  else if ((c.d_model | c.ffn | c.rq_dim | c.rq_ffn) & 7) r = "vector lengths must be multiples of 8";
   else if (frame_lds_bytes(c) > 160 * 1024) r = "depth-head keys/values do not fit in LDS";
   else if (c.rq_layers < 1) r = "no depth head";
   else {
