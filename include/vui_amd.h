@@ -117,9 +117,11 @@ int vui_ctx_fused(vui_ctx* ctx, int enable);
 /* Synchronous health check: VUI_EHIP if a fused launch gave up waiting for another workgroup. */
 int vui_ctx_status(vui_ctx* ctx);
 
-/* Profiling aid: fused launches made after this call let workgroup `workgroup` write up to `cap`
- * words (100 MHz clock << 8 | phase tag) into the device buffer buf (cap + 1 words, the last one
- * receives the count); buf = NULL switches it off.  No counterpart in the reference. */
+/* Profiling aid: fused launches made after this call let four workgroups (`workgroup`, +1, +8, +131;
+ * those beyond the grid do not exist) each write up to `cap` words (100 MHz clock << 8 | phase tag)
+ * into their region of the device buffer buf: 4 regions of cap + 1 words, the last word of a region
+ * receives the count in its low 32 bits and the launch's shader cycles above.  buf = NULL switches
+ * it off.  No counterpart in the reference. */
 int vui_debug_phase_clock(vui_ctx* ctx, uint64_t* buf, int cap, int workgroup);
 
 /* One backbone decode step for B rows (B <= max_batch).

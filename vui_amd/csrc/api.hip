@@ -217,7 +217,7 @@ static void fused_base(vui_ctx* ctx, FrameArgs& a) {
   a.w = ctx->wdev; a.n_slots = c.n_slots;
   a.ll = ctx->ll; a.epoch = ctx->ctl; a.arrive = ctx->ctl + 1; a.err = ctx->ctl + 2;
   a.prof = ctx->prof; a.prof_cap = ctx->prof_cap; a.prof_wg = ctx->prof_wg;
-  a.ns = ctx->ns; a.lds_kv_off = (int)(ctx->lds_bytes - (size_t)c.rq_layers * c.n_quantizers * 2 * c.rq_dim * 2);
+  a.ns = ctx->ns; a.lds_kv_off = (int)(ctx->lds_bytes - frame_rq_cache_bytes(c));
 }
 static bool use_fused(vui_ctx* ctx, int B) { return ctx->fused_ok && ctx->fused_on && B == 1; }
 

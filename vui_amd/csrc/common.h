@@ -108,6 +108,53 @@ __device__ __forceinline__ float wave_sum(float v) {
   v = group16_sum(v);
   return (lane_f(v, 0) + lane_f(v, 16)) + (lane_f(v, 32) + lane_f(v, 48));
 }
+// ---- reductions that stay in vector registers (gfx950 lane-swap instructions) ----
+// v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows of its
+// second, v_permlane32_swap the upper half of the first with the lower half of the second; applied to
+// two copies of one value and added, they fold rows 0+1 / 2+3 and then the two halves.
+__device__ __forceinline__ float rows_sum(float v) {  // in: per-row values; out: sum of the four rows, every lane
+  const uint32_t u = __float_as_uint(v);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const float s = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  const uint32_t w = __float_as_uint(s);
+  const auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+__device__ __forceinline__ float rows_max(float v) {
+  const uint32_t u = __float_as_uint(v);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const float s = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const uint32_t w = __float_as_uint(s);
+  const auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+// full-wave sum left in every lane, no scalar round trip
+__device__ __forceinline__ float wave_sum_v(float v) { return rows_sum(group16_sum(v)); }
+#define DPP_ROW_ROR4 0x124
+#define DPP_ROW_ROR8 0x128
+// Sums of four values at once: lane l returns the full-wave sum of value (l & 3).  Each step halves
+// the number of live values by pairing a select with a quad exchange.
+__device__ __forceinline__ float wave_sum4(float a, float b, float c, float d) {
+  const int lane = threadIdx.x & 63;
+  const bool o1 = lane & 1, o2 = lane & 2;
+  const float u = (o1 ? b : a) + dpp_f<DPP_QUAD_XOR1>(o1 ? a : b);  // lanes (l&1): partial of a / b over the lane pair
+  const float w = (o1 ? d : c) + dpp_f<DPP_QUAD_XOR1>(o1 ? c : d);
+  float z = (o2 ? w : u) + dpp_f<DPP_QUAD_XOR2>(o2 ? u : w);        // lane (l&3): partial of value l&3 over the quad
+  z += dpp_f<DPP_ROW_ROR4>(z);
+  z += dpp_f<DPP_ROW_ROR8>(z);
+  return rows_sum(z);
+}
+// two values: lane l returns the full-wave sum of value (l & 1)
+__device__ __forceinline__ float wave_sum2(float a, float b) {
+  const int lane = threadIdx.x & 63;
+  const bool o1 = lane & 1;
+  float z = (o1 ? b : a) + dpp_f<DPP_QUAD_XOR1>(o1 ? a : b);
+  z += dpp_f<DPP_QUAD_XOR2>(z);
+  z += dpp_f<DPP_ROW_ROR4>(z);
+  z += dpp_f<DPP_ROW_ROR8>(z);
+  return rows_sum(z);
+}
+
 __device__ __forceinline__ float group16_max(float v) {
   v = fmaxf(v, dpp_f<DPP_QUAD_XOR1>(v));
   v = fmaxf(v, dpp_f<DPP_QUAD_XOR2>(v));

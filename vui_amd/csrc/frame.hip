@@ -21,12 +21,31 @@
 
 #define FR_THREADS 256
 #define SPIN_LIMIT (1 << 21)
+#ifndef POLL_SLEEP
+#define POLL_SLEEP 0
+#endif
+#ifndef POLL_DELAY
+#define POLL_DELAY 0
+#endif
 
 __device__ __forceinline__ uint64_t ll_ld(const uint64_t* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ void ll_st(uint64_t* p, uint32_t payload, uint32_t epoch) {
   __hip_atomic_store(p, ((uint64_t)epoch << 32) | payload, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Vectors that every workgroup reads can be kept in LL_REP copies, copy r read by the workgroups with
+// index % LL_REP == r (those share an XCD); writers store all copies with one instruction (lanes
+// 0..LL_REP-1).  Measured: 8 copies shorten a bare exchange of <= 512 words between 256 workgroups by
+// 0.4-0.8 us in isolation but not inside this kernel, so one copy is used.
+#define LL_REP 1
+struct RepBuf { uint64_t* base; int n; };
+__device__ __forceinline__ RepBuf rep_alloc(uint64_t*& llp, int n) { RepBuf b = {llp, n}; llp += (size_t)LL_REP * n; return b; }
+__device__ __forceinline__ const uint64_t* rep_rd(const RepBuf& b) { return b.base + (size_t)(blockIdx.x & (LL_REP - 1)) * b.n; }
+// every lane of the wave calls this with the same (i, payload)
+__device__ __forceinline__ void rep_st(const RepBuf& b, int i, uint32_t payload, uint32_t epoch) {
+  const int lane = threadIdx.x & 63;
+  if (lane < LL_REP) ll_st(b.base + (size_t)lane * b.n + i, payload, epoch);
 }
 __device__ __forceinline__ uint32_t pack2(float a, float b) { return f2bf2(a, b); }
 
@@ -41,6 +60,7 @@ struct Ctl {
 // word and stops waiting for the rest of the launch, so every wave always reaches the end.
 template <typename F>
 __device__ __forceinline__ void ll_poll(const uint64_t* buf, int n, Ctl& c, F&& sink) {
+  if (POLL_DELAY) __builtin_amdgcn_s_sleep(POLL_DELAY);
   for (int base = 0; base < n; base += FR_THREADS * 4) {
     int idx[4];
     bool ok[4];
@@ -63,7 +83,7 @@ __device__ __forceinline__ void ll_poll(const uint64_t* buf, int n, Ctl& c, F&& 
         c.dead = 1;
         __hip_atomic_store(c.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
-      __builtin_amdgcn_s_sleep(1);
+      if (POLL_SLEEP) __builtin_amdgcn_s_sleep(POLL_SLEEP);
     }
   }
 }
@@ -144,7 +164,8 @@ __device__ __forceinline__ void gemv_prefetch(const bf16_t* W, const bf16_t* W2,
 
 // xp: K staged activations in LDS as packed bf16 pairs (K/2 words; every activation this kernel
 // multiplies is a bf16 value, so nothing is lost).  red: 4 x 4 floats of LDS.  epi(gp, v0, v1, u0, u1)
-// is called by one lane per finished pair with the fp32 dot products of rows 2gp, 2gp+1 (u*: second matrix).
+// is called by every lane of the finishing wave (same arguments in all lanes) with the fp32 dot products of
+// rows 2gp, 2gp+1 (u*: second matrix).
 template <int MAXC, bool DUAL, typename Epi>
 __device__ __forceinline__ void gemv_compute(const uint32_t* xp, const Plan& p, const WRegs<MAXC, DUAL>& r, float* red,
                                              Epi&& epi) {
@@ -176,14 +197,14 @@ __device__ __forceinline__ void gemv_compute(const uint32_t* xp, const Plan& p, 
   if (p.KS > 1) {  // uniform over the workgroup
     if (lane == 0) { red[wave * 4 + 0] = res[0][0]; red[wave * 4 + 1] = res[0][1]; red[wave * 4 + 2] = res[0][2]; red[wave * 4 + 3] = res[0][3]; }
     __syncthreads();
-    if (p.kpart == 0 && lane == 0) {
+    if (p.kpart == 0) {
       float t[4] = {0.f, 0.f, 0.f, 0.f};
       for (int k = 0; k < p.KS; ++k)
 #pragma unroll
         for (int j = 0; j < 4; ++j) t[j] += red[(wave + k) * 4 + j];
       epi(p.gp[0], t[0], t[1], t[2], t[3]);
     }
-  } else if (lane == 0) {
+  } else {
     if (p.nslots > 0) epi(p.gp[0], res[0][0], res[0][1], res[0][2], res[0][3]);
     if (p.nslots > 1) epi(p.gp[1], res[1][0], res[1][1], res[1][2], res[1][3]);
   }
@@ -261,10 +282,21 @@ __device__ __forceinline__ void poll_add(float* dst, const uint64_t* buf, int nw
 #define LDS_SAMP (LDS_MISC + 256)        // SampleShared
 #define LDS_FIXED (LDS_SAMP + 1280)
 
-// optional per-phase timestamps (100 MHz wall clock) written by one workgroup, for profiling
-#define TS(id)                                                                                    \
-  do {                                                                                            \
-    if (a.prof && wg == a.prof_wg && tid == 0 && nts < a.prof_cap) a.prof[nts++] = (wall_clock64() << 8) | (uint64_t)(id); \
+// optional per-phase timestamps (100 MHz wall clock) of four workgroups, for profiling: kept in LDS
+// as 16-bit deltas + 8-bit tags while the frame runs (a global store per stamp would sit in the
+// in-order memory queue in front of the weight loads) and written out at the end
+#define PROF_EVENTS 1000
+#define PROF_LDS_BYTES (PROF_EVENTS * 3 + 8)
+#define TS(id)                                                                      \
+  do {                                                                              \
+    if (prof_on && tid == 0 && nts < PROF_EVENTS) {                                 \
+      const uint64_t now_ = wall_clock64();                                         \
+      const uint64_t dl_ = now_ - ts_prev;                                          \
+      prof_dt[nts] = (uint16_t)(dl_ > 65535 ? 65535 : dl_);                         \
+      prof_id[nts] = (uint8_t)(id);                                                 \
+      ts_prev = now_;                                                               \
+      ++nts;                                                                        \
+    }                                                                               \
   } while (0)
 
 struct LayerP { const bf16_t *attn_norm, *wqkv, *wo, *mlp_norm, *w1, *w3, *w2; };
@@ -284,7 +316,7 @@ __device__ __forceinline__ void poll3(const uint64_t* p0, const uint64_t* p1, co
     if (!k2 && ((uint32_t)(v2 >> 32) == c.epoch || c.dead)) k2 = true;
     if (k0 && k1 && k2) break;
     if (++spins > SPIN_LIMIT) { c.dead = 1; __hip_atomic_store(c.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-    __builtin_amdgcn_s_sleep(1);
+    if (POLL_SLEEP) __builtin_amdgcn_s_sleep(POLL_SLEEP);
   }
   r0 = (uint32_t)v0; r1 = (uint32_t)v1; r2 = (uint32_t)v2;
 }
@@ -318,6 +350,14 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
   const uint32_t frame1 = a.frame_ctr1 ? (uint32_t)a.frame_ctr1[0] : 0u;
   int slot = 0, pos = 0;
   int nts = 0;
+  // four workgroups record: prof_wg, the next one (next XCD), +8 (same XCD), +131
+  const int prof_k = wg == a.prof_wg ? 0 : (wg == a.prof_wg + 1 ? 1 : (wg == a.prof_wg + 8 ? 2 : (wg == a.prof_wg + 131 ? 3 : -1)));
+  const bool prof_on = a.prof != nullptr && prof_k >= 0;
+  uint16_t* prof_dt = (uint16_t*)(smem + a.lds_prof_off);
+  uint8_t* prof_id = (uint8_t*)(smem + a.lds_prof_off + 2 * PROF_EVENTS);
+  const uint64_t ts_first = prof_on ? wall_clock64() : 0;
+  const uint64_t cyc_first = prof_on ? (uint64_t)clock64() : 0;
+  uint64_t ts_prev = ts_first;
   TS(0);
 
   // weight pointer tables into LDS (one pass, so no phase waits on a pointer load later)
@@ -447,6 +487,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           o0 = r0; o1 = r1;
         }
         const uint32_t pk = pack2(o0, o1);
+        if (lane != 0) return;
         ll_st(qkvbuf + gp, pk, ep);
         if (region == 1) *reinterpret_cast<uint32_t*>(kcl + ((size_t)slot * a.S + pos) * nkv + m) = pk;
         if (region == 2) *reinterpret_cast<uint32_t*>(vcl + ((size_t)slot * a.S + pos) * nkv + m) = pk;
@@ -571,8 +612,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       }
       TS(5);
       // ---- merge the splits: workgroup (h, 16-feature chunk); one wait for everything ----
-      uint64_t* attbuf = llp;
-      llp += d / 2;
+      const RepBuf attbuf = rep_alloc(llp, d / 2);
       if (mrg_on) {
         const int h = wg / cpd, cc = wg % cpd;
         const uint64_t* pb = part + (size_t)h * NS * (hd + 2);
@@ -594,44 +634,43 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           if (tid < 2 * ns_eff) ml[tid] = __uint_as_float(r2);
         }
         __syncthreads();
-        if (tid < 16) {
+        if (tid < 16 * LL_REP) {  // eight groups of 16 lanes compute the same 16 features, one copy each
+          const int f16 = tid & 15, rep = tid >> 4;
           float Mx = -INFINITY;
           for (int s = 0; s < ns_eff; ++s) Mx = fmaxf(Mx, ml[2 * s]);
           float Lt = 0.f, o = 0.f;
           for (int s = 0; s < ns_eff; ++s) {
             const float w = expf(ml[2 * s] - Mx);
             Lt = fmaf(w, ml[2 * s + 1], Lt);
-            o = fmaf(w, part_lds[s * 16 + tid], o);
+            o = fmaf(w, part_lds[s * 16 + f16], o);
           }
           const float val = o / Lt;
           const float nb = dpp_f<DPP_QUAD_XOR1>(val);  // neighbour feature
-          const int d0 = cc * 16 + tid;
-          if (!(tid & 1) && d0 < hd) ll_st(attbuf + (h * hd + d0) / 2, pack2(val, nb), ep);
+          const int d0 = cc * 16 + f16;
+          if (!(f16 & 1) && d0 < hd) ll_st(attbuf.base + (size_t)rep * attbuf.n + (h * hd + d0) / 2, pack2(val, nb), ep);
         }
       }
       TS(6);
       // ---- out_proj ----
-      uint64_t* obuf = llp;
-      llp += d / 2;
+      const RepBuf obuf = rep_alloc(llp, d / 2);
       {
         WRegs<2, false> w2;
         const Plan P_o = plan_of(n_o, d, wg, nwg, wave);
         gemv_prefetch<2, false>(Lw.wo, nullptr, d, P_o, w2);
-        poll_words(xp, attbuf, d / 2, c);
+        poll_words(xp, rep_rd(attbuf), d / 2, c);
         TS(7);
         gemv_compute<2, false>(xp, P_o, w2, red, [&](int gp, float v0, float v1, float, float) {
-          ll_st(obuf + gp, pack2(v0, v1), ep); });
+          rep_st(obuf, gp, pack2(v0, v1), ep); });
       }
       TS(8);
       // ---- SwiGLU ----
-      uint64_t* hbuf = llp;
-      llp += a.F / 2;
+      const RepBuf hbuf = rep_alloc(llp, a.F / 2);
       {
         WRegs<2, true> w3;
         const Plan P_sw = plan_of(n_sw, d, wg, nwg, wave);
         gemv_prefetch<2, true>(Lw.w1, Lw.w3, d, P_sw, w3);
         const NormW nw2 = load_normw(Lw.mlp_norm, d);
-        poll_add(xres, obuf, d / 2, c);
+        poll_add(xres, rep_rd(obuf), d / 2, c);
         TS(9);
         stage_norm(xres, nw2, a.eps, d, xp);
         __syncthreads();
@@ -639,23 +678,22 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
         gemv_compute<2, true>(xp, P_sw, w3, red, [&](int gp, float v0, float v1, float u0, float u1) {
           const float a0 = bf2f(f2bf(v0)), a1 = bf2f(f2bf(v1)), c0 = bf2f(f2bf(u0)), c1 = bf2f(f2bf(u1));
           const float s0 = bf2f(f2bf(a0 / (1.0f + expf(-a0)))), s1 = bf2f(f2bf(a1 / (1.0f + expf(-a1))));
-          ll_st(hbuf + gp, pack2(s0 * c0, s1 * c1), ep);
+          rep_st(hbuf, gp, pack2(s0 * c0, s1 * c1), ep);
         });
       }
       TS(11);
       // ---- W2 ----
-      uint64_t* yb = llp;
-      llp += d / 2;
+      const RepBuf yb = rep_alloc(llp, d / 2);
       {
         WRegs<4, false> w4;
         const Plan P_w2 = plan_of(n_o, a.F, wg, nwg, wave);
         gemv_prefetch<4, false>(Lw.w2, nullptr, a.F, P_w2, w4);
-        poll_words(xp, hbuf, a.F / 2, c);
+        poll_words(xp, rep_rd(hbuf), a.F / 2, c);
         TS(12);
         gemv_compute<4, false>(xp, P_w2, w4, red, [&](int gp, float v0, float v1, float, float) {
-          ll_st(yb + gp, pack2(v0, v1), ep); });
+          rep_st(yb, gp, pack2(v0, v1), ep); });
       }
-      ybuf = yb;
+      ybuf = rep_rd(yb);
       TS(13);
     }
     // ---- final norm, codec head, eos head ----
@@ -671,12 +709,11 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       poll_add(xres, ybuf, d / 2, c);
       stage_norm(xres, nwf, a.eps, d, xp);
       __syncthreads();
-      uint64_t* lgbuf = llp;
-      llp += a.CS / 2;
+      const RepBuf lgbuf = rep_alloc(llp, a.CS / 2);
       gemv_compute<2, false>(xp, p, wr, red, [&](int gp, float v0, float v1, float, float) {
         const uint32_t pk = pack2(v0, v1);
-        ll_st(lgbuf + gp, pk, ep);
-        if (a.cb0_out) *reinterpret_cast<uint32_t*>(a.cb0_out + 2 * gp) = pk;
+        rep_st(lgbuf, gp, pk, ep);
+        if (a.cb0_out && lane == 0) *reinterpret_cast<uint32_t*>(a.cb0_out + 2 * gp) = pk;
       });
       // eos logit: every workgroup (it is a 1 x d dot product), outputs by workgroup 0
       {
@@ -692,7 +729,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       }
       if (a.mode & FR_CB0) {
         const int E = (a.CS + FR_THREADS - 1) / FR_THREADS;
-        poll_set(lg, lgbuf, a.CS / 2, c);
+        poll_set(lg, rep_rd(lgbuf), a.CS / 2, c);
         const bool greedy = (a.topk0 == 1) || !(a.temp0 > 0.f);
         const float div = greedy ? 1.0f : a.temp0;
         const float* counts = (a.rep_counts && a.penalty > 1.0f) ? a.rep_counts : nullptr;
@@ -732,6 +769,9 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
               m_hd = pairs_of(CS / 2, wg, nwg);
     const NormW nw_rq = load_normw(g_rq_norm, R);
     // attention lane layout: QP key slots x PP feature parts per wave
+    const int QP8 = (Q + 7) & ~7;
+    // values of positions not yet written this frame are multiplied by weight zero: they must be finite
+    for (int i = tid; i < (a.rqL * 2 * R * QP8) / 8; i += FR_THREADS) reinterpret_cast<uint4*>(rqkv)[i] = make_uint4(0, 0, 0, 0);
     int PP = Q <= 16 ? 4 : (Q <= 32 ? 2 : 1);
     while (PP > 1 && ((rhd % PP) || ((rhd / PP) & 1))) PP >>= 1;
     const int fpp = rhd / PP;  // features per part, even
@@ -743,14 +783,13 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       // only pairs this wave really owns are inside pos_emb[0, R)
       const uint32_t pe0 = p.nslots > 0 ? *reinterpret_cast<const uint32_t*>(pos_emb + 2 * p.gp[0]) : 0u;
       const uint32_t pe1 = p.nslots > 1 ? *reinterpret_cast<const uint32_t*>(pos_emb + 2 * p.gp[1]) : 0u;
-      uint64_t* tb = llp;
-      llp += R / 2;
+      const RepBuf tb = rep_alloc(llp, R / 2);
       gemv_compute<2, false>(xp, p, wr, red, [&](int gp, float v0, float v1, float, float) {
         const uint32_t pe = (gp == p.gp[0]) ? pe0 : pe1;
         const float o0 = bf2f(f2bf(v0)) + __uint_as_float(pe << 16), o1 = bf2f(f2bf(v1)) + __uint_as_float(pe & 0xffff0000u);
-        ll_st(tb + gp, pack2(o0, o1), ep);
+        rep_st(tb, gp, pack2(o0, o1), ep);
       });
-      poll_set(xres, tb, R / 2, c);
+      poll_set(xres, rep_rd(tb), R / 2, c);
     } else {
       __syncthreads();
       for (int j = tid; j < R / 2; j += FR_THREADS) {
@@ -772,10 +811,13 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       const uint64_t* ybuf = nullptr;
       for (int l = 0; l < a.rqL; ++l) {
         const LayerP Lw = lp[a.L + l];
-        bf16_t* kst = rqkv + ((size_t)l * Q + t) * 2 * R;  // [k (R) | v (R)] of this layer and position
+        // depth-head cache of this layer in LDS, QP8 = Q rounded up to 8 positions:
+        //   keys    [R/8 chunks][QP8 positions][8 features]   (a lane group reads one position per lane: no bank conflicts)
+        //   values  [R features][QP8 positions]               (one feature's values over the positions are contiguous)
+        bf16_t* kcache = rqkv + (size_t)l * 2 * R * QP8;
+        bf16_t* vcache = kcache + (size_t)R * QP8;
         // ---- A: QKV ----
-        uint64_t* qkvb = llp;
-        llp += 3 * R / 2;
+        const RepBuf qkvb = rep_alloc(llp, 3 * R / 2);
         {
           TS(30);
           WRegs<2, false> wr;
@@ -787,20 +829,28 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           stage_norm(xres, nw1, a.rq_eps, R, xp);
           __syncthreads();
           gemv_compute<2, false>(xp, R_qkv, wr, red, [&](int gp, float v0, float v1, float, float) {
-            ll_st(qkvb + gp, pack2(v0, v1), ep); });
+            rep_st(qkvb, gp, pack2(v0, v1), ep); });
         }
         const bool kv_only = (t == 0 && l == a.rqL - 1);  // position 0 only feeds later keys/values
         // ---- B: attention (redundantly in every workgroup) + out_proj ----
-        uint64_t* ob = llp;
-        if (!kv_only) llp += R / 2;
+        RepBuf ob = {llp, R / 2};
+        if (!kv_only) ob = rep_alloc(llp, R / 2);
         {
           WRegs<2, false> wr;
           const Plan R_o = plan_of(m_o, R, wg, nwg, wave);
           if (!kv_only) gemv_prefetch<2, false>(Lw.wo, nullptr, R, R_o, wr);
           __syncthreads();  // xn (A's input) fully consumed before q overwrites it
-          ll_poll(qkvb, 3 * R / 2, c, [&](int i, uint32_t v) {
-            if (2 * i < R) xp[i] = v;                                             // q, packed
-            else *reinterpret_cast<uint32_t*>(kst + (2 * i - R)) = v;             // new key | value
+          ll_poll(rep_rd(qkvb), 3 * R / 2, c, [&](int i, uint32_t v) {
+            const int n = 2 * i;
+            if (n < R) xp[i] = v;  // q, packed
+            else if (n < 2 * R) {   // new key: features n-R, n-R+1 of position t
+              const int f = n - R;
+              *reinterpret_cast<uint32_t*>(kcache + ((size_t)(f >> 3) * QP8 + t) * 8 + (f & 7)) = v;
+            } else {                // new value
+              const int f = n - 2 * R;
+              vcache[(size_t)f * QP8 + t] = (bf16_t)(v & 0xffff);
+              vcache[(size_t)(f + 1) * QP8 + t] = (bf16_t)(v >> 16);
+            }
           });
           __syncthreads();
           if (kv_only) break;
@@ -808,59 +858,102 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           const int nk = t + 1;
           const int kj = lane / PP, part = lane % PP;
           const float scale = 1.0f / sqrtf((float)rhd);
-          for (int hh = wave; hh < a.rqH; hh += 4) {
-            // lane (key kj, part): partial dot over fpp features (fpp % 2 == 0)
-            float dsum = 0.f;
-            {
-              const int kk = min(kj, nk - 1);
-              const uint32_t* kp = reinterpret_cast<const uint32_t*>(rqkv + ((size_t)l * Q + kk) * 2 * R + hh * rhd + part * fpp);
-              const uint32_t* qp = xp + (hh * rhd + part * fpp) / 2;
-              if (!(fpp & 7)) {
-#pragma unroll 2
-                for (int i = 0; i < fpp / 2; i += 4)
-                  dsum = dot8_bf(*reinterpret_cast<const uint4*>(kp + i), *reinterpret_cast<const uint4*>(qp + i), dsum);
-              } else {
-                for (int i = 0; i < fpp / 2; ++i) dsum = dot2_bf(kp[i], qp[i], dsum);
+          // this wave's softmax weights of two heads as bf16 hi + lo parts: [head][hi 64 | lo 64]
+          bf16_t* pw_hi = reinterpret_cast<bf16_t*>(sc) + wave * 256;
+          bf16_t* pw_lo = pw_hi + 64;
+          // two heads per pass, written side by side so that their LDS round trips and reductions overlap
+          for (int hb0 = wave; hb0 < a.rqH; hb0 += 8) {
+            int hs[2];
+            hs[0] = hb0;
+            hs[1] = min(hb0 + 4, a.rqH - 1);  // a missing second head repeats a valid one and is not written
+            const bool second = hb0 + 4 < a.rqH;
+            const int kk = min(kj, nk - 1);
+            float dsum[2] = {0.f, 0.f};
+            if (!(fpp & 7)) {
+              for (int i = 0; i < fpp / 8; ++i) {
+                uint4 kr[2], qr[2];
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                  const int f0 = hs[h] * rhd + part * fpp + 8 * i;
+                  kr[h] = *reinterpret_cast<const uint4*>(kcache + ((size_t)(f0 >> 3) * QP8 + kk) * 8);
+                  qr[h] = *reinterpret_cast<const uint4*>(xp + f0 / 2);
+                }
+#pragma unroll
+                for (int h = 0; h < 2; ++h) dsum[h] = dot8_bf(kr[h], qr[h], dsum[h]);
+              }
+            } else {
+              for (int i = 0; i < fpp / 2; ++i)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                  const int f = hs[h] * rhd + part * fpp + 2 * i;
+                  dsum[h] = dot2_bf(*reinterpret_cast<const uint32_t*>(kcache + ((size_t)(f >> 3) * QP8 + kk) * 8 + (f & 7)), xp[f / 2], dsum[h]);
+                }
+            }
+            float pw[2], Ls[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              if (PP >= 2) dsum[h] += dpp_f<DPP_QUAD_XOR1>(dsum[h]);
+              if (PP >= 4) dsum[h] += dpp_f<DPP_QUAD_XOR2>(dsum[h]);
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              const float sco = (kj < nk) ? dsum[h] * scale : -INFINITY;
+              const float M = rows_max(group16_max(sco));
+              pw[h] = (kj < nk) ? __expf(sco - M) : 0.f;
+              Ls[h] = wave_sum_v(part == 0 ? pw[h] : 0.f);
+            }
+            // the weights go through LDS as bf16 pairs: p = hi + lo keeps 16 mantissa bits
+            if (part == 0) {
+#pragma unroll
+              for (int h = 0; h < 2; ++h) {
+                const bf16_t hi = f2bf(pw[h]);
+                pw_hi[h * 128 + kj] = hi;
+                pw_lo[h * 128 + kj] = f2bf(pw[h] - bf2f(hi));
               }
             }
-            if (PP >= 2) dsum += dpp_f<DPP_QUAD_XOR1>(dsum);
-            if (PP >= 4) dsum += dpp_f<DPP_QUAD_XOR2>(dsum);
-            const float sco = (kj < nk) ? dsum * scale : -INFINITY;
-            const float M = wave_max(sco);
-            const float pw = (kj < nk) ? expf(sco - M) : 0.f;
-            const float Ls = wave_sum(part == 0 ? pw : 0.f);
-            // lane = feature: weighted sum of the values
-            float o0 = 0.f, o1 = 0.f;
-            const bf16_t* vb = rqkv + ((size_t)l * Q) * 2 * R + R + hh * rhd;
-            const int f0 = min(lane, rhd - 1), f1 = min(lane + WAVE, rhd - 1);
-            for (int j = 0; j < nk; ++j) {
-              const float pj = lane_f(pw, j * PP);
-              o0 = fmaf(pj, bf2f(vb[(size_t)j * 2 * R + f0]), o0);
-              if (rhd > WAVE) o1 = fmaf(pj, bf2f(vb[(size_t)j * 2 * R + f1]), o1);
+            // lane = feature: dot product of the feature's values over the positions with the weights
+            float o0[2] = {0.f, 0.f}, o1[2] = {0.f, 0.f};
+            for (int j0 = 0; j0 < nk; j0 += 8) {
+              uint4 ph[2], pl[2], va[2], vb[2];
+#pragma unroll
+              for (int h = 0; h < 2; ++h) {
+                ph[h] = *reinterpret_cast<const uint4*>(pw_hi + h * 128 + j0);
+                pl[h] = *reinterpret_cast<const uint4*>(pw_lo + h * 128 + j0);
+                va[h] = *reinterpret_cast<const uint4*>(vcache + (size_t)(hs[h] * rhd + min(lane, rhd - 1)) * QP8 + j0);
+                if (rhd > WAVE) vb[h] = *reinterpret_cast<const uint4*>(vcache + (size_t)(hs[h] * rhd + min(lane + WAVE, rhd - 1)) * QP8 + j0);
+              }
+#pragma unroll
+              for (int h = 0; h < 2; ++h) {
+                o0[h] = dot8_bf(va[h], ph[h], o0[h]);
+                o0[h] = dot8_bf(va[h], pl[h], o0[h]);
+                if (rhd > WAVE) { o1[h] = dot8_bf(vb[h], ph[h], o1[h]); o1[h] = dot8_bf(vb[h], pl[h], o1[h]); }
+              }
             }
-            const float inv = 1.0f / Ls;
-            o0 *= inv; o1 *= inv;
-            const float n0 = dpp_f<DPP_QUAD_XOR1>(o0), n1 = dpp_f<DPP_QUAD_XOR1>(o1);  // neighbour features
-            if (!(lane & 1)) {
-              if (lane < rhd) xp[(R + hh * rhd + lane) / 2] = f2bf2(o0, n0);
-              if (lane + WAVE < rhd) xp[(R + hh * rhd + lane + WAVE) / 2] = f2bf2(o1, n1);
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              const float inv = __builtin_amdgcn_rcpf(Ls[h]);
+              const float a0 = o0[h] * inv, a1 = o1[h] * inv;
+              const float n0 = dpp_f<DPP_QUAD_XOR1>(a0), n1 = dpp_f<DPP_QUAD_XOR1>(a1);  // neighbour features
+              if (!(lane & 1) && (h == 0 || second)) {
+                if (lane < rhd) xp[(R + hs[h] * rhd + lane) / 2] = f2bf2(a0, n0);
+                if (lane + WAVE < rhd) xp[(R + hs[h] * rhd + lane + WAVE) / 2] = f2bf2(a1, n1);
+              }
             }
           }
           __syncthreads();
           TS(33);
           gemv_compute<2, false>(xp + R / 2, R_o, wr, red, [&](int gp, float v0, float v1, float, float) {
-            ll_st(ob + gp, pack2(v0, v1), ep); });
+            rep_st(ob, gp, pack2(v0, v1), ep); });
         }
         TS(34);
         // ---- C: SwiGLU ----
-        uint64_t* hb = llp;
-        llp += a.rqF / 2;
+        const RepBuf hb = rep_alloc(llp, a.rqF / 2);
         {
           WRegs<2, true> wr;
           const Plan R_sw = plan_of(m_sw, R, wg, nwg, wave);
           gemv_prefetch<2, true>(Lw.w1, Lw.w3, R, R_sw, wr);
           const NormW nw2 = load_normw(Lw.mlp_norm, R);
-          poll_add(xres, ob, R / 2, c);
+          poll_add(xres, rep_rd(ob), R / 2, c);
           TS(35);
           stage_norm(xres, nw2, a.rq_eps, R, xp);
           TS(70);
@@ -869,23 +962,22 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           gemv_compute<2, true>(xp, R_sw, wr, red, [&](int gp, float v0, float v1, float u0, float u1) {
             const float a0 = bf2f(f2bf(v0)), a1 = bf2f(f2bf(v1)), c0 = bf2f(f2bf(u0)), c1 = bf2f(f2bf(u1));
             const float s0 = bf2f(f2bf(a0 / (1.0f + expf(-a0)))), s1 = bf2f(f2bf(a1 / (1.0f + expf(-a1))));
-            ll_st(hb + gp, pack2(s0 * c0, s1 * c1), ep);
+            rep_st(hb, gp, pack2(s0 * c0, s1 * c1), ep);
           });
         }
         TS(36);
         // ---- D: W2 ----
-        uint64_t* yb = llp;
-        llp += R / 2;
+        const RepBuf yb = rep_alloc(llp, R / 2);
         {
           WRegs<4, false> wr;
           const Plan R_w2 = plan_of(m_o, a.rqF, wg, nwg, wave);
           gemv_prefetch<4, false>(Lw.w2, nullptr, a.rqF, R_w2, wr);
-          poll_words(xp, hb, a.rqF / 2, c);
+          poll_words(xp, rep_rd(hb), a.rqF / 2, c);
           TS(37);
           gemv_compute<4, false>(xp, R_w2, wr, red, [&](int gp, float v0, float v1, float, float) {
-            ll_st(yb + gp, pack2(v0, v1), ep); });
+            rep_st(yb, gp, pack2(v0, v1), ep); });
         }
-        ybuf = yb;
+        ybuf = rep_rd(yb);
       }
       if (t >= 1) {
         // ---- head t-1: logits of codebook t, then the draw in every workgroup ----
@@ -897,12 +989,11 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
         TS(41);
         stage_norm(xres, nw_rq, a.rq_eps, R, xp);
         __syncthreads();
-        uint64_t* lgbuf = llp;
-        llp += CS / 2;
+        const RepBuf lgbuf = rep_alloc(llp, CS / 2);
         gemv_compute<2, false>(xp, R_hd, wr, red, [&](int gp, float v0, float v1, float, float) {
-          ll_st(lgbuf + gp, pack2(v0, v1), ep); });
+          rep_st(lgbuf, gp, pack2(v0, v1), ep); });
         TS(42);
-        poll_set(lg, lgbuf, CS / 2, c);
+        poll_set(lg, rep_rd(lgbuf), CS / 2, c);
         TS(43);
         const int E = (CS + FR_THREADS - 1) / FR_THREADS;
         const bool greedy = (a.topk1 == 1) || !(a.temp1 > 0.f);
@@ -922,10 +1013,6 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
         }
         prev_code = block_sample<8>(lv, key, bias ? 0 : 16, CS, E, greedy, a.topk1, a.seed1, frame1, 0u, (uint32_t)t, ssh);
         TS(44);
-#ifdef VUI_SAMPLE_CLOCK
-        if (a.prof && wg == a.prof_wg && tid == 0)
-          for (int k = 0; k < 6; ++k) if (nts < a.prof_cap) a.prof[nts++] = (ssh.ts[k] << 8) | (uint64_t)(60 + k);
-#endif
         if (tid == 0) codes_l[t] = prev_code;
       }
     }
@@ -934,7 +1021,13 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
   // ------------------------------------------------------------------ bookkeeping by workgroup 0
   __syncthreads();
   TS(50);
-  if (a.prof && wg == a.prof_wg && tid == 0) a.prof[a.prof_cap] = (uint64_t)nts;
+  if (prof_on && tid == 0) {
+    uint64_t t = ts_first;
+    const int n = min(nts, a.prof_cap);
+    uint64_t* out = a.prof + (size_t)prof_k * (a.prof_cap + 1);
+    for (int i = 0; i < n; ++i) { t += prof_dt[i]; out[i] = (t << 8) | (uint64_t)prof_id[i]; }
+    out[a.prof_cap] = (uint64_t)n | (((uint64_t)clock64() - cyc_first) << 32);  // count | shader cycles of the launch
+  }
   if (wg == 0) {
     if ((a.mode & FR_CB0) && tid == 0) {
       if (a.code0_out) a.code0_out[0] = code0;
@@ -964,7 +1057,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       // every workgroup has read the epoch before it may change
       int spins = 0;
       while (__hip_atomic_load(a.arrive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (uint32_t)nwg && ++spins < SPIN_LIMIT)
-        __builtin_amdgcn_s_sleep(1);
+        if (POLL_SLEEP) __builtin_amdgcn_s_sleep(POLL_SLEEP);
       __hip_atomic_store(a.arrive, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(a.epoch, ep, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -974,21 +1067,26 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
 // ---------------------------------------------------------------------------------------------
 // host side
 size_t frame_ll_words(const vui_config& c, int ns) {
-  const size_t d = c.d_model, hd = c.head_dim;
-  size_t per_layer = (size_t)(c.n_heads + 2 * c.n_kv_heads) * hd / 2 + (size_t)c.n_heads * ns * (hd + 2) + d / 2 + d / 2 +
-                     c.ffn / 2 + d / 2;
-  size_t total = per_layer * c.n_layers + c.codebook_size / 2;
+  const size_t d = c.d_model, hd = c.head_dim, rep = LL_REP;
+  // per backbone layer: q/k/v and the attention partials once; attention output, out_proj, SwiGLU and W2 outputs in copies
+  size_t per_layer = (size_t)(c.n_heads + 2 * c.n_kv_heads) * hd / 2 + (size_t)c.n_heads * ns * (hd + 2) +
+                     rep * (d / 2 + d / 2 + c.ffn / 2 + d / 2);
+  size_t total = per_layer * c.n_layers + rep * (c.codebook_size / 2);
   const size_t R = c.rq_dim;
   size_t rq_layer = 3 * R / 2 + R / 2 + c.rq_ffn / 2 + R / 2;
-  total += R / 2 + (size_t)c.n_quantizers * (rq_layer * c.rq_layers + c.codebook_size / 2);
+  total += rep * (R / 2 + (size_t)c.n_quantizers * (rq_layer * c.rq_layers + c.codebook_size / 2));
   return total + 64;
 }
 
 static size_t frame_ptr_bytes(const vui_config& c) {
   return (((size_t)(c.n_layers + c.rq_layers) * sizeof(LayerP)) + 15) & ~(size_t)15;
 }
+// depth-head keys and values of every layer, positions rounded up to 8
+size_t frame_rq_cache_bytes(const vui_config& c) {
+  return (size_t)c.rq_layers * ((c.n_quantizers + 7) & ~7) * 2 * c.rq_dim * 2;
+}
 size_t frame_lds_bytes(const vui_config& c) {
-  return (size_t)LDS_FIXED + frame_ptr_bytes(c) + (size_t)c.rq_layers * c.n_quantizers * 2 * c.rq_dim * 2;
+  return (size_t)LDS_FIXED + frame_ptr_bytes(c) + frame_rq_cache_bytes(c);
 }
 
 bool frame_supported(const vui_config& c, int nwg, int ns, char* why, size_t why_len) {
@@ -1018,6 +1116,8 @@ bool frame_supported(const vui_config& c, int nwg, int ns, char* why, size_t why
   return r == nullptr;
 }
 
+size_t frame_prof_lds_bytes() { return (PROF_LDS_BYTES + 15) & ~(size_t)15; }
+
 int frame_max_resident(size_t lds_bytes, int* n_cu) {
   int dev = 0;
   HIP_TRY(hipGetDevice(&dev));
@@ -1026,7 +1126,9 @@ int frame_max_resident(size_t lds_bytes, int* n_cu) {
   // the attribute is per kernel, not per context: never lower it for another, larger context
   static size_t lds_attr = 0;
   if (lds_bytes > lds_attr) {
-    HIP_TRY(hipFuncSetAttribute((const void*)frame_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    // room for the optional phase-clock buffer where it fits
+    const size_t want = lds_bytes + frame_prof_lds_bytes() <= 160 * 1024 ? lds_bytes + frame_prof_lds_bytes() : lds_bytes;
+    HIP_TRY(hipFuncSetAttribute((const void*)frame_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)want));
     lds_attr = lds_bytes;
   }
   int occ = 0;
@@ -1035,7 +1137,13 @@ int frame_max_resident(size_t lds_bytes, int* n_cu) {
   return occ * prop.multiProcessorCount;
 }
 
-int launch_frame(const FrameArgs& a, int nwg, size_t lds_bytes, hipStream_t st) {
+int launch_frame(const FrameArgs& a_in, int nwg, size_t lds_bytes, hipStream_t st) {
+  FrameArgs a = a_in;
+  a.lds_prof_off = (int)lds_bytes;
+  if (a.prof) {
+    if (lds_bytes + frame_prof_lds_bytes() > 160 * 1024) { vui_set_error("no LDS left for the phase clock"); return VUI_EINVAL; }
+    lds_bytes += frame_prof_lds_bytes();
+  }
   hipLaunchKernelGGL(frame_kernel, dim3(nwg), dim3(FR_THREADS), lds_bytes, st, a);
   HIP_TRY(hipGetLastError());
   return VUI_OK;

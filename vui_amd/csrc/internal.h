@@ -176,12 +176,14 @@ struct FrameArgs {
   int lds_kv_off;  // byte offset of the depth-head K/V store in LDS
   uint64_t* prof;  // optional (prof_cap + 1) words: (clock << 8 | tag) per phase point, count in the last word
   int prof_cap, prof_wg;
+  int lds_prof_off;  // set by launch_frame: LDS offset of the stamp buffer
 };
 
 enum { FR_BACKBONE = 1, FR_CB0 = 2, FR_RQ = 4, FR_FINISH = 8 };
 
 size_t frame_ll_words(const vui_config& c, int ns);
 size_t frame_lds_bytes(const vui_config& c);
+size_t frame_rq_cache_bytes(const vui_config& c);
 bool frame_supported(const vui_config& c, int nwg, int ns, char* why, size_t why_len);
 int frame_max_resident(size_t lds_bytes, int* n_cu);
 int launch_frame(const FrameArgs& a, int nwg, size_t lds_bytes, hipStream_t st);
