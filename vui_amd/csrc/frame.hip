@@ -170,29 +170,41 @@ template <int MAXC, bool DUAL, typename Epi>
 __device__ __forceinline__ void gemv_compute(const uint32_t* xp, const Plan& p, const WRegs<MAXC, DUAL>& r, float* red,
                                              Epi&& epi) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  float res[2][4];
+  float res[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
   uint4 x[MAXC];
   if (p.nslots > 0) {
     // lanes beyond the K range hold zero weights; their reads are clamped to a staged chunk
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) x[i] = *reinterpret_cast<const uint4*>(xp + 4 * min(p.c0 + lane + WAVE * i, p.c1 - 1));
   }
+  float acc[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
     if (s < p.nslots) {
 #pragma unroll
       for (int i = 0; i < MAXC; ++i) {
 #pragma unroll
         for (int rr = 0; rr < 2; ++rr) {
-          acc[rr] = dot8_bf(r.a[s][rr][i], x[i], acc[rr]);
-          if (DUAL) acc[2 + rr] = dot8_bf(r.b[s][rr][i], x[i], acc[2 + rr]);
+          acc[s][rr] = dot8_bf(r.a[s][rr][i], x[i], acc[s][rr]);
+          if (DUAL) acc[s][2 + rr] = dot8_bf(r.b[s][rr][i], x[i], acc[s][2 + rr]);
         }
       }
     }
+  }
+  // several full-wave sums per butterfly; the totals are then spread to every lane of their quad
+  if (DUAL) {
 #pragma unroll
-    for (int j = 0; j < (DUAL ? 4 : 2); ++j) res[s][j] = (s < p.nslots) ? wave_sum(acc[j]) : 0.f;
-    if (!DUAL) res[s][2] = res[s][3] = 0.f;
+    for (int s = 0; s < 2; ++s)
+      if (s < p.nslots) {
+        const float z = wave_sum4(acc[s][0], acc[s][1], acc[s][2], acc[s][3]);
+        res[s][0] = dpp_f<0x00>(z); res[s][1] = dpp_f<0x55>(z); res[s][2] = dpp_f<0xAA>(z); res[s][3] = dpp_f<0xFF>(z);
+      }
+  } else if (p.nslots > 1) {
+    const float z = wave_sum4(acc[0][0], acc[0][1], acc[1][0], acc[1][1]);
+    res[0][0] = dpp_f<0x00>(z); res[0][1] = dpp_f<0x55>(z); res[1][0] = dpp_f<0xAA>(z); res[1][1] = dpp_f<0xFF>(z);
+  } else if (p.nslots > 0) {
+    const float z = wave_sum2(acc[0][0], acc[0][1]);
+    res[0][0] = dpp_f<0x00>(z); res[0][1] = dpp_f<0x55>(z);
   }
   if (p.KS > 1) {  // uniform over the workgroup
     if (lane == 0) { red[wave * 4 + 0] = res[0][0]; red[wave * 4 + 1] = res[0][1]; red[wave * 4 + 2] = res[0][2]; red[wave * 4 + 3] = res[0][3]; }
@@ -677,7 +689,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
         TS(10);
         gemv_compute<2, true>(xp, P_sw, w3, red, [&](int gp, float v0, float v1, float u0, float u1) {
           const float a0 = bf2f(f2bf(v0)), a1 = bf2f(f2bf(v1)), c0 = bf2f(f2bf(u0)), c1 = bf2f(f2bf(u1));
-          const float s0 = bf2f(f2bf(a0 / (1.0f + expf(-a0)))), s1 = bf2f(f2bf(a1 / (1.0f + expf(-a1))));
+          const float s0 = bf2f(f2bf(a0 * __builtin_amdgcn_rcpf(1.0f + __expf(-a0)))), s1 = bf2f(f2bf(a1 * __builtin_amdgcn_rcpf(1.0f + __expf(-a1))));
           rep_st(hbuf, gp, pack2(s0 * c0, s1 * c1), ep);
         });
       }
@@ -961,7 +973,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           TS(71);
           gemv_compute<2, true>(xp, R_sw, wr, red, [&](int gp, float v0, float v1, float u0, float u1) {
             const float a0 = bf2f(f2bf(v0)), a1 = bf2f(f2bf(v1)), c0 = bf2f(f2bf(u0)), c1 = bf2f(f2bf(u1));
-            const float s0 = bf2f(f2bf(a0 / (1.0f + expf(-a0)))), s1 = bf2f(f2bf(a1 / (1.0f + expf(-a1))));
+            const float s0 = bf2f(f2bf(a0 * __builtin_amdgcn_rcpf(1.0f + __expf(-a0)))), s1 = bf2f(f2bf(a1 * __builtin_amdgcn_rcpf(1.0f + __expf(-a1))));
             rep_st(hb, gp, pack2(s0 * c0, s1 * c1), ep);
           });
         }
