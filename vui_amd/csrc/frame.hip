@@ -292,16 +292,21 @@ __device__ __forceinline__ void poll_add(float* dst, const uint64_t* buf, int nw
 #define LDS_RED (LDS_QKV + 1536)         // 64 floats
 #define LDS_MISC (LDS_RED + 256)         // 64 ints: sampled codes of the frame
 #define LDS_SAMP (LDS_MISC + 256)        // SampleShared
-#define LDS_FIXED (LDS_SAMP + 1280)
+#define LDS_FIXED (LDS_SAMP + 1280)  // SampleShared with its optional stamps
 
 // optional per-phase timestamps (100 MHz wall clock) of four workgroups, for profiling: kept in LDS
 // as 16-bit deltas + 8-bit tags while the frame runs (a global store per stamp would sit in the
 // in-order memory queue in front of the weight loads) and written out at the end
 #define PROF_EVENTS 1000
+#ifdef VUI_SAMPLE_CLOCK
+#define PROF_KEEP(id) ((id) == 0 || (id) >= 40)  // room for the sampler's own stamps
+#else
+#define PROF_KEEP(id) true
+#endif
 #define PROF_LDS_BYTES (PROF_EVENTS * 3 + 8)
 #define TS(id)                                                                      \
   do {                                                                              \
-    if (prof_on && tid == 0 && nts < PROF_EVENTS) {                                 \
+    if (prof_on && tid == 0 && nts < PROF_EVENTS && PROF_KEEP(id)) {                                 \
       const uint64_t now_ = wall_clock64();                                         \
       const uint64_t dl_ = now_ - ts_prev;                                          \
       prof_dt[nts] = (uint16_t)(dl_ > 65535 ? 65535 : dl_);                         \
@@ -310,6 +315,23 @@ __device__ __forceinline__ void poll_add(float* dst, const uint64_t* buf, int nw
       ++nts;                                                                        \
     }                                                                               \
   } while (0)
+
+// a thread's E consecutive logits (elements tid*E ...) from the packed staging area
+__device__ __forceinline__ void load_logits8(const uint32_t* lgw, int E, int CS, float (&raw)[8]) {
+  const int tid = threadIdx.x;
+  if (E == 8 && !(CS & 7)) {
+    uint4 r = make_uint4(0, 0, 0, 0);
+    if (tid * 8 < CS) r = reinterpret_cast<const uint4*>(lgw)[tid];
+    raw[0] = bf_lo(r.x); raw[1] = bf_hi(r.x); raw[2] = bf_lo(r.y); raw[3] = bf_hi(r.y);
+    raw[4] = bf_lo(r.z); raw[5] = bf_hi(r.z); raw[6] = bf_lo(r.w); raw[7] = bf_hi(r.w);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int j = tid * E + e;
+      raw[e] = (e < E && j < CS) ? bf2f(reinterpret_cast<const bf16_t*>(lgw)[j]) : 0.f;
+    }
+  }
+}
 
 struct LayerP { const bf16_t *attn_norm, *wqkv, *wo, *mlp_norm, *w1, *w3, *w2; };
 
@@ -741,24 +763,25 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       }
       if (a.mode & FR_CB0) {
         const int E = (a.CS + FR_THREADS - 1) / FR_THREADS;
-        poll_set(lg, rep_rd(lgbuf), a.CS / 2, c);
+        poll_words((uint32_t*)lg, rep_rd(lgbuf), a.CS / 2, c);
         const bool greedy = (a.topk0 == 1) || !(a.temp0 > 0.f);
         const float div = greedy ? 1.0f : a.temp0;
         const float* counts = (a.rep_counts && a.penalty > 1.0f) ? a.rep_counts : nullptr;
-        float lv[8];
+        float lv[8], raw[8];
         uint32_t key[8];
+        load_logits8((const uint32_t*)lg, E, a.CS, raw);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           lv[e] = -INFINITY;
           key[e] = 0u;
           const int j = tid * E + e;
           if (e < E && j < a.CS) {
-            lv[e] = sample_value(lg[j], nullptr, j, counts, a.penalty, div);
-            key[e] = float_key(counts ? lv[e] : lg[j]);
+            lv[e] = sample_value(raw[e], nullptr, j, counts, a.penalty, div);
+            key[e] = float_key(counts ? lv[e] : raw[e]);
           }
         }
         TS(20);
-        code0 = block_sample<8>(lv, key, counts ? 0 : 16, a.CS, E, greedy, a.topk0, a.seed0, frame0, 0u, 0u, ssh);
+        code0 = block_sample<8>(lv, key, counts ? 0 : 16, a.CS, E, greedy, a.topk0, a.seed0, frame0, 0u, 0u, ssh, (int*)sc);
         TS(21);
       }
     }
@@ -1005,26 +1028,35 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
         gemv_compute<2, false>(xp, R_hd, wr, red, [&](int gp, float v0, float v1, float, float) {
           rep_st(lgbuf, gp, pack2(v0, v1), ep); });
         TS(42);
-        poll_set(lg, rep_rd(lgbuf), CS / 2, c);
+        poll_words((uint32_t*)lg, rep_rd(lgbuf), CS / 2, c);
         TS(43);
         const int E = (CS + FR_THREADS - 1) / FR_THREADS;
         const bool greedy = (a.topk1 == 1) || !(a.temp1 > 0.f);
         const float div = greedy ? 1.0f : a.temp1;
         const float* bias = a.logit_bias ? a.logit_bias + (size_t)(t - 1) * CS : nullptr;
-        float lv[8];
+        float lv[8], raw[8];
         uint32_t key[8];
+        load_logits8((const uint32_t*)lg, E, CS, raw);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           lv[e] = -INFINITY;
           key[e] = 0u;
           const int j = tid * E + e;
           if (e < E && j < CS) {
-            lv[e] = sample_value(lg[j], bias, j, nullptr, 1.0f, div);
-            key[e] = float_key(bias ? lv[e] : lg[j]);
+            lv[e] = sample_value(raw[e], bias, j, nullptr, 1.0f, div);
+            key[e] = float_key(bias ? lv[e] : raw[e]);
           }
         }
-        prev_code = block_sample<8>(lv, key, bias ? 0 : 16, CS, E, greedy, a.topk1, a.seed1, frame1, 0u, (uint32_t)t, ssh);
+        prev_code = block_sample<8>(lv, key, bias ? 0 : 16, CS, E, greedy, a.topk1, a.seed1, frame1, 0u, (uint32_t)t, ssh, (int*)sc);
         TS(44);
+#ifdef VUI_SAMPLE_CLOCK
+        if (prof_on && tid == 0) {
+          nts -= 1;  // replace stamp 44 by the sampler's own
+          ts_prev -= prof_dt[nts];
+          for (int k = 0; k < 8; ++k)
+            if (nts < PROF_EVENTS) { prof_dt[nts] = (uint16_t)(ssh.ts[k] - ts_prev); prof_id[nts] = (uint8_t)(60 + k); ts_prev = ssh.ts[k]; ++nts; }
+        }
+#endif
         if (tid == 0) codes_l[t] = prev_code;
       }
     }

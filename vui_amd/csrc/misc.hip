@@ -83,6 +83,7 @@ int launch_rope(int dtype, void* x, const float* table, const int32_t* pos, int 
 template <typename T, int EMAX>
 __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const SampleArgs p) {
   __shared__ SampleShared sh;
+  __shared__ __align__(16) int hist[HIST_WORDS];
   const int b = blockIdx.x, tid = threadIdx.x;
   const int CS = p.CS;
   const int E = (CS + SAMP_THREADS - 1) / SAMP_THREADS;  // contiguous elements per thread
@@ -108,7 +109,7 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const SampleArgs p
   }
   const uint32_t frame = p.frame_ctr ? (uint32_t)p.frame_ctr[0] : 0u;
   const int pick = block_sample<EMAX>(l, key, raw_keys ? 16 : 0, CS, E, greedy, p.top_k, p.seed, frame, (uint32_t)b,
-                                      (uint32_t)p.codebook, sh);
+                                      (uint32_t)p.codebook, sh, hist);
 
   if (tid == 0) {
     p.out[(size_t)b * p.out_stride + p.out_col] = (int64_t)pick;

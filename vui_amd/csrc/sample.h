@@ -31,8 +31,7 @@ struct SampleShared {
   float wsum[SAMP_THREADS / WAVE];
   int cnt[2][3 * SAMP_THREADS / WAVE];
   int pick;
-  int hist[256];   // 8-bit digit histogram of the 16-bit key search
-  int sel[2];      // chosen digit, count of keys above it
+  int sel[2][2];   // 16-bit key search, per round: chosen digit, count of keys above it
 #ifdef VUI_SAMPLE_CLOCK
   unsigned long long ts[8];
 #endif
@@ -42,32 +41,78 @@ struct SampleShared {
 #else
 #define SAMP_TS(k) do { } while (0)
 #endif
+// The 8-bit digit histogram of the 16-bit key search can be kept in HIST_COPIES copies (thread t adds
+// to copy t % HIST_COPIES) against serialised additions to one LDS word; measured, one copy is fastest.
+#define HIST_COPIES 1
+#define HIST_WORDS (HIST_COPIES * 256)
+
+// Wave 0 finds, in the 256-bin histogram (hist: HIST_WORDS ints of LDS), the largest digit whose suffix count (keys with digit >= it)
+// reaches `need`, stores {digit, keys above it} and clears the bins for the next round.
+__device__ __forceinline__ void hist_select(int* hist, int need, int* out) {
+  const int lane = threadIdx.x & 63;
+  int4 b = make_int4(0, 0, 0, 0);  // bins 4*lane .. 4*lane+3, summed over the copies
+#pragma unroll
+  for (int c = 0; c < HIST_COPIES; ++c) {
+    const int4 t = *reinterpret_cast<const int4*>(&hist[c * 256 + 4 * lane]);
+    *reinterpret_cast<int4*>(&hist[c * 256 + 4 * lane]) = make_int4(0, 0, 0, 0);
+    b.x += t.x; b.y += t.y; b.z += t.z; b.w += t.w;
+  }
+  const int s3 = b.w, s2 = s3 + b.z, s1 = s2 + b.y, s0 = s1 + b.x;  // suffix sums inside the lane
+  // exclusive suffix over the lanes: keys in the bins of higher lanes
+  int v = s0;
+  v += dpp_i<0x101>(v);  // row_shl:1 (a lane reads from higher lanes of its row, 0 from outside)
+  v += dpp_i<0x102>(v);
+  v += dpp_i<0x104>(v);
+  v += dpp_i<0x108>(v);
+  {
+    const int t3 = __builtin_amdgcn_readlane(v, 48), t2 = __builtin_amdgcn_readlane(v, 32), t1 = __builtin_amdgcn_readlane(v, 16);
+    const int row = lane >> 4;
+    v += (row <= 2 ? t3 : 0) + (row <= 1 ? t2 : 0) + (row <= 0 ? t1 : 0);
+  }
+  const int above = v - s0;
+  // bin k of this lane: suffix = above + s_k, suffix beyond it = suffix - bin_k
+  int digit = -1, over = 0;
+  if (above + s3 >= need && above < need) { digit = 4 * lane + 3; over = above; }
+  else if (above + s2 >= need && above + s3 < need) { digit = 4 * lane + 2; over = above + s3; }
+  else if (above + s1 >= need && above + s2 < need) { digit = 4 * lane + 1; over = above + s2; }
+  else if (above + s0 >= need && above + s1 < need) { digit = 4 * lane; over = above + s1; }
+  if (digit >= 0) { out[0] = digit; out[1] = over; }
+}
 
 // One draw from the values l[e] (element index tid*E + e, -inf beyond CS) held by a 256-thread
 // block.  RQ rule (src/vui/model.py:955-962): drop l < k-th largest, softmax, draw.  code-0 rule
 // (src/vui/engine.py:855-863): softmax, keep the top-k probabilities, renormalise, draw.  Both
 // are: keep {l >= k-th largest l}, weights exp(l - max), inverse CDF in index order with one
 // uniform.  greedy: the lowest index of the maximum.  Every thread returns the same pick.
+// hist: HIST_WORDS ints of LDS scratch (16-byte aligned) for the digit histograms.
 //
 // key[e] orders the elements for the top-k cut (any order-preserving image of l[e]); bits below
-// low_bit are known to carry no information (16 when the keys come from bf16 values), so the
-// search for the k-th largest key, two bits per barrier, only walks bits 31..low_bit and stops
-// as soon as exactly top_k keys lie above the candidate.
+// low_bit are known to carry no information (16 when the keys come from bf16 values).  16-bit keys:
+// two rounds of an 8-bit digit histogram; otherwise two bits per barrier over bits 31..low_bit,
+// stopping as soon as exactly top_k keys lie above the candidate.
 template <int EMAX>
 __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32_t (&key)[EMAX], int low_bit, int CS,
                                             int E, bool greedy, int top_k, uint64_t seed, uint32_t frame,
-                                            uint32_t row, uint32_t codebook, SampleShared& sh) {
+                                            uint32_t row, uint32_t codebook, SampleShared& sh, int* hist) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   SAMP_TS(0);
+  const uint32_t rnd = philox_u32(seed, frame, row, codebook, 0u);  // ahead of the first wait
+  const bool digits = top_k > 0 && top_k < CS && low_bit == 16 && !greedy;
   float m = -INFINITY; int mi = 0x7fffffff;
 #pragma unroll
   for (int e = 0; e < EMAX; ++e)
     if (e < E && l[e] > m) { m = l[e]; mi = tid * E + e; }
   {
-    const float wm = wave_max(m);
+    const float wm = rows_max(group16_max(m));
+    // the index of the maximum is the answer of a greedy draw and the fallback of a sampled one
     const int cand = wave_min_i((m == wm) ? mi : 0x7fffffff);
     if (lane == 0) { sh.sred[wave] = wm; sh.ired[wave] = cand; }
   }
+  if (digits) {
+#pragma unroll
+    for (int i = 0; i < HIST_WORDS / SAMP_THREADS; ++i) hist[tid + SAMP_THREADS * i] = 0;
+  }
+  if (tid == 0) sh.pick = -1;
   __syncthreads();
   float M = sh.sred[0]; int Mi = sh.ired[0];
 #pragma unroll
@@ -75,52 +120,28 @@ __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32
     if (sh.sred[w] > M) { M = sh.sred[w]; Mi = sh.ired[w]; }
     else if (sh.sred[w] == M) Mi = min(Mi, sh.ired[w]);
   }
-  __syncthreads();
-  if (greedy) return Mi;
+  if (greedy) { __syncthreads(); return Mi; }
   SAMP_TS(1);
 
   // key of the k-th largest value
   uint32_t thr = 0u;
-  if (top_k > 0 && top_k < CS && low_bit == 16) {
-    // 16-bit keys: two rounds of an 8-bit digit histogram in LDS (high byte, then low byte among the
-    // keys that share the chosen high byte); the digit is the largest one whose suffix count reaches k
+  if (digits) {
+    // high byte, then low byte among the keys that share the chosen high byte
     int need = top_k;
 #pragma unroll
     for (int round = 0; round < 2; ++round) {
       const int shift = round == 0 ? 24 : 16;
-      sh.hist[tid] = 0;  // SAMP_THREADS == 256 bins
-      __syncthreads();
 #pragma unroll
       for (int e = 0; e < EMAX; ++e)
         if (e < E && tid * E + e < CS && (round == 0 || (key[e] >> 24) == (thr >> 24)))
-          atomicAdd(&sh.hist[(key[e] >> shift) & 255], 1);
+          atomicAdd(&hist[(tid & (HIST_COPIES - 1)) * 256 + ((key[e] >> shift) & 255)], 1);
       __syncthreads();
-      // suffix sums over the 256 bins: thread t owns bin t; S(t) = sum of bins >= t
-      const int mine = sh.hist[tid];
-      // reverse inclusive scan: row_shl shifts (a lane reads from higher lanes of its row; lanes shifted in
-      // from outside read 0), then the totals of the higher rows
-      int v = mine;
-      v += dpp_i<0x101>(v);  // row_shl:1
-      v += dpp_i<0x102>(v);  // row_shl:2
-      v += dpp_i<0x104>(v);  // row_shl:4
-      v += dpp_i<0x108>(v);  // row_shl:8
-      {
-        const int t3 = __builtin_amdgcn_readlane(v, 48), t2 = __builtin_amdgcn_readlane(v, 32), t1 = __builtin_amdgcn_readlane(v, 16);
-        const int row = lane >> 4;
-        v += (row <= 2 ? t3 : 0) + (row <= 1 ? t2 : 0) + (row <= 0 ? t1 : 0);
-      }
-      if (lane == 0) sh.cnt[0][wave] = v;  // wave total
+      SAMP_TS(2 + 2 * round);
+      if (wave == 0) hist_select(hist, need, sh.sel[round]);
       __syncthreads();
-      int above = 0;  // keys in higher waves' bins
-#pragma unroll
-      for (int w = 0; w < SAMP_THREADS / WAVE; ++w) if (w > wave) above += sh.cnt[0][w];
-      const int suffix = v + above;          // keys with digit >= tid
-      const int suffix_next = suffix - mine; // keys with digit > tid
-      if (suffix >= need && suffix_next < need) { sh.sel[0] = tid; sh.sel[1] = suffix_next; }
-      __syncthreads();
-      thr |= (uint32_t)sh.sel[0] << shift;
-      need -= sh.sel[1];
-      __syncthreads();
+      SAMP_TS(3 + 2 * round);
+      thr |= (uint32_t)sh.sel[round][0] << shift;
+      need -= sh.sel[round][1];
     }
   } else if (top_k > 0 && top_k < CS) {
     int it = 0;
@@ -153,14 +174,13 @@ __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32
       if (tsel == top_k) break;  // exactly k keys are >= thr: the kept set is final
     }
   }
-  SAMP_TS(2);
   // weights, their total, and the inverse CDF in index order
   float wloc = 0.f;
   float pw[EMAX];
 #pragma unroll
   for (int e = 0; e < EMAX; ++e) {
     pw[e] = 0.f;
-    if (e < E && tid * E + e < CS && key[e] >= thr) pw[e] = expf(l[e] - M);
+    if (e < E && tid * E + e < CS && key[e] >= thr) pw[e] = __expf(l[e] - M);
     wloc += pw[e];
   }
   // inclusive scan over the wave: shifts inside each row of 16 lanes, then the row totals
@@ -174,15 +194,12 @@ __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32
     const int row = lane >> 4;
     incl += (row >= 1 ? t0 : 0.f) + (row >= 2 ? t1 : 0.f) + (row >= 3 ? t2 : 0.f);
   }
-  SAMP_TS(3);
+  SAMP_TS(6);
   if (lane == WAVE - 1) sh.wsum[wave] = incl;
-  if (tid == 0) sh.pick = -1;
   __syncthreads();
   float base = 0.f, total = 0.f;
 #pragma unroll
   for (int w = 0; w < SAMP_THREADS / WAVE; ++w) { if (w < wave) base += sh.wsum[w]; total += sh.wsum[w]; }
-  SAMP_TS(4);
-  const uint32_t rnd = philox_u32(seed, frame, row, codebook, 0u);
   const float u = (float)(rnd >> 8) * (1.0f / 16777216.0f);
   const float target = u * total;
   const float before = base + incl - wloc;  // sum of everything ahead of this thread
@@ -200,8 +217,8 @@ __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32
   }
   __syncthreads();
   const int pick = (sh.pick >= 0) ? sh.pick : Mi;
-  SAMP_TS(5);
-  __syncthreads();
+  SAMP_TS(7);
+  __syncthreads();  // the next draw may rewrite the shared state
   return pick;
 }
 
