@@ -292,7 +292,8 @@ __device__ __forceinline__ void poll_add(float* dst, const uint64_t* buf, int nw
 #define LDS_RED (LDS_QKV + 1536)         // 64 floats
 #define LDS_MISC (LDS_RED + 256)         // 64 ints: sampled codes of the frame
 #define LDS_SAMP (LDS_MISC + 256)        // SampleShared
-#define LDS_FIXED (LDS_SAMP + 1280)  // SampleShared with its optional stamps
+#define LDS_PTAB (LDS_SAMP + 1280)       // 64 floats: penalty^count, count = 0..63 (SampleShared with its optional stamps before it)
+#define LDS_FIXED (LDS_PTAB + 256)
 
 // optional per-phase timestamps (100 MHz wall clock) of four workgroups, for profiling: kept in LDS
 // as 16-bit deltas + 8-bit tags while the frame runs (a global store per stamp would sit in the
@@ -366,6 +367,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
   float* red = (float*)(smem + LDS_RED);
   int* codes_l = (int*)(smem + LDS_MISC);
   SampleShared& ssh = *(SampleShared*)(smem + LDS_SAMP);
+  float* ptab = (float*)(smem + LDS_PTAB);
   LayerP* lp = (LayerP*)(smem + LDS_FIXED);          // backbone layers, then depth-head layers
   bf16_t* rqkv = (bf16_t*)(smem + a.lds_kv_off);
 
@@ -408,6 +410,8 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
     }
     lp[i] = t;
   }
+  // repetition penalty factors by count; counts stay below the window, the rest falls back to powf
+  if ((a.mode & FR_CB0) && a.rep_counts && a.penalty > 1.0f && tid < 64) ptab[tid] = powf(a.penalty, (float)tid);
   const bf16_t* g_final_norm = (const bf16_t*)W.final_norm;
   const bf16_t* g_codec_head = (const bf16_t*)W.codec_head;
   const bf16_t* g_eos_w = (const bf16_t*)W.eos_w;
@@ -763,10 +767,23 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       }
       if (a.mode & FR_CB0) {
         const int E = (a.CS + FR_THREADS - 1) / FR_THREADS;
-        poll_words((uint32_t*)lg, rep_rd(lgbuf), a.CS / 2, c);
         const bool greedy = (a.topk0 == 1) || !(a.temp0 > 0.f);
         const float div = greedy ? 1.0f : a.temp0;
         const float* counts = (a.rep_counts && a.penalty > 1.0f) ? a.rep_counts : nullptr;
+        // this thread's repetition counts, fetched ahead of the wait for the logits
+        float cn[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (counts) {
+          if (E == 8 && !(a.CS & 7)) {
+            if (tid * 8 < a.CS) {
+              const float4 c0 = *reinterpret_cast<const float4*>(counts + tid * 8), c1 = *reinterpret_cast<const float4*>(counts + tid * 8 + 4);
+              cn[0] = c0.x; cn[1] = c0.y; cn[2] = c0.z; cn[3] = c0.w; cn[4] = c1.x; cn[5] = c1.y; cn[6] = c1.z; cn[7] = c1.w;
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { const int j = tid * E + e; if (e < E && j < a.CS) cn[e] = counts[j]; }
+          }
+        }
+        poll_words((uint32_t*)lg, rep_rd(lgbuf), a.CS / 2, c);
         float lv[8], raw[8];
         uint32_t key[8];
         load_logits8((const uint32_t*)lg, E, a.CS, raw);
@@ -776,7 +793,12 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           key[e] = 0u;
           const int j = tid * E + e;
           if (e < E && j < a.CS) {
-            lv[e] = sample_value(raw[e], nullptr, j, counts, a.penalty, div);
+            float v = raw[e];
+            if (counts) {  // src/vui/engine.py:571-576
+              const float f = (cn[e] >= 0.f && cn[e] < 64.f) ? ptab[(int)cn[e]] : powf(a.penalty, cn[e]);
+              v = (v > 0.f) ? v / f : v * f;
+            }
+            lv[e] = v / div;
             key[e] = float_key(counts ? lv[e] : raw[e]);
           }
         }

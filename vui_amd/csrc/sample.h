@@ -31,7 +31,7 @@ struct SampleShared {
   float wsum[SAMP_THREADS / WAVE];
   int cnt[2][3 * SAMP_THREADS / WAVE];
   int pick;
-  int sel[2][2];   // 16-bit key search, per round: chosen digit, count of keys above it
+  int sel[4][2];   // key search, per 8-bit round: chosen digit, count of keys above it
 #ifdef VUI_SAMPLE_CLOCK
   unsigned long long ts[8];
 #endif
@@ -87,8 +87,8 @@ __device__ __forceinline__ void hist_select(int* hist, int need, int* out) {
 // hist: HIST_WORDS ints of LDS scratch (16-byte aligned) for the digit histograms.
 //
 // key[e] orders the elements for the top-k cut (any order-preserving image of l[e]); bits below
-// low_bit are known to carry no information (16 when the keys come from bf16 values).  16-bit keys:
-// two rounds of an 8-bit digit histogram; otherwise two bits per barrier over bits 31..low_bit,
+// low_bit are known to carry no information (16 when the keys come from bf16 values).  low_bit 16 or 0:
+// two or four rounds of an 8-bit digit histogram; otherwise two bits per barrier over bits 31..low_bit,
 // stopping as soon as exactly top_k keys lie above the candidate.
 template <int EMAX>
 __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32_t (&key)[EMAX], int low_bit, int CS,
@@ -97,7 +97,7 @@ __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   SAMP_TS(0);
   const uint32_t rnd = philox_u32(seed, frame, row, codebook, 0u);  // ahead of the first wait
-  const bool digits = top_k > 0 && top_k < CS && low_bit == 16 && !greedy;
+  const bool digits = top_k > 0 && top_k < CS && (low_bit == 16 || low_bit == 0) && !greedy;
   float m = -INFINITY; int mi = 0x7fffffff;
 #pragma unroll
   for (int e = 0; e < EMAX; ++e)
@@ -126,14 +126,16 @@ __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32
   // key of the k-th largest value
   uint32_t thr = 0u;
   if (digits) {
-    // high byte, then low byte among the keys that share the chosen high byte
+    // one byte per round from the top, each among the keys that share the bytes chosen so far
     int need = top_k;
+    const int rounds = (32 - low_bit) / 8;
 #pragma unroll
-    for (int round = 0; round < 2; ++round) {
-      const int shift = round == 0 ? 24 : 16;
+    for (int round = 0; round < 4; ++round) {
+      if (round >= rounds) break;
+      const int shift = 24 - 8 * round;
 #pragma unroll
       for (int e = 0; e < EMAX; ++e)
-        if (e < E && tid * E + e < CS && (round == 0 || (key[e] >> 24) == (thr >> 24)))
+        if (e < E && tid * E + e < CS && (round == 0 || (key[e] >> (shift + 8)) == (thr >> (shift + 8))))
           atomicAdd(&hist[(tid & (HIST_COPIES - 1)) * 256 + ((key[e] >> shift) & 255)], 1);
       __syncthreads();
       SAMP_TS(2 + 2 * round);
