@@ -105,7 +105,7 @@ def gpu_bench(args):
 # HBM traffic of one frame_kernel launch on the default workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch) scaled by what the same counters read for a plain copy of known size;
 # see profiles/frame_kernel_e2e_b1.txt.  None until measured.
-MEASURED_TRAFFIC_BYTES = 518_986_473  # at cache length 596..651 (algorithmic 414.6 MB there): 1.25 x
+MEASURED_TRAFFIC_BYTES = 517_680_951  # at cache length 596..651 (algorithmic 414.6 MB there): 1.25 x
 
 
 def kernel_roofline(out, fb):
