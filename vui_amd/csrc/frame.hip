@@ -431,26 +431,38 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
     pos = a.seq_lens[slot];
     if (pos < 0) pos = 0;
     if (pos >= a.S) pos = a.S - 1;
-    // input embedding, redundantly in every workgroup (all row loads of a feature in flight together)
+    // input embedding, redundantly in every workgroup: the clamped table rows go through LDS once, then
+    // each thread sums feature pairs tid and tid + 256 with all row loads of both in flight together
     if (a.codes_in) {
-      const bf16_t* table = (const bf16_t*)W.audio_emb;
-      for (int k = tid; k < d; k += FR_THREADS) {
-        float s = 0.f;
-        for (int q0 = 0; q0 < a.Q; q0 += 16) {
-          bf16_t r[16];
+      const uint32_t* table = (const uint32_t*)W.audio_emb;
+      int* rows = codes_l;  // free until the depth head
+      for (int q = tid; q < a.Q; q += FR_THREADS) {
+        int64_t cc = a.codes_in[q];
+        cc = cc < 0 ? 0 : (cc >= a.CS ? a.CS - 1 : cc);
+        rows[q] = (int)(cc + (int64_t)q * a.CS);
+      }
+      __syncthreads();
+      float s0[2] = {0.f, 0.f}, s1[2] = {0.f, 0.f};
+      for (int q0 = 0; q0 < a.Q; q0 += 16) {
+        uint32_t r[2][16];
 #pragma unroll
-          for (int q = 0; q < 16; ++q) {
-            r[q] = 0;
-            if (q0 + q < a.Q) {
-              int64_t cc = a.codes_in[q0 + q];
-              cc = cc < 0 ? 0 : (cc >= a.CS ? a.CS - 1 : cc);
-              r[q] = table[(size_t)(cc + (int64_t)(q0 + q) * a.CS) * d + k];
-            }
+        for (int q = 0; q < 16; ++q) {
+          const int row = rows[min(q0 + q, a.Q - 1)];
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            const int j = tid + FR_THREADS * i;
+            r[i][q] = (q0 + q < a.Q && 2 * j < d) ? table[((size_t)row * d) / 2 + j] : 0u;
           }
-#pragma unroll
-          for (int q = 0; q < 16; ++q) if (q0 + q < a.Q) s += bf2f(r[q]);
         }
-        xres[k] = bf2f(f2bf(s));
+#pragma unroll
+        for (int q = 0; q < 16; ++q)
+#pragma unroll
+          for (int i = 0; i < 2; ++i) { s0[i] += bf_lo(r[i][q]); s1[i] += bf_hi(r[i][q]); }
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int j = tid + FR_THREADS * i;
+        if (2 * j < d) { const uint32_t pk = f2bf2(s0[i], s1[i]); xres[2 * j] = bf_lo(pk); xres[2 * j + 1] = bf_hi(pk); }
       }
     } else {
       for (int k = tid; k < d; k += FR_THREADS) xres[k] = bf2f(a.emb_in[k]);
