@@ -599,6 +599,134 @@ class OracleModel:
 
 
 # --------------------------------------------------------------------------------------
+# streaming control loop of one row
+# --------------------------------------------------------------------------------------
+FRAME_RATE = 12.5
+DEFAULT_WPS = 3.0  # engine.py:41
+GATE_RETRY_TEMPS = (0.5, 0.3)  # engine.py:1367
+
+
+def max_turn_frames(n_words: int, prompt_wps: float, max_turn_secs: float = 15.0, max_turn_wps: float = 0.0) -> int:
+    """Reference: GenConfig.max_turn_frames, engine.py:88-103."""
+    ceil = int(max_turn_secs * FRAME_RATE)
+    wps = max_turn_wps if max_turn_wps > 0 else prompt_wps
+    if wps <= 0:
+        wps = DEFAULT_WPS
+    if n_words <= 0:
+        return ceil
+    return min(int((n_words / wps * 1.6 + 0.6) * FRAME_RATE), ceil)
+
+
+def stream_row(model: "OracleModel", chunks, *, temperature: float = 0.9, top_k: int = 100, rq_top_k: int = 100,
+               rep_penalty: float = 1.1, rep_window: int = 24, eos_threshold: float = 0.45, min_secs: float = 0.5,
+               max_turn_secs: float = 15.0, max_secs: float = 30.0, n_codebooks: int = 0, max_turn_wps: float = 0.0,
+               gate_frames: int = 0, gate_entropy_max: float = 1.9, gate_retries: int = 2, seed: int = 0,
+               prompt_wps: float = 0.0, max_seq: int | None = None, slot: int = 0, cancel_after: int | None = None,
+               log: list | None = None) -> list[Tensor]:
+    """Restatement of Engine._stream_row (engine.py:1308-1521) on the oracle model, one turn with a
+    fresh repetition state.  chunks: list of (emb (T, d), n_words).  Returns the yielded code
+    frames.  The draw for frame f of the turn uses uniform01(seed, f, 0, codebook); a frame whose
+    EOS test ends the chunk still consumes its counter (the device step draws it before the test).
+    cancel_after: behave as if cancel were set once that many frames have been yielded.
+    log: receives ("retry", chunk, temp) / ("eos", chunk, step) / ("cap", chunk) events and the EOS
+    probability of every step as ("p", chunk, step, probability)."""
+    d = model.dims
+    max_frames = int(max_secs * FRAME_RATE)
+    min_frames = int(min_secs * FRAME_RATE)
+    max_seq = (max_seq if max_seq is not None else d.max_seqlen) - 10
+    s = torch.tensor([slot])
+    rep = RepState(d.codebook_size, rep_window)
+    out: list[Tensor] = []
+    fctr = 0
+
+    def cancelled() -> bool:
+        return cancel_after is not None and len(out) >= cancel_after
+
+    def probs_of(cb0, temp):
+        return torch.softmax(rep_penalise(cb0, rep.counts, rep_penalty) / temp, dim=-1)
+
+    def ent(p):
+        return float(-(p * p.clamp_min(1e-9).log()).sum(-1).mean())
+
+    def draw0(cb0, temp, k):
+        nonlocal fctr
+        c = sample_cb0(cb0, rep.counts, rep_penalty, temp, k, uniform01(seed, fctr, 0, 0))
+        if rep_penalty > 1.0:
+            rep.push(c)
+        return c
+
+    for ci, (emb, n_words) in enumerate(chunks):
+        if len(out) >= max_frames or int(model.seq_lens[slot]) >= max_seq or cancelled():
+            return out
+        use_gate = gate_frames > 0 and ci == 0
+        chunk_start = int(model.seq_lens[slot])
+        max_per_turn = max_turn_frames(n_words, prompt_wps, max_turn_secs, max_turn_wps)
+        retry_idx = 0
+        while True:
+            cur_temp = temperature
+            if retry_idx > 0:
+                cur_temp = GATE_RETRY_TEMPS[min(retry_idx - 1, len(GATE_RETRY_TEMPS) - 1)]
+                model.seq_lens[slot] = chunk_start
+                rep = RepState(d.codebook_size, rep_window)
+                if log is not None:
+                    log.append(("retry", ci, cur_temp))
+            hidden = model.prefill(emb, slot)[-1:]
+            cb0, _ = model.heads(hidden)
+            held: list[Tensor] = []
+            entropies: list[float] = []
+            if use_gate:
+                entropies.append(ent(probs_of(cb0, cur_temp)))
+            rq_k = rq_top_k if top_k != 1 else 1
+            c0 = draw0(cb0[0], cur_temp, 1 if top_k == 1 else 0)
+            frame = model.rq_generate(hidden, torch.tensor([c0]), cur_temp, rq_k, None, n_codebooks, seed, fctr)[0]
+            fctr += 1
+            (held if use_gate else out).append(frame)
+            retry = False
+            for step in range(1, max_per_turn):
+                if len(out) >= max_frames or int(model.seq_lens[slot]) >= max_seq:
+                    out.extend(held)
+                    if log is not None:
+                        log.append(("cap", ci))
+                    return out
+                if cancelled():
+                    return out
+                hidden, cb0, eos = model.decode_step(frame[None], s)
+                gathering = use_gate and len(held) < gate_frames
+                if gathering:
+                    entropies.append(ent(probs_of(cb0, cur_temp)))
+                c0 = draw0(cb0[0], cur_temp, top_k)
+                p_eos = float(torch.sigmoid(eos[0, 0].float()))
+                if log is not None:
+                    log.append(("p", ci, step, p_eos))
+                if step >= min_frames and p_eos > eos_threshold:
+                    out.extend(held)
+                    held = []
+                    fctr += 1
+                    if log is not None:
+                        log.append(("eos", ci, step))
+                    break
+                frame = model.rq_generate(hidden, torch.tensor([c0]), cur_temp, rq_k, None, n_codebooks, seed, fctr)[0]
+                fctr += 1
+                if gathering:
+                    held.append(frame)
+                    if len(held) == gate_frames:
+                        if sum(entropies) / len(entropies) > gate_entropy_max and retry_idx < gate_retries:
+                            retry = True
+                            break
+                        out.extend(held)
+                        held = []
+                        use_gate = False
+                else:
+                    out.append(frame)
+            if retry:
+                retry_idx += 1
+                continue
+            out.extend(held)
+            break
+    return out
+
+
+# --------------------------------------------------------------------------------------
 # deterministic synthetic weights (the benchmark's "random-init N(0, 0.02) from seed 0")
 # --------------------------------------------------------------------------------------
 def state_dict_shapes(d: Dims) -> dict[str, tuple[int, ...]]:

@@ -9,7 +9,8 @@ enter as embeddings or token ids.
 from __future__ import annotations
 
 import ctypes as C
-from dataclasses import dataclass
+from dataclasses import dataclass, replace
+from typing import Iterator
 
 import torch
 from torch import Tensor
@@ -18,6 +19,8 @@ from . import _lib
 from .model import MAX_BATCH, Graph, Vui, make_sample_params
 
 FRAME_RATE = 12.5  # codec frames per second (src/vui/qwen_codec.py:27-30)
+DEFAULT_WPS = 3.0  # words per second when the prompt gives none (src/vui/engine.py:41)
+GATE_RETRY_TEMPS = (0.5, 0.3)  # src/vui/engine.py:1367
 
 
 @dataclass(frozen=True)
@@ -35,8 +38,35 @@ class GenConfig:
     max_turn_secs: float = 15.0
     max_secs: float = 30.0
     n_codebooks: int = 0  # 0 = all Q quantizers
+    max_turn_wps: float = 0.0  # >0: override the words-per-second of the chunk duration cap
+    gate_frames: int = 0  # hallucination gate (engine.py:78-86): 0 = off
+    gate_entropy_max: float = 1.9
+    gate_retries: int = 2
     rq_top_k: int = 100  # the reference bakes top_k=100 into the RQ graphs (engine.py:393-397)
     seed: int = 0
+
+    def max_turn_frames(self, n_words: int, prompt_wps: float = 0.0) -> int:
+        """Frame cap of one chunk from its word count (src/vui/engine.py:88-103)."""
+        ceil = int(self.max_turn_secs * FRAME_RATE)
+        wps = self.max_turn_wps if self.max_turn_wps > 0 else prompt_wps
+        if wps <= 0:
+            wps = DEFAULT_WPS
+        if n_words <= 0:
+            return ceil
+        secs = n_words / wps * 1.6 + 0.6
+        return min(int(secs * FRAME_RATE), ceil)
+
+
+@dataclass
+class Chunk:
+    """One text chunk of a turn as the decode loop needs it: the embeddings of `[spk] text` (with
+    `[SC]` appended on a turn's last chunk) that Engine._add_agent_text writes (src/vui/engine.py:825-844;
+    tokenising and chunking the text is the caller's), the word count that caps the chunk's
+    length, and the speaker-change flag of chunk_text."""
+
+    emb: Tensor  # (1, T, d)
+    n_words: int = 0
+    sc: bool = False
 
 
 def _make_buckets(max_bs: int) -> list[int]:
@@ -65,6 +95,7 @@ class Row:
         self._idx = idx
         self._prompt_offset = 0
         self._closed = False
+        self.prompt_wps: float = 0.0
         self._slot = torch.tensor([idx], dtype=torch.int32, device=engine.device)
 
     @property
@@ -79,6 +110,15 @@ class Row:
         """Write a (1, T, d) embedding block at the row's offset; returns the final-norm output
         (1, T, d).  Engine._prefill_emb, src/vui/engine.py:674-694."""
         return self._engine._prefill_emb(self, emb)
+
+    def stream(self, chunks: "list[Chunk]", cfg: GenConfig = GenConfig(), cancel=None, *, reset_rep: bool = True,
+               final_turn: bool = False) -> Iterator[Tensor]:
+        """Streams the code frames of one assistant turn, chunk by chunk (Row.stream,
+        src/vui/engine.py:204-244; frames of codes instead of audio, the vocoder is not part of this
+        package).  cancel: object with is_set(), polled per frame."""
+        if self._engine.max_rows != 1:
+            raise RuntimeError(f"stream() requires Engine(max_rows=1), got {self._engine.max_rows}")
+        yield from self._engine._stream_row(self, chunks, cfg, cancel, reset_rep=reset_rep, final_turn=final_turn)
 
     def mark_prompt(self) -> int:
         self._prompt_offset = self.offset
@@ -310,8 +350,9 @@ class Engine:
             return hit
         nat = self.model._native
         dec = self.model.decoder
-        frames = torch.zeros(max_frames, B, self.Q, dtype=torch.long, device=self.device)
-        eos = torch.zeros(max_frames, B, dtype=torch.float32, device=self.device)
+        # max_frames == 0: no frame log, eos holds the (B) probabilities of the latest step
+        frames = torch.zeros(max_frames, B, self.Q, dtype=torch.long, device=self.device) if max_frames else None
+        eos = torch.zeros(max(max_frames, 1), B, dtype=torch.float32, device=self.device)
         sp0 = make_sample_params(cfg.temperature, cfg.top_k, cfg.seed, self._frame_ctr)
         sp1 = make_sample_params(cfg.temperature, cfg.rq_top_k if cfg.top_k != 1 else 1, cfg.seed, self._frame_ctr)
         use_rep = cfg.rep_penalty > 1.0
@@ -325,7 +366,7 @@ class Engine:
                 dec._k.data_ptr(), dec._v.data_ptr(), self._rep_counts.data_ptr() if use_rep else None,
                 _lib.ptr(self._rep_history) if win else None, self._rep_pos.data_ptr() if win else None,
                 float(cfg.rep_penalty), win, C.byref(sp0), C.byref(sp1), None, nq, self._g_hidden_out.data_ptr(),
-                self._g_cb0_out.data_ptr(), eos.data_ptr(), frames.data_ptr(), max_frames,
+                self._g_cb0_out.data_ptr(), eos.data_ptr(), _lib.ptr(frames), max_frames,
                 self._frame_ctr.data_ptr(), ns, st), "vui_frame_step")
 
         # captured without a warm-up run: the step mutates seq_lens, the rep state and the counter
@@ -375,3 +416,140 @@ class Engine:
                 torch.cuda.current_stream().synchronize()
         torch.cuda.current_stream().synchronize()
         return frames[:n_frames, :, :nq].clone(), eos[:n_frames].clone()
+
+    # ------------------------------------------------------------------ streaming single-row turn
+    def _penalised_probs(self, cb0: Tensor, counts: Tensor, cfg: GenConfig, temp: float) -> Tensor:
+        """softmax(rep_apply(cb0) / temp) as the reference forms it for the gate statistics
+        (src/vui/engine.py:571-576, 1412, 1455)."""
+        lf = cb0.float()
+        if cfg.rep_penalty > 1.0:
+            factor = torch.pow(torch.tensor(cfg.rep_penalty, device=lf.device), counts)
+            lf = torch.where(lf > 0, lf / factor, lf * factor)
+        return torch.softmax(lf / temp, dim=-1)
+
+    @torch.inference_mode()
+    def _stream_row(self, row: Row, chunks: "list[Chunk]", cfg: GenConfig, cancel=None, *, reset_rep: bool = True,
+                    final_turn: bool = False) -> Iterator[Tensor]:
+        """Per-frame streaming decode of one row; yields (Q',) int64 code frames.
+
+        The control flow of src/vui/engine.py:1308-1521: per chunk write its text, draw frame 0 from
+        the text's last hidden state (no top-k, engine.py:1411-1424), then one decode step per frame
+        until the EOS probability passes cfg.eos_threshold (after min_secs), the chunk's word-count
+        cap, cfg.max_secs or the cache limit; the optional gate holds the first cfg.gate_frames
+        frames of the first chunk, and on high mean entropy rewinds the cache to the chunk start and
+        retries colder.  A frame step here is one graph replay that also runs the depth head; when
+        the EOS test then ends the chunk, that frame is dropped (the reference tests before its depth
+        head runs: same frames out)."""
+        if not chunks:
+            return
+        max_frames = int(cfg.max_secs * FRAME_RATE)
+        min_frames = int(cfg.min_secs * FRAME_RATE)
+        max_seq = self.max_seq - 10
+        nq = cfg.n_codebooks if cfg.n_codebooks > 0 else self.Q
+        identity = row.idx == 0
+        slot_idx = None if identity else row._slot
+        codes_io = self._g_codes_in if identity else self._gc_codes_in
+        nat = self.model._native
+        stream = torch.cuda.current_stream()
+        if reset_rep:
+            self._rep_reset(cfg.rep_penalty, cfg.rep_window)
+            self._frame_ctr.zero_()  # draws are keyed by (seed, frame of the turn, row, codebook)
+        total_frames = 0
+        use_rep = cfg.rep_penalty > 1.0
+
+        def cancelled() -> bool:
+            return cancel is not None and cancel.is_set()
+
+        def entropy_top1(probs: Tensor) -> tuple[float, float]:
+            ent = -(probs * probs.clamp_min(1e-9).log()).sum(-1).mean().item()
+            return ent, probs.max(-1).values.mean().item()
+
+        last_idx = len(chunks) - 1
+        offset = row.offset
+        for ci, chunk in enumerate(chunks):
+            if total_frames >= max_frames or offset >= max_seq or cancelled():
+                return
+            # (speaker alternation on chunk.sc is the caller's: it picks the [spk] token inside chunk.emb)
+            use_gate = cfg.gate_frames > 0 and ci == 0 and reset_rep
+            chunk_start = offset
+            gate_target = cfg.gate_frames
+            max_per_turn = cfg.max_turn_frames(chunk.n_words, row.prompt_wps)
+            retry_idx = 0
+            while True:  # retry loop: a single pass unless the gate asks for a colder one
+                cur_temp = cfg.temperature
+                if retry_idx > 0:
+                    cur_temp = GATE_RETRY_TEMPS[min(retry_idx - 1, len(GATE_RETRY_TEMPS) - 1)]
+                    self.seq_lens[row.idx] = chunk_start
+                    self._rep_reset(cfg.rep_penalty, cfg.rep_window)
+                cfg_t = replace(cfg, temperature=cur_temp)
+                hidden = self._prefill_emb(row, chunk.emb)[:, -1]  # (1, d)
+                offset = chunk_start + chunk.emb.shape[1]
+                cb0 = self.model.codec_head(hidden)
+                held: list[Tensor] = []
+                entropies: list[float] = []
+                top1s: list[float] = []
+                if use_gate:
+                    e, p1 = entropy_top1(self._penalised_probs(cb0, self._rep_counts[row.idx:row.idx + 1], cfg, cur_temp))
+                    entropies.append(e)
+                    top1s.append(p1)
+                # frame 0 of the chunk: no top-k cut unless greedy
+                code0 = self._sample_cb0(cb0, cfg_t, top_k=1 if cfg.top_k == 1 else 0)
+                sp1 = make_sample_params(cur_temp, cfg.rq_top_k if cfg.top_k != 1 else 1, cfg.seed, self._frame_ctr)
+                _lib.check(nat.lib.vui_rq_generate(nat.handle, hidden.contiguous().data_ptr(), code0.data_ptr(), None, nq,
+                                                   C.byref(sp1), codes_io.data_ptr(), self.Q, 1, 1, stream.cuda_stream),
+                           "vui_rq_generate")
+                self._frame_ctr += 1
+                frame = codes_io[0, :nq].clone()
+                if use_gate:
+                    held.append(frame)
+                else:
+                    yield frame
+                    total_frames += 1
+                g, _, eos_now, _ = self._frame_graph(1, cfg_t, slot_idx, 0)
+                retry_triggered = False
+                for step in range(1, max_per_turn):
+                    if total_frames >= max_frames or offset >= max_seq:
+                        for hc in held:
+                            yield hc
+                            total_frames += 1
+                        return
+                    if cancelled():
+                        return
+                    gathering = use_gate and len(held) < gate_target
+                    counts_before = self._rep_counts[row.idx:row.idx + 1].clone() if (gathering and use_rep) else None
+                    g.replay()  # backbone step on the previous frame, code-0 draw + push, depth head
+                    offset += 1
+                    if gathering:
+                        cnt = counts_before if counts_before is not None else self._rep_counts[row.idx:row.idx + 1]
+                        e, p1 = entropy_top1(self._penalised_probs(self._g_cb0_out[0:1], cnt, cfg, cur_temp))
+                        entropies.append(e)
+                        top1s.append(p1)
+                    if step >= min_frames and eos_now[0, 0].item() > cfg.eos_threshold:
+                        for hc in held:
+                            yield hc
+                            total_frames += 1
+                        held = []
+                        break
+                    frame = codes_io[0, :nq].clone()
+                    if gathering:
+                        held.append(frame)
+                        if len(held) == gate_target:
+                            avg_e = sum(entropies) / len(entropies)
+                            if avg_e > cfg.gate_entropy_max and retry_idx < cfg.gate_retries:
+                                retry_triggered = True
+                                break
+                            for hc in held:
+                                yield hc
+                                total_frames += 1
+                            held = []
+                            use_gate = False
+                    else:
+                        yield frame
+                        total_frames += 1
+                if retry_triggered:
+                    retry_idx += 1
+                    continue
+                for hc in held:  # chunk shorter than the gate: flushed without a decision
+                    yield hc
+                    total_frames += 1
+                break
