@@ -453,9 +453,14 @@ class Vui:
                 state_dict = ck["model"]
         state_dict = {k.replace("module.", "").replace("text_embedding.", "token_emb."): v
                       for k, v in state_dict.items()}
-        cfg = Config.from_dict(config)
-        if "spk_proj.weight" in state_dict:
-            cfg.model.has_spk_proj = True
+        # older checkpoints carry the optional projections without their config flags
+        # (infer_optional_modules, src/vui/config.py:81-101); a flag present in the config wins
+        mcfg = dict(config.get("model") or {})
+        for flag, sentinel in (("has_sq_proj", "sq_proj.proj.0.weight"), ("has_wps_proj", "wps_proj.proj.0.weight"),
+                               ("has_spk_proj", "spk_proj.weight")):
+            if sentinel in state_dict and flag not in mcfg:
+                mcfg[flag] = True
+        cfg = Config.from_dict({**config, "model": mcfg})
         return Vui(cfg, state_dict, device=device, dtype=dtype)
 
     @staticmethod
