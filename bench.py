@@ -39,19 +39,18 @@ def frame_bytes(m, L_avg: float, esz: int = 2) -> dict:
 def gpu_bench(args):
     import torch
 
-    from oracle.vui_oracle import Dims, synthetic_state_dict  # weights generator only (shared with the tests)
-    from tests.util import dims_to_config
     from vui_amd.engine import Engine, GenConfig
     from vui_amd.model import Vui
+    from vui_amd.synthetic import nano_for_cache, synthetic_state_dict
 
     torch.manual_seed(0)
     n_prefix, n_text = 512, 64
     K, W = args.steps, args.warmup
-    d = Dims() if args.preset == "A" else Dims(rq_d_model=768, rq_n_layers=5, rq_n_heads=8, vocab_size=50534)
+    d = nano_for_cache(args.preset, 64).model  # architecture numbers
     max_seq = 64 * ((n_prefix + n_text + K + W + 2 + 63) // 64)
     t0 = time.time()
     sd = synthetic_state_dict(d, seed=0)
-    model = Vui(dims_to_config(d, max_seq), sd, device="cuda", dtype=torch.bfloat16)
+    model = Vui(nano_for_cache(args.preset, max_seq), sd, device="cuda", dtype=torch.bfloat16)
     eng = Engine(model=model, max_rows=1, max_seq=max_seq)
     row = eng.new_row()
     g = torch.Generator().manual_seed(0)
@@ -119,14 +118,14 @@ def kernel_roofline(out, fb):
             "traffic": MEASURED_TRAFFIC_BYTES, "us_per_launch": round(us, 2), "algorithmic_bytes": int(fb["frame"])}
 
 
-def suite(model, eng, d, sd):
+def suite(model, eng, d, sd, preset="A"):
     """Extra lines for the other benchmark configs: backbone step at KV 256/1024/4096, depth head alone,
     16 int8 streams with ragged caches."""
     import torch
 
-    from tests.util import dims_to_config
     from vui_amd.engine import Engine, GenConfig
     from vui_amd.model import Vui
+    from vui_amd.synthetic import nano_for_cache
 
     lines = []
     m = model.config.model
@@ -142,7 +141,7 @@ def suite(model, eng, d, sd):
         return e0.elapsed_time(e1) * 1e3 / n
 
     # config 2: backbone decode step, B=1, N(0,1) cache at three lengths (the walk over 200 steps is centred on L)
-    model2 = Vui(dims_to_config(d, 4608), sd, device="cuda", dtype=torch.bfloat16)
+    model2 = Vui(nano_for_cache(preset, 4608), sd, device="cuda", dtype=torch.bfloat16)
     eng2 = Engine(model=model2, max_rows=1, max_seq=4608)
     model2.decoder._k.normal_()
     model2.decoder._v.normal_()
@@ -166,10 +165,44 @@ def suite(model, eng, d, sd):
     b = frame_bytes(m, 0)["rq_unique"]
     lines.append({"config": "rq_head_b1", "frames": 1000, "us_per_frame": round(us, 2), "unique_bytes": int(b),
                   "achieved_GBs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4)})
+    # prompt ingestion: 576 positions (512 audio frames + 64 text tokens) in one pass per layer against the
+    # position-by-position path; flops = 2 x positions x backbone weights (attention is a few % more)
+    emb = (torch.randn(1, 576, m.d_model, generator=g) * 0.08).to(torch.bfloat16).cuda()
+    dec = model2.decoder
+
+    def prefill_once():
+        eng2.seq_lens[0] = 0
+        dec.forward_flash(emb, None)
+
+    prefill_once()
+    us_pass = timed(prefill_once, 5)
+    dec.PREFILL_MIN = 10 ** 9
+    prefill_once()
+    us_loop = timed(prefill_once, 2)
+    dec.PREFILL_MIN = 4
+    wparams = (frame_bytes(m, 0)["backbone"] - 67584 - m.n_quantizers * m.d_model * 2 - 3145728) / 2
+    fl = 2.0 * 576 * wparams
+    lines.append({"config": "prefill_b1", "positions": 576, "ms_one_pass": round(us_pass / 1e3, 3), "ms_position_by_position": round(us_loop / 1e3, 2),
+                  "achieved_TFLOPs": round(fl / us_pass / 1e6, 1), "mfma_frac": round(fl / us_pass / 1e6 / 2500.0, 4)})
+    # a streamed turn: one graph replay per frame plus the host's per-frame EOS read (Row.stream)
+    from vui_amd.engine import Chunk
+    eng2.seq_lens[0] = 0
+    row2 = eng2.new_row()
+    chunks = [Chunk(emb=emb[:, :16].contiguous(), n_words=40) for _ in range(4)]
+    cfg_s = GenConfig(eos_threshold=2.0, max_secs=60.0)
+    n_out = sum(1 for _ in row2.stream(chunks[:1], cfg_s))  # warm: graph capture
+    row2.reset()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    n_out = sum(1 for _ in row2.stream(chunks, cfg_s))
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    lines.append({"config": "stream_b1", "frames": n_out, "chunks": 4, "ms_per_frame_wall": round(dt * 1e3 / n_out, 4),
+                  "frames_per_s": round(n_out / dt, 1), "rtf": round(n_out / dt / 12.5, 2)})
     del eng2, model2
     # config 5: 16 streams, int8 backbone weights, ragged caches U[128, 2048]
     S = 2048 + 256
-    model5 = Vui(dims_to_config(d, S), sd, device="cuda", dtype=torch.bfloat16, int8=True)
+    model5 = Vui(nano_for_cache(preset, S), sd, device="cuda", dtype=torch.bfloat16, int8=True)
     eng5 = Engine(model=model5, max_rows=16, max_seq=S)
     model5.decoder._k.normal_()
     model5.decoder._v.normal_()
@@ -190,7 +223,7 @@ def suite(model, eng, d, sd):
     return lines
 
 
-def cpu_baseline(d, sd, n_frames: int = 12, n_ctx: int = 96):
+def cpu_baseline(preset, n_frames: int = 12, n_ctx: int = 96):
     """The CPU oracle (a port of the reference's fp32 CPU path) on a bounded sample of the same
     workload: a 96-position prefill, then n_frames greedy-free sampled frames; host cores of this box."""
     import torch
@@ -199,6 +232,8 @@ def cpu_baseline(d, sd, n_frames: int = 12, n_ctx: int = 96):
 
     threads = min(16, os.cpu_count() or 1)
     torch.set_num_threads(threads)
+    d = O.Dims() if preset == "A" else O.Dims(rq_d_model=768, rq_n_layers=5, rq_n_heads=8, vocab_size=50534)
+    sd = O.synthetic_state_dict(d, seed=0)
     o = O.OracleModel(d, sd, torch.float32, max_seqlen=n_ctx + n_frames + 8)
     g = torch.Generator().manual_seed(0)
     ids = torch.randint(0, d.vocab_size, (n_ctx,), generator=g)
@@ -232,9 +267,9 @@ def main():
     out, (model, eng, d, sd) = gpu_bench(args)
     if not args.no_roofline:
         out["roofline"] = kernel_roofline(out, out["frame_bytes"])
-    extra = suite(model, eng, d, sd) if args.suite else []
+    extra = suite(model, eng, d, sd, args.preset) if args.suite else []
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(d, sd)
+        out["cpu_baseline"] = cpu_baseline(args.preset)
     if args.calib:
         import torch
 

@@ -169,6 +169,18 @@ int vui_rq_generate(vui_ctx* ctx, const void* hidden, const int64_t* code0, cons
                     int n_q, const vui_sample_params* sp, int64_t* codes_out, int codes_stride, int zero_pad,
                     int B, vui_stream_t stream);
 
+/* Prompt ingestion: T new positions of ONE row in one pass per layer (GEMMs on the matrix cores,
+ * causal attention against the cache), bf16 weights only.
+ *   Decoder.forward_flash with T > 1 / Engine._prefill_emb  (model.py:534-549, engine.py:674-694)
+ * emb_in (T, d) bf16 device: the embeddings to append at positions pos0 .. pos0+T-1 of `slot`
+ * (pos0 is the slot's current length, passed from the host because the launch shapes depend on it);
+ * K/V rows are appended to the caches, seq_lens[slot] becomes pos0 + T, hidden_out (T, d) bf16
+ * receives the final-norm outputs.  scratch: device memory of vui_prefill_scratch_bytes(cfg, T,
+ * pos0 + T) bytes, 256-byte aligned; the library allocates nothing. */
+int64_t vui_prefill_scratch_bytes(const vui_config* cfg, int T, int L);
+int vui_prefill(vui_ctx* ctx, const void* emb_in, int T, int slot, int pos0, int32_t* seq_lens, void* k_cache,
+                void* v_cache, void* hidden_out, void* scratch, int64_t scratch_bytes, vui_stream_t stream);
+
 /* The whole per-frame step: backbone step on codes_io, code-0 sampling, RQ head; the new frame
  * is written back to codes_io (zero-padded to Q) so the call can be repeated or replayed.
  *   Engine._stream_row / _render_rows loop body (engine.py:1450-1485, 1011-1044)

@@ -62,6 +62,8 @@ SIGNATURES = {
     "vui_ctx_fused": (_I, [_P, _I]),
     "vui_ctx_status": (_I, [_P]),
     "vui_debug_phase_clock": (_I, [_P, _P, _I, _I]),
+    "vui_prefill_scratch_bytes": (_L, [C.POINTER(VuiConfigC), _I, _I]),
+    "vui_prefill": (_I, [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _L, _P]),
     "vui_backbone_step": (_I, [_P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _P]),
     "vui_sample_cb0": (_I, [_P, _P, _P, _P, _P, _F, _I, C.POINTER(SampleParamsC), _P, _I, _P]),
     "vui_rq_generate": (_I, [_P, _P, _P, _P, _I, C.POINTER(SampleParamsC), _P, _I, _I, _I, _P]),

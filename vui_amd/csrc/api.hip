@@ -228,6 +228,20 @@ static int check_batch(vui_ctx* ctx, int B, int n_splits) {
   return VUI_OK;
 }
 
+int64_t vui_prefill_scratch_bytes(const vui_config* c, int T, int L) {
+  if (!c || T < 1 || L < T) { vui_set_error("vui_prefill_scratch_bytes: bad arguments"); return VUI_EINVAL; }
+  return (int64_t)prefill_scratch_bytes(*c, T, L);
+}
+
+int vui_prefill(vui_ctx* ctx, const void* emb_in, int T, int slot, int pos0, int32_t* seq_lens, void* k_cache, void* v_cache,
+                void* hidden_out, void* scratch, int64_t scratch_bytes, vui_stream_t stream) {
+  if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
+  if (!emb_in || !seq_lens || !k_cache || !v_cache || !hidden_out || !scratch) { vui_set_error("vui_prefill: NULL argument"); return VUI_EINVAL; }
+  if (((uintptr_t)scratch & 255) || scratch_bytes < 0) { vui_set_error("vui_prefill: scratch must be 256-byte aligned"); return VUI_EINVAL; }
+  return launch_prefill(ctx->cfg, ctx->w, emb_in, T, slot, pos0, seq_lens, k_cache, v_cache, hidden_out, scratch,
+                        (size_t)scratch_bytes, (hipStream_t)stream);
+}
+
 int vui_backbone_step(vui_ctx* ctx, const int64_t* codes_in, const void* emb_in, const int32_t* slot_idx,
                       int32_t* seq_lens, const int32_t* seq_inc, int B, void* k_cache, void* v_cache, void* hidden_out,
                       void* cb0_out, void* eos_out, int n_splits, vui_stream_t stream) {

@@ -188,6 +188,11 @@ bool frame_supported(const vui_config& c, int nwg, int ns, char* why, size_t why
 int frame_max_resident(size_t lds_bytes, int* n_cu);
 int launch_frame(const FrameArgs& a, int nwg, size_t lds_bytes, hipStream_t st);
 
+// prefill.hip
+size_t prefill_scratch_bytes(const vui_config& c, int T, int L);
+int launch_prefill(const vui_config& c, const vui_weights& w, const void* emb, int T, int slot, int pos0, int32_t* seq_lens,
+                   void* k_cache, void* v_cache, void* out, void* scratch, size_t scratch_bytes, hipStream_t st);
+
 void vui_set_error(const char* fmt, ...);
 #define HIP_TRY(expr)                                                                  \
   do {                                                                                 \

@@ -1,0 +1,298 @@
+// Prompt ingestion: T > 1 new positions of one row through the backbone in one pass per layer.
+//
+//   Decoder.forward_flash / Engine._prefill_emb with T > 1  (src/vui/model.py:534-549, engine.py:674-694)
+//
+// bf16 only.  Per layer: row RMSNorm, QKV GEMM, RoPE + cache append, scores = q K^T (fp32, one
+// GEMM batched over heads against the cache itself), causal softmax (probabilities rounded to
+// bf16), transpose of the values, P V GEMM, out_proj GEMM with the residual add in its epilogue,
+// row RMSNorm, W1 / W3 GEMMs, SwiGLU product, W2 GEMM with residual.  Every GEMM is the same
+// matrix-core kernel: C (M x N) = X (M x K) W^T (N x K), K contiguous in both operands.
+//
+// Rounding points are those of the single-position step (one rounding after each linear, two in
+// the norm, products of the rotation rounded before their sum, residual sums rounded).
+#include "common.h"
+#include "internal.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 pf_bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float pf_floatx4;
+union PfU128 { uint4 u; pf_bf16x8 v; };
+__device__ __forceinline__ pf_bf16x8 pf_frag(const uint4& x) { PfU128 t; t.u = x; return t.v; }
+
+enum { PF_BF16 = 0, PF_RESID = 1, PF_F32_SCALE = 2 };
+
+struct PfGemm {
+  const bf16_t* X;   // activations (M x K), row stride ldx
+  const bf16_t* W;   // "weights" (N x K), row stride ldw
+  void* C;           // output (M x N), row stride ldc; bf16 (PF_BF16, PF_RESID: in place on the residual) or fp32
+  int M, N, K, ldx, ldw, ldc;
+  size_t xb, wb, cb;  // element offsets per batch index z: X + z*xb, W + (z / wgroup)*wb, C + z*cb
+  int wgroup;
+  float scale;
+};
+
+// Workgroup: 64 rows x 64 features, four waves in a 2 x 2 arrangement of 32 x 32 tiles, each four
+// v_mfma_f32_16x16x32_bf16 per K step of 32.  Operand A of the instruction is the weight tile (lane:
+// feature lane % 16, eight k from (lane / 16) * 8), operand B the activation tile (lane: row lane % 16,
+// same k): the lane then holds four consecutive features of one row.  Fragments go from global memory
+// straight to registers, the next step's loads are issued before this step's instructions.
+template <int EPI>
+__global__ __launch_bounds__(256) void pf_gemm_kernel(const PfGemm p) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int l16 = lane & 15, kg = lane >> 4;
+  const int z = blockIdx.z;
+  const int m0 = blockIdx.x * 64 + (wave & 1) * 32, n0 = blockIdx.y * 64 + (wave >> 1) * 32;
+  if (m0 >= p.M || n0 >= p.N) return;  // the whole 32 x 32 tile is outside
+  const bf16_t* X = p.X + (size_t)z * p.xb;
+  const bf16_t* W = p.W + (size_t)(z / p.wgroup) * p.wb;
+  const bf16_t* xr[2];
+  const bf16_t* wr[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    xr[j] = X + (size_t)min(m0 + 16 * j + l16, p.M - 1) * p.ldx + kg * 8;
+    wr[j] = W + (size_t)min(n0 + 16 * j + l16, p.N - 1) * p.ldw + kg * 8;
+  }
+  pf_floatx4 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = pf_floatx4{0.f, 0.f, 0.f, 0.f};
+  uint4 xa[2], wa[2], xn[2], wn[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) { xa[j] = *reinterpret_cast<const uint4*>(xr[j]); wa[j] = *reinterpret_cast<const uint4*>(wr[j]); }
+  for (int k = 0; k < p.K; k += 32) {
+    const int kn = (k + 32 < p.K) ? k + 32 : k;  // the last step reloads itself (unused)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) { xn[j] = *reinterpret_cast<const uint4*>(xr[j] + kn); wn[j] = *reinterpret_cast<const uint4*>(wr[j] + kn); }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)    // feature tile
+#pragma unroll
+      for (int j = 0; j < 2; ++j)  // row tile
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf_frag(wa[i]), pf_frag(xa[j]), acc[i][j], 0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) { xa[j] = xn[j]; wa[j] = wn[j]; }
+  }
+  // lane holds features n0 + 16 i + 4 kg + r (r = 0..3) of row m0 + 16 j + l16
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int m = m0 + 16 * j + l16, n = n0 + 16 * i + 4 * kg;
+      if (m >= p.M || n >= p.N) continue;
+      const pf_floatx4 a = acc[i][j];
+      if (EPI == PF_F32_SCALE) {
+        float* c = (float*)p.C + (size_t)z * p.cb + (size_t)m * p.ldc + n;
+        if (n + 3 < p.N) *reinterpret_cast<float4*>(c) = make_float4(a[0] * p.scale, a[1] * p.scale, a[2] * p.scale, a[3] * p.scale);
+        else for (int r = 0; r < 4; ++r) if (n + r < p.N) c[r] = a[r] * p.scale;
+      } else {
+        bf16_t* c = (bf16_t*)p.C + (size_t)z * p.cb + (size_t)m * p.ldc + n;
+        float v[4] = {a[0], a[1], a[2], a[3]};
+        if (EPI == PF_RESID) {  // x = rnd(x + rnd(y)), src/vui/model.py:367, 374
+          const uint2 old = *reinterpret_cast<const uint2*>(c);
+          v[0] = bf_lo(old.x) + bf2f(f2bf(v[0])); v[1] = bf_hi(old.x) + bf2f(f2bf(v[1]));
+          v[2] = bf_lo(old.y) + bf2f(f2bf(v[2])); v[3] = bf_hi(old.y) + bf2f(f2bf(v[3]));
+        }
+        if (n + 3 < p.N) *reinterpret_cast<uint2*>(c) = make_uint2(f2bf2(v[0], v[1]), f2bf2(v[2], v[3]));
+        else for (int r = 0; r < 4; ++r) if (n + r < p.N) c[r] = f2bf(v[r]);
+      }
+    }
+}
+
+// two-rounding RMSNorm of rows (src/vui/model.py:286-297); one wave per row
+__global__ __launch_bounds__(256) void pf_rownorm_kernel(const bf16_t* x, const bf16_t* w, bf16_t* y, int M, int K, float eps) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (row >= M) return;
+  const bf16_t* xr = x + (size_t)row * K;
+  float ss = 0.f;
+  for (int c = lane; c < K / 8; c += WAVE) {
+    float v[8];
+    El<bf16_t>::ld8(xr + c * 8, v);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss = fmaf(v[e], v[e], ss);
+  }
+  ss = wave_sum(ss);
+  const float r = 1.0f / sqrtf(ss / (float)K + eps);
+  for (int c = lane; c < K / 8; c += WAVE) {
+    float v[8], g[8], o[8];
+    El<bf16_t>::ld8(xr + c * 8, v);
+    El<bf16_t>::ld8(w + c * 8, g);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = bf2f(f2bf(v[e] * r)) * g[e];
+    El<bf16_t>::st8(y + (size_t)row * K + c * 8, o);
+  }
+}
+
+// interleaved rotation of q (in place) and k, append of k and v to the cache at positions pos0 + t
+// (src/vui/rope.py:16-77, model.py:234-247)
+__global__ __launch_bounds__(256) void pf_rope_append_kernel(bf16_t* qkv, bf16_t* kc, bf16_t* vc, const float* rope, int T,
+                                                             int nq, int nkv, int hd, int rope_dim, int pos0, int slot, int S) {
+  const int t = blockIdx.x;
+  const int pos = pos0 + t;
+  bf16_t* row = qkv + (size_t)t * (nq + 2 * nkv);
+  for (int pr = threadIdx.x; pr < (nq + 2 * nkv) / 2; pr += blockDim.x) {
+    const int n = 2 * pr;
+    uint32_t v = *reinterpret_cast<const uint32_t*>(row + n);
+    int region, m;
+    if (n < nq) { region = 0; m = n; }
+    else if (n < nq + nkv) { region = 1; m = n - nq; }
+    else { region = 2; m = n - nq - nkv; }
+    const int dd = m % hd;
+    if (region != 2 && dd < rope_dim) {
+      const float4 f = *reinterpret_cast<const float4*>(rope + ((size_t)pos * rope_dim + dd) * 2);  // cos, sin of dd and dd + 1
+      const float a = bf_lo(v), b = bf_hi(v);
+      v = f2bf2(rope_mix(a, f.x, -b, f.y), rope_mix(b, f.z, a, f.w));
+    }
+    if (region == 0) *reinterpret_cast<uint32_t*>(row + n) = v;
+    else *reinterpret_cast<uint32_t*>((region == 1 ? kc : vc) + ((size_t)slot * S + pos) * nkv + m) = v;
+  }
+}
+
+// causal softmax of one (head, query) row of scores; probabilities rounded to bf16, zero outside the
+// visible range [start, pos0 + t] up to the padded length
+__global__ __launch_bounds__(256) void pf_softmax_kernel(const float* scores, bf16_t* P, int T, int Lpad, int pos0, int window) {
+  const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const float* s = scores + ((size_t)h * T + t) * Lpad;
+  bf16_t* o = P + ((size_t)h * T + t) * Lpad;
+  const int len = pos0 + t + 1;
+  const int start = window > 0 ? max(0, len - 1 - window) : 0;
+  __shared__ float red[8];
+  float m = -INFINITY;
+  for (int j = start + tid; j < len; j += 256) m = fmaxf(m, s[j]);
+  m = wave_max(m);
+  if ((tid & 63) == 0) red[tid >> 6] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  float sum = 0.f;
+  for (int j = start + tid; j < len; j += 256) sum += expf(s[j] - m);
+  sum = wave_sum(sum);
+  if ((tid & 63) == 0) red[4 + (tid >> 6)] = sum;
+  __syncthreads();
+  sum = (red[4] + red[5]) + (red[6] + red[7]);
+  const float inv = 1.0f / sum;
+  for (int j = tid; j < Lpad; j += 256) o[j] = (j >= start && j < len) ? f2bf(expf(s[j] - m) * inv) : (bf16_t)0;
+}
+
+// values of one row's cache slab, (L x KV*hd) -> per KV head (hd x Lpad), zero beyond L
+__global__ __launch_bounds__(256) void pf_transpose_v_kernel(const bf16_t* vc, bf16_t* vt, int L, int Lpad, int nkv, int hd) {
+  __shared__ bf16_t tile[32][33];
+  const int j0 = blockIdx.x * 32, f0 = blockIdx.y * 32;  // f over nkv (= KV*hd)
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+  for (int r = ty; r < 32; r += 8) {
+    const int j = j0 + r, f = f0 + tx;
+    tile[r][tx] = (j < L && f < nkv) ? vc[(size_t)j * nkv + f] : (bf16_t)0;
+  }
+  __syncthreads();
+  for (int r = ty; r < 32; r += 8) {
+    const int f = f0 + r, j = j0 + tx;
+    if (f < nkv && j < Lpad) vt[(size_t)f * Lpad + j] = tile[tx][r];  // head = f / hd, feature f % hd: rows of hd x Lpad blocks
+  }
+}
+
+// h = rnd(rnd(silu(a)) * b) in place on a (src/vui/model.py:282)
+__global__ __launch_bounds__(256) void pf_swiglu_kernel(bf16_t* a, const bf16_t* b, size_t n8) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n8) return;
+  float x[8], y[8], o[8];
+  El<bf16_t>::ld8(a + i * 8, x);
+  El<bf16_t>::ld8(b + i * 8, y);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = bf2f(f2bf(x[e] / (1.0f + expf(-x[e])))) * y[e];
+  El<bf16_t>::st8(a + i * 8, o);
+}
+
+__global__ void pf_set_len_kernel(int32_t* seq_lens, int slot, int v) { seq_lens[slot] = v; }
+
+static int pf_gemm(int epi, const PfGemm& g, int batch, hipStream_t st) {
+  if (g.K % 32 || g.M < 1 || g.N < 1) { vui_set_error("prefill GEMM: K=%d must be a multiple of 32", g.K); return VUI_EINVAL; }
+  dim3 grid((g.M + 63) / 64, (g.N + 63) / 64, batch);
+  if (epi == PF_BF16) hipLaunchKernelGGL(pf_gemm_kernel<PF_BF16>, grid, dim3(256), 0, st, g);
+  else if (epi == PF_RESID) hipLaunchKernelGGL(pf_gemm_kernel<PF_RESID>, grid, dim3(256), 0, st, g);
+  else hipLaunchKernelGGL(pf_gemm_kernel<PF_F32_SCALE>, grid, dim3(256), 0, st, g);
+  HIP_TRY(hipGetLastError());
+  return VUI_OK;
+}
+
+static size_t pf_align(size_t b) { return (b + 255) & ~(size_t)255; }
+
+// scratch: residual x, normed xn, qkv, attention output, two FFN buffers, scores, probabilities, transposed values
+size_t prefill_scratch_bytes(const vui_config& c, int T, int L) {
+  const size_t d = c.d_model, nq = (size_t)c.n_heads * c.head_dim, nkv = (size_t)c.n_kv_heads * c.head_dim;
+  const size_t Lpad = ((size_t)L + 31) & ~(size_t)31;
+  size_t b = 0;
+  b += pf_align((size_t)T * d * 2) * 2;
+  b += pf_align((size_t)T * (nq + 2 * nkv) * 2);
+  b += pf_align((size_t)T * nq * 2);
+  b += pf_align((size_t)T * c.ffn * 2) * 2;
+  b += pf_align((size_t)c.n_heads * T * Lpad * 4);
+  b += pf_align((size_t)c.n_heads * T * Lpad * 2);
+  b += pf_align(nkv * Lpad * 2);
+  return b;
+}
+
+int launch_prefill(const vui_config& c, const vui_weights& w, const void* emb, int T, int slot, int pos0, int32_t* seq_lens,
+                   void* k_cache, void* v_cache, void* out, void* scratch, size_t scratch_bytes, hipStream_t st) {
+  const int d = c.d_model, H = c.n_heads, KV = c.n_kv_heads, hd = c.head_dim, F = c.ffn, S = c.max_seqlen;
+  const int nq = H * hd, nkv = KV * hd, L = pos0 + T, Lpad = (L + 31) & ~31;
+  if (c.dtype != VUI_DTYPE_BF16 || c.int8_backbone) { vui_set_error("prefill: bf16 weights only"); return VUI_EINVAL; }
+  if (T < 1 || pos0 < 0 || L > S) { vui_set_error("prefill: positions %d..%d outside the cache (S=%d)", pos0, L, S); return VUI_EINVAL; }
+  if (slot < 0 || slot >= c.n_slots) { vui_set_error("prefill: slot %d outside [0,%d)", slot, c.n_slots); return VUI_EINVAL; }
+  if ((d % 32) || (F % 32) || (hd % 32) || (nkv % 8) || (c.rope_dim & 1)) { vui_set_error("prefill: d_model, ffn, head_dim must be multiples of 32"); return VUI_EINVAL; }
+  if (scratch_bytes < prefill_scratch_bytes(c, T, L)) { vui_set_error("prefill: scratch of %zu bytes, %zu needed", scratch_bytes, prefill_scratch_bytes(c, T, L)); return VUI_EINVAL; }
+  char* sp = (char*)scratch;
+  auto take = [&](size_t bytes) { char* r = sp; sp += pf_align(bytes); return r; };
+  bf16_t* x = (bf16_t*)take((size_t)T * d * 2);
+  bf16_t* xn = (bf16_t*)take((size_t)T * d * 2);
+  bf16_t* qkv = (bf16_t*)take((size_t)T * (nq + 2 * nkv) * 2);
+  bf16_t* att = (bf16_t*)take((size_t)T * nq * 2);
+  bf16_t* fa = (bf16_t*)take((size_t)T * F * 2);
+  bf16_t* fb = (bf16_t*)take((size_t)T * F * 2);
+  float* scores = (float*)take((size_t)H * T * Lpad * 4);
+  bf16_t* P = (bf16_t*)take((size_t)H * T * Lpad * 2);
+  bf16_t* vt = (bf16_t*)take((size_t)nkv * Lpad * 2);
+  HIP_TRY(hipMemcpyAsync(x, emb, (size_t)T * d * 2, hipMemcpyDeviceToDevice, st));
+  const size_t slab = (size_t)c.n_slots * S * nkv;
+  const float scale = 1.0f / sqrtf((float)hd);
+  int rc;
+  for (int l = 0; l < c.n_layers; ++l) {
+    const vui_layer_weights& lw = w.layers[l];
+    bf16_t* kc = (bf16_t*)k_cache + slab * l;
+    bf16_t* vc = (bf16_t*)v_cache + slab * l;
+    hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)lw.attn_norm, xn, T, d, c.norm_eps);
+    PfGemm g{};
+    g.X = xn; g.W = (const bf16_t*)lw.wqkv; g.C = qkv; g.M = T; g.N = nq + 2 * nkv; g.K = d; g.ldx = d; g.ldw = d; g.ldc = nq + 2 * nkv;
+    g.wgroup = 1; g.scale = 1.f;
+    if ((rc = pf_gemm(PF_BF16, g, 1, st))) return rc;
+    hipLaunchKernelGGL(pf_rope_append_kernel, dim3(T), dim3(256), 0, st, qkv, kc, vc, w.rope_table, T, nq, nkv, hd, c.rope_dim, pos0,
+                       slot, S);
+    // scores[h] = q_h K_h^T * scale over the L cached positions of this slot
+    const bf16_t* krow = kc + (size_t)slot * S * nkv;
+    const bf16_t* vrow = vc + (size_t)slot * S * nkv;
+    PfGemm s{};
+    s.X = qkv; s.ldx = nq + 2 * nkv; s.xb = hd; s.W = krow; s.ldw = nkv; s.wb = hd; s.wgroup = H / KV; s.C = scores; s.ldc = Lpad;
+    s.cb = (size_t)T * Lpad; s.M = T; s.N = L; s.K = hd; s.scale = scale;
+    if ((rc = pf_gemm(PF_F32_SCALE, s, H, st))) return rc;
+    hipLaunchKernelGGL(pf_softmax_kernel, dim3(T, H), dim3(256), 0, st, scores, P, T, Lpad, pos0, c.window);
+    hipLaunchKernelGGL(pf_transpose_v_kernel, dim3(Lpad / 32, (nkv + 31) / 32), dim3(256), 0, st, vrow, vt, L, Lpad, nkv, hd);
+    PfGemm o{};
+    o.X = P; o.ldx = Lpad; o.xb = (size_t)T * Lpad; o.W = vt; o.ldw = Lpad; o.wb = (size_t)hd * Lpad; o.wgroup = H / KV; o.C = att;
+    o.ldc = nq; o.cb = hd; o.M = T; o.N = hd; o.K = Lpad; o.scale = 1.f;
+    if ((rc = pf_gemm(PF_BF16, o, H, st))) return rc;
+    PfGemm wo{};
+    wo.X = att; wo.ldx = nq; wo.W = (const bf16_t*)lw.wo; wo.ldw = nq; wo.C = x; wo.ldc = d; wo.M = T; wo.N = d; wo.K = nq; wo.wgroup = 1;
+    if ((rc = pf_gemm(PF_RESID, wo, 1, st))) return rc;
+    hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)lw.mlp_norm, xn, T, d, c.norm_eps);
+    PfGemm f1{};
+    f1.X = xn; f1.ldx = d; f1.W = (const bf16_t*)lw.w1; f1.ldw = d; f1.C = fa; f1.ldc = F; f1.M = T; f1.N = F; f1.K = d; f1.wgroup = 1;
+    if ((rc = pf_gemm(PF_BF16, f1, 1, st))) return rc;
+    f1.W = (const bf16_t*)lw.w3; f1.C = fb;
+    if ((rc = pf_gemm(PF_BF16, f1, 1, st))) return rc;
+    const size_t n8 = (size_t)T * F / 8;
+    hipLaunchKernelGGL(pf_swiglu_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, st, fa, fb, n8);
+    PfGemm f2{};
+    f2.X = fa; f2.ldx = F; f2.W = (const bf16_t*)lw.w2; f2.ldw = F; f2.C = x; f2.ldc = d; f2.M = T; f2.N = d; f2.K = F; f2.wgroup = 1;
+    if ((rc = pf_gemm(PF_RESID, f2, 1, st))) return rc;
+  }
+  hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)w.final_norm, (bf16_t*)out, T, d, c.norm_eps);
+  hipLaunchKernelGGL(pf_set_len_kernel, dim3(1), dim3(1), 0, st, seq_lens, slot, L);
+  HIP_TRY(hipGetLastError());
+  return VUI_OK;
+}

@@ -246,6 +246,7 @@ class Decoder:
                                               m.rope_theta_rescale_factor).to(model.device)
         self.flash_kv_caches: list[FlashKVCache] | None = None
         self._k = self._v = None
+        self._prefill_scratch: Tensor | None = None
 
     def allocate_flash_kv_cache(self, batch_size: int, device, dtype=torch.bfloat16, max_seqlen: int | None = None):
         """src/vui/model.py:473-495.  One allocation per K and V, laid out (layers, slots, S, KV, hd);
@@ -294,6 +295,9 @@ class Decoder:
         B, T, d = x.shape
         if B > MAX_BATCH:
             raise ValueError(f"batch {B} > {MAX_BATCH}")
+        model = self._model
+        if B == 1 and T >= self.PREFILL_MIN and model.dtype == torch.bfloat16 and not model.int8:
+            return self._prefill(x, slot_idx)
         out = torch.empty_like(x)
         st = torch.cuda.current_stream().cuda_stream
         ns = self.default_splits(B)
@@ -303,6 +307,35 @@ class Decoder:
             self._step(codes=None, emb=xt, slot_idx=slot_idx, seq_inc=None, B=B, hidden_out=ht, cb0_out=None,
                        eos_out=None, n_splits=ns, stream=st)
             out[:, t] = ht
+        return out
+
+    PREFILL_MIN = 4      # shorter blocks go position by position through the decode step
+    PREFILL_CHUNK = 1024  # positions per pass: bounds the score scratch (heads x chunk x cache length)
+
+    def _prefill(self, x: Tensor, slot_idx: Tensor | None) -> Tensor:
+        """One row, T positions: the matrix-core pass of the native library, in chunks."""
+        model = self._model
+        nat = model._native
+        seq_lens = self.flash_kv_caches[0].seq_lens
+        slot = 0 if slot_idx is None else int(slot_idx[0])
+        pos = int(seq_lens[slot])
+        T = x.shape[1]
+        if pos + T > self._k.shape[2]:
+            raise ValueError(f"prefill of {T} positions at offset {pos} exceeds the cache length {self._k.shape[2]}")
+        out = torch.empty_like(x)
+        st = torch.cuda.current_stream().cuda_stream
+        for t0 in range(0, T, self.PREFILL_CHUNK):
+            n = min(self.PREFILL_CHUNK, T - t0)
+            need = nat.lib.vui_prefill_scratch_bytes(C.byref(nat.cfg), n, pos + n)
+            if need < 0:
+                raise RuntimeError(f"vui_prefill_scratch_bytes failed: {_lib.last_error()}")
+            if self._prefill_scratch is None or self._prefill_scratch.numel() < need + 256:
+                self._prefill_scratch = torch.empty(need + 256, dtype=torch.uint8, device=x.device)
+            base = (self._prefill_scratch.data_ptr() + 255) & ~255
+            xc = x[0, t0:t0 + n].contiguous()
+            _lib.check(nat.lib.vui_prefill(nat.handle, xc.data_ptr(), n, slot, pos, seq_lens.data_ptr(), self._k.data_ptr(),
+                                           self._v.data_ptr(), out[0, t0:t0 + n].data_ptr(), base, need, st), "vui_prefill")
+            pos += n
         return out
 
 
