@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--preset A|B] [--no-cpu]
 
-Workload (BASELINE.json config 4, end-to-end streaming at batch 1): random-init weights
+Workload (benchmark configuration 4, end-to-end streaming at batch 1): random-init weights
 N(0, 0.02) from seed 0 in the Vui Nano architecture, a synthetic voice prefix of 512 codec
 frames (uniform token ids) plus 64 uniform text tokens prefilled into the KV cache, then K
 codec frames generated with the whole per-frame step (backbone step, code-0 sampling with

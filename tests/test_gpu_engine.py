@@ -154,7 +154,7 @@ def test_batched_and_bucketed_steps():
 
 
 def test_int8_batch16_ragged_vs_oracle():
-    """BASELINE config 5 at full dims: 16 streams, ragged cache lengths in [128, 2048], backbone linears
+    """Benchmark configuration 5 at full dims: 16 streams, ragged cache lengths in [128, 2048], backbone linears
     as weight-only int8 (per-row scales): logits against the oracle evaluating the same int8 weights
     (dequantise-then-matmul), tolerance 2^-5 * max|logit|."""
     S = 2112

@@ -200,7 +200,7 @@ def test_sampler_matches_oracle_draws(lib, CS, top_k):
 
 
 def test_sampler_histogram(lib):
-    """Chi-square of 20000 device draws against the analytic top-k softmax (BASELINE config 3's
+    """Chi-square of 20000 device draws against the analytic top-k softmax (benchmark configuration 3's
     distribution-level check)."""
     g = torch.Generator().manual_seed(5)
     CS, k = 2048, 50

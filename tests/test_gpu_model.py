@@ -98,7 +98,7 @@ def _nano_models(dt, int8=False, n_slots=1, S=256, preset_dims=None):
 
 
 def test_config1_greedy_grid_fp32():
-    """BASELINE config 1: Vui Nano dims, fp32 N(0,0.02) weights from seed 0, 32 uniform text ids,
+    """Benchmark configuration 1: Vui Nano dims, fp32 N(0,0.02) weights from seed 0, 32 uniform text ids,
     greedy 64 frames x 16 codebooks: the token grid equals the reference's."""
     g = np.load(os.path.join(GOLDEN, "nano_grid.npz"))
     d = O.Dims()
