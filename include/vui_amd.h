@@ -114,6 +114,9 @@ int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream);
  * fused form on/off, -1 only queries; returns 1 when the fused form will be used, else 0 (then
  * vui_last_error() says why it is unavailable).  No counterpart in the reference. */
 int vui_ctx_fused(vui_ctx* ctx, int enable);
+/* 1 when the depth head of 2..16 rows runs as one persistent kernel (bf16, enough resident workgroups, the
+ * fused form switched on), else 0 and vui_last_error() says why.  No counterpart in the reference. */
+int vui_ctx_rq_batch(vui_ctx* ctx);
 /* Synchronous health check: VUI_EHIP if a fused launch gave up waiting for another workgroup. */
 int vui_ctx_status(vui_ctx* ctx);
 
@@ -176,7 +179,9 @@ int vui_rq_generate(vui_ctx* ctx, const void* hidden, const int64_t* code0, cons
  * (pos0 is the slot's current length, passed from the host because the launch shapes depend on it);
  * K/V rows are appended to the caches, seq_lens[slot] becomes pos0 + T, hidden_out (T, d) bf16
  * receives the final-norm outputs.  scratch: device memory of vui_prefill_scratch_bytes(cfg, T,
- * pos0 + T) bytes, 256-byte aligned; the library allocates nothing. */
+ * pos0 + T) bytes, 256-byte aligned; the library allocates nothing.  vui_prefill_scratch_bytes returns
+ * VUI_EINVAL for a configuration the pass does not take (fp32 or int8 weights, d_model / ffn / head_dim
+ * not multiples of 32): such prompts go position by position through vui_backbone_step. */
 int64_t vui_prefill_scratch_bytes(const vui_config* cfg, int T, int L);
 int vui_prefill(vui_ctx* ctx, const void* emb_in, int T, int slot, int pos0, int32_t* seq_lens, void* k_cache,
                 void* v_cache, void* hidden_out, void* scratch, int64_t scratch_bytes, vui_stream_t stream);

@@ -41,10 +41,19 @@ struct vui_ctx {
   char fused_why[96];
   uint64_t* prof;
   int prof_cap, prof_wg;
+  // persistent depth head for 2..16 rows
+  int rqb_ok;
+  char rqb_why[96];
 };
 
 #define FUSED_NWG 256
 #define FUSED_NS 32
+
+// the batch-1 frame kernel and the batched depth head never run at the same time: one exchange area
+static size_t ll_words_needed(const vui_config& c) {
+  const size_t a = frame_ll_words(c, FUSED_NS), b = (c.dtype == VUI_DTYPE_BF16 && c.rq_layers > 0) ? rq_batch_ll_words(c) : 0;
+  return a > b ? a : b;
+}
 
 struct Carve {
   size_t off = 0;
@@ -100,7 +109,7 @@ static size_t carve(const vui_config* c, int Bm, vui_ctx* x) {
   TAKE(rq_logits, void*, (size_t)Bm * c->codebook_size * e);
   TAKE(code0, int64_t*, Bm * 8);
   TAKE(eos_prob, float*, Bm * 4);
-  TAKE(ll, uint64_t*, frame_ll_words(*c, FUSED_NS) * 8);
+  TAKE(ll, uint64_t*, ll_words_needed(*c) * 8);
   TAKE(wdev, vui_weights*, sizeof(vui_weights));
   TAKE(ctl, uint32_t*, 256);
 #undef TAKE
@@ -167,7 +176,7 @@ int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream) {
   int rc = launch_fill_u32(ctx->counter, 0u, (int64_t)ctx->max_batch * ctx->cfg.n_heads, st);
   if (rc) return rc;
   // fused frame kernel: exchange words and control words start at zero (epoch 0 = "never written")
-  ctx->ll_words = frame_ll_words(ctx->cfg, FUSED_NS);
+  ctx->ll_words = ll_words_needed(ctx->cfg);
   if ((rc = launch_fill_u32((uint32_t*)ctx->ll, 0u, (int64_t)ctx->ll_words * 2, st))) return rc;
   if ((rc = launch_fill_u32(ctx->ctl, 0u, 64, st))) return rc;
   HIP_TRY(hipMemcpyAsync(ctx->wdev, &ctx->w, sizeof(vui_weights), hipMemcpyHostToDevice, st));
@@ -184,6 +193,14 @@ int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream) {
     if (cap >= ctx->nwg) ctx->fused_ok = 1;
     else snprintf(ctx->fused_why, sizeof(ctx->fused_why), "only %d workgroups can be resident (%d CUs), %d needed", cap, n_cu, ctx->nwg);
   }
+  ctx->rqb_ok = 0;
+  ctx->rqb_why[0] = 0;
+  if (rq_batch_supported(ctx->cfg, ctx->nwg, ctx->rqb_why, sizeof(ctx->rqb_why))) {
+    const int cap = rq_batch_max_resident(rq_batch_lds_bytes(ctx->cfg));
+    if (cap < 0) return cap;
+    if (cap >= ctx->nwg) ctx->rqb_ok = 1;
+    else snprintf(ctx->rqb_why, sizeof(ctx->rqb_why), "only %d workgroups can be resident, %d needed", cap, ctx->nwg);
+  }
   return VUI_OK;
 }
 
@@ -192,6 +209,12 @@ int vui_ctx_fused(vui_ctx* ctx, int enable) {
   if (enable >= 0) ctx->fused_on = enable ? 1 : 0;
   if (!ctx->fused_ok && ctx->fused_why[0]) vui_set_error("fused frame kernel unavailable: %s", ctx->fused_why);
   return (ctx->fused_ok && ctx->fused_on) ? 1 : 0;
+}
+
+int vui_ctx_rq_batch(vui_ctx* ctx) {
+  if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
+  if (!ctx->rqb_ok && ctx->rqb_why[0]) vui_set_error("batched depth-head kernel unavailable: %s", ctx->rqb_why);
+  return (ctx->rqb_ok && ctx->fused_on) ? 1 : 0;
 }
 
 int vui_debug_phase_clock(vui_ctx* ctx, uint64_t* buf, int cap, int workgroup) {
@@ -230,6 +253,8 @@ static int check_batch(vui_ctx* ctx, int B, int n_splits) {
 
 int64_t vui_prefill_scratch_bytes(const vui_config* c, int T, int L) {
   if (!c || T < 1 || L < T) { vui_set_error("vui_prefill_scratch_bytes: bad arguments"); return VUI_EINVAL; }
+  char why[96];
+  if (!prefill_supported(*c, why, sizeof(why))) { vui_set_error("prefill pass unavailable: %s", why); return VUI_EINVAL; }
   return (int64_t)prefill_scratch_bytes(*c, T, L);
 }
 
@@ -399,6 +424,9 @@ int vui_rq_generate(vui_ctx* ctx, const void* hidden, const int64_t* code0, cons
     a.codes_out = codes_out; a.codes_stride = codes_stride; a.zero_pad = zero_pad;
     return launch_frame(a, ctx->nwg, ctx->lds_bytes, st);
   }
+  if (ctx->rqb_ok && ctx->fused_on && B > 1)
+    return launch_rq_batch(c, ctx->wdev, hidden, code0, logit_bias, n_q, sp->temperature, sp->top_k, sp->seed, sp->frame_ctr,
+                           codes_out, codes_stride, zero_pad, B, ctx->ll, ctx->ctl, ctx->nwg, st);
   const int R = c.rq_dim, CS = c.codebook_size;
   const char* pos_emb = (const char*)ctx->w.rq_pos_emb;
   const size_t rowb = (size_t)R * ctx->esz;

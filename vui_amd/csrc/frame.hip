@@ -19,74 +19,7 @@
 #include "sample.h"
 #include <stdio.h>
 
-#define FR_THREADS 256
-#define SPIN_LIMIT (1 << 21)
-#ifndef POLL_SLEEP
-#define POLL_SLEEP 0
-#endif
-#ifndef POLL_DELAY
-#define POLL_DELAY 0
-#endif
-
-__device__ __forceinline__ uint64_t ll_ld(const uint64_t* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void ll_st(uint64_t* p, uint32_t payload, uint32_t epoch) {
-  __hip_atomic_store(p, ((uint64_t)epoch << 32) | payload, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-// Vectors that every workgroup reads can be kept in LL_REP copies, copy r read by the workgroups with
-// index % LL_REP == r (those share an XCD); writers store all copies with one instruction (lanes
-// 0..LL_REP-1).  Measured: 8 copies shorten a bare exchange of <= 512 words between 256 workgroups by
-// 0.4-0.8 us in isolation but not inside this kernel, so one copy is used.
-#define LL_REP 1
-struct RepBuf { uint64_t* base; int n; };
-__device__ __forceinline__ RepBuf rep_alloc(uint64_t*& llp, int n) { RepBuf b = {llp, n}; llp += (size_t)LL_REP * n; return b; }
-__device__ __forceinline__ const uint64_t* rep_rd(const RepBuf& b) { return b.base + (size_t)(blockIdx.x & (LL_REP - 1)) * b.n; }
-// every lane of the wave calls this with the same (i, payload)
-__device__ __forceinline__ void rep_st(const RepBuf& b, int i, uint32_t payload, uint32_t epoch) {
-  const int lane = threadIdx.x & 63;
-  if (lane < LL_REP) ll_st(b.base + (size_t)lane * b.n + i, payload, epoch);
-}
-__device__ __forceinline__ uint32_t pack2(float a, float b) { return f2bf2(a, b); }
-
-struct Ctl {
-  uint32_t epoch;
-  uint32_t* err;
-  int dead;
-};
-
-// Wait until words [0, n) of buf carry the current epoch; sink(i, payload) once per word.
-// Threads take words tid, tid+256, ...  A thread that exceeds the spin limit raises the error
-// word and stops waiting for the rest of the launch, so every wave always reaches the end.
-template <typename F>
-__device__ __forceinline__ void ll_poll(const uint64_t* buf, int n, Ctl& c, F&& sink) {
-  if (POLL_DELAY) __builtin_amdgcn_s_sleep(POLL_DELAY);
-  for (int base = 0; base < n; base += FR_THREADS * 4) {
-    int idx[4];
-    bool ok[4];
-    uint64_t v[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) { idx[i] = base + (int)threadIdx.x + FR_THREADS * i; ok[i] = idx[i] >= n; }
-    int spins = 0;
-    while (true) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) if (!ok[i]) v[i] = ll_ld(buf + idx[i]);
-      bool all = true;
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (!ok[i]) {
-          if ((uint32_t)(v[i] >> 32) == c.epoch || c.dead) { ok[i] = true; sink(idx[i], (uint32_t)v[i]); }
-          else all = false;
-        }
-      if (all) break;
-      if (++spins > SPIN_LIMIT) {
-        c.dead = 1;
-        __hip_atomic_store(c.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-      if (POLL_SLEEP) __builtin_amdgcn_s_sleep(POLL_SLEEP);
-    }
-  }
-}
+#include "ll.h"
 
 // ---- per-workgroup slice of a GEMV: adjacent row pairs, dealt round-robin over workgroups ----
 struct Plan {
@@ -335,26 +268,6 @@ __device__ __forceinline__ void load_logits8(const uint32_t* lgw, int E, int CS,
 }
 
 struct LayerP { const bf16_t *attn_norm, *wqkv, *wo, *mlp_norm, *w1, *w3, *w2; };
-
-// wait for up to 3 scattered words per thread (nullptr = none); returns payloads
-__device__ __forceinline__ void poll3(const uint64_t* p0, const uint64_t* p1, const uint64_t* p2, Ctl& c, uint32_t& r0,
-                                      uint32_t& r1, uint32_t& r2) {
-  bool k0 = p0 == nullptr, k1 = p1 == nullptr, k2 = p2 == nullptr;
-  uint64_t v0 = 0, v1 = 0, v2 = 0;
-  int spins = 0;
-  while (true) {
-    if (!k0) v0 = ll_ld(p0);
-    if (!k1) v1 = ll_ld(p1);
-    if (!k2) v2 = ll_ld(p2);
-    if (!k0 && ((uint32_t)(v0 >> 32) == c.epoch || c.dead)) k0 = true;
-    if (!k1 && ((uint32_t)(v1 >> 32) == c.epoch || c.dead)) k1 = true;
-    if (!k2 && ((uint32_t)(v2 >> 32) == c.epoch || c.dead)) k2 = true;
-    if (k0 && k1 && k2) break;
-    if (++spins > SPIN_LIMIT) { c.dead = 1; __hip_atomic_store(c.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-    if (POLL_SLEEP) __builtin_amdgcn_s_sleep(POLL_SLEEP);
-  }
-  r0 = (uint32_t)v0; r1 = (uint32_t)v1; r2 = (uint32_t)v2;
-}
 
 __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];

@@ -188,8 +188,18 @@ bool frame_supported(const vui_config& c, int nwg, int ns, char* why, size_t why
 int frame_max_resident(size_t lds_bytes, int* n_cu);
 int launch_frame(const FrameArgs& a, int nwg, size_t lds_bytes, hipStream_t st);
 
+// rqbatch.hip
+size_t rq_batch_ll_words(const vui_config& c);
+size_t rq_batch_lds_bytes(const vui_config& c);
+bool rq_batch_supported(const vui_config& c, int nwg, char* why, size_t why_len);
+int rq_batch_max_resident(size_t lds_bytes);
+int launch_rq_batch(const vui_config& c, const vui_weights* wdev, const void* hidden, const int64_t* code0, const float* logit_bias,
+                    int n_q, float temp, int topk, uint64_t seed, const int32_t* frame_ctr, int64_t* codes_out, int codes_stride,
+                    int zero_pad, int B, uint64_t* ll, uint32_t* ctl, int nwg, hipStream_t st);
+
 // prefill.hip
 size_t prefill_scratch_bytes(const vui_config& c, int T, int L);
+bool prefill_supported(const vui_config& c, char* why, size_t why_len);
 int launch_prefill(const vui_config& c, const vui_weights& w, const void* emb, int T, int slot, int pos0, int32_t* seq_lens,
                    void* k_cache, void* v_cache, void* out, void* scratch, size_t scratch_bytes, hipStream_t st);
 

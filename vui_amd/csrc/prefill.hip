@@ -12,6 +12,7 @@
 // the norm, products of the rotation rounded before their sum, residual sums rounded).
 #include "common.h"
 #include "internal.h"
+#include <stdio.h>
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 pf_bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float pf_floatx4;
@@ -228,14 +229,24 @@ size_t prefill_scratch_bytes(const vui_config& c, int T, int L) {
   return b;
 }
 
+bool prefill_supported(const vui_config& c, char* why, size_t why_len) {
+  const char* r = nullptr;
+  const int nkv = c.n_kv_heads * c.head_dim;
+  if (c.dtype != VUI_DTYPE_BF16 || c.int8_backbone) r = "bf16 weights only";
+  else if ((c.d_model % 32) || (c.ffn % 32) || (c.head_dim % 32) || (nkv % 8) || (c.rope_dim & 1)) r = "d_model, ffn and head_dim must be multiples of 32";
+  else if (c.n_kv_heads < 1 || c.n_heads % c.n_kv_heads) r = "heads must be a multiple of KV heads";
+  if (r && why) snprintf(why, why_len, "%s", r);
+  return r == nullptr;
+}
+
 int launch_prefill(const vui_config& c, const vui_weights& w, const void* emb, int T, int slot, int pos0, int32_t* seq_lens,
                    void* k_cache, void* v_cache, void* out, void* scratch, size_t scratch_bytes, hipStream_t st) {
   const int d = c.d_model, H = c.n_heads, KV = c.n_kv_heads, hd = c.head_dim, F = c.ffn, S = c.max_seqlen;
   const int nq = H * hd, nkv = KV * hd, L = pos0 + T, Lpad = (L + 31) & ~31;
-  if (c.dtype != VUI_DTYPE_BF16 || c.int8_backbone) { vui_set_error("prefill: bf16 weights only"); return VUI_EINVAL; }
+  char why[96];
+  if (!prefill_supported(c, why, sizeof(why))) { vui_set_error("prefill: %s", why); return VUI_EINVAL; }
   if (T < 1 || pos0 < 0 || L > S) { vui_set_error("prefill: positions %d..%d outside the cache (S=%d)", pos0, L, S); return VUI_EINVAL; }
   if (slot < 0 || slot >= c.n_slots) { vui_set_error("prefill: slot %d outside [0,%d)", slot, c.n_slots); return VUI_EINVAL; }
-  if ((d % 32) || (F % 32) || (hd % 32) || (nkv % 8) || (c.rope_dim & 1)) { vui_set_error("prefill: d_model, ffn, head_dim must be multiples of 32"); return VUI_EINVAL; }
   if (scratch_bytes < prefill_scratch_bytes(c, T, L)) { vui_set_error("prefill: scratch of %zu bytes, %zu needed", scratch_bytes, prefill_scratch_bytes(c, T, L)); return VUI_EINVAL; }
   char* sp = (char*)scratch;
   auto take = [&](size_t bytes) { char* r = sp; sp += pf_align(bytes); return r; };

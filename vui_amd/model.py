@@ -172,6 +172,10 @@ class _Native:
         """Query (-1) or switch (1/0) the one-kernel form of the batch-1 bf16 calls."""
         return bool(self.lib.vui_ctx_fused(self.handle, enable))
 
+    def rq_batch(self) -> bool:
+        """True when the depth head of 2..16 rows runs as one persistent kernel."""
+        return bool(self.lib.vui_ctx_rq_batch(self.handle))
+
     def status(self) -> None:
         _lib.check(self.lib.vui_ctx_status(self.handle), "vui_ctx_status")
 
@@ -247,6 +251,7 @@ class Decoder:
         self.flash_kv_caches: list[FlashKVCache] | None = None
         self._k = self._v = None
         self._prefill_scratch: Tensor | None = None
+        self._prefill_ok: bool | None = None
 
     def allocate_flash_kv_cache(self, batch_size: int, device, dtype=torch.bfloat16, max_seqlen: int | None = None):
         """src/vui/model.py:473-495.  One allocation per K and V, laid out (layers, slots, S, KV, hd);
@@ -296,7 +301,7 @@ class Decoder:
         if B > MAX_BATCH:
             raise ValueError(f"batch {B} > {MAX_BATCH}")
         model = self._model
-        if B == 1 and T >= self.PREFILL_MIN and model.dtype == torch.bfloat16 and not model.int8:
+        if B == 1 and T >= self.PREFILL_MIN and self._prefill_available():
             return self._prefill(x, slot_idx)
         out = torch.empty_like(x)
         st = torch.cuda.current_stream().cuda_stream
@@ -311,6 +316,13 @@ class Decoder:
 
     PREFILL_MIN = 4      # shorter blocks go position by position through the decode step
     PREFILL_CHUNK = 1024  # positions per pass: bounds the score scratch (heads x chunk x cache length)
+
+    def _prefill_available(self) -> bool:
+        """The one-pass form takes bf16 weights and dims that are multiples of 32 (the library decides)."""
+        if self._prefill_ok is None:
+            nat = self._model._native
+            self._prefill_ok = nat.lib.vui_prefill_scratch_bytes(C.byref(nat.cfg), 1, 1) >= 0
+        return self._prefill_ok
 
     def _prefill(self, x: Tensor, slot_idx: Tensor | None) -> Tensor:
         """One row, T positions: the matrix-core pass of the native library, in chunks."""
