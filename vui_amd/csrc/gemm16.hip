@@ -1,4 +1,4 @@
-// Skinny GEMM for 9..16 activation rows on the matrix cores: y (B, N) = x (B, K) W^T (N, K).
+// Skinny GEMM for 2..16 activation rows on the matrix cores: y (B, N) = x (B, K) W^T (N, K).
 //
 // One workgroup owns 16 consecutive output features; its four waves split K in steps of 64 and
 // each issues v_mfma_f32_16x16x32_bf16 with A = a 16 x 32 weight tile (lane i: feature i % 16,
@@ -18,6 +18,9 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
 #define G16_THREADS 256
 #define G16_MAXS 8  // K steps (of 64) per wave held in registers: K <= 2048
+// from two rows on the matrix-core form wins over one wave per row pair (measured, bf16 and int8 weights:
+// a 4-row int8 backbone step 1.6 ms -> see the benchmark); a single row stays on the GEMV
+#define G16_MIN_ROWS 2
 
 union U128 { uint4 u; bf16x8 v; };
 
@@ -216,7 +219,7 @@ static int launch_g16(const GemvArgs& a, hipStream_t st) {
 }
 
 bool gemm16_supported(const GemvArgs& a) {
-  return a.dtype == VUI_DTYPE_BF16 && a.B > 8 && a.B <= 16 && (a.K % 16) == 0 && a.K <= G16_MAXS * 4 * 64 &&
+  return a.dtype == VUI_DTYPE_BF16 && a.B >= G16_MIN_ROWS && a.B <= 16 && (a.K % 16) == 0 && a.K <= G16_MAXS * 4 * 64 &&
          g16_lds(a.K, a.epi == EPI_SWIGLU) <= 150 * 1024;
 }
 

@@ -233,7 +233,7 @@ int launch_gemv(const GemvArgs& a, hipStream_t st) {
   }
   const bool dual = a.epi == EPI_SWIGLU;
   if (gemm16_supported(a)) {
-    // 9..16 rows: the matrix-core form computes the N outputs; the extra row and the position
+    // 2..16 rows: the matrix-core form computes the N outputs; the extra row and the position
     // update, if any, go through this kernel's extra block alone (N = 0 main blocks)
     int rc = launch_gemm16(a, st);
     if (rc || !a.Wx) return rc;
