@@ -938,9 +938,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           poll_add(xres, rep_rd(ob), R / 2, c);
           TS(35);
           stage_norm(xres, nw2, a.rq_eps, R, xp);
-          TS(70);
           __syncthreads();
-          TS(71);
           gemv_compute<2, true>(xp, R_sw, wr, red, [&](int gp, float v0, float v1, float u0, float u1) {
             const float a0 = bf2f(f2bf(v0)), a1 = bf2f(f2bf(v1)), c0 = bf2f(f2bf(u0)), c1 = bf2f(f2bf(u1));
             const float s0 = bf2f(f2bf(a0 * __builtin_amdgcn_rcpf(1.0f + __expf(-a0)))), s1 = bf2f(f2bf(a1 * __builtin_amdgcn_rcpf(1.0f + __expf(-a1))));

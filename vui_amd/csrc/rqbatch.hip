@@ -617,9 +617,12 @@ int rq_batch_max_resident(size_t lds_bytes) {
   return occ * prop.multiProcessorCount;
 }
 
+#ifdef VUI_RB_CLOCK
+// profiling builds only: where the next launches drop the phase stamps of workgroup wg
 static unsigned long long* g_rb_dbg = nullptr;
 static int g_rb_dbg_wg = 0;
 extern "C" void vui_debug_rq_batch_clock(unsigned long long* buf, int wg) { g_rb_dbg = buf; g_rb_dbg_wg = wg; }
+#endif
 
 int launch_rq_batch(const vui_config& c, const vui_weights* wdev, const void* hidden, const int64_t* code0, const float* logit_bias,
                     int n_q, float temp, int topk, uint64_t seed, const int32_t* frame_ctr, int64_t* codes_out, int codes_stride,
@@ -630,7 +633,11 @@ int launch_rq_batch(const vui_config& c, const vui_weights* wdev, const void* hi
   a.CS = c.codebook_size; a.n_q = n_q; a.rq_eps = c.rq_norm_eps; a.w = wdev; a.hidden = (const uint16_t*)hidden; a.code0 = code0;
   a.codes_out = codes_out; a.codes_stride = codes_stride; a.zero_pad = zero_pad; a.logit_bias = logit_bias; a.temp = temp;
   a.topk = topk; a.seed = seed; a.frame_ctr = frame_ctr; a.ll = ll; a.epoch = ctl; a.arrive = ctl + 1; a.err = ctl + 2;
+#ifdef VUI_RB_CLOCK
   a.dbg = g_rb_dbg; a.dbg_wg = g_rb_dbg_wg;
+#else
+  a.dbg = nullptr; a.dbg_wg = 0;
+#endif
   const RbLayout l = rb_layout(c);
   a.xs = rb_xs(c); a.off_xp = (int)l.xp; a.off_red = (int)l.red; a.off_misc = (int)l.misc; a.off_att = (int)l.att; a.off_kv = (int)l.kv;
   hipLaunchKernelGGL(rq_batch_kernel, dim3(nwg), dim3(FR_THREADS), l.total, st, a);
