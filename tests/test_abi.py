@@ -19,7 +19,8 @@ def lib():
 
 
 def declared_functions():
-    src = open(os.path.join(ROOT, "include", "vui_amd.h")).read()
+    inc = os.path.join(ROOT, "include")
+    src = "".join(open(os.path.join(inc, f)).read() for f in sorted(os.listdir(inc)) if f.endswith(".h"))
     src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
     return sorted(set(re.findall(r"\b(vui_[a-z0-9_]+)\s*\(", src)))
 

@@ -49,7 +49,16 @@ class SampleParamsC(C.Structure):
                 ("frame_ctr", C.c_void_p)]
 
 
-# name -> (restype, argtypes); every symbol include/vui_amd.h declares
+class CodecConfigC(C.Structure):
+    """vui_codec_config (include/vui_codec.h)."""
+    _fields_ = [(n, C.c_int32) for n in (
+        "n_codebooks", "codebook_size", "codebook_dim", "vq_dim", "n_semantic", "latent_dim", "d_model", "n_layers",
+        "n_heads", "head_dim", "mlp_dim", "max_seq")] + [
+        ("rope_theta", C.c_float), ("n_up", C.c_int32), ("up_ratios", C.c_int32 * 4), ("decoder_dim", C.c_int32),
+        ("n_rates", C.c_int32), ("rates", C.c_int32 * 8)]
+
+
+# name -> (restype, argtypes); every symbol include/*.h declares
 _P, _I, _L, _F = C.c_void_p, C.c_int, C.c_int64, C.c_float
 SIGNATURES = {
     "vui_last_error": (C.c_char_p, []),
@@ -65,6 +74,14 @@ SIGNATURES = {
     "vui_debug_phase_clock": (_I, [_P, _P, _I, _I]),
     "vui_prefill_scratch_bytes": (_L, [C.POINTER(VuiConfigC), _I, _I]),
     "vui_prefill": (_I, [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _L, _P]),
+    "vui_codec_hop": (C.c_int32, [C.POINTER(CodecConfigC)]),
+    "vui_codec_n_tensors": (C.c_int32, [C.POINTER(CodecConfigC)]),
+    "vui_codec_workspace_bytes": (_L, [C.POINTER(CodecConfigC)]),
+    "vui_codec_init": (_I, [C.POINTER(CodecConfigC), C.POINTER(_P), C.c_int32, _P, _L, _P, C.POINTER(_P)]),
+    "vui_codec_destroy": (None, [_P]),
+    "vui_codec_reset": (_I, [_P, _P]),
+    "vui_codec_decode_frame": (_I, [_P, _P, C.c_int32, _P, _P]),
+    "vui_codec_status": (_L, [_P, _P]),
     "vui_backbone_step": (_I, [_P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _P]),
     "vui_sample_cb0": (_I, [_P, _P, _P, _P, _P, _F, _I, C.POINTER(SampleParamsC), _P, _I, _P]),
     "vui_rq_generate": (_I, [_P, _P, _P, _P, _I, C.POINTER(SampleParamsC), _P, _I, _I, _I, _P]),

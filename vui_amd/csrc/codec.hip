@@ -1,0 +1,826 @@
+// Streaming vocoder frame step: codes of one codec frame -> hop audio samples, fp32.
+//
+// Reference: QwenCodecDecoder.forward in streaming mode (src/vui/qwen_codec.py:1191-1224) with its
+// building blocks CausalConv1d (:45-101), CausalTransConv1d (:112-158), SplitResidualVQ.decode (:263-270),
+// DecTransformer._forward_streaming (:1048-1076), ConvNeXtBlock (:832-848), DecoderBlock (:863-879),
+// SnakeBeta (:820-829).
+//
+// Layout.  Activations are channel-major (C, columns).  Every conv input lives in a ring of 2^k columns
+// per channel that keeps the last `pad` columns of earlier frames in front of the current ones: frame f
+// occupies columns (f*T + pad + t) mod 2^k, so no history is ever copied; a device counter holds f.
+// The activation that precedes a conv (snake) is applied by the producer's epilogue, which writes the
+// raw value (for residuals) and the activated value (into the consumer's ring) in one pass.
+//
+// One GEMM kernel serves every conv, transposed conv and linear layer: out (M x T) = W (M x taps*Cin) .
+// X, X[(tap, ci)][t] = ring[ci][t + tap*dil].  Weights are repacked once to tap-major (taps, M, Cin) so a
+// lane reads 32 contiguous bytes of one output row; a transposed conv with kernel 2*stride is the
+// two-tap conv over (previous column, current column) with M = Cout*stride rows whose results are
+// scattered to column t*stride + r.  A workgroup owns 16 output rows x 16*TT columns; its waves split
+// the (tap, 32-channel) units, multiply on v_mfma_f32_16x16x4_f32 with both operands read straight from
+// global memory / L2 one step ahead, and add their parts through LDS in a fixed order.
+#include "common.h"
+#include "internal.h"
+#include "../../include/vui_codec.h"
+
+#include <math.h>
+#include <new>
+#include <stdio.h>
+#include <string.h>
+#include <vector>
+
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+struct Ring {
+  float* p;
+  int rs;     // columns per channel (power of two)
+  int mask;   // rs - 1
+  int pad;    // history columns in front of a frame
+  int tstep;  // columns a frame adds (0: plain buffer, always at column 0)
+};
+
+__device__ __forceinline__ int ring_base(const Ring& r, int f) { return (f * r.tstep) & r.mask; }
+__device__ __forceinline__ float* ring_ptr(const Ring& r, int base, int c, int col) {
+  return r.p + (size_t)c * r.rs + ((base + col) & r.mask);
+}
+
+enum { IN_PLAIN = 0, IN_RMS = 1, IN_SILU_MUL = 2 };
+enum { EPI_NONE = 0, EPI_GELU = 1, EPI_RES = 2, EPI_SCALE_RES = 3 };
+
+struct CvGemm {
+  const float* W;     // (taps, M, Cin)
+  const float* bias;  // row m uses bias[m / bias_div]; may be null
+  int M, Cin, taps, dil, T;
+  int bias_div;
+  Ring in;
+  int in_mode;
+  const float* in_w;  // norm weight (IN_RMS)
+  float eps;
+  int epi;
+  const float* scale;  // per output channel (EPI_SCALE_RES)
+  Ring res;
+  int tc_stride;  // > 0: row m -> channel m / s, column t*s + m % s
+  Ring out_raw;   // p may be null
+  Ring out_act;   // p may be null: snake with (ea, ib) of the consumer
+  const float* ea;
+  const float* ib;
+  const int* ctr;  // frames started; this frame is *ctr - 1
+  int nw, tt;      // launch shape (host side)
+};
+
+template <int TT> struct Pf { static constexpr int N = TT == 1 ? 3 : (TT == 2 ? 2 : 1); };
+
+template <int TT>
+__global__ __launch_bounds__(1024) void cv_gemm_kernel(const CvGemm p) {
+  extern __shared__ __align__(16) float red[];  // nw x TT x 64 x 4
+  constexpr int PF = Pf<TT>::N;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, nw = blockDim.x >> 6;
+  const int r16 = lane & 15, g = lane >> 4;
+  const int m0 = blockIdx.x * 16, t0 = blockIdx.y * (16 * TT);
+  const int f = *p.ctr - 1;
+  const int ib_ = ring_base(p.in, f);
+  const int G = p.Cin >> 5, U = p.taps * G;
+  const int M = p.M, Cin = p.Cin;
+
+  float rstd = 1.f;
+  if (p.in_mode == IN_RMS) {  // one column
+    float ss = 0.f;
+    for (int c = lane; c < Cin; c += WAVE) {
+      const float v = *ring_ptr(p.in, ib_, c, p.in.pad);
+      ss = fmaf(v, v, ss);
+    }
+    ss = wave_sum(ss);
+    rstd = 1.0f / sqrtf(ss / (float)Cin + p.eps);
+  }
+
+  float4 a_nx[PF][2], a_cu[PF][2];
+  float b_nx[PF][TT][8], b_cu[PF][TT][8];
+  floatx4 acc[TT];
+#pragma unroll
+  for (int tt = 0; tt < TT; ++tt) acc[tt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  auto load = [&](int u0, float4 (&a)[PF][2], float (&b)[PF][TT][8]) {
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const int u = u0 + i * nw;
+      const bool on = u < U;
+      const int tap = on ? u / G : 0, grp = on ? u % G : 0;
+      const int ci0 = grp * 32 + g * 8;
+      const float* wp = p.W + ((size_t)tap * M + m0 + r16) * Cin + ci0;
+      a[i][0] = on ? *reinterpret_cast<const float4*>(wp) : make_float4(0.f, 0.f, 0.f, 0.f);
+      a[i][1] = on ? *reinterpret_cast<const float4*>(wp + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt) {
+        const int t = t0 + tt * 16 + r16;
+        const bool bon = on && t < p.T;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          float v = 0.f;
+          if (bon) {
+            const int ci = ci0 + j;
+            if (p.in_mode == IN_SILU_MUL) {
+              const float ga = *ring_ptr(p.in, ib_, ci, p.in.pad + t);
+              const float up = *ring_ptr(p.in, ib_, ci + Cin, p.in.pad + t);
+              v = ga / (1.0f + expf(-ga)) * up;
+            } else {
+              v = *ring_ptr(p.in, ib_, ci, t + tap * p.dil);
+              if (p.in_mode == IN_RMS) v = v * rstd * p.in_w[ci];
+            }
+          }
+          b[i][tt][j] = v;
+        }
+      }
+    }
+  };
+
+  load(wave, a_nx, b_nx);
+  for (int u0 = wave; u0 < U; u0 += PF * nw) {
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      a_cu[i][0] = a_nx[i][0]; a_cu[i][1] = a_nx[i][1];
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) b_cu[i][tt][j] = b_nx[i][tt][j];
+    }
+    if (u0 + PF * nw < U) load(u0 + PF * nw, a_nx, b_nx);
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const float av[8] = {a_cu[i][0].x, a_cu[i][0].y, a_cu[i][0].z, a_cu[i][0].w,
+                           a_cu[i][1].x, a_cu[i][1].y, a_cu[i][1].z, a_cu[i][1].w};
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt)
+          acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[j], b_cu[i][tt][j], acc[tt], 0, 0, 0);
+    }
+  }
+
+  // add the waves' parts in a fixed order
+#pragma unroll
+  for (int tt = 0; tt < TT; ++tt)
+    *reinterpret_cast<float4*>(red + ((size_t)(wave * TT + tt) * 64 + lane) * 4) =
+        make_float4(acc[tt][0], acc[tt][1], acc[tt][2], acc[tt][3]);
+  __syncthreads();
+  const int rb = ring_base(p.res, f), ob = ring_base(p.out_raw, f), ab = ring_base(p.out_act, f);
+  for (int idx = tid; idx < TT * 64; idx += blockDim.x) {
+    const int tt = idx >> 6, l = idx & 63;
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int w = 0; w < nw; ++w) {
+      const float4 q = *reinterpret_cast<const float4*>(red + ((size_t)(w * TT + tt) * 64 + l) * 4);
+      v[0] += q.x; v[1] += q.y; v[2] += q.z; v[3] += q.w;
+    }
+    const int t = t0 + tt * 16 + (l & 15);
+    if (t >= p.T) continue;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = m0 + 4 * (l >> 4) + r;
+      if (m >= M) continue;
+      float y = v[r];
+      if (p.bias) y += p.bias[m / p.bias_div];
+      int ch = m, col = t;
+      if (p.tc_stride > 0) { ch = m / p.tc_stride; col = t * p.tc_stride + m % p.tc_stride; }
+      if (p.epi == EPI_GELU) y = 0.5f * y * (1.0f + erff(y * 0.70710678118654752f));
+      else if (p.epi == EPI_RES) y = *ring_ptr(p.res, rb, ch, p.res.pad + col) + y;
+      else if (p.epi == EPI_SCALE_RES) y = *ring_ptr(p.res, rb, ch, p.res.pad + col) + p.scale[ch] * y;
+      if (p.out_raw.p) *ring_ptr(p.out_raw, ob, ch, p.out_raw.pad + col) = y;
+      if (p.out_act.p) {
+        const float s = sinf(y * p.ea[ch]);
+        *ring_ptr(p.out_act, ab, ch, p.out_act.pad + col) = y + p.ib[ch] * s * s;
+      }
+    }
+  }
+}
+
+// ---- codebook rows of one frame: [sum of the semantic rows | sum of the acoustic rows]; starts the frame ----
+struct CvVq {
+  const int64_t* codes;
+  int n_q, n_sem, CS, cd;
+  const float* embed;  // (n_codebooks, CS, cd)
+  float* x;            // (2*cd) as a one-column plain buffer with rs = 1
+  int* ctr;
+  int* err;
+  int max_seq;
+};
+
+__global__ __launch_bounds__(256) void cv_vq_kernel(const CvVq p) {
+  for (int c = threadIdx.x; c < p.cd; c += blockDim.x) {
+    float s0 = 0.f, s1 = 0.f;
+    for (int i = 0; i < p.n_q; ++i) {
+      long code = p.codes[i];
+      if (code < 0 || code >= p.CS) { code = code < 0 ? 0 : p.CS - 1; if (c == 0) *p.err = 1; }
+      const float e = p.embed[((size_t)i * p.CS + code) * p.cd + c];
+      if (i < p.n_sem) s0 += e; else s1 += e;
+    }
+    p.x[c] = s0;
+    p.x[p.cd + c] = s1;
+  }
+  if (threadIdx.x == 0) {
+    int f = *p.ctr;
+    if (f >= p.max_seq) { *p.err = 2; f = p.max_seq - 1; }  // stay on the last position: nothing runs out of bounds
+    *p.ctr = f + 1;
+  }
+}
+
+// ---- pre-transformer attention of one new position: rotate-half RoPE, cache append, softmax, P.V ----
+struct CvAttn {
+  const float* qkv;  // (3*A): q | k | v
+  float* kc;         // (H, max_seq, hd)
+  float* vc;
+  float* out;        // (A)
+  const float* inv_freq;  // (hd/2)
+  int H, hd, max_seq;
+  const int* ctr;
+};
+
+__global__ __launch_bounds__(256) void cv_attn_kernel(const CvAttn p) {
+  extern __shared__ float sm[];  // q[hd] | sc[max_seq] | part[4][hd] | red[8]
+  float* q = sm;
+  float* sc = q + p.hd;
+  float* part = sc + p.max_seq;
+  float* red = part + 4 * p.hd;
+  const int h = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int hd = p.hd, half = hd >> 1, A = p.H * hd;
+  const int pos = *p.ctr - 1;
+  float* kh = p.kc + (size_t)h * p.max_seq * hd;
+  float* vh = p.vc + (size_t)h * p.max_seq * hd;
+  if (tid < hd) {
+    const float ang = (float)pos * p.inv_freq[tid % half];
+    const float cs = cosf(ang), sn = sinf(ang);
+    const float* qq = p.qkv + h * hd;
+    const float* kk = p.qkv + A + h * hd;
+    const float qr = tid < half ? -qq[tid + half] : qq[tid - half];
+    const float kr = tid < half ? -kk[tid + half] : kk[tid - half];
+    q[tid] = qq[tid] * cs + qr * sn;
+    kh[(size_t)pos * hd + tid] = kk[tid] * cs + kr * sn;
+    vh[(size_t)pos * hd + tid] = p.qkv[2 * A + h * hd + tid];
+  }
+  __syncthreads();  // this workgroup's own cache row is visible to all its threads after the barrier
+  const float scale = 1.0f / sqrtf((float)hd);
+  for (int j = wave; j <= pos; j += 4) {
+    float d = lane < hd ? q[lane] * kh[(size_t)j * hd + lane] : 0.f;
+    d = wave_sum(d);
+    if (lane == 0) sc[j] = d * scale;
+  }
+  __syncthreads();
+  float mx = -INFINITY;
+  for (int j = tid; j <= pos; j += 256) mx = fmaxf(mx, sc[j]);
+  mx = wave_max(mx);
+  if (lane == 0) red[wave] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  float sum = 0.f;
+  for (int j = tid; j <= pos; j += 256) { const float e = expf(sc[j] - mx); sc[j] = e; sum += e; }
+  sum = wave_sum(sum);
+  if (lane == 0) red[4 + wave] = sum;
+  __syncthreads();
+  sum = (red[4] + red[5]) + (red[6] + red[7]);
+  float o = 0.f;
+  if (lane < hd)
+    for (int j = wave; j <= pos; j += 4) o = fmaf(sc[j], vh[(size_t)j * hd + lane], o);
+  if (lane < hd) part[wave * hd + lane] = o;
+  __syncthreads();
+  if (tid < hd) p.out[h * hd + tid] = ((part[tid] + part[hd + tid]) + (part[2 * hd + tid] + part[3 * hd + tid])) / sum;
+}
+
+// ---- depthwise causal conv (k taps) + LayerNorm over channels, one workgroup per column ----
+struct CvDwLn {
+  Ring in;           // pad = k - 1
+  const float* w;    // (C, k)
+  const float* b;    // (C)
+  const float* lnw;
+  const float* lnb;
+  float* out;        // (C, rs_out) plain
+  int rs_out, C, k;
+  float eps;
+  const int* ctr;
+};
+
+#define DW_MAXC 8  // channels per thread
+
+__global__ __launch_bounds__(256) void cv_dwln_kernel(const CvDwLn p) {
+  __shared__ float red[8];
+  const int t = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int f = *p.ctr - 1, base = ring_base(p.in, f);
+  float v[DW_MAXC];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < DW_MAXC; ++i) {
+    const int c = tid + 256 * i;
+    v[i] = 0.f;
+    if (c < p.C) {
+      float a = p.b[c];
+      for (int k = 0; k < p.k; ++k) a = fmaf(p.w[c * p.k + k], *ring_ptr(p.in, base, c, t + k), a);
+      v[i] = a;
+      s += a;
+    }
+  }
+  s = wave_sum(s);
+  if (lane == 0) red[wave] = s;
+  __syncthreads();
+  const float mean = ((red[0] + red[1]) + (red[2] + red[3])) / (float)p.C;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < DW_MAXC; ++i) {
+    const int c = tid + 256 * i;
+    if (c < p.C) { const float d = v[i] - mean; q = fmaf(d, d, q); }
+  }
+  q = wave_sum(q);
+  if (lane == 0) red[4 + wave] = q;
+  __syncthreads();
+  const float rstd = 1.0f / sqrtf(((red[4] + red[5]) + (red[6] + red[7])) / (float)p.C + p.eps);
+#pragma unroll
+  for (int i = 0; i < DW_MAXC; ++i) {
+    const int c = tid + 256 * i;
+    if (c < p.C) p.out[(size_t)c * p.rs_out + t] = (v[i] - mean) * rstd * p.lnw[c] + p.lnb[c];
+  }
+}
+
+// ---- last conv: one output channel, k taps, clamp to [-1, 1]; 64 samples x 4 channel quarters per workgroup ----
+struct CvFinal {
+  Ring in;         // pad = k - 1
+  const float* w;  // (C, k)
+  const float* b;  // (1)
+  float* audio;
+  int C, k, T;
+  const int* ctr;
+};
+
+__global__ __launch_bounds__(256) void cv_final_kernel(const CvFinal p) {
+  __shared__ float part[4][64];
+  const int tid = threadIdx.x, qd = tid >> 6, l = tid & 63;
+  const int t = blockIdx.x * 64 + l;
+  const int f = *p.ctr - 1, base = ring_base(p.in, f);
+  float a = 0.f;
+  if (t < p.T) {
+    const int c0 = (p.C * qd) / 4, c1 = (p.C * (qd + 1)) / 4;
+    for (int c = c0; c < c1; ++c)
+      for (int k = 0; k < p.k; ++k) a = fmaf(p.w[c * p.k + k], *ring_ptr(p.in, base, c, t + k), a);
+  }
+  part[qd][l] = a;
+  __syncthreads();
+  if (qd == 0 && t < p.T) {
+    const float y = ((part[0][l] + part[1][l]) + (part[2][l] + part[3][l])) + p.b[0];
+    p.audio[t] = fminf(1.0f, fmaxf(-1.0f, y));
+  }
+}
+
+// ---- one-time repacking ----
+__global__ void cv_pack_conv_kernel(const float* w, float* wp, int Cout, int Cin, int K) {  // (Cout,Cin,K) -> (K,Cout,Cin)
+  const size_t n = (size_t)Cout * Cin * K;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const int ci = (int)(i % Cin);
+    const int co = (int)((i / Cin) % Cout);
+    const int k = (int)(i / ((size_t)Cin * Cout));
+    wp[i] = w[((size_t)co * Cin + ci) * K + k];
+  }
+}
+// ConvTranspose1d (Cin, Cout, K = taps*s) -> (taps, Cout*s, Cin); tap `taps-1` multiplies the current column
+__global__ void cv_pack_tconv_kernel(const float* w, float* wp, int Cin, int Cout, int s, int taps) {
+  const size_t n = (size_t)taps * Cout * s * Cin;
+  const int K = taps * s;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const int ci = (int)(i % Cin);
+    const int m = (int)((i / Cin) % ((size_t)Cout * s));
+    const int tap = (int)(i / ((size_t)Cin * Cout * s));
+    const int co = m / s, r = m % s;
+    wp[i] = w[((size_t)ci * Cout + co) * K + r + (taps - 1 - tap) * s];
+  }
+}
+// rows of src (M, K) into dst (M, ld) at column offset off
+__global__ void cv_copy_rows_kernel(const float* src, float* dst, int M, int K, int ld, int off) {
+  const size_t n = (size_t)M * K;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    dst[(i / K) * ld + off + (i % K)] = src[i];
+}
+__global__ void cv_snake_tab_kernel(const float* alpha, const float* beta, float* ea, float* ib, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) { ea[i] = expf(alpha[i]); ib[i] = 1.0f / (expf(beta[i]) + 1e-9f); }
+}
+__global__ void cv_fill_kernel(float* p, size_t n, float v) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
+}
+__global__ void cv_set_int_kernel(int* p, int v0, int v1) { p[0] = v0; p[1] = v1; }
+
+// =================================== host side ===================================
+struct Step {
+  int kind;  // 0 gemm, 1 attn, 2 dwln
+  CvGemm g;
+  CvAttn a;
+  CvDwLn d;
+};
+
+struct vui_codec {
+  vui_codec_config cfg;
+  int hop;
+  char* ws;
+  int64_t ws_bytes;
+  float* state0;  // start of the zeroed-on-reset region (rings)
+  size_t state_floats;
+  int* ctr;  // [0] frames started since reset, [1] error flag
+  CvVq vq;
+  std::vector<Step> steps;
+  CvFinal fin;
+};
+
+static int ipow2(int n) { int r = 1; while (r < n) r <<= 1; return r; }
+
+static int cv_check(const vui_codec_config* c) {
+  if (!c) { vui_set_error("NULL codec config"); return VUI_EINVAL; }
+  if (c->n_up < 0 || c->n_up > 4 || c->n_rates < 1 || c->n_rates > 8) { vui_set_error("codec: n_up=%d / n_rates=%d outside the supported range", c->n_up, c->n_rates); return VUI_EINVAL; }
+  if (c->n_codebooks < 1 || c->n_semantic < 1 || c->n_semantic > c->n_codebooks || c->codebook_size < 1) { vui_set_error("codec: bad codebook layout"); return VUI_EINVAL; }
+  const int A = c->n_heads * c->head_dim;
+  int dims32[] = {2 * c->codebook_dim, c->vq_dim, c->latent_dim, c->d_model, A, c->mlp_dim, 4 * c->latent_dim, c->decoder_dim};
+  for (int v : dims32)
+    if (v < 32 || (v % 32)) { vui_set_error("codec: every layer width must be a multiple of 32 (got %d)", v); return VUI_EINVAL; }
+  if (c->head_dim > 64 || (c->head_dim & 1) || c->n_heads < 1) { vui_set_error("codec: head_dim=%d unsupported (even, <= 64)", c->head_dim); return VUI_EINVAL; }
+  if (c->max_seq < 1 || c->max_seq > 4096) { vui_set_error("codec: max_seq=%d outside [1,4096]", c->max_seq); return VUI_EINVAL; }
+  if (c->latent_dim > 256 * DW_MAXC) { vui_set_error("codec: latent_dim=%d above %d", c->latent_dim, 256 * DW_MAXC); return VUI_EINVAL; }
+  int dim = c->decoder_dim;
+  for (int i = 0; i < c->n_rates; ++i) {
+    if (c->rates[i] < 1 || (dim % 64)) { vui_set_error("codec: decoder stage %d: width %d must be a multiple of 64, rate >= 1", i, dim); return VUI_EINVAL; }
+    dim /= 2;
+  }
+  for (int i = 0; i < c->n_up; ++i)
+    if (c->up_ratios[i] < 1) { vui_set_error("codec: bad upsample ratio"); return VUI_EINVAL; }
+  return VUI_OK;
+}
+
+int32_t vui_codec_hop(const vui_codec_config* c) {
+  if (cv_check(c)) return VUI_EINVAL;
+  int h = 1;
+  for (int i = 0; i < c->n_up; ++i) h *= c->up_ratios[i];
+  for (int i = 0; i < c->n_rates; ++i) h *= c->rates[i];
+  return h;
+}
+
+int32_t vui_codec_n_tensors(const vui_codec_config* c) {
+  if (cv_check(c)) return VUI_EINVAL;
+  return 2 * 2 + c->n_codebooks + 2 + 2 + 11 * c->n_layers + 3 + 11 * c->n_up + 2 + c->n_rates * (4 + 3 * 8) + 2 + 2;
+}
+
+// Bump allocator over the workspace; with base == nullptr it only measures.
+struct Arena {
+  char* base;
+  size_t off = 0;
+  float* take(size_t floats) {
+    float* p = base ? (float*)(base + off) : nullptr;
+    off += (floats * 4 + 255) & ~(size_t)255;
+    return p;
+  }
+};
+
+static Ring mk_ring(Arena& ar, int C, int pad, int T, bool stream) {
+  Ring r;
+  r.rs = ipow2(pad + T);
+  r.mask = r.rs - 1;
+  r.pad = pad;
+  r.tstep = stream ? T : 0;
+  r.p = ar.take((size_t)C * r.rs);
+  return r;
+}
+static Ring no_ring() { Ring r; r.p = nullptr; r.rs = 1; r.mask = 0; r.pad = 0; r.tstep = 0; return r; }
+
+static void grid_for(size_t n, dim3& g) { size_t b = (n + 255) / 256; g = dim3((unsigned)(b > 4096 ? 4096 : (b ? b : 1))); }
+
+// Lays out the workspace and (when tensors != nullptr) packs weights and records the launch plan.
+static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const* tensors, char* ws, hipStream_t st, int64_t* need) {
+  Arena ar{ws};
+  const bool real = ws != nullptr && tensors != nullptr;
+  int ti = 0;
+  auto next = [&]() -> const float* { return real ? (const float*)tensors[ti++] : (ti++, nullptr); };
+  auto pack_copy = [&](const float* src, float* dst, int M, int K, int ld, int off) {
+    if (!real) return;
+    dim3 g; grid_for((size_t)M * K, g);
+    hipLaunchKernelGGL(cv_copy_rows_kernel, g, dim3(256), 0, st, src, dst, M, K, ld, off);
+  };
+  auto pack_conv = [&](const float* src, int Cout, int Cin, int K) -> float* {
+    float* dst = ar.take((size_t)Cout * Cin * K);
+    if (real) { dim3 g; grid_for((size_t)Cout * Cin * K, g); hipLaunchKernelGGL(cv_pack_conv_kernel, g, dim3(256), 0, st, src, dst, Cout, Cin, K); }
+    return dst;
+  };
+  auto pack_tconv = [&](const float* src, int Cin, int Cout, int s, int taps) -> float* {
+    float* dst = ar.take((size_t)taps * Cout * s * Cin);
+    if (real) { dim3 g; grid_for((size_t)taps * Cout * s * Cin, g); hipLaunchKernelGGL(cv_pack_tconv_kernel, g, dim3(256), 0, st, src, dst, Cin, Cout, s, taps); }
+    return dst;
+  };
+  auto vec = [&](const float* src, int n) -> float* { float* dst = ar.take(n); pack_copy(src, dst, 1, n, n, 0); return dst; };
+  struct Snake { float* ea; float* ib; };
+  auto snake = [&](int n) -> Snake {
+    const float* al = next(); const float* be = next();
+    Snake s{ar.take(n), ar.take(n)};
+    if (real) hipLaunchKernelGGL(cv_snake_tab_kernel, dim3((n + 255) / 256), dim3(256), 0, st, al, be, s.ea, s.ib, n);
+    return s;
+  };
+  int* ctr = (int*)ar.take(64);
+  auto gemm = [&](const float* W, const float* bias, int M, int Cin, int taps, int dil, int T, const Ring& in) -> CvGemm {
+    CvGemm g;
+    memset(&g, 0, sizeof(g));
+    g.W = W; g.bias = bias; g.M = M; g.Cin = Cin; g.taps = taps; g.dil = dil; g.T = T; g.bias_div = 1;
+    g.in = in; g.in_mode = IN_PLAIN; g.eps = 1e-6f; g.epi = EPI_NONE;
+    g.res = no_ring(); g.out_raw = no_ring(); g.out_act = no_ring(); g.ctr = ctr;
+    g.tt = T <= 16 ? 1 : (T <= 32 ? 2 : 4);
+    const int U = taps * (Cin / 32);
+    const int pf = g.tt == 1 ? 3 : (g.tt == 2 ? 2 : 1);
+    int nw = (U + 2 * pf - 1) / (2 * pf);
+    g.nw = nw < 4 ? 4 : (nw > 16 ? 16 : nw);
+    return g;
+  };
+  auto push_gemm = [&](const CvGemm& g) { if (real) { Step s; memset((void*)&s, 0, sizeof(s)); s.kind = 0; s.g = g; cc->steps.push_back(s); } };
+
+  const int cd = c->codebook_dim, CS = c->codebook_size, L = c->latent_dim, D = c->d_model, A = c->n_heads * c->head_dim;
+  // ---- quantizer: [semantic | acoustic] rows times [W_sem | W_ac] ----
+  float* embed = ar.take((size_t)c->n_codebooks * CS * cd);
+  float* Wvq = ar.take((size_t)c->vq_dim * 2 * cd);
+  {
+    int cb = 0;
+    for (int grp = 0; grp < 2; ++grp) {
+      const int n = grp == 0 ? c->n_semantic : c->n_codebooks - c->n_semantic;
+      next();  // input_proj: encoder side only
+      const float* op = next();
+      pack_copy(op, Wvq, c->vq_dim, cd, 2 * cd, grp * cd);
+      for (int i = 0; i < n; ++i, ++cb) pack_copy(next(), embed + (size_t)cb * CS * cd, CS, cd, cd, 0);
+    }
+  }
+  // ---- state region (zeroed by reset) starts here: all rings ----
+  const size_t state_begin = ar.off;
+  Ring pre_in = mk_ring(ar, c->vq_dim, 2, 1, true);
+  std::vector<Ring> dw_in, tc_in, ru_in;
+  int T = 1;
+  for (int i = 0; i < c->n_up; ++i) { T *= c->up_ratios[i]; dw_in.push_back(mk_ring(ar, L, 6, T, true)); }
+  const int T_lat = T;
+  Ring dec0_in = mk_ring(ar, L, 6, T_lat, true);
+  {
+    int dim = c->decoder_dim, t = T_lat;
+    for (int i = 0; i < c->n_rates; ++i) {
+      tc_in.push_back(mk_ring(ar, dim, 1, t, true));
+      t *= c->rates[i];
+      dim /= 2;
+      for (int j = 0; j < 3; ++j) { const int dil = j == 0 ? 1 : (j == 1 ? 3 : 9); ru_in.push_back(mk_ring(ar, dim, 6 * dil, t, true)); }
+    }
+  }
+  int fin_dim = c->decoder_dim >> c->n_rates;
+  const int hop = vui_codec_hop(c);
+  Ring fin_in = mk_ring(ar, fin_dim, 6, hop, true);
+  const size_t state_end = ar.off;
+  // ---- plain activation buffers ----
+  Ring vqx = mk_ring(ar, 2 * cd, 0, 1, false);
+  Ring pre_out = mk_ring(ar, L, 0, 1, false);
+  Ring xres = mk_ring(ar, D, 0, 1, false);
+  Ring qkv = mk_ring(ar, 3 * A, 0, 1, false);
+  Ring att = mk_ring(ar, A, 0, 1, false);
+  Ring gu = mk_ring(ar, 2 * c->mlp_dim, 0, 1, false);
+  float* kc = ar.take((size_t)c->n_layers * A * c->max_seq);
+  float* vc = ar.take((size_t)c->n_layers * A * c->max_seq);
+  float* inv_freq = ar.take(c->head_dim / 2);
+  if (real) {
+    std::vector<float> h(c->head_dim / 2);
+    // 1 / theta^(2i/dim) in fp32, as torch evaluates it (qwen_codec.py:164)
+    for (int i = 0; i < c->head_dim / 2; ++i) h[i] = 1.0f / powf(c->rope_theta, (float)(2 * i) / (float)c->head_dim);
+    HIP_TRY(hipMemcpyAsync(inv_freq, h.data(), h.size() * 4, hipMemcpyHostToDevice, st));
+    HIP_TRY(hipStreamSynchronize(st));  // h goes out of scope
+  }
+
+  // ---- pre_conv, pre_transformer ----
+  {
+    CvGemm g = gemm(Wvq, nullptr, c->vq_dim, 2 * cd, 1, 1, 1, vqx);
+    g.out_raw = pre_in;
+    push_gemm(g);
+    const float* w = next(); const float* b = next();
+    g = gemm(pack_conv(w, L, c->vq_dim, 3), vec(b, L), L, c->vq_dim, 3, 1, 1, pre_in);
+    g.out_raw = pre_out;
+    push_gemm(g);
+    w = next(); b = next();
+    float* Wi = ar.take((size_t)D * L);
+    pack_copy(w, Wi, D, L, L, 0);
+    g = gemm(Wi, vec(b, D), D, L, 1, 1, 1, pre_out);
+    g.out_raw = xres;
+    push_gemm(g);
+  }
+  for (int l = 0; l < c->n_layers; ++l) {
+    const float* ln1 = next();
+    float* Wqkv = ar.take((size_t)3 * A * D);
+    for (int i = 0; i < 3; ++i) pack_copy(next(), Wqkv + (size_t)i * A * D, A, D, D, 0);
+    float* Wo = ar.take((size_t)D * A);
+    pack_copy(next(), Wo, D, A, A, 0);
+    const float* asc = next();
+    const float* ln2 = next();
+    float* Wgu = ar.take((size_t)2 * c->mlp_dim * D);
+    for (int i = 0; i < 2; ++i) pack_copy(next(), Wgu + (size_t)i * c->mlp_dim * D, c->mlp_dim, D, D, 0);
+    float* Wd = ar.take((size_t)D * c->mlp_dim);
+    pack_copy(next(), Wd, D, c->mlp_dim, c->mlp_dim, 0);
+    const float* msc = next();
+    CvGemm g = gemm(Wqkv, nullptr, 3 * A, D, 1, 1, 1, xres);
+    g.in_mode = IN_RMS; g.in_w = vec(ln1, D); g.out_raw = qkv;
+    push_gemm(g);
+    if (real) {
+      Step s; memset((void*)&s, 0, sizeof(s)); s.kind = 1;
+      s.a.qkv = qkv.p; s.a.kc = kc + (size_t)l * A * c->max_seq; s.a.vc = vc + (size_t)l * A * c->max_seq;
+      s.a.out = att.p; s.a.inv_freq = inv_freq; s.a.H = c->n_heads; s.a.hd = c->head_dim; s.a.max_seq = c->max_seq; s.a.ctr = ctr;
+      cc->steps.push_back(s);
+    }
+    g = gemm(Wo, nullptr, D, A, 1, 1, 1, att);
+    g.epi = EPI_SCALE_RES; g.scale = vec(asc, D); g.res = xres; g.out_raw = xres;
+    push_gemm(g);
+    g = gemm(Wgu, nullptr, 2 * c->mlp_dim, D, 1, 1, 1, xres);
+    g.in_mode = IN_RMS; g.in_w = vec(ln2, D); g.out_raw = gu;
+    push_gemm(g);
+    g = gemm(Wd, nullptr, D, c->mlp_dim, 1, 1, 1, gu);
+    g.in_mode = IN_SILU_MUL; g.epi = EPI_SCALE_RES; g.scale = vec(msc, D); g.res = xres; g.out_raw = xres;
+    push_gemm(g);
+  }
+  Ring cur = mk_ring(ar, L, 0, 1, false);  // output of the transformer = input of the first upsample stage
+  {
+    const float* nw = next(); const float* w = next(); const float* b = next();
+    float* Wout = ar.take((size_t)L * D);
+    pack_copy(w, Wout, L, D, D, 0);
+    CvGemm g = gemm(Wout, vec(b, L), L, D, 1, 1, 1, xres);
+    g.in_mode = IN_RMS; g.in_w = vec(nw, D);
+    g.out_raw = c->n_up ? cur : dec0_in;
+    push_gemm(g);
+  }
+  // ---- upsample stages: transposed conv (kernel = stride) + ConvNeXt block ----
+  T = 1;
+  for (int i = 0; i < c->n_up; ++i) {
+    const int r = c->up_ratios[i], Tin = T;
+    T *= r;
+    const float* w = next(); const float* b = next();
+    CvGemm g = gemm(pack_tconv(w, L, L, r, 1), vec(b, L), L * r, L, 1, 1, Tin, cur);
+    g.bias_div = r; g.tc_stride = r; g.out_raw = dw_in[i];
+    push_gemm(g);
+    const float* dww = next(); const float* dwb = next(); const float* lnw = next(); const float* lnb = next();
+    Ring ln = mk_ring(ar, L, 0, T, false);
+    float* dwwp = vec(dww, L * 7); float* dwbp = vec(dwb, L); float* lnwp = vec(lnw, L); float* lnbp = vec(lnb, L);
+    if (real) {
+      Step s; memset((void*)&s, 0, sizeof(s)); s.kind = 2;
+      s.d.in = dw_in[i]; s.d.w = dwwp; s.d.b = dwbp; s.d.lnw = lnwp; s.d.lnb = lnbp;
+      s.d.out = ln.p; s.d.rs_out = ln.rs; s.d.C = L; s.d.k = 7; s.d.eps = 1e-6f; s.d.ctr = ctr;
+      s.g.T = T;  // grid
+      cc->steps.push_back(s);
+    }
+    const float* w1 = next(); const float* b1 = next(); const float* w2 = next(); const float* b2 = next(); const float* gam = next();
+    Ring pw = mk_ring(ar, 4 * L, 0, T, false);
+    float* W1 = ar.take((size_t)4 * L * L);
+    pack_copy(w1, W1, 4 * L, L, L, 0);
+    g = gemm(W1, vec(b1, 4 * L), 4 * L, L, 1, 1, T, ln);
+    g.epi = EPI_GELU; g.out_raw = pw;
+    push_gemm(g);
+    float* W2 = ar.take((size_t)L * 4 * L);
+    pack_copy(w2, W2, L, 4 * L, 4 * L, 0);
+    g = gemm(W2, vec(b2, L), L, 4 * L, 1, 1, T, pw);
+    g.epi = EPI_SCALE_RES; g.scale = vec(gam, L); g.res = dw_in[i];
+    if (i + 1 < c->n_up) { cur = mk_ring(ar, L, 0, T, false); g.out_raw = cur; } else g.out_raw = dec0_in;
+    push_gemm(g);
+  }
+  // ---- BigVGAN-style decoder ----
+  {
+    int dim = c->decoder_dim;
+    const float* w = next(); const float* b = next();
+    CvGemm g0 = gemm(pack_conv(w, dim, L, 7), vec(b, dim), dim, L, 7, 1, T_lat, dec0_in);
+    int t = T_lat;
+    CvGemm pending = g0;  // its out_act is the first block's snake, known once the block's tensors are read
+    for (int i = 0; i < c->n_rates; ++i) {
+      const int rate = c->rates[i], out = dim / 2, tin = t;
+      t *= rate;
+      Snake s0 = snake(dim);
+      pending.out_act = tc_in[i]; pending.ea = s0.ea; pending.ib = s0.ib;
+      push_gemm(pending);
+      const float* tw = next(); const float* tb = next();
+      CvGemm tg = gemm(pack_tconv(tw, dim, out, rate, 2), vec(tb, out), out * rate, dim, 2, 1, tin, tc_in[i]);
+      tg.bias_div = rate; tg.tc_stride = rate;
+      Ring R = mk_ring(ar, out, 0, t, false);
+      Ring hbuf = mk_ring(ar, out, 0, t, false);
+      tg.out_raw = R;
+      pending = tg;
+      for (int j = 0; j < 3; ++j) {
+        const int dil = j == 0 ? 1 : (j == 1 ? 3 : 9);
+        const Ring& rin = ru_in[i * 3 + j];
+        Snake a1 = snake(out);
+        pending.out_act = rin; pending.ea = a1.ea; pending.ib = a1.ib;
+        push_gemm(pending);
+        const float* w1 = next(); const float* b1 = next();
+        Snake a2 = snake(out);
+        const float* w2 = next(); const float* b2 = next();
+        CvGemm c1 = gemm(pack_conv(w1, out, out, 7), vec(b1, out), out, out, 7, dil, t, rin);
+        c1.out_act = hbuf; c1.ea = a2.ea; c1.ib = a2.ib;
+        push_gemm(c1);
+        float* W2 = ar.take((size_t)out * out);
+        pack_copy(w2, W2, out, out, out, 0);
+        CvGemm c2 = gemm(W2, vec(b2, out), out, out, 1, 1, t, hbuf);
+        c2.epi = EPI_RES; c2.res = R;
+        if (j < 2) c2.out_raw = R;
+        pending = c2;
+      }
+      dim = out;
+    }
+    Snake sf = snake(dim);
+    pending.out_act = fin_in; pending.ea = sf.ea; pending.ib = sf.ib;
+    push_gemm(pending);
+    const float* fw = next(); const float* fb = next();
+    float* fwp = vec(fw, dim * 7); float* fbp = vec(fb, 1);
+    if (real) {
+      cc->fin.in = fin_in; cc->fin.w = fwp; cc->fin.b = fbp; cc->fin.audio = nullptr; cc->fin.C = dim; cc->fin.k = 7; cc->fin.T = hop; cc->fin.ctr = ctr;
+    }
+  }
+  if (need) *need = (int64_t)ar.off;
+  if (real) {
+    cc->ctr = ctr;
+    cc->state0 = (float*)(ws + state_begin);
+    cc->state_floats = (state_end - state_begin) / 4;
+    cc->vq.codes = nullptr; cc->vq.n_q = 0; cc->vq.n_sem = c->n_semantic; cc->vq.CS = CS; cc->vq.cd = cd;
+    cc->vq.embed = embed; cc->vq.x = vqx.p; cc->vq.ctr = ctr; cc->vq.err = ctr + 1; cc->vq.max_seq = c->max_seq;
+    if (ti != vui_codec_n_tensors(c)) { vui_set_error("codec: internal tensor count %d != %d", ti, vui_codec_n_tensors(c)); return VUI_EINVAL; }
+    HIP_TRY(hipGetLastError());
+  }
+  return VUI_OK;
+}
+
+int64_t vui_codec_workspace_bytes(const vui_codec_config* c) {
+  if (cv_check(c)) return VUI_EINVAL;
+  int64_t need = 0;
+  if (cv_build(nullptr, c, nullptr, nullptr, nullptr, &need)) return VUI_EINVAL;
+  return need;
+}
+
+int vui_codec_reset(vui_codec* c, vui_stream_t stream) {
+  if (!c) { vui_set_error("NULL codec"); return VUI_EINVAL; }
+  hipStream_t st = (hipStream_t)stream;
+  dim3 g; grid_for(c->state_floats, g);
+  hipLaunchKernelGGL(cv_fill_kernel, g, dim3(256), 0, st, c->state0, c->state_floats, 0.0f);
+  hipLaunchKernelGGL(cv_set_int_kernel, dim3(1), dim3(1), 0, st, c->ctr, 0, 0);
+  HIP_TRY(hipGetLastError());
+  return VUI_OK;
+}
+
+int vui_codec_init(const vui_codec_config* cfg, const void* const* tensors, int32_t n_tensors, void* workspace,
+                   int64_t workspace_bytes, vui_stream_t stream, vui_codec** out) {
+  if (!out) { vui_set_error("NULL out"); return VUI_EINVAL; }
+  *out = nullptr;
+  int rc = cv_check(cfg);
+  if (rc) return rc;
+  if (!tensors || !workspace) { vui_set_error("NULL argument"); return VUI_EINVAL; }
+  if (n_tensors != vui_codec_n_tensors(cfg)) { vui_set_error("codec: %d tensors given, %d expected", n_tensors, vui_codec_n_tensors(cfg)); return VUI_EINVAL; }
+  for (int i = 0; i < n_tensors; ++i)
+    if (!tensors[i]) { vui_set_error("codec: tensor %d is NULL", i); return VUI_EINVAL; }
+  const int64_t need = vui_codec_workspace_bytes(cfg);
+  if (need < 0) return (int)need;
+  if (workspace_bytes < need) { vui_set_error("workspace too small: %lld < %lld", (long long)workspace_bytes, (long long)need); return VUI_ENOMEM; }
+  if (((uintptr_t)workspace) & 255) { vui_set_error("workspace must be 256-byte aligned"); return VUI_EINVAL; }
+  vui_codec* c = new (std::nothrow) vui_codec();
+  if (!c) { vui_set_error("out of host memory"); return VUI_ENOMEM; }
+  c->cfg = *cfg; c->hop = vui_codec_hop(cfg); c->ws = (char*)workspace; c->ws_bytes = workspace_bytes;
+  rc = cv_build(c, cfg, tensors, (char*)workspace, (hipStream_t)stream, nullptr);
+  if (!rc) rc = vui_codec_reset(c, stream);
+  if (rc) { delete c; return rc; }
+  // kernels with more than 64 KB of dynamic LDS need the attribute (16 waves x 4 tiles at most)
+  *out = c;
+  return VUI_OK;
+}
+
+void vui_codec_destroy(vui_codec* c) { delete c; }
+
+static int launch_cv_gemm(const CvGemm& g, hipStream_t st) {
+  if (g.M % 16 || g.Cin % 32 || g.T < 1) { vui_set_error("codec gemm: bad shape M=%d Cin=%d T=%d", g.M, g.Cin, g.T); return VUI_EINVAL; }
+  const dim3 grid(g.M / 16, (g.T + 16 * g.tt - 1) / (16 * g.tt));
+  const dim3 block(64 * g.nw);
+  const size_t lds = (size_t)g.nw * g.tt * 64 * 4 * 4;
+  if (g.tt == 1) hipLaunchKernelGGL(cv_gemm_kernel<1>, grid, block, lds, st, g);
+  else if (g.tt == 2) hipLaunchKernelGGL(cv_gemm_kernel<2>, grid, block, lds, st, g);
+  else hipLaunchKernelGGL(cv_gemm_kernel<4>, grid, block, lds, st, g);
+  return VUI_OK;
+}
+
+int vui_codec_decode_frame(vui_codec* c, const int64_t* codes, int32_t n_q, float* audio_out, vui_stream_t stream) {
+  if (!c) { vui_set_error("NULL codec"); return VUI_EINVAL; }
+  if (!codes || !audio_out) { vui_set_error("NULL argument"); return VUI_EINVAL; }
+  if (n_q < 1 || n_q > c->cfg.n_codebooks) { vui_set_error("n_q=%d outside [1,%d]", n_q, c->cfg.n_codebooks); return VUI_EINVAL; }
+  hipStream_t st = (hipStream_t)stream;
+  CvVq vq = c->vq;
+  vq.codes = codes; vq.n_q = n_q;
+  hipLaunchKernelGGL(cv_vq_kernel, dim3(1), dim3(256), 0, st, vq);
+  for (const Step& s : c->steps) {
+    if (s.kind == 0) {
+      int rc = launch_cv_gemm(s.g, st);
+      if (rc) return rc;
+    } else if (s.kind == 1) {
+      const size_t lds = (size_t)(s.a.hd + s.a.max_seq + 4 * s.a.hd + 8) * 4;
+      hipLaunchKernelGGL(cv_attn_kernel, dim3(s.a.H), dim3(256), lds, st, s.a);
+    } else {
+      hipLaunchKernelGGL(cv_dwln_kernel, dim3(s.g.T), dim3(256), 0, st, s.d);
+    }
+  }
+  CvFinal fin = c->fin;
+  fin.audio = audio_out;
+  hipLaunchKernelGGL(cv_final_kernel, dim3((fin.T + 63) / 64), dim3(256), 0, st, fin);
+  HIP_TRY(hipGetLastError());
+  return VUI_OK;
+}
+
+int64_t vui_codec_status(vui_codec* c, vui_stream_t stream) {
+  if (!c) { vui_set_error("NULL codec"); return VUI_EINVAL; }
+  int h[2] = {0, 0};
+  HIP_TRY(hipMemcpyAsync(h, c->ctr, sizeof(h), hipMemcpyDeviceToHost, (hipStream_t)stream));
+  HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+  if (h[1] == 1) { vui_set_error("codec: a code outside [0, %d) was clamped", c->cfg.codebook_size); return VUI_EINVAL; }
+  if (h[1] == 2) { vui_set_error("codec: more than max_seq=%d frames since the last reset", c->cfg.max_seq); return VUI_EINVAL; }
+  return h[0];
+}
