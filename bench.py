@@ -13,6 +13,7 @@ from __future__ import annotations
 
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -118,6 +119,42 @@ def kernel_roofline(out, fb):
             "traffic": MEASURED_TRAFFIC_BYTES, "us_per_launch": round(us, 2), "algorithmic_bytes": int(fb["frame"])}
 
 
+def vocoder_line():
+    """Streaming vocoder (fp32) at the reference's dims: codes of one frame -> 1920 samples from its captured
+    graph, 200 frames.  Bytes = every weight one frame must read (all but the encoder-side projections and
+    the unused codebook rows)."""
+    import torch
+
+    from vui_amd.codec import CodecConfig, QwenCodecDecoder, codec_state_dict_shapes
+    from vui_amd.synthetic import synthetic_codec_state_dict
+
+    ccfg = CodecConfig()
+    voc = QwenCodecDecoder(synthetic_codec_state_dict(ccfg, 0), ccfg)
+    voc.setup_streaming_graph(1)
+    g = torch.Generator().manual_seed(0)
+    voc._stream_codes_in.copy_(torch.randint(0, ccfg.codebook_size, (ccfg.n_codebooks,), generator=g).cuda())
+    shapes = codec_state_dict_shapes(ccfg)
+    cb = sum(math.prod(v) for k, v in shapes.items() if not (k.startswith("quantizer") and "input_proj" in k))
+    cb -= sum(math.prod(v) for k, v in shapes.items() if k.endswith("embed"))
+    cb = (cb + ccfg.n_codebooks * ccfg.codebook_dim) * 4
+    gr = voc._graphs[ccfg.n_codebooks]
+    n = 200
+    with voc.streaming(1):
+        for _ in range(3):
+            gr.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            gr.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / n
+    return voc, {"config": "vocoder_b1", "dtype": "f32", "frames": n, "us_per_frame": round(us, 1), "samples_per_frame": voc.hop,
+                 "rtf": round(1e6 / us / 12.5, 1), "weight_bytes": int(cb), "achieved_GBs": round(cb / us / 1e3, 1),
+                 "hbm_frac": round(cb / us / 1e3 / HBM_PEAK_GBS, 4)}
+
+
 def suite(model, eng, d, sd, preset="A"):
     """Extra lines for the other benchmark configs: backbone step at KV 256/1024/4096, depth head alone,
     16 int8 streams with ragged caches."""
@@ -199,7 +236,27 @@ def suite(model, eng, d, sd, preset="A"):
     dt = time.perf_counter() - t0
     lines.append({"config": "stream_b1", "frames": n_out, "chunks": 4, "ms_per_frame_wall": round(dt * 1e3 / n_out, 4),
                   "frames_per_s": round(n_out / dt, 1), "rtf": round(n_out / dt / 12.5, 2)})
-    del eng2, model2
+    # streaming vocoder, then a streamed turn with audio out (decode step + vocoder per frame, codes stay on
+    # the device)
+    voc, line = vocoder_line()
+    lines.append(line)
+    eng2.codec = voc
+    eng2.seq_lens[0] = 0
+    row3 = row2
+    from vui_amd.codec import CodecCtx
+    row3._codec_ctx = CodecCtx(voc)
+    row3.reset()
+    n_out = sum(1 for _ in row3.stream_audio(chunks[:1], cfg_s))
+    row3.reset()
+    row3._codec_ctx.reset()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    n_out = sum(1 for _ in row3.stream_audio(chunks, cfg_s))
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    lines.append({"config": "stream_b1_audio", "frames": n_out, "chunks": 4, "ms_per_frame_wall": round(dt * 1e3 / n_out, 4),
+                  "frames_per_s": round(n_out / dt, 1), "rtf": round(n_out / dt / 12.5, 2)})
+    del eng2, model2, voc
     # config 5: 16 streams, int8 backbone weights, ragged caches U[128, 2048]
     S = 2048 + 256
     model5 = Vui(nano_for_cache(preset, S), sd, device="cuda", dtype=torch.bfloat16, int8=True)
@@ -259,11 +316,16 @@ def main():
     ap.add_argument("--suite", action="store_true", help="also print one JSON line per further benchmark config")
     ap.add_argument("--calib", action="store_true",
                     help="end with three plain 512 MiB device copies (reference points for hardware counters)")
+    ap.add_argument("--vocoder-only", action="store_true",
+                    help="print only the vocoder line (the run rocprofv3 summaries of the vocoder kernels come from)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (streams are independent); "
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.vocoder_only:
+        print(json.dumps(vocoder_line()[1]))
+        return
     out, (model, eng, d, sd) = gpu_bench(args)
     if not args.no_roofline:
         out["roofline"] = kernel_roofline(out, out["frame_bytes"])

@@ -109,6 +109,10 @@ def load() -> C.CDLL:
     if not os.path.exists(LIB_PATH):
         raise RuntimeError(
             f"{LIB_PATH} is missing: build it with `python -m vui_amd.build` (there is no fallback path)")
+    # one HIP runtime per process: PyTorch brings its own copy, so it is loaded first and the library binds
+    # to that one (loaded the other way round, kernels launched from here find no device)
+    import torch  # noqa: F401
+
     lib = C.CDLL(LIB_PATH)
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError if the library does not export it

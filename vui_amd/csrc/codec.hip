@@ -43,8 +43,10 @@ __device__ __forceinline__ float* ring_ptr(const Ring& r, int base, int c, int c
   return r.p + (size_t)c * r.rs + ((base + col) & r.mask);
 }
 
-enum { IN_PLAIN = 0, IN_RMS = 1, IN_SILU_MUL = 2 };
-enum { EPI_NONE = 0, EPI_GELU = 1, EPI_RES = 2, EPI_SCALE_RES = 3 };
+// IN_RMS: the input column is RMS-normalised; the norm weight is folded into W when it is packed and
+// 1/rms multiplies the sums.  EPI_SILU_PAIR: rows (2i, 2i+1) hold gate_i and up_i; channel i = silu(gate) * up.
+enum { IN_PLAIN = 0, IN_RMS = 1 };
+enum { EPI_NONE = 0, EPI_GELU = 1, EPI_RES = 2, EPI_SCALE_RES = 3, EPI_SILU_PAIR = 4 };
 
 struct CvGemm {
   const float* W;     // (taps, M, Cin)
@@ -53,7 +55,6 @@ struct CvGemm {
   int bias_div;
   Ring in;
   int in_mode;
-  const float* in_w;  // norm weight (IN_RMS)
   float eps;
   int epi;
   const float* scale;  // per output channel (EPI_SCALE_RES)
@@ -64,46 +65,53 @@ struct CvGemm {
   const float* ea;
   const float* ib;
   const int* ctr;  // frames started; this frame is *ctr - 1
-  int nw, tt;      // launch shape (host side)
+  int splits;      // workgroups that share one tile's (tap, channel) units; > 1: parts meet in `part`
+  float* part;     // (tiles, splits, TT*64*4) partial sums
+  int* cnt;        // (tiles) arrival counters, zero between launches
+  int tt;          // 16-column blocks per tile (host side: picks the instantiation)
 };
 
-template <int TT> struct Pf { static constexpr int N = TT == 1 ? 3 : (TT == 2 ? 2 : 1); };
+// device-scope relaxed accesses: they bypass the per-XCD L2s, so another workgroup's value is seen
+__device__ __forceinline__ void st_dev(float* p, float a, float b) {
+  __hip_atomic_store(reinterpret_cast<uint64_t*>(p), ((uint64_t)__float_as_uint(b) << 32) | __float_as_uint(a),
+                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t ld_dev(const float* p) {
+  return __hip_atomic_load(reinterpret_cast<const uint64_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
+// units a wave keeps in registers per round (both operands, double-buffered): 2 * NU * (8 + 8*TT) VGPRs
+template <int TT> struct Nu { static constexpr int N = TT == 1 ? 8 : (TT == 2 ? 5 : 3); };
+
+#define CV_NW 4  // waves per workgroup
+
+// One 16-row x 16*TT-column output tile.  `red` is CV_NW * TT * 64 * 4 floats of LDS.
 template <int TT>
-__global__ __launch_bounds__(1024) void cv_gemm_kernel(const CvGemm p) {
-  extern __shared__ __align__(16) float red[];  // nw x TT x 64 x 4
-  constexpr int PF = Pf<TT>::N;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, nw = blockDim.x >> 6;
+__device__ __forceinline__ void cv_gemm_tile(const CvGemm& p, const int m0, const int t0, const int f, float* red,
+                                             const int tile, const int part_idx) {
+  constexpr int NU = Nu<TT>::N;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int r16 = lane & 15, g = lane >> 4;
-  const int m0 = blockIdx.x * 16, t0 = blockIdx.y * (16 * TT);
-  const int f = *p.ctr - 1;
   const int ib_ = ring_base(p.in, f);
-  const int G = p.Cin >> 5, U = p.taps * G;
+  const int G = p.Cin >> 5, Uall = p.taps * G;
   const int M = p.M, Cin = p.Cin;
+  // this workgroup's share of the units: [ub, U)
+  const int per = (Uall + p.splits - 1) / p.splits;
+  const int ub = part_idx * per, U = min(Uall, ub + per);
 
-  float rstd = 1.f;
-  if (p.in_mode == IN_RMS) {  // one column
-    float ss = 0.f;
-    for (int c = lane; c < Cin; c += WAVE) {
-      const float v = *ring_ptr(p.in, ib_, c, p.in.pad);
-      ss = fmaf(v, v, ss);
-    }
-    ss = wave_sum(ss);
-    rstd = 1.0f / sqrtf(ss / (float)Cin + p.eps);
-  }
-
-  float4 a_nx[PF][2], a_cu[PF][2];
-  float b_nx[PF][TT][8], b_cu[PF][TT][8];
+  float4 a0[NU][2], a1[NU][2];
+  float b0[NU][TT][8], b1[NU][TT][8];
   floatx4 acc[TT];
 #pragma unroll
   for (int tt = 0; tt < TT; ++tt) acc[tt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  auto load = [&](int u0, float4 (&a)[PF][2], float (&b)[PF][TT][8]) {
+  // requests the operands of units u0, u0 + NW, ... (NU of them); nothing is waited for here
+  auto load = [&](int u0, float4 (&a)[NU][2], float (&b)[NU][TT][8]) {
 #pragma unroll
-    for (int i = 0; i < PF; ++i) {
-      const int u = u0 + i * nw;
+    for (int i = 0; i < NU; ++i) {
+      const int u = u0 + i * CV_NW;
       const bool on = u < U;
-      const int tap = on ? u / G : 0, grp = on ? u % G : 0;
+      const int tap = on ? u / G : 0, grp = on ? u - tap * G : 0;
       const int ci0 = grp * 32 + g * 8;
       const float* wp = p.W + ((size_t)tap * M + m0 + r16) * Cin + ci0;
       a[i][0] = on ? *reinterpret_cast<const float4*>(wp) : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -112,46 +120,43 @@ __global__ __launch_bounds__(1024) void cv_gemm_kernel(const CvGemm p) {
       for (int tt = 0; tt < TT; ++tt) {
         const int t = t0 + tt * 16 + r16;
         const bool bon = on && t < p.T;
+        const float* xp = ring_ptr(p.in, ib_, bon ? ci0 : 0, bon ? t + tap * p.dil : 0);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          float v = 0.f;
-          if (bon) {
-            const int ci = ci0 + j;
-            if (p.in_mode == IN_SILU_MUL) {
-              const float ga = *ring_ptr(p.in, ib_, ci, p.in.pad + t);
-              const float up = *ring_ptr(p.in, ib_, ci + Cin, p.in.pad + t);
-              v = ga / (1.0f + expf(-ga)) * up;
-            } else {
-              v = *ring_ptr(p.in, ib_, ci, t + tap * p.dil);
-              if (p.in_mode == IN_RMS) v = v * rstd * p.in_w[ci];
-            }
-          }
-          b[i][tt][j] = v;
-        }
+        for (int j = 0; j < 8; ++j) b[i][tt][j] = bon ? xp[(size_t)j * p.in.rs] : 0.f;
       }
     }
   };
-
-  load(wave, a_nx, b_nx);
-  for (int u0 = wave; u0 < U; u0 += PF * nw) {
+  auto mma = [&](const float4 (&a)[NU][2], const float (&b)[NU][TT][8]) {
 #pragma unroll
-    for (int i = 0; i < PF; ++i) {
-      a_cu[i][0] = a_nx[i][0]; a_cu[i][1] = a_nx[i][1];
-#pragma unroll
-      for (int tt = 0; tt < TT; ++tt)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) b_cu[i][tt][j] = b_nx[i][tt][j];
-    }
-    if (u0 + PF * nw < U) load(u0 + PF * nw, a_nx, b_nx);
-#pragma unroll
-    for (int i = 0; i < PF; ++i) {
-      const float av[8] = {a_cu[i][0].x, a_cu[i][0].y, a_cu[i][0].z, a_cu[i][0].w,
-                           a_cu[i][1].x, a_cu[i][1].y, a_cu[i][1].z, a_cu[i][1].w};
+    for (int i = 0; i < NU; ++i) {
+      const float av[8] = {a[i][0].x, a[i][0].y, a[i][0].z, a[i][0].w, a[i][1].x, a[i][1].y, a[i][1].z, a[i][1].w};
 #pragma unroll
       for (int j = 0; j < 8; ++j)
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt)
-          acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[j], b_cu[i][tt][j], acc[tt], 0, 0, 0);
+          acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[j], b[i][tt][j], acc[tt], 0, 0, 0);
+    }
+  };
+
+  constexpr int STEP = NU * CV_NW;
+  load(ub + wave, a0, b0);
+  // 1/rms of the input column while the first operands are in flight; applied to the sums at the end
+  float rstd = 1.f;
+  if (p.in_mode == IN_RMS) {
+    float ss = 0.f;
+    for (int c = lane; c < Cin; c += WAVE) {
+      const float v = *ring_ptr(p.in, ib_, c, p.in.pad);
+      ss = fmaf(v, v, ss);
+    }
+    ss = wave_sum(ss);
+    rstd = 1.0f / sqrtf(ss / (float)Cin + p.eps);
+  }
+  for (int u0 = ub + wave; u0 < U; u0 += 2 * STEP) {
+    if (u0 + STEP < U) load(u0 + STEP, a1, b1);
+    mma(a0, b0);
+    if (u0 + STEP < U) {
+      if (u0 + 2 * STEP < U) load(u0 + 2 * STEP, a0, b0);
+      mma(a1, b1);
     }
   }
 
@@ -162,20 +167,60 @@ __global__ __launch_bounds__(1024) void cv_gemm_kernel(const CvGemm p) {
         make_float4(acc[tt][0], acc[tt][1], acc[tt][2], acc[tt][3]);
   __syncthreads();
   const int rb = ring_base(p.res, f), ob = ring_base(p.out_raw, f), ab = ring_base(p.out_act, f);
-  for (int idx = tid; idx < TT * 64; idx += blockDim.x) {
-    const int tt = idx >> 6, l = idx & 63;
-    float v[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int w = 0; w < nw; ++w) {
-      const float4 q = *reinterpret_cast<const float4*>(red + ((size_t)(w * TT + tt) * 64 + l) * 4);
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  if (tid < TT * 64) {
+#pragma unroll
+    for (int w = 0; w < CV_NW; ++w) {
+      const float4 q = *reinterpret_cast<const float4*>(red + ((size_t)w * TT * 64 + tid) * 4);
       v[0] += q.x; v[1] += q.y; v[2] += q.z; v[3] += q.w;
     }
+  }
+  if (p.splits > 1) {
+    // parts of a tile meet in memory; the workgroup that arrives last adds them in part order and finishes
+    __shared__ int last;
+    float* mine = p.part + (((size_t)tile * p.splits + part_idx) * TT * 64 + tid) * 4;
+    if (tid < TT * 64) { st_dev(mine, v[0], v[1]); st_dev(mine + 2, v[2], v[3]); }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the write-through stores have completed
+    __syncthreads();
+    if (tid == 0) {
+      const int old = __hip_atomic_fetch_add(p.cnt + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      last = old == p.splits - 1;
+      if (last) __hip_atomic_store(p.cnt + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!last) return;
+    if (tid < TT * 64) {
+      uint64_t q[8][2];
+#pragma unroll
+      for (int z = 0; z < 8; ++z) {
+        const float* src = p.part + (((size_t)tile * p.splits + z) * TT * 64 + tid) * 4;
+        q[z][0] = z < p.splits ? ld_dev(src) : 0;
+        q[z][1] = z < p.splits ? ld_dev(src + 2) : 0;
+      }
+      v[0] = v[1] = v[2] = v[3] = 0.f;
+#pragma unroll
+      for (int z = 0; z < 8; ++z) {
+        v[0] += __uint_as_float((uint32_t)q[z][0]); v[1] += __uint_as_float((uint32_t)(q[z][0] >> 32));
+        v[2] += __uint_as_float((uint32_t)q[z][1]); v[3] += __uint_as_float((uint32_t)(q[z][1] >> 32));
+      }
+    }
+  }
+  if (tid < TT * 64) {
+    const int tt = tid >> 6, l = tid & 63;
     const int t = t0 + tt * 16 + (l & 15);
-    if (t >= p.T) continue;
+    if (t >= p.T) return;
+    if (p.epi == EPI_SILU_PAIR) {  // one column per frame
+#pragma unroll
+      for (int r = 0; r < 4; r += 2) {
+        const float ga = v[r] * rstd, up = v[r + 1] * rstd;
+        *ring_ptr(p.out_raw, ob, (m0 + 4 * (l >> 4) + r) >> 1, p.out_raw.pad + t) = ga / (1.0f + expf(-ga)) * up;
+      }
+      return;
+    }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int m = m0 + 4 * (l >> 4) + r;
-      if (m >= M) continue;
-      float y = v[r];
+      float y = v[r] * rstd;
       if (p.bias) y += p.bias[m / p.bias_div];
       int ch = m, col = t;
       if (p.tc_stride > 0) { ch = m / p.tc_stride; col = t * p.tc_stride + m % p.tc_stride; }
@@ -189,6 +234,12 @@ __global__ __launch_bounds__(1024) void cv_gemm_kernel(const CvGemm p) {
       }
     }
   }
+}
+
+template <int TT>
+__global__ __launch_bounds__(CV_NW * 64) void cv_gemm_kernel(const CvGemm p) {
+  __shared__ __align__(16) float red[CV_NW * TT * 64 * 4];
+  cv_gemm_tile<TT>(p, blockIdx.x * 16, blockIdx.y * (16 * TT), *p.ctr - 1, red, blockIdx.y * gridDim.x + blockIdx.x, blockIdx.z);
 }
 
 // ---- codebook rows of one frame: [sum of the semantic rows | sum of the acoustic rows]; starts the frame ----
@@ -205,11 +256,20 @@ struct CvVq {
 __global__ __launch_bounds__(256) void cv_vq_kernel(const CvVq p) {
   for (int c = threadIdx.x; c < p.cd; c += blockDim.x) {
     float s0 = 0.f, s1 = 0.f;
-    for (int i = 0; i < p.n_q; ++i) {
-      long code = p.codes[i];
-      if (code < 0 || code >= p.CS) { code = code < 0 ? 0 : p.CS - 1; if (c == 0) *p.err = 1; }
-      const float e = p.embed[((size_t)i * p.CS + code) * p.cd + c];
-      if (i < p.n_sem) s0 += e; else s1 += e;
+    for (int i0 = 0; i0 < p.n_q; i0 += 16) {  // 16 codes, then their 16 rows, are requested together
+      long code[16];
+      float e[16];
+#pragma unroll
+      for (int k = 0; k < 16; ++k) code[k] = i0 + k < p.n_q ? p.codes[i0 + k] : 0;
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        if (code[k] < 0 || code[k] >= p.CS) { code[k] = code[k] < 0 ? 0 : p.CS - 1; if (c == 0) *p.err = 1; }
+        e[k] = i0 + k < p.n_q ? p.embed[((size_t)(i0 + k) * p.CS + code[k]) * p.cd + c] : 0.f;
+      }
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {  // the reference's order: codebook after codebook
+        if (i0 + k < p.n_sem) s0 += e[k]; else s1 += e[k];
+      }
     }
     p.x[c] = s0;
     p.x[p.cd + c] = s1;
@@ -255,11 +315,29 @@ __global__ __launch_bounds__(256) void cv_attn_kernel(const CvAttn p) {
     vh[(size_t)pos * hd + tid] = p.qkv[2 * A + h * hd + tid];
   }
   __syncthreads();  // this workgroup's own cache row is visible to all its threads after the barrier
+  // scores: a group of 16 lanes per key (features l16, l16 + 16, ...), four keys of a group in flight
   const float scale = 1.0f / sqrtf((float)hd);
-  for (int j = wave; j <= pos; j += 4) {
-    float d = lane < hd ? q[lane] * kh[(size_t)j * hd + lane] : 0.f;
-    d = wave_sum(d);
-    if (lane == 0) sc[j] = d * scale;
+  const int grp = tid >> 4, l16 = tid & 15, E = hd >> 4;
+  float qe[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) qe[e] = e < E ? q[l16 + 16 * e] : 0.f;
+  for (int j0 = grp; j0 <= pos; j0 += 64) {
+    float kv[4][4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + 16 * u;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) kv[u][e] = (j <= pos && e < E) ? kh[(size_t)j * hd + l16 + 16 * e] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + 16 * u;
+      float d = 0.f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) d = fmaf(qe[e], kv[u][e], d);
+      d = group16_sum(d);
+      if (l16 == 0 && j <= pos) sc[j] = d * scale;
+    }
   }
   __syncthreads();
   float mx = -INFINITY;
@@ -274,10 +352,18 @@ __global__ __launch_bounds__(256) void cv_attn_kernel(const CvAttn p) {
   if (lane == 0) red[4 + wave] = sum;
   __syncthreads();
   sum = (red[4] + red[5]) + (red[6] + red[7]);
+  // P.V: wave w takes keys w, w + 4, ...; eight rows in flight
   float o = 0.f;
-  if (lane < hd)
-    for (int j = wave; j <= pos; j += 4) o = fmaf(sc[j], vh[(size_t)j * hd + lane], o);
-  if (lane < hd) part[wave * hd + lane] = o;
+  if (lane < hd) {
+    for (int j0 = wave; j0 <= pos; j0 += 32) {
+      float vv[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) { const int j = j0 + 4 * u; vv[u] = j <= pos ? vh[(size_t)j * hd + lane] : 0.f; }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) { const int j = j0 + 4 * u; o = fmaf(j <= pos ? sc[j] : 0.f, vv[u], o); }
+    }
+    part[wave * hd + lane] = o;
+  }
   __syncthreads();
   if (tid < hd) p.out[h * hd + tid] = ((part[tid] + part[hd + tid]) + (part[2 * hd + tid] + part[3 * hd + tid])) / sum;
 }
@@ -346,20 +432,32 @@ struct CvFinal {
 };
 
 __global__ __launch_bounds__(256) void cv_final_kernel(const CvFinal p) {
-  __shared__ float part[4][64];
+  extern __shared__ float xs[];  // C x (64 + k - 1) window of the ring, then 4 x 64 partial sums
   const int tid = threadIdx.x, qd = tid >> 6, l = tid & 63;
-  const int t = blockIdx.x * 64 + l;
+  const int t0 = blockIdx.x * 64, W = 64 + p.k - 1;
   const int f = *p.ctr - 1, base = ring_base(p.in, f);
-  float a = 0.f;
-  if (t < p.T) {
-    const int c0 = (p.C * qd) / 4, c1 = (p.C * (qd + 1)) / 4;
-    for (int c = c0; c < c1; ++c)
-      for (int k = 0; k < p.k; ++k) a = fmaf(p.w[c * p.k + k], *ring_ptr(p.in, base, c, t + k), a);
+  const int n = p.C * W;
+  for (int i0 = tid; i0 < n; i0 += 256 * 8) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + 256 * u;
+      v[u] = i < n ? *ring_ptr(p.in, base, i / W, t0 + i % W) : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) { const int i = i0 + 256 * u; if (i < n) xs[i] = v[u]; }
   }
-  part[qd][l] = a;
   __syncthreads();
+  float a = 0.f;
+  const int c0 = (p.C * qd) / 4, c1 = (p.C * (qd + 1)) / 4;
+  for (int c = c0; c < c1; ++c)
+    for (int k = 0; k < p.k; ++k) a = fmaf(p.w[c * p.k + k], xs[c * W + l + k], a);
+  float* part = xs + n;
+  part[qd * 64 + l] = a;
+  __syncthreads();
+  const int t = t0 + l;
   if (qd == 0 && t < p.T) {
-    const float y = ((part[0][l] + part[1][l]) + (part[2][l] + part[3][l])) + p.b[0];
+    const float y = ((part[l] + part[64 + l]) + (part[128 + l] + part[192 + l])) + p.b[0];
     p.audio[t] = fminf(1.0f, fmaxf(-1.0f, y));
   }
 }
@@ -392,6 +490,11 @@ __global__ void cv_copy_rows_kernel(const float* src, float* dst, int M, int K, 
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
     dst[(i / K) * ld + off + (i % K)] = src[i];
 }
+// W (M, K) *= w (K) along every row
+__global__ void cv_scale_cols_kernel(float* W, const float* w, int M, int K) {
+  const size_t n = (size_t)M * K;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) W[i] *= w[i % K];
+}
 __global__ void cv_snake_tab_kernel(const float* alpha, const float* beta, float* ea, float* ib, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) { ea[i] = expf(alpha[i]); ib[i] = 1.0f / (expf(beta[i]) + 1e-9f); }
@@ -417,6 +520,8 @@ struct vui_codec {
   float* state0;  // start of the zeroed-on-reset region (rings)
   size_t state_floats;
   int* ctr;  // [0] frames started since reset, [1] error flag
+  int* cnt;  // arrival counters of split tiles
+  size_t part_floats = 0, cnt_ints = 0;
   CvVq vq;
   std::vector<Step> steps;
   CvFinal fin;
@@ -432,7 +537,8 @@ static int cv_check(const vui_codec_config* c) {
   int dims32[] = {2 * c->codebook_dim, c->vq_dim, c->latent_dim, c->d_model, A, c->mlp_dim, 4 * c->latent_dim, c->decoder_dim};
   for (int v : dims32)
     if (v < 32 || (v % 32)) { vui_set_error("codec: every layer width must be a multiple of 32 (got %d)", v); return VUI_EINVAL; }
-  if (c->head_dim > 64 || (c->head_dim & 1) || c->n_heads < 1) { vui_set_error("codec: head_dim=%d unsupported (even, <= 64)", c->head_dim); return VUI_EINVAL; }
+  if (c->head_dim > 64 || (c->head_dim & 15) || c->n_heads < 1) { vui_set_error("codec: head_dim=%d unsupported (a multiple of 16, <= 64)", c->head_dim); return VUI_EINVAL; }
+  if ((c->decoder_dim >> c->n_rates) * (64 + 6) * 4 > 60000) { vui_set_error("codec: last stage too wide"); return VUI_EINVAL; }
   if (c->max_seq < 1 || c->max_seq > 4096) { vui_set_error("codec: max_seq=%d outside [1,4096]", c->max_seq); return VUI_EINVAL; }
   if (c->latent_dim > 256 * DW_MAXC) { vui_set_error("codec: latent_dim=%d above %d", c->latent_dim, 256 * DW_MAXC); return VUI_EINVAL; }
   int dim = c->decoder_dim;
@@ -483,7 +589,8 @@ static Ring no_ring() { Ring r; r.p = nullptr; r.rs = 1; r.mask = 0; r.pad = 0; 
 static void grid_for(size_t n, dim3& g) { size_t b = (n + 255) / 256; g = dim3((unsigned)(b > 4096 ? 4096 : (b ? b : 1))); }
 
 // Lays out the workspace and (when tensors != nullptr) packs weights and records the launch plan.
-static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const* tensors, char* ws, hipStream_t st, int64_t* need) {
+static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const* tensors, char* ws, hipStream_t st, int64_t* need,
+                    size_t part_cap, size_t cnt_cap, size_t* part_need, size_t* cnt_need) {
   Arena ar{ws};
   const bool real = ws != nullptr && tensors != nullptr;
   int ti = 0;
@@ -503,6 +610,11 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
     if (real) { dim3 g; grid_for((size_t)taps * Cout * s * Cin, g); hipLaunchKernelGGL(cv_pack_tconv_kernel, g, dim3(256), 0, st, src, dst, Cin, Cout, s, taps); }
     return dst;
   };
+  auto fold_norm = [&](float* W, const float* w, int M, int K) {
+    if (!real) return;
+    dim3 g; grid_for((size_t)M * K, g);
+    hipLaunchKernelGGL(cv_scale_cols_kernel, g, dim3(256), 0, st, W, w, M, K);
+  };
   auto vec = [&](const float* src, int n) -> float* { float* dst = ar.take(n); pack_copy(src, dst, 1, n, n, 0); return dst; };
   struct Snake { float* ea; float* ib; };
   auto snake = [&](int n) -> Snake {
@@ -512,17 +624,31 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
     return s;
   };
   int* ctr = (int*)ar.take(64);
+  // meeting place of split tiles: sized by a first pass (the sizes do not depend on the pointers)
+  size_t part_floats = 0, cnt_ints = 0;
+  float* part = ar.take(part_cap);
+  int* cnt = (int*)ar.take(cnt_cap);
   auto gemm = [&](const float* W, const float* bias, int M, int Cin, int taps, int dil, int T, const Ring& in) -> CvGemm {
     CvGemm g;
     memset(&g, 0, sizeof(g));
     g.W = W; g.bias = bias; g.M = M; g.Cin = Cin; g.taps = taps; g.dil = dil; g.T = T; g.bias_div = 1;
     g.in = in; g.in_mode = IN_PLAIN; g.eps = 1e-6f; g.epi = EPI_NONE;
     g.res = no_ring(); g.out_raw = no_ring(); g.out_act = no_ring(); g.ctr = ctr;
-    g.tt = T <= 16 ? 1 : (T <= 32 ? 2 : 4);
+    // the widest tile that still gives ~200 workgroups; then workgroups share a tile's units until ~768
+    // are in flight, as long as every wave keeps at least four units
     const int U = taps * (Cin / 32);
-    const int pf = g.tt == 1 ? 3 : (g.tt == 2 ? 2 : 1);
-    int nw = (U + 2 * pf - 1) / (2 * pf);
-    g.nw = nw < 4 ? 4 : (nw > 16 ? 16 : nw);
+    auto tiles = [&](int tt) { return (M / 16) * ((T + 16 * tt - 1) / (16 * tt)); };
+    g.tt = (T > 32 && tiles(4) >= 200) ? 4 : ((T > 16 && tiles(2) >= 200) ? 2 : 1);
+    int sp = 1;
+    if (U >= 64) {
+      sp = (768 + tiles(g.tt) - 1) / tiles(g.tt);
+      if (sp > U / 16) sp = U / 16;
+      if (sp > 8) sp = 8;
+      if (sp < 1) sp = 1;
+    }
+    g.splits = sp; g.part = part; g.cnt = cnt;
+    if ((size_t)tiles(g.tt) * sp * g.tt * 256 > part_floats) part_floats = (size_t)tiles(g.tt) * sp * g.tt * 256;
+    if ((size_t)tiles(g.tt) > cnt_ints) cnt_ints = tiles(g.tt);
     return g;
   };
   auto push_gemm = [&](const CvGemm& g) { if (real) { Step s; memset((void*)&s, 0, sizeof(s)); s.kind = 0; s.g = g; cc->steps.push_back(s); } };
@@ -568,7 +694,7 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
   Ring xres = mk_ring(ar, D, 0, 1, false);
   Ring qkv = mk_ring(ar, 3 * A, 0, 1, false);
   Ring att = mk_ring(ar, A, 0, 1, false);
-  Ring gu = mk_ring(ar, 2 * c->mlp_dim, 0, 1, false);
+  Ring gu = mk_ring(ar, c->mlp_dim, 0, 1, false);
   float* kc = ar.take((size_t)c->n_layers * A * c->max_seq);
   float* vc = ar.take((size_t)c->n_layers * A * c->max_seq);
   float* inv_freq = ar.take(c->head_dim / 2);
@@ -600,17 +726,19 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
     const float* ln1 = next();
     float* Wqkv = ar.take((size_t)3 * A * D);
     for (int i = 0; i < 3; ++i) pack_copy(next(), Wqkv + (size_t)i * A * D, A, D, D, 0);
+    fold_norm(Wqkv, ln1, 3 * A, D);
     float* Wo = ar.take((size_t)D * A);
     pack_copy(next(), Wo, D, A, A, 0);
     const float* asc = next();
     const float* ln2 = next();
-    float* Wgu = ar.take((size_t)2 * c->mlp_dim * D);
-    for (int i = 0; i < 2; ++i) pack_copy(next(), Wgu + (size_t)i * c->mlp_dim * D, c->mlp_dim, D, D, 0);
+    float* Wgu = ar.take((size_t)2 * c->mlp_dim * D);  // rows interleaved: gate_0, up_0, gate_1, up_1, ...
+    for (int i = 0; i < 2; ++i) pack_copy(next(), Wgu, c->mlp_dim, D, 2 * D, i * D);
+    fold_norm(Wgu, ln2, 2 * c->mlp_dim, D);
     float* Wd = ar.take((size_t)D * c->mlp_dim);
     pack_copy(next(), Wd, D, c->mlp_dim, c->mlp_dim, 0);
     const float* msc = next();
     CvGemm g = gemm(Wqkv, nullptr, 3 * A, D, 1, 1, 1, xres);
-    g.in_mode = IN_RMS; g.in_w = vec(ln1, D); g.out_raw = qkv;
+    g.in_mode = IN_RMS; g.out_raw = qkv;
     push_gemm(g);
     if (real) {
       Step s; memset((void*)&s, 0, sizeof(s)); s.kind = 1;
@@ -622,10 +750,10 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
     g.epi = EPI_SCALE_RES; g.scale = vec(asc, D); g.res = xres; g.out_raw = xres;
     push_gemm(g);
     g = gemm(Wgu, nullptr, 2 * c->mlp_dim, D, 1, 1, 1, xres);
-    g.in_mode = IN_RMS; g.in_w = vec(ln2, D); g.out_raw = gu;
+    g.in_mode = IN_RMS; g.epi = EPI_SILU_PAIR; g.out_raw = gu;
     push_gemm(g);
     g = gemm(Wd, nullptr, D, c->mlp_dim, 1, 1, 1, gu);
-    g.in_mode = IN_SILU_MUL; g.epi = EPI_SCALE_RES; g.scale = vec(msc, D); g.res = xres; g.out_raw = xres;
+    g.epi = EPI_SCALE_RES; g.scale = vec(msc, D); g.res = xres; g.out_raw = xres;
     push_gemm(g);
   }
   Ring cur = mk_ring(ar, L, 0, 1, false);  // output of the transformer = input of the first upsample stage
@@ -633,8 +761,9 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
     const float* nw = next(); const float* w = next(); const float* b = next();
     float* Wout = ar.take((size_t)L * D);
     pack_copy(w, Wout, L, D, D, 0);
+    fold_norm(Wout, nw, L, D);
     CvGemm g = gemm(Wout, vec(b, L), L, D, 1, 1, 1, xres);
-    g.in_mode = IN_RMS; g.in_w = vec(nw, D);
+    g.in_mode = IN_RMS;
     g.out_raw = c->n_up ? cur : dec0_in;
     push_gemm(g);
   }
@@ -722,8 +851,11 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
     }
   }
   if (need) *need = (int64_t)ar.off;
+  if (part_need) *part_need = part_floats;
+  if (cnt_need) *cnt_need = cnt_ints;
   if (real) {
-    cc->ctr = ctr;
+    if (part_floats > part_cap || cnt_ints > cnt_cap) { vui_set_error("codec: internal scratch sizing"); return VUI_EINVAL; }
+    cc->ctr = ctr; cc->cnt = cnt; cc->cnt_ints = cnt_cap;
     cc->state0 = (float*)(ws + state_begin);
     cc->state_floats = (state_end - state_begin) / 4;
     cc->vq.codes = nullptr; cc->vq.n_q = 0; cc->vq.n_sem = c->n_semantic; cc->vq.CS = CS; cc->vq.cd = cd;
@@ -737,7 +869,9 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
 int64_t vui_codec_workspace_bytes(const vui_codec_config* c) {
   if (cv_check(c)) return VUI_EINVAL;
   int64_t need = 0;
-  if (cv_build(nullptr, c, nullptr, nullptr, nullptr, &need)) return VUI_EINVAL;
+  size_t pf = 0, ci = 0;
+  if (cv_build(nullptr, c, nullptr, nullptr, nullptr, nullptr, 0, 0, &pf, &ci)) return VUI_EINVAL;
+  if (cv_build(nullptr, c, nullptr, nullptr, nullptr, &need, pf, ci, nullptr, nullptr)) return VUI_EINVAL;
   return need;
 }
 
@@ -768,7 +902,13 @@ int vui_codec_init(const vui_codec_config* cfg, const void* const* tensors, int3
   vui_codec* c = new (std::nothrow) vui_codec();
   if (!c) { vui_set_error("out of host memory"); return VUI_ENOMEM; }
   c->cfg = *cfg; c->hop = vui_codec_hop(cfg); c->ws = (char*)workspace; c->ws_bytes = workspace_bytes;
-  rc = cv_build(c, cfg, tensors, (char*)workspace, (hipStream_t)stream, nullptr);
+  size_t pf = 0, ci = 0;
+  rc = cv_build(nullptr, cfg, nullptr, nullptr, nullptr, nullptr, 0, 0, &pf, &ci);
+  if (!rc) rc = cv_build(c, cfg, tensors, (char*)workspace, (hipStream_t)stream, nullptr, pf, ci, nullptr, nullptr);
+  if (!rc) {
+    dim3 g; grid_for(ci, g);
+    hipLaunchKernelGGL(cv_fill_kernel, g, dim3(256), 0, (hipStream_t)stream, (float*)c->cnt, ci, 0.0f);
+  }
   if (!rc) rc = vui_codec_reset(c, stream);
   if (rc) { delete c; return rc; }
   // kernels with more than 64 KB of dynamic LDS need the attribute (16 waves x 4 tiles at most)
@@ -780,12 +920,11 @@ void vui_codec_destroy(vui_codec* c) { delete c; }
 
 static int launch_cv_gemm(const CvGemm& g, hipStream_t st) {
   if (g.M % 16 || g.Cin % 32 || g.T < 1) { vui_set_error("codec gemm: bad shape M=%d Cin=%d T=%d", g.M, g.Cin, g.T); return VUI_EINVAL; }
-  const dim3 grid(g.M / 16, (g.T + 16 * g.tt - 1) / (16 * g.tt));
-  const dim3 block(64 * g.nw);
-  const size_t lds = (size_t)g.nw * g.tt * 64 * 4 * 4;
-  if (g.tt == 1) hipLaunchKernelGGL(cv_gemm_kernel<1>, grid, block, lds, st, g);
-  else if (g.tt == 2) hipLaunchKernelGGL(cv_gemm_kernel<2>, grid, block, lds, st, g);
-  else hipLaunchKernelGGL(cv_gemm_kernel<4>, grid, block, lds, st, g);
+  const dim3 grid(g.M / 16, (g.T + 16 * g.tt - 1) / (16 * g.tt), g.splits);
+  const dim3 block(64 * CV_NW);
+  if (g.tt == 1) hipLaunchKernelGGL(cv_gemm_kernel<1>, grid, block, 0, st, g);
+  else if (g.tt == 2) hipLaunchKernelGGL(cv_gemm_kernel<2>, grid, block, 0, st, g);
+  else hipLaunchKernelGGL(cv_gemm_kernel<4>, grid, block, 0, st, g);
   return VUI_OK;
 }
 
@@ -810,7 +949,7 @@ int vui_codec_decode_frame(vui_codec* c, const int64_t* codes, int32_t n_q, floa
   }
   CvFinal fin = c->fin;
   fin.audio = audio_out;
-  hipLaunchKernelGGL(cv_final_kernel, dim3((fin.T + 63) / 64), dim3(256), 0, st, fin);
+  hipLaunchKernelGGL(cv_final_kernel, dim3((fin.T + 63) / 64), dim3(256), (size_t)(fin.C * (64 + fin.k - 1) + 256) * 4, st, fin);
   HIP_TRY(hipGetLastError());
   return VUI_OK;
 }

@@ -97,6 +97,12 @@ class Row:
         self._closed = False
         self.prompt_wps: float = 0.0
         self._slot = torch.tensor([idx], dtype=torch.int32, device=engine.device)
+        # rolling vocoder context of the row (src/vui/engine.py:172); None without a codec
+        self._codec_ctx = None
+        if engine.codec is not None:
+            from .codec import CodecCtx
+
+            self._codec_ctx = CodecCtx(engine.codec)
 
     @property
     def idx(self) -> int:
@@ -119,6 +125,18 @@ class Row:
         if self._engine.max_rows != 1:
             raise RuntimeError(f"stream() requires Engine(max_rows=1), got {self._engine.max_rows}")
         yield from self._engine._stream_row(self, chunks, cfg, cancel, reset_rep=reset_rep, final_turn=final_turn)
+
+    def stream_audio(self, chunks: "list[Chunk]", cfg: GenConfig = GenConfig(), cancel=None, *, reset_rep: bool = True,
+                     final_turn: bool = False) -> Iterator[Tensor]:
+        """`stream` with every frame passed through the row's vocoder context: yields audio (1, 1, 1920)
+        per frame, as Row.stream of the reference does (src/vui/engine.py:204-244, 1349-1356, 1537-1546).
+        The vocoder stream is seeded once per session from the row's buffered codes."""
+        if self._codec_ctx is None:
+            raise RuntimeError("stream_audio() needs Engine(codec=...)")
+        if self._codec_ctx._stack is None:
+            self._codec_ctx.prefill(n_codebooks=cfg.n_codebooks)
+        for codes in self.stream(chunks, cfg, cancel, reset_rep=reset_rep, final_turn=final_turn):
+            yield self._engine._stream_decode_frame(self, codes, cfg.n_codebooks)
 
     def mark_prompt(self) -> int:
         self._prompt_offset = self.offset
@@ -316,6 +334,19 @@ class Engine:
     def _release_row(self, row: Row) -> None:
         self._rows.pop(row.idx, None)
         self._free.add(row.idx)
+        if row._codec_ctx is not None:
+            row._codec_ctx.reset()
+
+    def _stream_decode_frame(self, row: Row, frame_codes: Tensor, n_codebooks: int) -> Tensor:
+        """One frame of codes (Q',) -> audio through the row's vocoder context; fewer codebooks are
+        decoded as such but stored zero-padded to Q (src/vui/engine.py:1537-1546)."""
+        if frame_codes.shape[0] < self.Q:
+            padded = torch.zeros(self.Q, device=self.device, dtype=frame_codes.dtype)
+            padded[: frame_codes.shape[0]] = frame_codes
+            frame_codes = padded
+        codes_t = frame_codes.unsqueeze(0).unsqueeze(-1)
+        decode_codes = codes_t[:, :n_codebooks] if n_codebooks > 0 else codes_t
+        return row._codec_ctx.decode_frame(decode_codes, store_codes=codes_t)
 
     def reset(self) -> None:
         for row in list(self._rows.values()):

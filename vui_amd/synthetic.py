@@ -70,3 +70,42 @@ def nano_for_cache(preset: str, max_seqlen: int) -> Config:
     cfg.model.max_text_tokens = max_seqlen - cfg.model.n_quantizers
     cfg.model.max_audio_tokens = 0
     return cfg
+
+
+def synthetic_codec_state_dict(cfg, seed: int = 0) -> dict[str, Tensor]:
+    """Deterministic fp32 vocoder weights (vui_amd.codec.CodecConfig) that keep activations O(1) through
+    its ~60 layers: linear and conv weights N(0, 1/fan_in), biases N(0, 0.05), norm weights 1 + N(0, 0.1),
+    snake log-rates N(0, 0.3), residual scales N(0.3, 0.1), codebooks N(0, 1); the closing 1x1 conv of every
+    residual unit is scaled by 0.3 and the last conv by 0.12.  Each key draws from its own CPU generator
+    seeded with (seed, key index)."""
+    import math
+
+    from .codec import codec_state_dict_shapes
+
+    sd = {}
+    for idx, (k, shape) in enumerate(codec_state_dict_shapes(cfg).items()):
+        g = torch.Generator().manual_seed(seed * 1000003 + 7919 + idx)
+        r = torch.randn(shape, generator=g)
+        if k.endswith("embed"):
+            t = r
+        elif k.endswith(("alpha", "beta")):
+            t = 0.3 * r
+        elif k.endswith(("attn_scale", "mlp_scale", "gamma")):
+            t = 0.3 + 0.1 * r
+        elif k.endswith("norm.weight"):
+            t = 1.0 + 0.1 * r
+        elif k.endswith(".bias"):
+            t = 0.05 * r
+        elif len(shape) == 3 and (".block.1." in k or (k.startswith("upsample") and ".0.conv" in k)):
+            stride = shape[2] if k.startswith("upsample") else shape[2] // 2
+            t = r / math.sqrt(shape[0] * shape[2] / stride)
+        elif len(shape) == 3:
+            t = r / math.sqrt(shape[1] * shape[2])
+            if "conv2.conv" in k:
+                t = 0.3 * t
+            elif shape[0] == 1:
+                t = 0.12 * t
+        else:
+            t = r / math.sqrt(shape[-1])
+        sd[k] = t.contiguous()
+    return sd
