@@ -25,6 +25,7 @@
 #include <math.h>
 #include <new>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 #include <vector>
 
@@ -80,42 +81,53 @@ __device__ __forceinline__ uint64_t ld_dev(const float* p) {
   return __hip_atomic_load(reinterpret_cast<const uint64_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// units a wave keeps in registers per round (both operands, double-buffered): 2 * NU * (8 + 8*TT) VGPRs
-template <int TT> struct Nu { static constexpr int N = TT == 1 ? 8 : (TT == 2 ? 5 : 3); };
+// units a wave keeps in registers per round: NU * (8 + 8*TT) VGPRs, twice that when the rounds are
+// double-buffered (DB: for tiles whose waves need several rounds; one wave per SIMD).  Tiles that fit one
+// round use the single-buffered form, which leaves room for two or three waves per SIMD.
+template <int TT, bool DB> struct Nu { static constexpr int N = TT == 1 ? 8 : (TT == 2 ? (DB ? 5 : 6) : 3); };
 
 #define CV_NW 4  // waves per workgroup
 
 // One 16-row x 16*TT-column output tile.  `red` is CV_NW * TT * 64 * 4 floats of LDS.
-template <int TT>
-__device__ __forceinline__ void cv_gemm_tile(const CvGemm& p, const int m0, const int t0, const int f, float* red,
+template <int TT, bool DB>
+__device__ __forceinline__ void cv_gemm_tile(const CvGemm& p, const int m0, const int t0, float* red,
                                              const int tile, const int part_idx) {
-  constexpr int NU = Nu<TT>::N;
+  constexpr int NU = Nu<TT, DB>::N;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int r16 = lane & 15, g = lane >> 4;
-  const int ib_ = ring_base(p.in, f);
   const int G = p.Cin >> 5, Uall = p.taps * G;
   const int M = p.M, Cin = p.Cin;
   // this workgroup's share of the units: [ub, U)
   const int per = (Uall + p.splits - 1) / p.splits;
   const int ub = part_idx * per, U = min(Uall, ub + per);
 
-  float4 a0[NU][2], a1[NU][2];
-  float b0[NU][TT][8], b1[NU][TT][8];
+  float4 a0[NU][2], a1[DB ? NU : 1][2];
+  float b0[NU][TT][8], b1[DB ? NU : 1][TT][8];
   floatx4 acc[TT];
 #pragma unroll
   for (int tt = 0; tt < TT; ++tt) acc[tt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  // requests the operands of units u0, u0 + NW, ... (NU of them); nothing is waited for here
-  auto load = [&](int u0, float4 (&a)[NU][2], float (&b)[NU][TT][8]) {
+  // request the operands of units u0, u0 + NW, ... (NU of them); nothing is waited for here.  The weights
+  // do not depend on the frame counter, so the first round asks for them before the counter is needed.
+  auto load_a = [&](int u0, auto& a) {
+#pragma unroll
+    for (int i = 0; i < NU; ++i) {
+      const int u = u0 + i * CV_NW;
+      const bool on = u < U;
+      const int tap = on ? u / G : 0, grp = on ? u - tap * G : 0;
+      const float* wp = p.W + ((size_t)tap * M + m0 + r16) * Cin + grp * 32 + g * 8;
+      a[i][0] = on ? *reinterpret_cast<const float4*>(wp) : make_float4(0.f, 0.f, 0.f, 0.f);
+      a[i][1] = on ? *reinterpret_cast<const float4*>(wp + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  };
+  int ib_ = 0;
+  auto load_b = [&](int u0, auto& b) {
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
       const int u = u0 + i * CV_NW;
       const bool on = u < U;
       const int tap = on ? u / G : 0, grp = on ? u - tap * G : 0;
       const int ci0 = grp * 32 + g * 8;
-      const float* wp = p.W + ((size_t)tap * M + m0 + r16) * Cin + ci0;
-      a[i][0] = on ? *reinterpret_cast<const float4*>(wp) : make_float4(0.f, 0.f, 0.f, 0.f);
-      a[i][1] = on ? *reinterpret_cast<const float4*>(wp + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
       for (int tt = 0; tt < TT; ++tt) {
         const int t = t0 + tt * 16 + r16;
@@ -126,7 +138,8 @@ __device__ __forceinline__ void cv_gemm_tile(const CvGemm& p, const int m0, cons
       }
     }
   };
-  auto mma = [&](const float4 (&a)[NU][2], const float (&b)[NU][TT][8]) {
+  auto load = [&](int u0, auto& a, auto& b) { load_a(u0, a); load_b(u0, b); };
+  auto mma = [&](const auto& a, const auto& b) {
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
       const float av[8] = {a[i][0].x, a[i][0].y, a[i][0].z, a[i][0].w, a[i][1].x, a[i][1].y, a[i][1].z, a[i][1].w};
@@ -139,7 +152,29 @@ __device__ __forceinline__ void cv_gemm_tile(const CvGemm& p, const int m0, cons
   };
 
   constexpr int STEP = NU * CV_NW;
-  load(ub + wave, a0, b0);
+  load_a(ub + wave, a0);
+  const int f = *p.ctr - 1;
+  ib_ = ring_base(p.in, f);
+  load_b(ub + wave, b0);
+  // what the epilogue adds is requested now as well
+  const int rb = ring_base(p.res, f), ob = ring_base(p.out_raw, f), ab = ring_base(p.out_act, f);
+  float e_bias[4] = {0.f, 0.f, 0.f, 0.f}, e_res[4] = {0.f, 0.f, 0.f, 0.f}, e_sc[4] = {1.f, 1.f, 1.f, 1.f};
+  float e_ea[4] = {0.f, 0.f, 0.f, 0.f}, e_ib[4] = {0.f, 0.f, 0.f, 0.f};
+  if (tid < TT * 64) {
+    const int t = t0 + (tid >> 6) * 16 + (tid & 15);
+    if (t < p.T) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = m0 + 4 * ((tid & 63) >> 4) + r;
+        int ch = m, col = t;
+        if (p.tc_stride > 0) { ch = m / p.tc_stride; col = t * p.tc_stride + m % p.tc_stride; }
+        if (p.bias) e_bias[r] = p.bias[m / p.bias_div];
+        if (p.epi == EPI_RES || p.epi == EPI_SCALE_RES) e_res[r] = *ring_ptr(p.res, rb, ch, p.res.pad + col);
+        if (p.epi == EPI_SCALE_RES) e_sc[r] = p.scale[ch];
+        if (p.out_act.p) { e_ea[r] = p.ea[ch]; e_ib[r] = p.ib[ch]; }
+      }
+    }
+  }
   // 1/rms of the input column while the first operands are in flight; applied to the sums at the end
   float rstd = 1.f;
   if (p.in_mode == IN_RMS) {
@@ -151,12 +186,19 @@ __device__ __forceinline__ void cv_gemm_tile(const CvGemm& p, const int m0, cons
     ss = wave_sum(ss);
     rstd = 1.0f / sqrtf(ss / (float)Cin + p.eps);
   }
-  for (int u0 = ub + wave; u0 < U; u0 += 2 * STEP) {
-    if (u0 + STEP < U) load(u0 + STEP, a1, b1);
-    mma(a0, b0);
-    if (u0 + STEP < U) {
-      if (u0 + 2 * STEP < U) load(u0 + 2 * STEP, a0, b0);
-      mma(a1, b1);
+  if constexpr (DB) {
+    for (int u0 = ub + wave; u0 < U; u0 += 2 * STEP) {
+      if (u0 + STEP < U) load(u0 + STEP, a1, b1);
+      mma(a0, b0);
+      if (u0 + STEP < U) {
+        if (u0 + 2 * STEP < U) load(u0 + 2 * STEP, a0, b0);
+        mma(a1, b1);
+      }
+    }
+  } else {
+    for (int u0 = ub + wave; u0 < U; u0 += STEP) {
+      if (u0 != ub + wave) load(u0, a0, b0);
+      mma(a0, b0);
     }
   }
 
@@ -166,7 +208,6 @@ __device__ __forceinline__ void cv_gemm_tile(const CvGemm& p, const int m0, cons
     *reinterpret_cast<float4*>(red + ((size_t)(wave * TT + tt) * 64 + lane) * 4) =
         make_float4(acc[tt][0], acc[tt][1], acc[tt][2], acc[tt][3]);
   __syncthreads();
-  const int rb = ring_base(p.res, f), ob = ring_base(p.out_raw, f), ab = ring_base(p.out_act, f);
   float v[4] = {0.f, 0.f, 0.f, 0.f};
   if (tid < TT * 64) {
 #pragma unroll
@@ -220,17 +261,16 @@ __device__ __forceinline__ void cv_gemm_tile(const CvGemm& p, const int m0, cons
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int m = m0 + 4 * (l >> 4) + r;
-      float y = v[r] * rstd;
-      if (p.bias) y += p.bias[m / p.bias_div];
+      float y = v[r] * rstd + e_bias[r];
       int ch = m, col = t;
       if (p.tc_stride > 0) { ch = m / p.tc_stride; col = t * p.tc_stride + m % p.tc_stride; }
       if (p.epi == EPI_GELU) y = 0.5f * y * (1.0f + erff(y * 0.70710678118654752f));
-      else if (p.epi == EPI_RES) y = *ring_ptr(p.res, rb, ch, p.res.pad + col) + y;
-      else if (p.epi == EPI_SCALE_RES) y = *ring_ptr(p.res, rb, ch, p.res.pad + col) + p.scale[ch] * y;
+      else if (p.epi == EPI_RES) y = e_res[r] + y;
+      else if (p.epi == EPI_SCALE_RES) y = e_res[r] + e_sc[r] * y;
       if (p.out_raw.p) *ring_ptr(p.out_raw, ob, ch, p.out_raw.pad + col) = y;
       if (p.out_act.p) {
-        const float s = sinf(y * p.ea[ch]);
-        *ring_ptr(p.out_act, ab, ch, p.out_act.pad + col) = y + p.ib[ch] * s * s;
+        const float s = sinf(y * e_ea[r]);
+        *ring_ptr(p.out_act, ab, ch, p.out_act.pad + col) = y + e_ib[r] * s * s;
       }
     }
   }
@@ -239,7 +279,12 @@ __device__ __forceinline__ void cv_gemm_tile(const CvGemm& p, const int m0, cons
 template <int TT>
 __global__ __launch_bounds__(CV_NW * 64) void cv_gemm_kernel(const CvGemm p) {
   __shared__ __align__(16) float red[CV_NW * TT * 64 * 4];
-  cv_gemm_tile<TT>(p, blockIdx.x * 16, blockIdx.y * (16 * TT), *p.ctr - 1, red, blockIdx.y * gridDim.x + blockIdx.x, blockIdx.z);
+  cv_gemm_tile<TT, true>(p, blockIdx.x * 16, blockIdx.y * (16 * TT), red, blockIdx.y * gridDim.x + blockIdx.x, blockIdx.z);
+}
+template <int TT>
+__global__ __launch_bounds__(CV_NW * 64, 2) void cv_gemm1_kernel(const CvGemm p) {
+  __shared__ __align__(16) float red[CV_NW * TT * 64 * 4];
+  cv_gemm_tile<TT, false>(p, blockIdx.x * 16, blockIdx.y * (16 * TT), red, blockIdx.y * gridDim.x + blockIdx.x, blockIdx.z);
 }
 
 // ---- codebook rows of one frame: [sum of the semantic rows | sum of the acoustic rows]; starts the frame ----
@@ -366,6 +411,365 @@ __global__ __launch_bounds__(256) void cv_attn_kernel(const CvAttn p) {
   }
   __syncthreads();
   if (tid < hd) p.out[h * hd + tid] = ((part[tid] + part[hd + tid]) + (part[2 * hd + tid] + part[3 * hd + tid])) / sum;
+}
+
+// =============================================================================================
+// The one-column trunk as ONE persistent kernel: codebook rows -> quantizer projection -> pre_conv
+// -> input_proj -> the transformer layers -> output_proj -> first upsampling transposed conv.
+// These 46 steps have one column each (1-3 MB of weights), so as separate launches they run at the
+// cost of a dependent launch.  Here 256 workgroups (one per CU) walk the same list of phases; every
+// workgroup owns a few rows of every matrix, keeps the residual stream and the current input vector
+// in LDS, requests the weights of the next phase before it waits, and passes results as 8-byte
+// words = fp32 payload + launch epoch (device-scope relaxed atomics: a word showing the epoch is the
+// data).  Exchange buffers are never reused inside a launch.  Every wait is bounded.
+// =============================================================================================
+#include "ll.h"
+
+struct TrunkLayer {
+  const float* Wqkv; const float* Wo; const float* asc; const float* Wgu; const float* Wd; const float* msc;
+  float* kc; float* vc;
+};
+
+struct CvTrunk {
+  const int64_t* codes;
+  int n_q, n_sem, CS, cd;
+  const float* embed;
+  int* ctr;
+  int* err;
+  int max_seq;
+  const float* Wvq; int vq_dim;
+  const float* Wpre; const float* bpre; int L;
+  Ring pre_in;
+  const float* Win; const float* bin; int D;
+  int n_layers, H, hd, mlp;
+  const TrunkLayer* layers;
+  const float* inv_freq;
+  const float* Wout; const float* bout;
+  const float* Wt0; const float* bt0; int r0;  // Wt0 == nullptr: no upsampling stage, `out` takes the latent
+  Ring out;
+  uint64_t* ll;
+  uint32_t* epoch; uint32_t* arrive; uint32_t* lerr;
+  float eps;
+};
+
+#define TR_MAXR 3  // rows per wave and phase
+#define TR_MAXC 6  // float4 chunks per lane and row: K <= 1536
+
+struct TrRows { float4 w[TR_MAXR][TR_MAXC]; };
+
+// rows r_lo + wave, r_lo + wave + 4, ... below r_hi of W (M x K): request them
+template <int MAXR, int MAXC>
+__device__ __forceinline__ void tr_prefetch(const float* W, int K, int r_lo, int r_hi, TrRows& rr) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+  for (int i = 0; i < MAXR; ++i) {
+    const int row = r_lo + wave + 4 * i;
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+      const int k = (lane + 64 * c) * 4;
+      const bool on = row < r_hi && k < K;
+      rr.w[i][c] = on ? *reinterpret_cast<const float4*>(W + (size_t)row * K + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  }
+}
+// dot products of those rows with xs (K floats in LDS); epi(row, sum) runs in every lane of the wave
+template <int MAXR, int MAXC, typename F>
+__device__ __forceinline__ void tr_compute(const float* xs, int K, int r_lo, int r_hi, const TrRows& rr, F&& epi) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+  for (int i = 0; i < MAXR; ++i) {
+    const int row = r_lo + wave + 4 * i;
+    if (row < r_hi) {
+      float s = 0.f;
+#pragma unroll
+      for (int c = 0; c < MAXC; ++c) {
+        const int k = (lane + 64 * c) * 4;
+        if (k < K) {
+          const float4 x = *reinterpret_cast<const float4*>(xs + k);
+          s = fmaf(rr.w[i][c].x, x.x, s); s = fmaf(rr.w[i][c].y, x.y, s);
+          s = fmaf(rr.w[i][c].z, x.z, s); s = fmaf(rr.w[i][c].w, x.w, s);
+        }
+      }
+      s = wave_sum(s);
+      epi(row, s);
+    }
+  }
+}
+
+__device__ __forceinline__ void tr_rows(int M, int wg, int nwg, int& lo, int& hi) {
+  const int per = (M + nwg - 1) / nwg;
+  lo = min(M, wg * per);
+  hi = min(M, lo + per);
+}
+
+__device__ __forceinline__ float tr_rstd(const float* x, int n, float eps, float* red) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  float ss = 0.f;
+  for (int i = tid; i < n; i += FR_THREADS) ss = fmaf(x[i], x[i], ss);
+  ss = wave_sum(ss);
+  __syncthreads();
+  if (lane == 0) red[wave] = ss;
+  __syncthreads();
+  return 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)n + eps);
+}
+
+__global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
+  extern __shared__ __align__(16) float tsm[];
+  // xs: current input vector (<= 1536) | x: residual stream (D) | q (hd) | sc (max_seq) | part (4*hd) | red (16)
+  float* xs = tsm;
+  float* x = xs + 1536;
+  float* q = x + a.D;
+  float* sc = q + 64;  // max_seq + 192: scores, and before them the raw q | k | v of the head
+  float* part = sc + a.max_seq + 192;
+  float* red = part + 4 * 64;
+  const int wg = blockIdx.x, nwg = gridDim.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  Ctl c;
+  c.epoch = __hip_atomic_load(a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+  c.err = a.lerr;
+  c.dead = 0;
+  const uint32_t ep = c.epoch;
+  int f = *a.ctr;
+  const bool over = f >= a.max_seq;
+  if (over) f = a.max_seq - 1;  // stay on the last position: nothing runs out of bounds
+  // the epoch and the frame counter have been read before this workgroup reports its arrival
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  if (tid == 0) __hip_atomic_fetch_add(a.arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+  uint64_t* ll = a.ll;
+  auto take = [&](int n) { uint64_t* p = ll; ll += n; return p; };
+  auto put = [&](uint64_t* buf, int i, float v) { ll_st(buf + i, __float_as_uint(v), ep); };
+  auto get = [&](const uint64_t* buf, int n, float* dst) {
+    ll_poll(buf, n, c, [&](int i, uint32_t v) { dst[i] = __uint_as_float(v); });
+    __syncthreads();
+  };
+  TrRows rr;
+  int lo, hi;
+  const int cd = a.cd, V = a.vq_dim, L = a.L, D = a.D, A = a.H * a.hd, hd = a.hd, mlp = a.mlp;
+
+  // ---- quantizer projection: rows of [W_sem | W_ac] against [sum of semantic rows | sum of acoustic rows] ----
+  tr_rows(V, wg, nwg, lo, hi);
+  tr_prefetch<1, 2>(a.Wvq, 2 * cd, lo, hi, rr);
+  for (int ch = tid; ch < cd; ch += FR_THREADS) {  // every workgroup sums the codebook rows itself
+    float s0 = 0.f, s1 = 0.f;
+    for (int i0 = 0; i0 < a.n_q; i0 += 16) {
+      long code[16];
+      float e[16];
+#pragma unroll
+      for (int k = 0; k < 16; ++k) code[k] = i0 + k < a.n_q ? a.codes[i0 + k] : 0;
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        if (code[k] < 0 || code[k] >= a.CS) { code[k] = code[k] < 0 ? 0 : a.CS - 1; if (ch == 0 && wg == 0) *a.err = 1; }
+        e[k] = i0 + k < a.n_q ? a.embed[((size_t)(i0 + k) * a.CS + code[k]) * cd + ch] : 0.f;
+      }
+#pragma unroll
+      for (int k = 0; k < 16; ++k) { if (i0 + k < a.n_sem) s0 += e[k]; else s1 += e[k]; }
+    }
+    xs[ch] = s0;
+    xs[cd + ch] = s1;
+  }
+  __syncthreads();
+  uint64_t* b_y1 = take(V);
+  const int pbase = ring_base(a.pre_in, f);
+  tr_compute<1, 2>(xs, 2 * cd, lo, hi, rr, [&](int row, float s) {
+    if (lane == 0) { put(b_y1, row, s); *ring_ptr(a.pre_in, pbase, row, a.pre_in.pad) = s; }
+  });
+  // ---- pre_conv: three taps = the two previous frames' columns and this one ----
+  tr_rows(L, wg, nwg, lo, hi);
+  {
+    const int wave_row = lo + wave;  // one row per wave: (3, L, V) tap-major
+#pragma unroll
+    for (int cc = 0; cc < TR_MAXC; ++cc) {
+      const int k = (lane + 64 * cc) * 4;  // index into [tap][ci]
+      const int tap = k / V, ci = k - tap * V;
+      const bool on = wave_row < hi && k < 3 * V;
+      rr.w[0][cc] = on ? *reinterpret_cast<const float4*>(a.Wpre + ((size_t)tap * L + wave_row) * V + ci) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  }
+  __syncthreads();  // xs is free again
+  for (int i = tid; i < 2 * V; i += FR_THREADS) xs[i] = *ring_ptr(a.pre_in, pbase, i % V, i / V);
+  ll_poll(b_y1, V, c, [&](int i, uint32_t v) { xs[2 * V + i] = __uint_as_float(v); });
+  __syncthreads();
+  uint64_t* b_pre = take(L);
+  tr_compute<1, TR_MAXC>(xs, 3 * V, lo, hi, rr, [&](int row, float s) { if (lane == 0) put(b_pre, row, s + a.bpre[row]); });
+  // ---- input_proj ----
+  tr_rows(D, wg, nwg, lo, hi);
+  tr_prefetch<1, 4>(a.Win, L, lo, hi, rr);
+  __syncthreads();
+  get(b_pre, L, xs);
+  uint64_t* b_x = take(D);
+  tr_compute<1, 4>(xs, L, lo, hi, rr, [&](int row, float s) { if (lane == 0) put(b_x, row, s + a.bin[row]); });
+  {
+    int qlo, qhi;
+    tr_rows(3 * A, wg, nwg, qlo, qhi);
+    tr_prefetch<TR_MAXR, 2>(a.layers[0].Wqkv, D, qlo, qhi, rr);
+  }
+  get(b_x, D, x);
+
+  const float att_scale = 1.0f / sqrtf((float)hd);
+  for (int l = 0; l < a.n_layers; ++l) {
+    const TrunkLayer& W = a.layers[l];
+    // ---- q, k, v rows (norm weight folded in; 1/rms multiplies the sums) ----
+    const float r1 = tr_rstd(x, D, a.eps, red);
+    tr_rows(3 * A, wg, nwg, lo, hi);
+    uint64_t* b_qkv = take(3 * A);
+    tr_compute<TR_MAXR, 2>(x, D, lo, hi, rr, [&](int row, float s) { if (lane == 0) put(b_qkv, row, s * r1); });
+    uint64_t* b_att = take(A);
+    int olo, ohi;
+    tr_rows(D, wg, nwg, olo, ohi);
+    tr_prefetch<1, 4>(W.Wo, A, olo, ohi, rr);
+    // ---- attention: workgroup h owns head h ----
+    if (wg < a.H) {
+      const int h = wg, half = hd >> 1, pos = f;
+      float* kh = W.kc + (size_t)h * a.max_seq * hd;
+      float* vh = W.vc + (size_t)h * a.max_seq * hd;
+      float* kvn = part;  // this position's rotated key | value
+      __syncthreads();
+      if (tid < 3 * hd) {
+        const int which = tid / hd, i = tid - which * hd;
+        const uint64_t* src = b_qkv + which * A + h * hd + i;
+        uint64_t v = ll_ld(src);
+        int spins = 0;
+        while ((uint32_t)(v >> 32) != ep && !c.dead) {
+          v = ll_ld(src);
+          if (++spins > SPIN_LIMIT) { c.dead = 1; __hip_atomic_store(c.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+        }
+        sc[which * hd + i] = __uint_as_float((uint32_t)v);  // raw q | k | v
+      }
+      __syncthreads();
+      if (tid < hd) {
+        const float ang = (float)pos * a.inv_freq[tid % half];
+        const float cs = cosf(ang), sn = sinf(ang);
+        const float* qq = sc;
+        const float* kk = sc + hd;
+        const float qr = tid < half ? -qq[tid + half] : qq[tid - half];
+        const float kr = tid < half ? -kk[tid + half] : kk[tid - half];
+        q[tid] = qq[tid] * cs + qr * sn;
+        const float kn = kk[tid] * cs + kr * sn, vn = sc[2 * hd + tid];
+        kvn[tid] = kn; kvn[hd + tid] = vn;
+        kh[(size_t)pos * hd + tid] = kn;
+        vh[(size_t)pos * hd + tid] = vn;
+      }
+      __syncthreads();
+      const int grp = tid >> 4, l16 = tid & 15, E = hd >> 4;
+      float qe[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) qe[e] = e < E ? q[l16 + 16 * e] : 0.f;
+      __syncthreads();  // sc is rewritten below
+      for (int j0 = grp; j0 <= pos; j0 += 64) {
+        float kv[4][4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int j = j0 + 16 * u;
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            kv[u][e] = (j <= pos && e < E) ? (j == pos ? kvn[l16 + 16 * e] : kh[(size_t)j * hd + l16 + 16 * e]) : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int j = j0 + 16 * u;
+          float d = 0.f;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) d = fmaf(qe[e], kv[u][e], d);
+          d = group16_sum(d);
+          if (l16 == 0 && j <= pos) sc[j] = d * att_scale;
+        }
+      }
+      __syncthreads();
+      float mx = -INFINITY;
+      for (int j = tid; j <= pos; j += FR_THREADS) mx = fmaxf(mx, sc[j]);
+      mx = wave_max(mx);
+      if (lane == 0) red[wave] = mx;
+      __syncthreads();
+      mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+      float sum = 0.f;
+      for (int j = tid; j <= pos; j += FR_THREADS) { const float e = expf(sc[j] - mx); sc[j] = e; sum += e; }
+      sum = wave_sum(sum);
+      if (lane == 0) red[4 + wave] = sum;
+      __syncthreads();
+      sum = (red[4] + red[5]) + (red[6] + red[7]);
+      float o = 0.f;
+      if (lane < hd) {
+        for (int j0 = wave; j0 <= pos; j0 += 32) {
+          float vv[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) { const int j = j0 + 4 * u; vv[u] = j <= pos ? (j == pos ? kvn[hd + lane] : vh[(size_t)j * hd + lane]) : 0.f; }
+#pragma unroll
+          for (int u = 0; u < 8; ++u) { const int j = j0 + 4 * u; o = fmaf(j <= pos ? sc[j] : 0.f, vv[u], o); }
+        }
+      }
+      __syncthreads();  // kvn (= part) has been read
+      if (lane < hd) part[wave * hd + lane] = o;
+      __syncthreads();
+      if (tid < hd) put(b_att, h * hd + tid, ((part[tid] + part[hd + tid]) + (part[2 * hd + tid] + part[3 * hd + tid])) / sum);
+    }
+    // ---- out_proj, residual with per-channel scale ----
+    get(b_att, A, xs);
+    uint64_t* b_o = take(D);
+    tr_compute<1, 4>(xs, A, olo, ohi, rr, [&](int row, float s) { if (lane == 0) put(b_o, row, s); });
+    int glo, ghi;
+    tr_rows(mlp, wg, nwg, glo, ghi);  // channels; rows 2i, 2i + 1 are gate_i, up_i
+    glo *= 2; ghi *= 2;
+    tr_prefetch<TR_MAXR, 2>(W.Wgu, D, glo, ghi, rr);
+    ll_poll(b_o, D, c, [&](int i, uint32_t v) { x[i] += W.asc[i] * __uint_as_float(v); });
+    // ---- gate / up rows interleaved: channel i = silu(gate_i) * up_i ----
+    const float r2 = tr_rstd(x, D, a.eps, red);
+    uint64_t* b_h = take(mlp);
+    {
+      // a wave's rows glo + wave + 4 i alternate between gate and up of different channels: pair through LDS
+      float* pair = part;
+      tr_compute<TR_MAXR, 2>(x, D, glo, ghi, rr, [&](int row, float s) { if (lane == 0) pair[row - glo] = s * r2; });
+      __syncthreads();
+      for (int i = tid; 2 * i + 1 < ghi - glo; i += FR_THREADS) {
+        const float ga = pair[2 * i], up = pair[2 * i + 1];
+        put(b_h, (glo >> 1) + i, ga / (1.0f + expf(-ga)) * up);
+      }
+    }
+    int dlo, dhi;
+    tr_rows(D, wg, nwg, dlo, dhi);
+    tr_prefetch<1, 4>(W.Wd, mlp, dlo, dhi, rr);
+    get(b_h, mlp, xs);
+    uint64_t* b_d = take(D);
+    tr_compute<1, 4>(xs, mlp, dlo, dhi, rr, [&](int row, float s) { if (lane == 0) put(b_d, row, s); });
+    if (l + 1 < a.n_layers) {
+      int qlo, qhi;
+      tr_rows(3 * A, wg, nwg, qlo, qhi);
+      tr_prefetch<TR_MAXR, 2>(a.layers[l + 1].Wqkv, D, qlo, qhi, rr);
+    } else {
+      int plo, phi;
+      tr_rows(L, wg, nwg, plo, phi);
+      tr_prefetch<1, 2>(a.Wout, D, plo, phi, rr);
+    }
+    ll_poll(b_d, D, c, [&](int i, uint32_t v) { x[i] += W.msc[i] * __uint_as_float(v); });
+  }
+  // ---- final norm (folded) + output_proj ----
+  const float r3 = tr_rstd(x, D, a.eps, red);
+  tr_rows(L, wg, nwg, lo, hi);
+  const int obase = ring_base(a.out, f);
+  if (a.Wt0 == nullptr) {
+    tr_compute<1, 2>(x, D, lo, hi, rr, [&](int row, float s) {
+      if (lane == 0) *ring_ptr(a.out, obase, row, a.out.pad) = s * r3 + a.bout[row];
+    });
+  } else {
+    uint64_t* b_lat = take(L);
+    tr_compute<1, 2>(x, D, lo, hi, rr, [&](int row, float s) { if (lane == 0) put(b_lat, row, s * r3 + a.bout[row]); });
+    // ---- first upsampling stage: transposed conv with kernel = stride: row m -> channel m / r0, column m % r0 ----
+    tr_rows(L * a.r0, wg, nwg, lo, hi);
+    tr_prefetch<TR_MAXR, 4>(a.Wt0, L, lo, hi, rr);
+    __syncthreads();
+    get(b_lat, L, xs);
+    tr_compute<TR_MAXR, 4>(xs, L, lo, hi, rr, [&](int row, float s) {
+      if (lane == 0) *ring_ptr(a.out, obase, row / a.r0, a.out.pad + row % a.r0) = s + a.bt0[row / a.r0];
+    });
+  }
+  if (wg == 0 && tid == 0) {
+    // every workgroup has read the epoch and the frame counter before they may change
+    int spins = 0;
+    while (__hip_atomic_load(a.arrive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (uint32_t)nwg && ++spins < SPIN_LIMIT) {}
+    __hip_atomic_store(a.arrive, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(a.epoch, ep, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (over) *a.err = 2;
+    *a.ctr = f + 1;
+  }
 }
 
 // ---- depthwise causal conv (k taps) + LayerNorm over channels, one workgroup per column ----
@@ -525,6 +929,12 @@ struct vui_codec {
   CvVq vq;
   std::vector<Step> steps;
   CvFinal fin;
+  // the persistent form of the one-column steps (0: the kernel sequence runs them)
+  CvTrunk trunk;
+  int trunk_steps = 0;  // leading entries of `steps` the trunk kernel replaces (the codebook kernel as well)
+  int trunk_wgs = 0;
+  size_t trunk_lds = 0;
+  int use_trunk = 1;
 };
 
 static int ipow2(int n) { int r = 1; while (r < n) r <<= 1; return r; }
@@ -624,6 +1034,10 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
     return s;
   };
   int* ctr = (int*)ar.take(64);
+  // launch-shape targets (overridable for tuning runs)
+  const char* e1 = getenv("VUI_CV_TILES_MIN");
+  const char* e2 = getenv("VUI_CV_WG_TARGET");
+  const int tiles_min = e1 ? atoi(e1) : 200, wg_target = e2 ? atoi(e2) : 768;
   // meeting place of split tiles: sized by a first pass (the sizes do not depend on the pointers)
   size_t part_floats = 0, cnt_ints = 0;
   float* part = ar.take(part_cap);
@@ -638,10 +1052,10 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
     // are in flight, as long as every wave keeps at least four units
     const int U = taps * (Cin / 32);
     auto tiles = [&](int tt) { return (M / 16) * ((T + 16 * tt - 1) / (16 * tt)); };
-    g.tt = (T > 32 && tiles(4) >= 200) ? 4 : ((T > 16 && tiles(2) >= 200) ? 2 : 1);
+    g.tt = (T > 32 && tiles(4) >= tiles_min) ? 4 : ((T > 16 && tiles(2) >= tiles_min) ? 2 : 1);
     int sp = 1;
     if (U >= 64) {
-      sp = (768 + tiles(g.tt) - 1) / tiles(g.tt);
+      sp = (wg_target + tiles(g.tt) - 1) / tiles(g.tt);
       if (sp > U / 16) sp = U / 16;
       if (sp > 8) sp = 8;
       if (sp < 1) sp = 1;
@@ -698,6 +1112,11 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
   float* kc = ar.take((size_t)c->n_layers * A * c->max_seq);
   float* vc = ar.take((size_t)c->n_layers * A * c->max_seq);
   float* inv_freq = ar.take(c->head_dim / 2);
+  // persistent trunk: exchange words (never reused inside a launch), layer table, epoch / arrival / error words
+  const size_t ll_words = (size_t)c->vq_dim + L + D + (size_t)c->n_layers * (3 * A + A + D + c->mlp_dim + D) + L;
+  uint64_t* ll = (uint64_t*)ar.take(ll_words * 2);
+  TrunkLayer* tl_dev = (TrunkLayer*)ar.take((sizeof(TrunkLayer) * c->n_layers + 3) / 4);
+  uint32_t* tctl = (uint32_t*)ar.take(64);
   if (real) {
     std::vector<float> h(c->head_dim / 2);
     // 1 / theta^(2i/dim) in fp32, as torch evaluates it (qwen_codec.py:164)
@@ -707,6 +1126,9 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
   }
 
   // ---- pre_conv, pre_transformer ----
+  CvTrunk tk;
+  memset((void*)&tk, 0, sizeof(tk));
+  std::vector<TrunkLayer> tl(c->n_layers);
   {
     CvGemm g = gemm(Wvq, nullptr, c->vq_dim, 2 * cd, 1, 1, 1, vqx);
     g.out_raw = pre_in;
@@ -715,12 +1137,14 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
     g = gemm(pack_conv(w, L, c->vq_dim, 3), vec(b, L), L, c->vq_dim, 3, 1, 1, pre_in);
     g.out_raw = pre_out;
     push_gemm(g);
+    tk.Wvq = Wvq; tk.vq_dim = c->vq_dim; tk.Wpre = g.W; tk.bpre = g.bias; tk.L = L; tk.pre_in = pre_in;
     w = next(); b = next();
     float* Wi = ar.take((size_t)D * L);
     pack_copy(w, Wi, D, L, L, 0);
     g = gemm(Wi, vec(b, D), D, L, 1, 1, 1, pre_out);
     g.out_raw = xres;
     push_gemm(g);
+    tk.Win = g.W; tk.bin = g.bias; tk.D = D;
   }
   for (int l = 0; l < c->n_layers; ++l) {
     const float* ln1 = next();
@@ -749,12 +1173,15 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
     g = gemm(Wo, nullptr, D, A, 1, 1, 1, att);
     g.epi = EPI_SCALE_RES; g.scale = vec(asc, D); g.res = xres; g.out_raw = xres;
     push_gemm(g);
+    tl[l].Wqkv = Wqkv; tl[l].Wo = Wo; tl[l].asc = g.scale; tl[l].Wgu = Wgu; tl[l].Wd = Wd;
+    tl[l].kc = kc + (size_t)l * A * c->max_seq; tl[l].vc = vc + (size_t)l * A * c->max_seq;
     g = gemm(Wgu, nullptr, 2 * c->mlp_dim, D, 1, 1, 1, xres);
     g.in_mode = IN_RMS; g.epi = EPI_SILU_PAIR; g.out_raw = gu;
     push_gemm(g);
     g = gemm(Wd, nullptr, D, c->mlp_dim, 1, 1, 1, gu);
     g.epi = EPI_SCALE_RES; g.scale = vec(msc, D); g.res = xres; g.out_raw = xres;
     push_gemm(g);
+    tl[l].msc = g.scale;
   }
   Ring cur = mk_ring(ar, L, 0, 1, false);  // output of the transformer = input of the first upsample stage
   {
@@ -766,7 +1193,9 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
     g.in_mode = IN_RMS;
     g.out_raw = c->n_up ? cur : dec0_in;
     push_gemm(g);
+    tk.Wout = g.W; tk.bout = g.bias; tk.out = dec0_in;
   }
+  int trunk_steps = real ? (int)cc->steps.size() : 0;
   // ---- upsample stages: transposed conv (kernel = stride) + ConvNeXt block ----
   T = 1;
   for (int i = 0; i < c->n_up; ++i) {
@@ -776,6 +1205,7 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
     CvGemm g = gemm(pack_tconv(w, L, L, r, 1), vec(b, L), L * r, L, 1, 1, Tin, cur);
     g.bias_div = r; g.tc_stride = r; g.out_raw = dw_in[i];
     push_gemm(g);
+    if (i == 0) { tk.Wt0 = g.W; tk.bt0 = g.bias; tk.r0 = r; tk.out = dw_in[0]; if (real) trunk_steps = (int)cc->steps.size(); }
     const float* dww = next(); const float* dwb = next(); const float* lnw = next(); const float* lnb = next();
     Ring ln = mk_ring(ar, L, 0, T, false);
     float* dwwp = vec(dww, L * 7); float* dwbp = vec(dwb, L); float* lnwp = vec(lnw, L); float* lnbp = vec(lnb, L);
@@ -854,6 +1284,20 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
   if (part_need) *part_need = part_floats;
   if (cnt_need) *cnt_need = cnt_ints;
   if (real) {
+    tk.codes = nullptr; tk.n_q = 0; tk.n_sem = c->n_semantic; tk.CS = CS; tk.cd = cd; tk.embed = embed;
+    tk.ctr = ctr; tk.err = ctr + 1; tk.max_seq = c->max_seq;
+    tk.n_layers = c->n_layers; tk.H = c->n_heads; tk.hd = c->head_dim; tk.mlp = c->mlp_dim;
+    tk.layers = tl_dev; tk.inv_freq = inv_freq; tk.ll = ll; tk.epoch = tctl; tk.arrive = tctl + 1; tk.lerr = tctl + 2;
+    tk.eps = 1e-6f;
+    HIP_TRY(hipMemcpyAsync(tl_dev, tl.data(), sizeof(TrunkLayer) * c->n_layers, hipMemcpyHostToDevice, st));
+    {
+      dim3 g; grid_for(ll_words * 2, g);
+      hipLaunchKernelGGL(cv_fill_kernel, g, dim3(256), 0, st, (float*)ll, ll_words * 2, 0.0f);
+      hipLaunchKernelGGL(cv_fill_kernel, dim3(1), dim3(64), 0, st, (float*)tctl, (size_t)16, 0.0f);
+    }
+    HIP_TRY(hipStreamSynchronize(st));  // tl goes out of scope
+    cc->trunk = tk;
+    cc->trunk_steps = trunk_steps;
     if (part_floats > part_cap || cnt_ints > cnt_cap) { vui_set_error("codec: internal scratch sizing"); return VUI_EINVAL; }
     cc->ctr = ctr; cc->cnt = cnt; cc->cnt_ints = cnt_cap;
     cc->state0 = (float*)(ws + state_begin);
@@ -911,7 +1355,26 @@ int vui_codec_init(const vui_codec_config* cfg, const void* const* tensors, int3
   }
   if (!rc) rc = vui_codec_reset(c, stream);
   if (rc) { delete c; return rc; }
-  // kernels with more than 64 KB of dynamic LDS need the attribute (16 waves x 4 tiles at most)
+  // the persistent trunk needs all its workgroups resident at once and the per-wave row counts it was built for
+  {
+    const vui_codec_config& k = c->cfg;
+    const int A = k.n_heads * k.head_dim;
+    c->trunk_lds = (size_t)(1536 + k.d_model + 64 + k.max_seq + 192 + 256 + 16) * 4;
+    int dev = 0, cus = 0, per_cu = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)cv_trunk_kernel, FR_THREADS, c->trunk_lds));
+    int nwg = cus * per_cu < 256 ? cus * per_cu : 256;
+    auto fits = [&](int M, int K, int maxr, int maxc) { return nwg > 0 && ((M + nwg - 1) / nwg + 3) / 4 <= maxr && K <= 256 * maxc && K % 4 == 0; };
+    const bool ok = nwg >= k.n_heads && fits(k.vq_dim, 2 * k.codebook_dim, 1, 2) && fits(k.latent_dim, 3 * k.vq_dim, 1, TR_MAXC) &&
+                    fits(k.d_model, k.latent_dim, 1, 4) && fits(3 * A, k.d_model, TR_MAXR, 2) && fits(k.d_model, A, 1, 4) &&
+                    2 * ((k.mlp_dim + nwg - 1) / nwg) <= 4 * TR_MAXR && fits(k.d_model, k.mlp_dim, 1, 4) && fits(k.latent_dim, k.d_model, 1, 2) &&
+                    (k.n_up == 0 || fits(k.latent_dim * k.up_ratios[0], k.latent_dim, TR_MAXR, 4)) && k.head_dim <= 64 &&
+                    k.d_model <= 1536 && A <= 1536 && k.mlp_dim <= 1536 && k.latent_dim <= 1536 && 3 * k.vq_dim <= 1536;
+    c->trunk_wgs = ok ? nwg : 0;
+    const char* e = getenv("VUI_CODEC_TRUNK");
+    c->use_trunk = e ? atoi(e) : 1;
+  }
   *out = c;
   return VUI_OK;
 }
@@ -922,9 +1385,18 @@ static int launch_cv_gemm(const CvGemm& g, hipStream_t st) {
   if (g.M % 16 || g.Cin % 32 || g.T < 1) { vui_set_error("codec gemm: bad shape M=%d Cin=%d T=%d", g.M, g.Cin, g.T); return VUI_EINVAL; }
   const dim3 grid(g.M / 16, (g.T + 16 * g.tt - 1) / (16 * g.tt), g.splits);
   const dim3 block(64 * CV_NW);
-  if (g.tt == 1) hipLaunchKernelGGL(cv_gemm_kernel<1>, grid, block, 0, st, g);
-  else if (g.tt == 2) hipLaunchKernelGGL(cv_gemm_kernel<2>, grid, block, 0, st, g);
-  else hipLaunchKernelGGL(cv_gemm_kernel<4>, grid, block, 0, st, g);
+  // units a wave of one part works through; one single-buffered round holds 8 / 6 / 3 of them
+  const int U = g.taps * (g.Cin / 32), per_wave = ((U + g.splits - 1) / g.splits + CV_NW - 1) / CV_NW;
+  const bool one_round = per_wave <= (g.tt == 1 ? 8 : (g.tt == 2 ? 6 : 3));
+  if (one_round) {
+    if (g.tt == 1) hipLaunchKernelGGL(cv_gemm1_kernel<1>, grid, block, 0, st, g);
+    else if (g.tt == 2) hipLaunchKernelGGL(cv_gemm1_kernel<2>, grid, block, 0, st, g);
+    else hipLaunchKernelGGL(cv_gemm1_kernel<4>, grid, block, 0, st, g);
+  } else {
+    if (g.tt == 1) hipLaunchKernelGGL(cv_gemm_kernel<1>, grid, block, 0, st, g);
+    else if (g.tt == 2) hipLaunchKernelGGL(cv_gemm_kernel<2>, grid, block, 0, st, g);
+    else hipLaunchKernelGGL(cv_gemm_kernel<4>, grid, block, 0, st, g);
+  }
   return VUI_OK;
 }
 
@@ -933,10 +1405,19 @@ int vui_codec_decode_frame(vui_codec* c, const int64_t* codes, int32_t n_q, floa
   if (!codes || !audio_out) { vui_set_error("NULL argument"); return VUI_EINVAL; }
   if (n_q < 1 || n_q > c->cfg.n_codebooks) { vui_set_error("n_q=%d outside [1,%d]", n_q, c->cfg.n_codebooks); return VUI_EINVAL; }
   hipStream_t st = (hipStream_t)stream;
-  CvVq vq = c->vq;
-  vq.codes = codes; vq.n_q = n_q;
-  hipLaunchKernelGGL(cv_vq_kernel, dim3(1), dim3(256), 0, st, vq);
-  for (const Step& s : c->steps) {
+  size_t first = 0;
+  if (c->use_trunk && c->trunk_wgs > 0) {
+    CvTrunk tk = c->trunk;
+    tk.codes = codes; tk.n_q = n_q;
+    hipLaunchKernelGGL(cv_trunk_kernel, dim3(c->trunk_wgs), dim3(FR_THREADS), c->trunk_lds, st, tk);
+    first = (size_t)c->trunk_steps;
+  } else {
+    CvVq vq = c->vq;
+    vq.codes = codes; vq.n_q = n_q;
+    hipLaunchKernelGGL(cv_vq_kernel, dim3(1), dim3(256), 0, st, vq);
+  }
+  for (size_t si = first; si < c->steps.size(); ++si) {
+    const Step& s = c->steps[si];
     if (s.kind == 0) {
       int rc = launch_cv_gemm(s.g, st);
       if (rc) return rc;
