@@ -97,9 +97,12 @@ __device__ __forceinline__ void cv_gemm_tile(const CvGemm& p, const int m0, cons
   const int r16 = lane & 15, g = lane >> 4;
   const int G = p.Cin >> 5, Uall = p.taps * G;
   const int M = p.M, Cin = p.Cin;
-  // this workgroup's share of the units: [ub, U)
+  // this workgroup's share of the units, and in it this wave's contiguous run [ub, U): a wave walks along
+  // its 16 weight rows, 128 bytes of each per unit
   const int per = (Uall + p.splits - 1) / p.splits;
-  const int ub = part_idx * per, U = min(Uall, ub + per);
+  const int wb = part_idx * per, we = min(Uall, wb + per);
+  const int per_wave = (we - wb + CV_NW - 1) / CV_NW;
+  const int ub = min(we, wb + wave * per_wave), U = min(we, ub + per_wave);
 
   float4 a0[NU][2], a1[DB ? NU : 1][2];
   float b0[NU][TT][8], b1[DB ? NU : 1][TT][8];
@@ -112,7 +115,7 @@ __device__ __forceinline__ void cv_gemm_tile(const CvGemm& p, const int m0, cons
   auto load_a = [&](int u0, auto& a) {
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
-      const int u = u0 + i * CV_NW;
+      const int u = u0 + i;
       const bool on = u < U;
       const int tap = on ? u / G : 0, grp = on ? u - tap * G : 0;
       const float* wp = p.W + ((size_t)tap * M + m0 + r16) * Cin + grp * 32 + g * 8;
@@ -124,7 +127,7 @@ __device__ __forceinline__ void cv_gemm_tile(const CvGemm& p, const int m0, cons
   auto load_b = [&](int u0, auto& b) {
 #pragma unroll
     for (int i = 0; i < NU; ++i) {
-      const int u = u0 + i * CV_NW;
+      const int u = u0 + i;
       const bool on = u < U;
       const int tap = on ? u / G : 0, grp = on ? u - tap * G : 0;
       const int ci0 = grp * 32 + g * 8;
@@ -151,11 +154,11 @@ __device__ __forceinline__ void cv_gemm_tile(const CvGemm& p, const int m0, cons
     }
   };
 
-  constexpr int STEP = NU * CV_NW;
-  load_a(ub + wave, a0);
+  constexpr int STEP = NU;
+  load_a(ub, a0);
   const int f = *p.ctr - 1;
   ib_ = ring_base(p.in, f);
-  load_b(ub + wave, b0);
+  load_b(ub, b0);
   // what the epilogue adds is requested now as well
   const int rb = ring_base(p.res, f), ob = ring_base(p.out_raw, f), ab = ring_base(p.out_act, f);
   float e_bias[4] = {0.f, 0.f, 0.f, 0.f}, e_res[4] = {0.f, 0.f, 0.f, 0.f}, e_sc[4] = {1.f, 1.f, 1.f, 1.f};
@@ -187,7 +190,7 @@ __device__ __forceinline__ void cv_gemm_tile(const CvGemm& p, const int m0, cons
     rstd = 1.0f / sqrtf(ss / (float)Cin + p.eps);
   }
   if constexpr (DB) {
-    for (int u0 = ub + wave; u0 < U; u0 += 2 * STEP) {
+    for (int u0 = ub; u0 < U; u0 += 2 * STEP) {
       if (u0 + STEP < U) load(u0 + STEP, a1, b1);
       mma(a0, b0);
       if (u0 + STEP < U) {
@@ -196,8 +199,8 @@ __device__ __forceinline__ void cv_gemm_tile(const CvGemm& p, const int m0, cons
       }
     }
   } else {
-    for (int u0 = ub + wave; u0 < U; u0 += STEP) {
-      if (u0 != ub + wave) load(u0, a0, b0);
+    for (int u0 = ub; u0 < U; u0 += STEP) {
+      if (u0 != ub) load(u0, a0, b0);
       mma(a0, b0);
     }
   }
@@ -836,11 +839,13 @@ struct CvFinal {
 };
 
 __global__ __launch_bounds__(256) void cv_final_kernel(const CvFinal p) {
-  extern __shared__ float xs[];  // C x (64 + k - 1) window of the ring, then 4 x 64 partial sums
+  extern __shared__ float xs[];  // C x (64 + k - 1) window of the ring | 4 x 64 partial sums | C x k weights
   const int tid = threadIdx.x, qd = tid >> 6, l = tid & 63;
   const int t0 = blockIdx.x * 64, W = 64 + p.k - 1;
-  const int f = *p.ctr - 1, base = ring_base(p.in, f);
   const int n = p.C * W;
+  float* ws = xs + n + 256;
+  for (int i = tid; i < p.C * p.k; i += 256) ws[i] = p.w[i];
+  const int f = *p.ctr - 1, base = ring_base(p.in, f);
   for (int i0 = tid; i0 < n; i0 += 256 * 8) {
     float v[8];
 #pragma unroll
@@ -855,7 +860,7 @@ __global__ __launch_bounds__(256) void cv_final_kernel(const CvFinal p) {
   float a = 0.f;
   const int c0 = (p.C * qd) / 4, c1 = (p.C * (qd + 1)) / 4;
   for (int c = c0; c < c1; ++c)
-    for (int k = 0; k < p.k; ++k) a = fmaf(p.w[c * p.k + k], xs[c * W + l + k], a);
+    for (int k = 0; k < p.k; ++k) a = fmaf(ws[c * p.k + k], xs[c * W + l + k], a);
   float* part = xs + n;
   part[qd * 64 + l] = a;
   __syncthreads();
@@ -1035,9 +1040,10 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
   };
   int* ctr = (int*)ar.take(64);
   // launch-shape targets (overridable for tuning runs)
-  const char* e1 = getenv("VUI_CV_TILES_MIN");
+  const char* e1 = getenv("VUI_CV_TT");
   const char* e2 = getenv("VUI_CV_WG_TARGET");
-  const int tiles_min = e1 ? atoi(e1) : 200, wg_target = e2 ? atoi(e2) : 768;
+  const char* e3 = getenv("VUI_CV_WG_TARGET2");
+  const int tt_force = e1 ? atoi(e1) : 0, wg_target = e2 ? atoi(e2) : 512, wg_target2 = e3 ? atoi(e3) : 200;
   // meeting place of split tiles: sized by a first pass (the sizes do not depend on the pointers)
   size_t part_floats = 0, cnt_ints = 0;
   float* part = ar.take(part_cap);
@@ -1048,14 +1054,20 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
     g.W = W; g.bias = bias; g.M = M; g.Cin = Cin; g.taps = taps; g.dil = dil; g.T = T; g.bias_div = 1;
     g.in = in; g.in_mode = IN_PLAIN; g.eps = 1e-6f; g.epi = EPI_NONE;
     g.res = no_ring(); g.out_raw = no_ring(); g.out_act = no_ring(); g.ctr = ctr;
-    // the widest tile that still gives ~200 workgroups; then workgroups share a tile's units until ~768
-    // are in flight, as long as every wave keeps at least four units
+    // Tile width: the one that pads the columns least, the wider one on a tie (a wave reuses its weight
+    // registers for every 16-column block).  Then workgroups share a tile's units until about 512 (one
+    // column block: the layer streams weights) or 200 (wider: the layer computes) are in flight, each wave
+    // keeping at least four units.  Measured per layer shape on MI355X.
     const int U = taps * (Cin / 32);
     auto tiles = [&](int tt) { return (M / 16) * ((T + 16 * tt - 1) / (16 * tt)); };
-    g.tt = (T > 32 && tiles(4) >= tiles_min) ? 4 : ((T > 16 && tiles(2) >= tiles_min) ? 2 : 1);
+    g.tt = 1;
+    for (int tt : {2, 4})
+      if (T > 8 * tt && tiles(tt) * tt <= tiles(g.tt) * g.tt) g.tt = tt;
+    if (tt_force > 0 && T > 8 * tt_force) g.tt = tt_force;
     int sp = 1;
     if (U >= 64) {
-      sp = (wg_target + tiles(g.tt) - 1) / tiles(g.tt);
+      const int target = g.tt == 1 ? wg_target : wg_target2;
+      sp = (2 * target + tiles(g.tt)) / (2 * tiles(g.tt));  // rounded
       if (sp > U / 16) sp = U / 16;
       if (sp > 8) sp = 8;
       if (sp < 1) sp = 1;
@@ -1430,7 +1442,7 @@ int vui_codec_decode_frame(vui_codec* c, const int64_t* codes, int32_t n_q, floa
   }
   CvFinal fin = c->fin;
   fin.audio = audio_out;
-  hipLaunchKernelGGL(cv_final_kernel, dim3((fin.T + 63) / 64), dim3(256), (size_t)(fin.C * (64 + fin.k - 1) + 256) * 4, st, fin);
+  hipLaunchKernelGGL(cv_final_kernel, dim3((fin.T + 63) / 64), dim3(256), (size_t)(fin.C * (64 + fin.k - 1) + 256 + fin.C * fin.k) * 4, st, fin);
   HIP_TRY(hipGetLastError());
   return VUI_OK;
 }
