@@ -105,6 +105,10 @@ def test_rope(lib, dt, hd, rope_dim):
     (4, 2, 16, 64, [0, 5, 63], 3, 0),
     (4, 2, 16, 64, [40, 5, 63], 2, 7),
     (8, 8, 96, 512, [300], 1, 0),
+    # many rows, many pieces, short and empty pieces
+    (8, 8, 96, 2304, [127, 2047, 600, 1, 0, 999, 1500, 64], 32, 0),
+    (4, 4, 16, 256, [0, 5, 63, 255, 100, 31, 32, 33], 32, 0),
+    (2, 2, 32, 256, [200, 5, 63, 255, 100, 31, 32, 33], 64, 50),
 ])
 def test_decode_attn(lib, dt, H, KV, hd, S, lens, splits, window):
     """Append + attention over ragged lengths with slot indirection, against the textbook softmax."""

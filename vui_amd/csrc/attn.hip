@@ -3,11 +3,13 @@
 //
 // Backbone: caches are (slots, S, KV, hd); the key range [start, len) of a (row, head) is cut
 // into n_splits contiguous pieces, one workgroup each.  A group of 16 lanes owns one key
-// (8 features per lane, 16-byte loads), so a 256-thread workgroup works on 16 keys at a time.
-// Scores of the piece go to LDS, the piece maximum is taken over the workgroup, then
-// exp-weights multiply V.  Each piece writes (max, sum, acc[hd]); a second small kernel merges the
-// pieces of each (row, head) (a kernel boundary is cheaper here than device-scope fences in 256
-// workgroups, which cost ~40 us per launch on the eight non-coherent L2s).
+// (8 features per lane, 16-byte loads), so a 256-thread workgroup works on 16 keys at a time, and
+// every group has four keys AND their values in flight per step: one pass with a running maximum
+// (scores never go to memory).  The 16 groups are merged through LDS into the piece's
+// (max, sum, acc[hd]).  Pieces of a (row, head) meet in memory: each workgroup writes its piece with
+// device-scope write-through stores, waits for them to complete and bumps an arrival counter; the
+// last arriver merges all pieces in piece order and writes the output (and zeroes the counter for
+// the next launch).  No second kernel, no cache flush.
 //
 // Reference: flash_attn_with_kvcache call in MHA.forward_flash, src/vui/model.py:242-258
 // (causal, one query at position seq_len; window (w, 0)); F.scaled_dot_product_attention in
@@ -19,11 +21,11 @@
 #define ATT_KEYS_PER_ITER 16  // 4 waves x 4 lane-groups
 
 template <typename T>
-__global__ __launch_bounds__(ATT_THREADS) void decode_attn_kernel(const AttnArgs p, const int max_chunk) {
-  extern __shared__ float sc[];  // max_chunk scores
-  __shared__ float red[ATT_KEYS_PER_ITER];
-  __shared__ float accs[4][4][128];
-  __shared__ float lsum[ATT_KEYS_PER_ITER];
+__global__ __launch_bounds__(ATT_THREADS) void decode_attn_kernel(const AttnArgs p) {
+  __shared__ float gm[ATT_KEYS_PER_ITER], gl[ATT_KEYS_PER_ITER], gw[ATT_KEYS_PER_ITER];
+  __shared__ float gacc[ATT_KEYS_PER_ITER][128];
+  __shared__ __align__(8) float fin[130];  // max, sum, acc[hd]
+  __shared__ int s_last;
 
   const int b = blockIdx.z, h = blockIdx.y, sp = blockIdx.x;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, grp = lane >> 4, l16 = lane & 15;
@@ -36,7 +38,6 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attn_kernel(const AttnArgs
   const int n = len - start;
   int chunk = (n + p.n_splits - 1) / p.n_splits;
   chunk = (chunk + ATT_KEYS_PER_ITER - 1) / ATT_KEYS_PER_ITER * ATT_KEYS_PER_ITER;
-  chunk = min(chunk, max_chunk);
   const int lo = start + sp * chunk;
   const int hi = min(lo + chunk, len);
   const int kvh = h / (p.H / p.KV);
@@ -52,103 +53,122 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attn_kernel(const AttnArgs
   const T* kbase = (const T*)p.kc + ((size_t)slot * p.S) * rowstride + kvh * hd + l16 * 8;
   const T* vbase = (const T*)p.vc + ((size_t)slot * p.S) * rowstride + kvh * hd + l16 * 8;
 
-  // pass 1: scores (four keys per lane group in flight)
-  float mloc = -INFINITY;
-  for (int j0 = lo + g; j0 < hi; j0 += 4 * ATT_KEYS_PER_ITER) {
-    float k8[4][8];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int j = j0 + u * ATT_KEYS_PER_ITER;
-      if (act && j < hi) El<T>::ld8(kbase + (size_t)j * rowstride, k8[u]);
-    }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int j = j0 + u * ATT_KEYS_PER_ITER;
-      if (j < hi) {
-        float d = 0.f;
-        if (act) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) d = fmaf(q8[e], k8[u][e], d);
-        }
-        d = group16_sum(d) * scale;
-        if (l16 == 0) sc[j - lo] = d;
-        mloc = fmaxf(mloc, d);
-      }
-    }
-  }
-  if (l16 == 0) red[g] = mloc;
-  __syncthreads();
-  float M = -INFINITY;
-#pragma unroll
-  for (int i = 0; i < ATT_KEYS_PER_ITER; ++i) M = fmaxf(M, red[i]);
-
-  // pass 2: weights and P.V
-  float acc[8];
+  float m = -INFINITY, l = 0.f, acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-  float l = 0.f;
   for (int j0 = lo + g; j0 < hi; j0 += 4 * ATT_KEYS_PER_ITER) {
-    float v8[4][8];
+    float k8[4][8], v8[4][8];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int j = j0 + u * ATT_KEYS_PER_ITER;
-      if (act && j < hi) El<T>::ld8(vbase + (size_t)j * rowstride, v8[u]);
-    }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int j = j0 + u * ATT_KEYS_PER_ITER;
-      if (j < hi) {
-        const float pw = expf(sc[j - lo] - M);
-        l += pw;
-        if (act) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) acc[e] = fmaf(pw, v8[u][e], acc[e]);
-        }
+      for (int e = 0; e < 8; ++e) { k8[u][e] = 0.f; v8[u][e] = 0.f; }
+      if (act && j < hi) {
+        El<T>::ld8(kbase + (size_t)j * rowstride, k8[u]);
+        El<T>::ld8(vbase + (size_t)j * rowstride, v8[u]);
       }
     }
+    float s[4];
+    float mn = m;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      float d = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) d = fmaf(q8[e], k8[u][e], d);
+      d = group16_sum(d) * scale;
+      s[u] = (j0 + u * ATT_KEYS_PER_ITER < hi) ? d : -INFINITY;
+      mn = fmaxf(mn, s[u]);
+    }
+    // j0 < hi: at least one of the four keys is real, so mn is finite
+    const float r = expf(m - mn);  // 0 on the first step (m = -inf)
+    l *= r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] *= r;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float pw = expf(s[u] - mn);  // 0 for a key beyond the piece
+      l += pw;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = fmaf(pw, v8[u][e], acc[e]);
+    }
+    m = mn;
   }
+  // the 16 groups of the workgroup -> one piece
+  if (l16 == 0) { gm[g] = m; gl[g] = l; }
   if (act) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) accs[wave][grp][l16 * 8 + e] = acc[e];
+    for (int e = 0; e < 8; ++e) gacc[g][l16 * 8 + e] = acc[e];
   }
-  if (l16 == 0) lsum[g] = l;
+  __syncthreads();
+  if (tid < ATT_KEYS_PER_ITER) {
+    float M = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < ATT_KEYS_PER_ITER; ++i) M = fmaxf(M, gm[i]);
+    gw[tid] = (gm[tid] == -INFINITY) ? 0.f : expf(gm[tid] - M);
+    if (tid == 0) fin[0] = M;
+  }
+  __syncthreads();
+  if (tid < hd) {
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < ATT_KEYS_PER_ITER; ++i) o = fmaf(gw[i], gacc[i][tid], o);
+    fin[2 + tid] = o;
+  }
+  if (tid == 128) {
+    float L = 0.f;
+#pragma unroll
+    for (int i = 0; i < ATT_KEYS_PER_ITER; ++i) L = fmaf(gw[i], gl[i], L);
+    fin[1] = L;
+  }
   __syncthreads();
 
-  float* part = p.part + (((size_t)b * p.H + h) * p.n_splits + sp) * (hd + 2);
-  if (tid < hd) {
-    float s = 0.f;
-#pragma unroll
-    for (int w = 0; w < 4; ++w)
-#pragma unroll
-      for (int gg = 0; gg < 4; ++gg) s += accs[w][gg][tid];
-    part[2 + tid] = s;
+  const int pw_ = hd + 2;  // floats per piece (even: hd is a multiple of 8)
+  float* pbase = p.part + (((size_t)b * p.H + h) * p.n_splits) * pw_;
+  if (p.n_splits > 1) {
+    if (tid < pw_ / 2) st_dev(pbase + (size_t)sp * pw_ + 2 * tid, fin[2 * tid], fin[2 * tid + 1]);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the write-through stores have completed
+    __syncthreads();
+    if (tid == 0) {
+      uint32_t* cnt = p.counter + (size_t)b * p.H + h;
+      const uint32_t old = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = old == (uint32_t)p.n_splits - 1u;
+      if (s_last) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!s_last) return;
   }
-  if (tid == 0) {
-    float s = 0.f;
+  // merge of the pieces: out = sum_s w_s acc_s / sum_s w_s l_s, w_s = exp(m_s - max m), in piece order.
+  // All pieces are fetched into LDS with one round of loads (a chain of dependent device-scope loads
+  // would cost a memory round trip each).
+  extern __shared__ __align__(8) float pieces[];  // n_splits x (hd + 2)
+  if (p.n_splits > 1) {
+    const int np = p.n_splits * pw_ / 2;
+    for (int i0 = tid; i0 < np; i0 += ATT_THREADS * 8) {
+      uint64_t v[8];
 #pragma unroll
-    for (int i = 0; i < ATT_KEYS_PER_ITER; ++i) s += lsum[i];
-    part[0] = M;
-    part[1] = s;
+      for (int u = 0; u < 8; ++u) { const int i = i0 + ATT_THREADS * u; v[u] = i < np ? ld_dev(pbase + 2 * i) : 0; }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = i0 + ATT_THREADS * u;
+        if (i < np) { pieces[2 * i] = lo_f(v[u]); pieces[2 * i + 1] = hi_f(v[u]); }
+      }
+    }
+    __syncthreads();
   }
-
-}
-
-// merge of the pieces of one (row, head): out = sum_s w_s acc_s / sum_s w_s l_s, w_s = exp(m_s - max m)
-template <typename T>
-__global__ __launch_bounds__(128) void attn_merge_kernel(const AttnArgs p) {
-  const int b = blockIdx.y, h = blockIdx.x, tid = threadIdx.x;
-  const int hd = p.hd;
-  const float* pb = p.part + (((size_t)b * p.H + h) * p.n_splits) * (hd + 2);
   if (tid < hd) {
-    float Mx = -INFINITY;
-    for (int s = 0; s < p.n_splits; ++s) Mx = fmaxf(Mx, pb[(size_t)s * (hd + 2)]);
-    float L = 0.f, o = 0.f;
-    for (int s = 0; s < p.n_splits; ++s) {
-      const float* ps = pb + (size_t)s * (hd + 2);
-      const float ms = ps[0];
-      const float w = (ms == -INFINITY) ? 0.f : expf(ms - Mx);
-      L = fmaf(w, ps[1], L);
-      o = fmaf(w, ps[2 + tid], o);
+    float o, L;
+    if (p.n_splits > 1) {
+      float Mx = -INFINITY;
+      for (int s0 = 0; s0 < p.n_splits; ++s0) Mx = fmaxf(Mx, pieces[s0 * pw_]);
+      o = 0.f; L = 0.f;
+      for (int s0 = 0; s0 < p.n_splits; ++s0) {
+        const float ms = pieces[s0 * pw_];
+        const float w = (ms == -INFINITY) ? 0.f : expf(ms - Mx);
+        L = fmaf(w, pieces[s0 * pw_ + 1], L);
+        o = fmaf(w, pieces[s0 * pw_ + 2 + tid], o);
+      }
+    } else {
+      o = fin[2 + tid]; L = fin[1];
     }
     El<T>::st((T*)p.out + (size_t)b * p.H * hd + h * hd + tid, o / L);
   }
@@ -159,21 +179,11 @@ int launch_decode_attn(const AttnArgs& a, hipStream_t st) {
     vui_set_error("decode_attn: unsupported shape hd=%d H=%d KV=%d splits=%d", a.hd, a.H, a.KV, a.n_splits);
     return VUI_EINVAL;
   }
-  int max_chunk = (a.S + a.n_splits - 1) / a.n_splits;
-  max_chunk = (max_chunk + ATT_KEYS_PER_ITER - 1) / ATT_KEYS_PER_ITER * ATT_KEYS_PER_ITER;
-  if ((size_t)max_chunk * 4 > 60000) {
-    vui_set_error("decode_attn: S=%d needs more than %d key splits", a.S, a.n_splits);
-    return VUI_EINVAL;
-  }
+  if (a.n_splits > 1 && (!a.part || !a.counter)) { vui_set_error("decode_attn: split pieces need scratch"); return VUI_EINVAL; }
   dim3 grid(a.n_splits, a.H, a.B);
-  dim3 mgrid(a.H, a.B);
-  if (a.dtype == VUI_DTYPE_F32) {
-    hipLaunchKernelGGL(decode_attn_kernel<float>, grid, dim3(ATT_THREADS), max_chunk * 4, st, a, max_chunk);
-    hipLaunchKernelGGL(attn_merge_kernel<float>, mgrid, dim3(128), 0, st, a);
-  } else {
-    hipLaunchKernelGGL(decode_attn_kernel<bf16_t>, grid, dim3(ATT_THREADS), max_chunk * 4, st, a, max_chunk);
-    hipLaunchKernelGGL(attn_merge_kernel<bf16_t>, mgrid, dim3(128), 0, st, a);
-  }
+  const size_t lds = a.n_splits > 1 ? (size_t)a.n_splits * (a.hd + 2) * 4 : 0;  // the pieces, for the last arriver
+  if (a.dtype == VUI_DTYPE_F32) hipLaunchKernelGGL(decode_attn_kernel<float>, grid, dim3(ATT_THREADS), lds, st, a);
+  else hipLaunchKernelGGL(decode_attn_kernel<bf16_t>, grid, dim3(ATT_THREADS), lds, st, a);
   HIP_TRY(hipGetLastError());
   return VUI_OK;
 }

@@ -72,15 +72,6 @@ struct CvGemm {
   int tt;          // 16-column blocks per tile (host side: picks the instantiation)
 };
 
-// device-scope relaxed accesses: they bypass the per-XCD L2s, so another workgroup's value is seen
-__device__ __forceinline__ void st_dev(float* p, float a, float b) {
-  __hip_atomic_store(reinterpret_cast<uint64_t*>(p), ((uint64_t)__float_as_uint(b) << 32) | __float_as_uint(a),
-                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ uint64_t ld_dev(const float* p) {
-  return __hip_atomic_load(reinterpret_cast<const uint64_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 // units a wave keeps in registers per round: NU * (8 + 8*TT) VGPRs, twice that when the rounds are
 // double-buffered (DB: for tiles whose waves need several rounds; one wave per SIMD).  Tiles that fit one
 // round use the single-buffered form, which leaves room for two or three waves per SIMD.

@@ -193,3 +193,17 @@ __device__ __forceinline__ float rope_mix(float a, float c, float b, float s) {
 }
 
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
+
+// ---- values that workgroups of one launch hand to each other ----
+// Device-scope relaxed accesses bypass the per-XCD L2s (write-through stores, loads served from memory), so
+// another workgroup's value is seen without a cache flush.  After such stores `s_waitcnt vmcnt(0)` means
+// they have completed; a counter incremented afterwards tells the last arriver that everything is there.
+__device__ __forceinline__ void st_dev(float* p, float a, float b) {
+  __hip_atomic_store(reinterpret_cast<uint64_t*>(p), ((uint64_t)__float_as_uint(b) << 32) | __float_as_uint(a),
+                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t ld_dev(const float* p) {
+  return __hip_atomic_load(reinterpret_cast<const uint64_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float lo_f(uint64_t v) { return __uint_as_float((uint32_t)v); }
+__device__ __forceinline__ float hi_f(uint64_t v) { return __uint_as_float((uint32_t)(v >> 32)); }

@@ -287,11 +287,10 @@ class Decoder:
             _lib.ptr(eos_out), n_splits, stream), "vui_backbone_step")
 
     def default_splits(self, B: int) -> int:
-        """Key-range splits per (row, head): enough workgroups to keep every CU streaming keys (about
-        2048 over the whole launch, measured best on 16 ragged rows of 128..2048 keys), at most 32 per
-        (row, head)."""
+        """Key-range pieces per (row, head): about 1024 workgroups over the launch (measured on 16 ragged
+        rows of 128..2048 keys), at most 32 pieces."""
         H = self._model.config.model.n_heads
-        return max(1, min(32, 2048 // max(1, B * H)))
+        return max(1, min(32, 1024 // max(1, B * H)))
 
     def forward_flash(self, x: Tensor, positions: Tensor, per_sample_positions: bool = False,
                       slot_idx: Tensor | None = None) -> Tensor:
