@@ -155,6 +155,65 @@ def vocoder_line():
                  "hbm_frac": round(cb / us / 1e3 / HBM_PEAK_GBS, 4)}
 
 
+def b16_line(sd, preset="A", n=100):
+    """Config 5: 16 streams, int8 backbone weights, ragged caches U[128, 2048] filled N(0, 1), n frame steps
+    from one captured graph (backbone kernel sequence + persistent depth head)."""
+    import torch
+
+    from vui_amd.engine import Engine, GenConfig
+    from vui_amd.model import Vui
+    from vui_amd.synthetic import nano_for_cache
+
+    S = 2048 + 256
+    model5 = Vui(nano_for_cache(preset, S), sd, device="cuda", dtype=torch.bfloat16, int8=True)
+    m = model5.config.model
+    eng5 = Engine(model=model5, max_rows=16, max_seq=S)
+    model5.decoder._k.normal_()
+    model5.decoder._v.normal_()
+    g = torch.Generator().manual_seed(5)
+    lens = torch.randint(128, 2049, (16,), generator=g)
+    rows = [eng5.new_row() for _ in range(16)]
+    eng5.seq_lens[:16] = lens.to(torch.int32).cuda()
+    hid16 = torch.randn(16, m.d_model, generator=g).to(torch.bfloat16).cuda()
+    eng5.generate(rows, hid16, 1, GenConfig())
+    gr5, _, _, _ = eng5._frame_graph(16, GenConfig(), None, n + 4)
+    eng5.seq_lens[:16] = lens.to(torch.int32).cuda()
+    for _ in range(3):
+        gr5.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(n):
+        gr5.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / n
+    kv_bytes = float((lens.float() + 3 + n / 2 + 1).sum()) * 2 * m.kv_heads * m.head_dim * 2 * m.n_layers
+    wbytes = frame_bytes(m, 0, 1)["backbone"] - (m.n_quantizers * m.d_model + 2 * m.kv_heads * m.head_dim * 2 * m.n_layers)
+    return {"config": "e2e_b16_int8_ragged", "us_per_frame_step": round(us, 1), "aggregate_frames_per_s": round(16e6 / us, 1),
+            "kv_bytes": int(kv_bytes), "int8_weight_bytes": int(wbytes), "achieved_GBs": round((kv_bytes + wbytes) / us / 1e3, 1)}
+
+
+def copy_line():
+    """The practical bandwidth ceiling of the box: a plain 1 GiB device-to-device copy (reads + writes)."""
+    import torch
+
+    src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_(0, 255)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(10):
+        dst.copy_(src)
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / 10
+    return {"config": "device_copy_1GiB", "us": round(us, 1), "read_plus_write_GBs": round(2 * (1 << 30) / us / 1e3, 1),
+            "frac_of_8TBs": round(2 * (1 << 30) / us / 1e3 / HBM_PEAK_GBS, 3)}
+
+
 def suite(model, eng, d, sd, preset="A"):
     """Extra lines for the other benchmark configs: backbone step at KV 256/1024/4096, depth head alone,
     16 int8 streams with ragged caches."""
@@ -257,26 +316,8 @@ def suite(model, eng, d, sd, preset="A"):
     lines.append({"config": "stream_b1_audio", "frames": n_out, "chunks": 4, "ms_per_frame_wall": round(dt * 1e3 / n_out, 4),
                   "frames_per_s": round(n_out / dt, 1), "rtf": round(n_out / dt / 12.5, 2)})
     del eng2, model2, voc
-    # config 5: 16 streams, int8 backbone weights, ragged caches U[128, 2048]
-    S = 2048 + 256
-    model5 = Vui(nano_for_cache(preset, S), sd, device="cuda", dtype=torch.bfloat16, int8=True)
-    eng5 = Engine(model=model5, max_rows=16, max_seq=S)
-    model5.decoder._k.normal_()
-    model5.decoder._v.normal_()
-    lens = torch.randint(128, 2049, (16,), generator=g)
-    rows = [eng5.new_row() for _ in range(16)]
-    eng5.seq_lens[:16] = lens.to(torch.int32).cuda()
-    hid16 = torch.randn(16, m.d_model, generator=g).to(torch.bfloat16).cuda()
-    n = 100
-    eng5.generate(rows, hid16, 1, GenConfig())
-    gr5, _, _, _ = eng5._frame_graph(16, GenConfig(), None, n + 1)
-    eng5.seq_lens[:16] = lens.to(torch.int32).cuda()
-    us = timed(gr5.replay, n)
-    kv_bytes = float((lens.float() + n / 2 + 1).sum()) * 2 * m.kv_heads * m.head_dim * 2 * m.n_layers
-    wbytes = frame_bytes(m, 0, 1)["backbone"] - (m.n_quantizers * m.d_model + 2 * m.kv_heads * m.head_dim * 2 * m.n_layers)
-    lines.append({"config": "e2e_b16_int8_ragged", "us_per_frame_step": round(us, 1), "aggregate_frames_per_s": round(16e6 / us, 1),
-                  "kv_bytes": int(kv_bytes), "int8_weight_bytes": int(wbytes),
-                  "achieved_GBs": round((kv_bytes + wbytes) / us / 1e3, 1)})
+    lines.append(b16_line(sd, preset))
+    lines.append(copy_line())
     return lines
 
 
@@ -316,6 +357,8 @@ def main():
     ap.add_argument("--suite", action="store_true", help="also print one JSON line per further benchmark config")
     ap.add_argument("--calib", action="store_true",
                     help="end with three plain 512 MiB device copies (reference points for hardware counters)")
+    ap.add_argument("--b16-only", action="store_true",
+                    help="print only the 16-stream int8 line (the run its rocprofv3 summaries come from)")
     ap.add_argument("--vocoder-only", action="store_true",
                     help="print only the vocoder line (the run rocprofv3 summaries of the vocoder kernels come from)")
     args = ap.parse_args()
@@ -325,6 +368,12 @@ def main():
         sys.exit(2)
     if args.vocoder_only:
         print(json.dumps(vocoder_line()[1]))
+        return
+    if args.b16_only:
+        from vui_amd.synthetic import nano_for_cache, synthetic_state_dict
+
+        n = args.steps if args.steps != 750 else 100  # --steps shortens the run for counter collection
+        print(json.dumps(b16_line(synthetic_state_dict(nano_for_cache(args.preset, 64).model, seed=0), args.preset, n)))
         return
     out, (model, eng, d, sd) = gpu_bench(args)
     if not args.no_roofline:
