@@ -194,6 +194,39 @@ def b16_line(sd, preset="A", n=100):
             "kv_bytes": int(kv_bytes), "int8_weight_bytes": int(wbytes), "achieved_GBs": round((kv_bytes + wbytes) / us / 1e3, 1)}
 
 
+def serve_line(sd, preset="A", n_requests=32, max_rows=16):
+    """Continuous batching as a served workload (Engine.render_continuous): n_requests requests, each a
+    256-position prompt and two text chunks of 16 positions / 5 words, through max_rows rows (bf16); EOS off,
+    so every chunk runs to its 40-frame cap.  Wall clock includes prompt ingestion, the host loop, the
+    per-step EOS read and the refills."""
+    import torch
+
+    from vui_amd.engine import Chunk, Engine, GenConfig, RenderRequest
+    from vui_amd.model import Vui
+    from vui_amd.synthetic import nano_for_cache
+
+    S = 512
+    model = Vui(nano_for_cache(preset, S), sd, device="cuda", dtype=torch.bfloat16)
+    m = model.config.model
+    eng = Engine(model=model, max_rows=max_rows, max_seq=S)
+    g = torch.Generator().manual_seed(9)
+
+    def emb(n):
+        return (torch.randn(1, n, m.d_model, generator=g) * 0.08).to(torch.bfloat16).cuda()
+
+    reqs = [RenderRequest(chunks=[Chunk(emb=emb(16), n_words=5) for _ in range(2)], prompt_emb=emb(256)) for _ in range(n_requests)]
+    cfg = GenConfig(eos_threshold=2.0)
+    eng.render_continuous(reqs[:max_rows + 1], cfg)  # warm: graph capture for every bucket on the way down
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    out = eng.render_continuous(reqs, cfg)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    n_frames = sum(len(o) for o in out)
+    return {"config": "continuous_batching_b16", "requests": n_requests, "rows": max_rows, "frames": n_frames,
+            "wall_s": round(dt, 3), "aggregate_frames_per_s": round(n_frames / dt, 1), "rtf_aggregate": round(n_frames / dt / 12.5, 1)}
+
+
 def copy_line():
     """The practical bandwidth ceiling of the box: a plain 1 GiB device-to-device copy (reads + writes)."""
     import torch
@@ -317,6 +350,7 @@ def suite(model, eng, d, sd, preset="A"):
                   "frames_per_s": round(n_out / dt, 1), "rtf": round(n_out / dt / 12.5, 2)})
     del eng2, model2, voc
     lines.append(b16_line(sd, preset))
+    lines.append(serve_line(sd, preset))
     lines.append(copy_line())
     return lines
 

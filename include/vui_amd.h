@@ -152,6 +152,9 @@ typedef struct vui_sample_params {
   int32_t top_k;          /* 1 = greedy (lowest index of the maximum), <= 0 = no truncation */
   uint64_t seed;
   const int32_t* frame_ctr; /* device (1) int32 frame number, or NULL for frame 0 */
+  const int32_t* state_rows; /* device (B) int32 or NULL: row b of a code-0 call uses the repetition state and the
+                                random-stream row of state_rows[b] (continuous batching: the physical slot,
+                                Engine._rep_apply_slots / _rep_push_slots, engine.py:594-616) */
 } vui_sample_params;
 
 /* Code-0 sampler with repetition penalty for B rows:

@@ -726,6 +726,128 @@ def stream_row(model: "OracleModel", chunks, *, temperature: float = 0.9, top_k:
     return out
 
 
+def _get_bucket(n: int, max_rows: int) -> int:
+    """Smallest bucket holding n rows; buckets are the powers of two below max_rows and max_rows itself
+    (engine.py:134-154)."""
+    b = 1
+    while b < n:
+        b *= 2
+    return min(b, max_rows)
+
+
+def render_continuous(model: "OracleModel", requests, *, max_rows: int, temperature: float = 0.9, top_k: int = 100,
+                      rq_top_k: int = 100, rep_penalty: float = 1.1, eos_threshold: float = 0.45,
+                      min_secs: float = 0.5, max_turn_secs: float = 15.0, max_secs: float = 30.0,
+                      n_codebooks: int = 0, max_turn_wps: float = 0.0, seed: int = 0, max_seq: int | None = None,
+                      log: list | None = None) -> list[Tensor]:
+    """Restatement of Engine.render_continuous (engine.py:1112-1302) on the oracle model (n_slots >=
+    max_rows).  requests: list of (prompt_emb (T, d) or None, chunks [(emb (T, d), n_words)], prompt_wps).
+    Returns the frames (T_i, Q') of every request in input order.
+
+    Rules kept from the reference: the queue is served in order into the lowest free slot; a slot's
+    repetition counts start at zero and never age (no window); a chunk's first frame is drawn from the
+    text's last hidden state without top-k (unless greedy); every step draws for all active slots, and a slot
+    whose EOS flag is up after min_secs or whose chunk reached its frame cap drops that step's frame and
+    starts its next chunk; max_secs or the cache limit end the request (that step's frame is dropped too);
+    freed slots are refilled before the next step.  The draw of sampling event e (a chunk start or a
+    step) for slot s uses uniform01(seed, e, s, 0); the depth head of that event uses frame e with rows
+    numbered by position in the sorted slot list.
+    log: receives ("start", request, slot) / ("next", request, chunk) / ("end", request, reason, frames)
+    and ("step", tuple(sorted slots), bucket)."""
+    d = model.dims
+    max_frames = int(max_secs * FRAME_RATE)
+    min_frames = int(min_secs * FRAME_RATE)
+    max_seq = (max_seq if max_seq is not None else d.max_seqlen) - 10
+    greedy = top_k == 1
+    rq_k = 1 if greedy else rq_top_k
+    counts = torch.zeros(max_rows, d.codebook_size)
+    frames: list[list[Tensor]] = [[] for _ in requests]
+    pending = list(range(len(requests)))
+    free = set(range(max_rows))
+    active: dict[int, dict] = {}
+    event = 0
+
+    def draw(cb0_row: Tensor, slot: int, k: int) -> int:
+        c = sample_cb0(cb0_row, counts[slot], rep_penalty, temperature, k, uniform01(seed, event, slot, 0))
+        if rep_penalty > 1.0:
+            counts[slot, c] += 1.0
+        return c
+
+    def advance(info: dict) -> bool:
+        nonlocal event
+        if info["ci"] >= len(info["chunks"]):
+            return False
+        emb, n_words = info["chunks"][info["ci"]]
+        info["max_turn"] = max_turn_frames(n_words, info["wps"], max_turn_secs, max_turn_wps)
+        hidden = model.prefill(emb, info["slot"])[-1:]
+        cb0, _ = model.heads(hidden)
+        c0 = draw(cb0[0], info["slot"], 1 if greedy else 0)
+        info["last"] = model.rq_generate(hidden, torch.tensor([c0]), temperature, rq_k, None, n_codebooks, seed, event)[0]
+        event += 1
+        frames[info["req"]].append(info["last"])
+        info["n"] += 1
+        info["turn"] = 1
+        info["off"] = int(model.seq_lens[info["slot"]])
+        if log is not None:
+            log.append(("next", info["req"], info["ci"]))
+        return True
+
+    def backfill() -> None:
+        while pending and free:
+            ri = pending.pop(0)
+            prompt, chunks, wps = requests[ri]
+            slot = min(free)
+            free.remove(slot)
+            model.seq_lens[slot] = 0
+            counts[slot].zero_()
+            if log is not None:
+                log.append(("start", ri, slot))
+            if prompt is not None and prompt.shape[0] > 0:
+                model.prefill(prompt, slot)
+            info = dict(req=ri, slot=slot, chunks=chunks, wps=wps, ci=0, n=0, turn=0, max_turn=0, off=0, last=None)
+            if not chunks or not advance(info):
+                free.add(slot)
+                continue
+            active[slot] = info
+
+    backfill()
+    while active:
+        slots = sorted(active)
+        if log is not None:
+            log.append(("step", tuple(slots), _get_bucket(len(slots), max_rows)))
+        codes = torch.stack([active[s]["last"] for s in slots])
+        hidden, cb0, eos = model.decode_step(codes, torch.tensor(slots))
+        for s in slots:
+            active[s]["off"] += 1
+        c0 = torch.tensor([draw(cb0[i], s, top_k) for i, s in enumerate(slots)])
+        flags = torch.sigmoid(eos.float()).flatten() > eos_threshold
+        new = model.rq_generate(hidden, c0, temperature, rq_k, None, n_codebooks, seed, event)
+        event += 1
+        gone = []
+        for i, s in enumerate(slots):
+            info = active[s]
+            if info["n"] >= max_frames or info["off"] >= max_seq:
+                gone.append((s, "cap"))
+                continue
+            if (info["turn"] >= min_frames and bool(flags[i])) or info["turn"] >= info["max_turn"]:
+                info["ci"] += 1
+                if not advance(info):
+                    gone.append((s, "done"))
+                continue
+            info["last"] = new[i]
+            frames[info["req"]].append(new[i])
+            info["n"] += 1
+            info["turn"] += 1
+        for s, why in gone:
+            info = active.pop(s)
+            free.add(s)
+            if log is not None:
+                log.append(("end", info["req"], why, info["n"]))
+        backfill()
+    q = n_codebooks if n_codebooks > 0 else d.n_quantizers
+    return [torch.stack(f) if f else torch.zeros(0, q, dtype=torch.long) for f in frames]
+
+
 # --------------------------------------------------------------------------------------
 # deterministic synthetic weights (the benchmark's "random-init N(0, 0.02) from seed 0")
 # --------------------------------------------------------------------------------------

@@ -46,7 +46,7 @@ class WeightsC(C.Structure):
 
 class SampleParamsC(C.Structure):
     _fields_ = [("temperature", C.c_float), ("top_k", C.c_int32), ("seed", C.c_uint64),
-                ("frame_ctr", C.c_void_p)]
+                ("frame_ctr", C.c_void_p), ("state_rows", C.c_void_p)]
 
 
 class CodecConfigC(C.Structure):

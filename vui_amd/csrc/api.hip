@@ -349,6 +349,7 @@ static SampleArgs sample_base(const vui_sample_params* sp) {
   SampleArgs s;
   memset(&s, 0, sizeof(s));
   s.temperature = sp->temperature; s.top_k = sp->top_k; s.seed = sp->seed; s.frame_ctr = sp->frame_ctr;
+  s.state_rows = sp->state_rows;
   return s;
 }
 

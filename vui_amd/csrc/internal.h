@@ -100,6 +100,7 @@ struct SampleArgs {
   int top_k;
   uint64_t seed;
   const int32_t* frame_ctr;
+  const int32_t* state_rows;  // (B) or nullptr: repetition state / random-stream row of row b
   int codebook;  // Philox counter word 2
   int CS, B;
   int64_t* out;  // out[b * out_stride + out_col]

@@ -90,7 +90,8 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const SampleArgs p
   const T* lg = (const T*)p.logits + (size_t)b * CS;
   const bool greedy = (p.top_k == 1) || !(p.temperature > 0.f);
   const float div = greedy ? 1.0f : p.temperature;
-  const float* counts = (p.rep_counts && p.penalty > 1.0f) ? p.rep_counts + (size_t)b * CS : nullptr;
+  const int sb = p.state_rows ? p.state_rows[b] : b;  // row of the repetition state and of the random stream
+  const float* counts = (p.rep_counts && p.penalty > 1.0f) ? p.rep_counts + (size_t)sb * CS : nullptr;
 
   // untouched bf16 logits order the elements with 16-bit keys; bias or penalty need all 32 bits
   const bool raw_keys = sizeof(T) == 2 && !p.bias && !counts;
@@ -108,14 +109,14 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const SampleArgs p
     }
   }
   const uint32_t frame = p.frame_ctr ? (uint32_t)p.frame_ctr[0] : 0u;
-  const int pick = block_sample<EMAX>(l, key, raw_keys ? 16 : 0, CS, E, greedy, p.top_k, p.seed, frame, (uint32_t)b,
+  const int pick = block_sample<EMAX>(l, key, raw_keys ? 16 : 0, CS, E, greedy, p.top_k, p.seed, frame, (uint32_t)sb,
                                       (uint32_t)p.codebook, sh, hist);
 
   if (tid == 0) {
     p.out[(size_t)b * p.out_stride + p.out_col] = (int64_t)pick;
     if (counts)
-      rep_push(p.rep_counts + (size_t)b * CS, p.rep_hist ? p.rep_hist + (size_t)b * p.window : nullptr,
-               p.rep_pos ? p.rep_pos + b * 2 : nullptr, p.window, pick);
+      rep_push(p.rep_counts + (size_t)sb * CS, p.rep_hist ? p.rep_hist + (size_t)sb * p.window : nullptr,
+               p.rep_pos ? p.rep_pos + sb * 2 : nullptr, p.window, pick);
     if (p.eos_prob) {
       const float z = El<T>::ld((const T*)p.eos_logit + b);
       p.eos_prob[b] = 1.0f / (1.0f + expf(-z));

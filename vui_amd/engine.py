@@ -69,6 +69,30 @@ class Chunk:
     sc: bool = False
 
 
+@dataclass
+class RenderRequest:
+    """One request of `Engine.render_continuous` (RenderRequest, src/vui/engine.py:107-117, with the text
+    side already embedded): `prompt_emb` (1, T, d) is what Row.prefill / add_user would have written (voice
+    prompt, user turn), `chunks` the agent text chunk by chunk."""
+
+    chunks: "list[Chunk]"
+    prompt_emb: Tensor | None = None
+    prompt_wps: float = 0.0
+
+
+@dataclass
+class _ActiveSlot:
+    row: "Row"
+    request_idx: int
+    chunks: "list[Chunk]"
+    chunk_idx: int = 0
+    frame_count: int = 0
+    turn_count: int = 0
+    max_turn_frames: int = 0
+    seq_offset: int = 0
+    last_codes: Tensor | None = None
+
+
 def _make_buckets(max_bs: int) -> list[int]:
     """src/vui/engine.py:134-142."""
     buckets, b = [], 1
@@ -447,6 +471,131 @@ class Engine:
                 torch.cuda.current_stream().synchronize()
         torch.cuda.current_stream().synchronize()
         return frames[:n_frames, :, :nq].clone(), eos[:n_frames].clone()
+
+    # ------------------------------------------------------------------ continuous batching
+    @torch.inference_mode()
+    def render_continuous(self, requests: "list[RenderRequest]", cfg: GenConfig = GenConfig()) -> list[Tensor]:
+        """Continuous batching over bucketed step graphs (Engine.render_continuous,
+        src/vui/engine.py:1112-1302): more requests than rows are accepted, a slot is freed when its
+        request ends and refilled from the queue at once.  Per step: one bucketed backbone step with slot
+        indirection (padding rows write to the spare slot), code 0 per active slot with the slot's own
+        repetition counts (no window here, engine.py:594-616), EOS flags, one batched depth-head call at the
+        bucket size, then per-slot bookkeeping (EOS after min_secs or the chunk's frame cap start the next
+        chunk; max_secs or the cache limit end the request).  Returns the codes (T_i, Q') of every request in
+        input order (the reference decodes them to audio with the offline vocoder pass)."""
+        if not requests:
+            return []
+        model, nat = self.model, self.model._native
+        max_frames = int(cfg.max_secs * FRAME_RATE)
+        min_frames = int(cfg.min_secs * FRAME_RATE)
+        max_seq = self.max_seq - 10
+        nq = cfg.n_codebooks if cfg.n_codebooks > 0 else self.Q
+        greedy = cfg.top_k == 1
+        use_rep = cfg.rep_penalty > 1.0
+        frame_bufs: list[list[Tensor]] = [[] for _ in requests]
+        pending = list(range(len(requests)))
+        active: dict[int, _ActiveSlot] = {}
+        self._rep_counts.zero_()
+        self._frame_ctr.zero_()
+        stream = torch.cuda.current_stream()
+        sp_rq = make_sample_params(cfg.temperature, cfg.rq_top_k if not greedy else 1, cfg.seed, self._frame_ctr)
+        one_slot = torch.zeros(1, dtype=torch.int32, device=self.device)
+        rq_code0 = torch.zeros(self._buckets[-1], dtype=torch.long, device=self.device)
+        rq_out = torch.zeros(self._buckets[-1], self.Q, dtype=torch.long, device=self.device)
+
+        def sample(cb0: Tensor, slots: Tensor, top_k: int, out: Tensor | None = None) -> Tensor:
+            B = cb0.shape[0]
+            sp = make_sample_params(cfg.temperature, top_k, cfg.seed, self._frame_ctr, state_rows=slots)
+            out = out if out is not None else torch.empty(B, dtype=torch.long, device=self.device)
+            _lib.check(nat.lib.vui_sample_cb0(nat.handle, cb0.contiguous().data_ptr(),
+                                              self._rep_counts.data_ptr() if use_rep else None, None, None,
+                                              float(cfg.rep_penalty), 0, C.byref(sp), out.data_ptr(), B, stream.cuda_stream),
+                       "vui_sample_cb0")
+            return out
+
+        def depth_head(hidden: Tensor, code0: Tensor, B: int) -> Tensor:
+            _lib.check(nat.lib.vui_rq_generate(nat.handle, hidden.contiguous().data_ptr(), code0.data_ptr(), None, nq,
+                                               C.byref(sp_rq), rq_out.data_ptr(), self.Q, 1, B, stream.cuda_stream),
+                       "vui_rq_generate")
+            return rq_out[:B, :nq]
+
+        def advance_slot(info: _ActiveSlot) -> bool:
+            """Write the next chunk's text, draw its first frame; False when no chunk is left."""
+            if info.chunk_idx >= len(info.chunks):
+                return False
+            chunk = info.chunks[info.chunk_idx]
+            row = info.row
+            info.max_turn_frames = cfg.max_turn_frames(chunk.n_words, row.prompt_wps)
+            hidden = self._prefill_emb(row, chunk.emb)[:, -1]
+            cb0 = model.codec_head(hidden)
+            one_slot.fill_(row.idx)
+            code0 = sample(cb0, one_slot, 1 if greedy else 0)
+            info.last_codes = depth_head(hidden, code0, 1)[0].clone()
+            self._frame_ctr += 1
+            frame_bufs[info.request_idx].append(info.last_codes)
+            info.frame_count += 1
+            info.turn_count = 1
+            info.seq_offset = row.offset
+            return True
+
+        def backfill() -> None:
+            while pending and self._free:
+                req_idx = pending.pop(0)
+                req = requests[req_idx]
+                row = self.new_row()
+                self._rep_counts[row.idx].zero_()
+                row.prompt_wps = req.prompt_wps
+                if req.prompt_emb is not None and req.prompt_emb.shape[1] > 0:
+                    self._prefill_emb(row, req.prompt_emb)
+                if not req.chunks:
+                    row.close()
+                    continue
+                info = _ActiveSlot(row=row, request_idx=req_idx, chunks=req.chunks)
+                if not advance_slot(info):
+                    row.close()
+                    continue
+                active[row.idx] = info
+
+        backfill()
+        while active:
+            slot_list = sorted(active)
+            B_active = len(slot_list)
+            B_bucket = _get_bucket(B_active, self._buckets)
+            self._g_seq_inc.zero_()
+            for qi, slot in enumerate(slot_list):
+                info = active[slot]
+                self._gc_codes_in[qi].zero_()
+                self._gc_codes_in[qi, : info.last_codes.shape[0]] = info.last_codes
+            slots_t = torch.tensor(slot_list, dtype=torch.int32, device=self.device)
+            self._g_slot_idx[:B_active] = slots_t
+            self._g_seq_inc[slots_t.long()] = 1
+            hidden_all, cb0_all, eos_all = self._bucketed_decode_step(B_active)
+            for slot in slot_list:
+                active[slot].seq_offset += 1
+            sample(cb0_all, slots_t, cfg.top_k, out=rq_code0[:B_active])
+            eos_flags = (torch.sigmoid(eos_all.float()).flatten() > cfg.eos_threshold).cpu()
+            frames_all = depth_head(self._gc_hidden_out[:B_bucket], rq_code0, B_bucket)[:B_active].clone()
+            self._frame_ctr += 1
+            to_remove: list[int] = []
+            for qi, slot in enumerate(slot_list):
+                info = active[slot]
+                if info.frame_count >= max_frames or info.seq_offset >= max_seq:
+                    to_remove.append(slot)
+                    continue
+                turn_n = info.turn_count
+                if (turn_n >= min_frames and bool(eos_flags[qi])) or turn_n >= info.max_turn_frames:
+                    info.chunk_idx += 1
+                    if not advance_slot(info):
+                        to_remove.append(slot)
+                    continue
+                info.last_codes = frames_all[qi]
+                frame_bufs[info.request_idx].append(info.last_codes)
+                info.frame_count += 1
+                info.turn_count += 1
+            for slot in to_remove:
+                active.pop(slot).row.close()
+            backfill()
+        return [torch.stack(b) if b else torch.zeros(0, nq, dtype=torch.long, device=self.device) for b in frame_bufs]
 
     # ------------------------------------------------------------------ streaming single-row turn
     def _penalised_probs(self, cb0: Tensor, counts: Tensor, cfg: GenConfig, temp: float) -> Tensor:

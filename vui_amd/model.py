@@ -222,8 +222,10 @@ class Graph:
             pass
 
 
-def make_sample_params(temperature: float, top_k: int | None, seed: int, frame_ctr: Tensor | None):
+def make_sample_params(temperature: float, top_k: int | None, seed: int, frame_ctr: Tensor | None,
+                       state_rows: Tensor | None = None):
     sp = _lib.SampleParamsC()
+    sp.state_rows = state_rows.data_ptr() if state_rows is not None else None
     sp.temperature = float(temperature)
     sp.top_k = int(top_k) if top_k is not None else 0
     sp.seed = int(seed) & 0xFFFFFFFFFFFFFFFF
