@@ -1030,11 +1030,8 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
     return s;
   };
   int* ctr = (int*)ar.take(64);
-  // launch-shape targets (overridable for tuning runs)
-  const char* e1 = getenv("VUI_CV_TT");
-  const char* e2 = getenv("VUI_CV_WG_TARGET");
-  const char* e3 = getenv("VUI_CV_WG_TARGET2");
-  const int tt_force = e1 ? atoi(e1) : 0, wg_target = e2 ? atoi(e2) : 512, wg_target2 = e3 ? atoi(e3) : 200;
+  // launch-shape targets: workgroups in flight for weight-streaming (one column block) and for wider tiles
+  const int wg_target = 512, wg_target2 = 200;
   // meeting place of split tiles: sized by a first pass (the sizes do not depend on the pointers)
   size_t part_floats = 0, cnt_ints = 0;
   float* part = ar.take(part_cap);
@@ -1054,7 +1051,6 @@ static int cv_build(vui_codec* cc, const vui_codec_config* c, const void* const*
     g.tt = 1;
     for (int tt : {2, 4})
       if (T > 8 * tt && tiles(tt) * tt <= tiles(g.tt) * g.tt) g.tt = tt;
-    if (tt_force > 0 && T > 8 * tt_force) g.tt = tt_force;
     int sp = 1;
     if (U >= 64) {
       const int target = g.tt == 1 ? wg_target : wg_target2;
