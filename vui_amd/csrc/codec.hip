@@ -446,7 +446,7 @@ struct CvTrunk {
   float eps;
 };
 
-#define TR_MAXR 3  // rows per wave and phase
+#define TR_MAXR 4  // rows per wave and phase
 #define TR_MAXC 6  // float4 chunks per lane and row: K <= 1536
 
 struct TrRows { float4 w[TR_MAXR][TR_MAXC]; };
@@ -494,6 +494,17 @@ __device__ __forceinline__ void tr_rows(int M, int wg, int nwg, int& lo, int& hi
   const int per = (M + nwg - 1) / nwg;
   lo = min(M, wg * per);
   hi = min(M, lo + per);
+}
+
+// q/k/v rows: the head-owning workgroups (the first H) stay out of this phase when enough others exist; they
+// use the time to fetch their key / value history
+__device__ __forceinline__ void tr_rows_qkv(int M, int wg, int nwg, int H, int& lo, int& hi) {
+  if (nwg >= 4 * H) {
+    if (wg < H) { lo = hi = M; return; }
+    tr_rows(M, wg - H, nwg - H, lo, hi);
+  } else {
+    tr_rows(M, wg, nwg, lo, hi);
+  }
 }
 
 __device__ __forceinline__ float tr_rstd(const float* x, int n, float eps, float* red) {
@@ -594,17 +605,47 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
   tr_compute<1, 4>(xs, L, lo, hi, rr, [&](int row, float s) { if (lane == 0) put(b_x, row, s + a.bin[row]); });
   {
     int qlo, qhi;
-    tr_rows(3 * A, wg, nwg, qlo, qhi);
+    tr_rows_qkv(3 * A, wg, nwg, a.H, qlo, qhi);
     tr_prefetch<TR_MAXR, 2>(a.layers[0].Wqkv, D, qlo, qhi, rr);
   }
   get(b_x, D, x);
 
   const float att_scale = 1.0f / sqrtf((float)hd);
+  // rotation of this position: the same for every layer, computed once and before any q arrives
+  float rope_cs = 1.f, rope_sn = 0.f;
+  if (wg < a.H && tid < hd) {
+    const float ang = (float)f * a.inv_freq[tid % (hd >> 1)];
+    rope_cs = cosf(ang);
+    rope_sn = sinf(ang);
+  }
   for (int l = 0; l < a.n_layers; ++l) {
     const TrunkLayer& W = a.layers[l];
+    // The head's workgroup asks for its whole key / value history now (at most 256 earlier positions: 16 per
+    // lane group, 4 features per lane), long before the new q arrives: attention then runs from registers,
+    // whatever the position.
+    float kreg[16][4], vreg[16][4];
+    if (wg < a.H) {
+      const float* kh = W.kc + (size_t)wg * a.max_seq * hd;
+      const float* vh = W.vc + (size_t)wg * a.max_seq * hd;
+      const int g16 = tid >> 4, c16 = tid & 15, E = hd >> 4;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int j = g16 + 16 * i;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { kreg[i][e] = 0.f; vreg[i][e] = 0.f; }
+        if (16 * i < f) {  // uniform: blocks of 16 positions that do not exist yet cost nothing
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const bool on = j < f && e < E;
+            kreg[i][e] = on ? kh[(size_t)j * hd + c16 + 16 * e] : 0.f;
+            vreg[i][e] = on ? vh[(size_t)j * hd + c16 + 16 * e] : 0.f;
+          }
+        }
+      }
+    }
     // ---- q, k, v rows (norm weight folded in; 1/rms multiplies the sums) ----
     const float r1 = tr_rstd(x, D, a.eps, red);
-    tr_rows(3 * A, wg, nwg, lo, hi);
+    tr_rows_qkv(3 * A, wg, nwg, a.H, lo, hi);
     uint64_t* b_qkv = take(3 * A);
     tr_compute<TR_MAXR, 2>(x, D, lo, hi, rr, [&](int row, float s) { if (lane == 0) put(b_qkv, row, s * r1); });
     uint64_t* b_att = take(A);
@@ -631,8 +672,7 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
       }
       __syncthreads();
       if (tid < hd) {
-        const float ang = (float)pos * a.inv_freq[tid % half];
-        const float cs = cosf(ang), sn = sinf(ang);
+        const float cs = rope_cs, sn = rope_sn;
         const float* qq = sc;
         const float* kk = sc + hd;
         const float qr = tid < half ? -qq[tid + half] : qq[tid - half];
@@ -649,23 +689,15 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) qe[e] = e < E ? q[l16 + 16 * e] : 0.f;
       __syncthreads();  // sc is rewritten below
-      for (int j0 = grp; j0 <= pos; j0 += 64) {
-        float kv[4][4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int j = j0 + 16 * u;
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            kv[u][e] = (j <= pos && e < E) ? (j == pos ? kvn[l16 + 16 * e] : kh[(size_t)j * hd + l16 + 16 * e]) : 0.f;
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int j = j0 + 16 * u;
+      for (int i = 0; i < 16; ++i) {
+        const int j = grp + 16 * i;
+        if (j <= pos) {  // uniform over the 16 lanes of a group
           float d = 0.f;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) d = fmaf(qe[e], kv[u][e], d);
+          for (int e = 0; e < 4; ++e) d = fmaf(qe[e], (j == pos && e < E) ? kvn[l16 + 16 * e] : kreg[i][e], d);
           d = group16_sum(d);
-          if (l16 == 0 && j <= pos) sc[j] = d * att_scale;
+          if (l16 == 0) sc[j] = d * att_scale;
         }
       }
       __syncthreads();
@@ -681,20 +713,28 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
       if (lane == 0) red[4 + wave] = sum;
       __syncthreads();
       sum = (red[4] + red[5]) + (red[6] + red[7]);
-      float o = 0.f;
-      if (lane < hd) {
-        for (int j0 = wave; j0 <= pos; j0 += 32) {
-          float vv[8];
+      // P.V per lane group over its own keys, then the 16 groups are added in order (xs is free here)
+      float o4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int u = 0; u < 8; ++u) { const int j = j0 + 4 * u; vv[u] = j <= pos ? (j == pos ? kvn[hd + lane] : vh[(size_t)j * hd + lane]) : 0.f; }
+      for (int i = 0; i < 16; ++i) {
+        const int j = grp + 16 * i;
+        if (j <= pos) {
+          const float pj = sc[j];
 #pragma unroll
-          for (int u = 0; u < 8; ++u) { const int j = j0 + 4 * u; o = fmaf(j <= pos ? sc[j] : 0.f, vv[u], o); }
+          for (int e = 0; e < 4; ++e) o4[e] = fmaf(pj, (j == pos && e < E) ? kvn[hd + l16 + 16 * e] : vreg[i][e], o4[e]);
         }
       }
-      __syncthreads();  // kvn (= part) has been read
-      if (lane < hd) part[wave * hd + lane] = o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) if (e < E) xs[grp * hd + l16 + 16 * e] = o4[e];
       __syncthreads();
-      if (tid < hd) put(b_att, h * hd + tid, ((part[tid] + part[hd + tid]) + (part[2 * hd + tid] + part[3 * hd + tid])) / sum);
+      if (tid < hd) {
+        float o = 0.f;
+#pragma unroll
+        for (int gg = 0; gg < 16; ++gg) o += xs[gg * hd + tid];
+        part[tid] = o / sum;  // kvn (= part) has been read by everyone
+      }
+      __syncthreads();
+      if (tid < hd) put(b_att, h * hd + tid, part[tid]);
     }
     // ---- out_proj, residual with per-channel scale ----
     get(b_att, A, xs);
@@ -726,7 +766,7 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
     tr_compute<1, 4>(xs, mlp, dlo, dhi, rr, [&](int row, float s) { if (lane == 0) put(b_d, row, s); });
     if (l + 1 < a.n_layers) {
       int qlo, qhi;
-      tr_rows(3 * A, wg, nwg, qlo, qhi);
+      tr_rows_qkv(3 * A, wg, nwg, a.H, qlo, qhi);
       tr_prefetch<TR_MAXR, 2>(a.layers[l + 1].Wqkv, D, qlo, qhi, rr);
     } else {
       int plo, phi;
@@ -1364,11 +1404,12 @@ int vui_codec_init(const vui_codec_config* cfg, const void* const* tensors, int3
     HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)cv_trunk_kernel, FR_THREADS, c->trunk_lds));
     int nwg = cus * per_cu < 256 ? cus * per_cu : 256;
+    auto fits_n = [&](int M, int K, int maxr, int maxc, int n) { return n > 0 && ((M + n - 1) / n + 3) / 4 <= maxr && K <= 256 * maxc && K % 4 == 0; };
     auto fits = [&](int M, int K, int maxr, int maxc) { return nwg > 0 && ((M + nwg - 1) / nwg + 3) / 4 <= maxr && K <= 256 * maxc && K % 4 == 0; };
     const bool ok = nwg >= k.n_heads && fits(k.vq_dim, 2 * k.codebook_dim, 1, 2) && fits(k.latent_dim, 3 * k.vq_dim, 1, TR_MAXC) &&
-                    fits(k.d_model, k.latent_dim, 1, 4) && fits(3 * A, k.d_model, TR_MAXR, 2) && fits(k.d_model, A, 1, 4) &&
+                    fits(k.d_model, k.latent_dim, 1, 4) && fits_n(3 * A, k.d_model, TR_MAXR, 2, nwg >= 4 * k.n_heads ? nwg - k.n_heads : nwg) && fits(k.d_model, A, 1, 4) &&
                     2 * ((k.mlp_dim + nwg - 1) / nwg) <= 4 * TR_MAXR && fits(k.d_model, k.mlp_dim, 1, 4) && fits(k.latent_dim, k.d_model, 1, 2) &&
-                    (k.n_up == 0 || fits(k.latent_dim * k.up_ratios[0], k.latent_dim, TR_MAXR, 4)) && k.head_dim <= 64 &&
+                    (k.n_up == 0 || fits(k.latent_dim * k.up_ratios[0], k.latent_dim, TR_MAXR, 4)) && k.head_dim <= 64 && k.max_seq <= 256 &&
                     k.d_model <= 1536 && A <= 1536 && k.mlp_dim <= 1536 && k.latent_dim <= 1536 && 3 * k.vq_dim <= 1536;
     c->trunk_wgs = ok ? nwg : 0;
     const char* e = getenv("VUI_CODEC_TRUNK");
