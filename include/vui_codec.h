@@ -76,6 +76,14 @@ int vui_codec_reset(vui_codec* c, vui_stream_t stream);
  * frames between two resets; further frames raise the status flag and reuse the last position. */
 int vui_codec_decode_frame(vui_codec* c, const int64_t* codes, int32_t n_q, float* audio_out, vui_stream_t stream);
 
+/* The one-column steps of a frame (codebook rows ... first upsampling conv) run as one persistent kernel when
+ * the device can keep 256 workgroups resident and the dimensions fit, otherwise as separate launches (same
+ * sums in another order).  enable = 1/0 switches the persistent form on/off, -1 only queries; returns 1 when
+ * it will be used, else 0.  No counterpart in the reference.  Do not run two persistent kernels of this library
+ * (this one, the batch-1 frame kernel, the batched depth head) on different streams at the same time: each
+ * needs all its workgroups resident. */
+int vui_codec_persistent(vui_codec* c, int enable);
+
 /* Synchronous: frames decoded since the last reset (reads a device counter on `stream`), or a negative
  * code; VUI_EINVAL after a code outside [0, codebook_size) or a frame beyond max_seq was seen. */
 int64_t vui_codec_status(vui_codec* c, vui_stream_t stream);

@@ -104,19 +104,21 @@ def test_small_graph_replays_equal_eager(small):
         dec._graphs.clear()
 
 
-def test_persistent_trunk_equals_kernel_sequence(small, monkeypatch):
-    """The one-column steps run as one persistent kernel by default; VUI_CODEC_TRUNK=0 keeps them as
-    separate launches.  Same sums in another order."""
+def test_persistent_trunk_equals_kernel_sequence(small):
+    """The one-column steps run as one persistent kernel by default; switched off they are separate
+    launches.  Same sums in another order."""
     d, ora, dec = small
-    assert dec.lib is not None
-    monkeypatch.setenv("VUI_CODEC_TRUNK", "0")
-    seq = native(d, O.synthetic_codec_state_dict(d, seed=4))
-    monkeypatch.delenv("VUI_CODEC_TRUNK")
+    assert dec.persistent()
     g = torch.Generator().manual_seed(8)
     codes = torch.randint(0, d.codebook_size, (1, d.n_codebooks, 12), generator=g).cuda()
-    a, b = dec(codes), seq(codes)
-    assert err(a, b.cpu()) < 2e-5
-    assert err(seq(codes[:, :2]), ora.forward(codes[:, :2].cpu())) < TOL
+    a = dec(codes).clone()
+    try:
+        assert not dec.persistent(0)
+        b = dec(codes).clone()
+        assert err(a, b.cpu()) < 2e-5
+        assert err(dec(codes[:, :2]), ora.forward(codes[:, :2].cpu())) < TOL
+    finally:
+        assert dec.persistent(1)
 
 
 def test_errors_are_reported(small):

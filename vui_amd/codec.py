@@ -10,7 +10,6 @@ from __future__ import annotations
 
 import ctypes as C
 import math
-from contextlib import contextmanager
 from dataclasses import dataclass
 
 import torch
@@ -281,6 +280,11 @@ class QwenCodecDecoder:
         if n < 0:
             raise RuntimeError(_lib.last_error())
         return int(n)
+
+    def persistent(self, enable: int = -1) -> bool:
+        """Whether the one-column steps of a frame run as one persistent kernel; enable = 1/0 switches it
+        (captured graphs keep the form they were captured with)."""
+        return bool(self.lib.vui_codec_persistent(self.handle, int(enable)))
 
     def setup_streaming_graph(self, batch_size: int = 1, n_q: int | None = None, **_) -> None:
         """Captures the one-frame step as a HIP graph over static in/out buffers

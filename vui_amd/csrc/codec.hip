@@ -25,7 +25,6 @@
 #include <math.h>
 #include <new>
 #include <stdio.h>
-#include <stdlib.h>
 #include <string.h>
 #include <vector>
 
@@ -1412,14 +1411,19 @@ int vui_codec_init(const vui_codec_config* cfg, const void* const* tensors, int3
                     (k.n_up == 0 || fits(k.latent_dim * k.up_ratios[0], k.latent_dim, TR_MAXR, 4)) && k.head_dim <= 64 && k.max_seq <= 256 &&
                     k.d_model <= 1536 && A <= 1536 && k.mlp_dim <= 1536 && k.latent_dim <= 1536 && 3 * k.vq_dim <= 1536;
     c->trunk_wgs = ok ? nwg : 0;
-    const char* e = getenv("VUI_CODEC_TRUNK");
-    c->use_trunk = e ? atoi(e) : 1;
+    c->use_trunk = 1;
   }
   *out = c;
   return VUI_OK;
 }
 
 void vui_codec_destroy(vui_codec* c) { delete c; }
+
+int vui_codec_persistent(vui_codec* c, int enable) {
+  if (!c) { vui_set_error("NULL codec"); return 0; }
+  if (enable >= 0) c->use_trunk = enable ? 1 : 0;
+  return c->use_trunk && c->trunk_wgs > 0;
+}
 
 static int launch_cv_gemm(const CvGemm& g, hipStream_t st) {
   if (g.M % 16 || g.Cin % 32 || g.T < 1) { vui_set_error("codec gemm: bad shape M=%d Cin=%d T=%d", g.M, g.Cin, g.T); return VUI_EINVAL; }
