@@ -155,6 +155,43 @@ def vocoder_line():
                  "hbm_frac": round(cb / us / 1e3 / HBM_PEAK_GBS, 4)}
 
 
+def prefill_line(model2, eng2, g, loop_too=True, reps=5):
+    """Prompt ingestion: 576 positions (512 audio frames + 64 text tokens) in one pass per layer against the
+    position-by-position path; flops = 2 x positions x backbone weights (attention is a few % more)."""
+    import torch
+
+    m = model2.config.model
+    emb = (torch.randn(1, 576, m.d_model, generator=g) * 0.08).to(torch.bfloat16).cuda()
+    dec = model2.decoder
+
+    def prefill_once():
+        eng2.seq_lens[0] = 0
+        dec.forward_flash(emb, None)
+
+    def timed(fn, n):
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / n
+
+    prefill_once()
+    us_pass = timed(prefill_once, reps)
+    us_loop = 0.0
+    if loop_too:
+        dec.PREFILL_MIN = 10 ** 9
+        prefill_once()
+        us_loop = timed(prefill_once, 2)
+        dec.PREFILL_MIN = 4
+    wparams = (frame_bytes(m, 0)["backbone"] - 67584 - m.n_quantizers * m.d_model * 2 - 3145728) / 2
+    fl = 2.0 * 576 * wparams
+    return {"config": "prefill_b1", "positions": 576, "ms_one_pass": round(us_pass / 1e3, 3), "ms_position_by_position": round(us_loop / 1e3, 2),
+            "achieved_TFLOPs": round(fl / us_pass / 1e6, 1), "mfma_frac": round(fl / us_pass / 1e6 / 2500.0, 4)}
+
+
 def b16_line(sd, preset="A", n=100):
     """Config 5: 16 streams, int8 backbone weights, ragged caches U[128, 2048] filled N(0, 1), n frame steps
     from one captured graph (backbone kernel sequence + persistent depth head)."""
@@ -294,25 +331,8 @@ def suite(model, eng, d, sd, preset="A"):
     b = frame_bytes(m, 0)["rq_unique"]
     lines.append({"config": "rq_head_b1", "frames": 1000, "us_per_frame": round(us, 2), "unique_bytes": int(b),
                   "achieved_GBs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4)})
-    # prompt ingestion: 576 positions (512 audio frames + 64 text tokens) in one pass per layer against the
-    # position-by-position path; flops = 2 x positions x backbone weights (attention is a few % more)
+    lines.append(prefill_line(model2, eng2, g))
     emb = (torch.randn(1, 576, m.d_model, generator=g) * 0.08).to(torch.bfloat16).cuda()
-    dec = model2.decoder
-
-    def prefill_once():
-        eng2.seq_lens[0] = 0
-        dec.forward_flash(emb, None)
-
-    prefill_once()
-    us_pass = timed(prefill_once, 5)
-    dec.PREFILL_MIN = 10 ** 9
-    prefill_once()
-    us_loop = timed(prefill_once, 2)
-    dec.PREFILL_MIN = 4
-    wparams = (frame_bytes(m, 0)["backbone"] - 67584 - m.n_quantizers * m.d_model * 2 - 3145728) / 2
-    fl = 2.0 * 576 * wparams
-    lines.append({"config": "prefill_b1", "positions": 576, "ms_one_pass": round(us_pass / 1e3, 3), "ms_position_by_position": round(us_loop / 1e3, 2),
-                  "achieved_TFLOPs": round(fl / us_pass / 1e6, 1), "mfma_frac": round(fl / us_pass / 1e6 / 2500.0, 4)})
     # a streamed turn: one graph replay per frame plus the host's per-frame EOS read (Row.stream)
     from vui_amd.engine import Chunk
     eng2.seq_lens[0] = 0
@@ -391,6 +411,8 @@ def main():
     ap.add_argument("--suite", action="store_true", help="also print one JSON line per further benchmark config")
     ap.add_argument("--calib", action="store_true",
                     help="end with three plain 512 MiB device copies (reference points for hardware counters)")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="print only the prompt-ingestion line, one-pass path only (the run its rocprofv3 summary comes from)")
     ap.add_argument("--b16-only", action="store_true",
                     help="print only the 16-stream int8 line (the run its rocprofv3 summaries come from)")
     ap.add_argument("--vocoder-only", action="store_true",
@@ -402,6 +424,18 @@ def main():
         sys.exit(2)
     if args.vocoder_only:
         print(json.dumps(vocoder_line()[1]))
+        return
+    if args.prefill_only:
+        import torch
+
+        from vui_amd.engine import Engine
+        from vui_amd.model import Vui
+        from vui_amd.synthetic import nano_for_cache, synthetic_state_dict
+
+        sd = synthetic_state_dict(nano_for_cache(args.preset, 64).model, seed=0)
+        model2 = Vui(nano_for_cache(args.preset, 1024), sd, device="cuda", dtype=torch.bfloat16)
+        eng2 = Engine(model=model2, max_rows=1, max_seq=1024)
+        print(json.dumps(prefill_line(model2, eng2, torch.Generator().manual_seed(0), loop_too=False, reps=20)))
         return
     if args.b16_only:
         from vui_amd.synthetic import nano_for_cache, synthetic_state_dict
