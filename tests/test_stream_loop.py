@@ -181,3 +181,55 @@ def test_engine_stream_sampled_and_cancel():
     eng2 = Engine(model=model, max_rows=2, max_seq=320)
     with pytest.raises(RuntimeError):
         next(iter(eng2.new_row().stream(ch, cfg)))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("graph", [False, True])
+def test_stream_audio_equals_vocoder_oracle_on_streamed_codes(graph):
+    """Row.stream_audio: every frame of Row.stream passed through the row's vocoder context.  Same turn, same
+    seed: the audio is the vocoder oracle's for the codes Row.stream yields; an early stop by the consumer
+    leaves the row and the vocoder context usable."""
+    import dataclasses
+
+    from oracle import codec_oracle as CO
+    from tests.util import make_model
+    from vui_amd.codec import CodecConfig, QwenCodecDecoder
+    from vui_amd.engine import Chunk, Engine, GenConfig
+
+    d = tiny_dims(max_seqlen=320)
+    sd = O.synthetic_state_dict(d, **TINY_SD)
+    cd = CO.CodecDims(n_codebooks=4, codebook_size=32, codebook_dim=16, vq_dim=32, latent_dim=64, d_model=32,
+                      n_layers=2, n_heads=2, head_dim=16, mlp_dim=64, max_seq=130, up_ratios=(2, 2),
+                      decoder_dim=128, rates=(3, 2))
+    csd = CO.synthetic_codec_state_dict(cd, seed=4)
+    dec = QwenCodecDecoder(csd, CodecConfig(**dataclasses.asdict(cd)), device="cuda")
+    if graph:
+        dec.setup_streaming_graph(1)
+    model = make_model(d, sd, torch.bfloat16, max_seqlen=320)
+    ch = [Chunk(emb=e[None].cuda().to(torch.bfloat16), n_words=w) for e, w in _chunks(d, 2, words=3)]
+    cfg = GenConfig(eos_threshold=2.0, rep_window=4, top_k=5)
+    eng = Engine(model=model, codec=dec, max_rows=1, max_seq=320)
+    row = eng.new_row()
+    audio = [a.clone().cpu() for a in row.stream_audio(ch, cfg)]
+    row.reset()
+    row._codec_ctx.reset()
+    it = row.stream_audio(ch, cfg)  # the consumer walks away after three frames
+    for _ in range(3):
+        next(it)
+    it.close()
+    row.reset()
+    row._codec_ctx.reset()
+    again = [a.clone().cpu() for a in row.stream_audio(ch, cfg)]
+    assert len(again) == len(audio) and all(torch.equal(a, b) for a, b in zip(again, audio))
+    row.reset()
+    row._codec_ctx.reset()
+    codes = [f.cpu() for f in row.stream(ch, cfg)]
+    n = 2 * cfg.max_turn_frames(3)
+    assert len(audio) == len(codes) == n
+    ora = CO.CodecDecoderOracle(cd, csd)
+    ora.open_stream()
+    for i in range(n):  # fewer frames than the context's cold restart after 125
+        ref = ora.forward(codes[i].view(1, -1, 1))
+        assert audio[i].shape == (1, 1, cd.hop) and float((audio[i] - ref).abs().max()) < 2e-4, i
+    ora.close_stream()
+    row.close()
