@@ -5,8 +5,8 @@
 // bf16 only.  Per layer: row RMSNorm, QKV GEMM, RoPE + cache append, scores = q K^T (fp32, one
 // GEMM batched over heads against the cache itself), causal softmax (probabilities rounded to
 // bf16), transpose of the values, P V GEMM, out_proj GEMM with the residual add in its epilogue,
-// row RMSNorm, W1 / W3 GEMMs, SwiGLU product, W2 GEMM with residual.  Every GEMM is the same
-// matrix-core kernel: C (M x N) = X (M x K) W^T (N x K), K contiguous in both operands.
+// row RMSNorm, one GEMM over W1 and W3 with the SwiGLU product in its epilogue, W2 GEMM with residual.
+// Every GEMM is C (M x N) = X (M x K) W^T (N x K), K contiguous in both operands, on the matrix cores.
 //
 // Rounding points are those of the single-position step (one rounding after each linear, two in
 // the norm, products of the rotation rounded before their sum, residual sums rounded).
@@ -19,25 +19,24 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float pf_floatx4;
 union PfU128 { uint4 u; pf_bf16x8 v; };
 __device__ __forceinline__ pf_bf16x8 pf_frag(const uint4& x) { PfU128 t; t.u = x; return t.v; }
 
-enum { PF_BF16 = 0, PF_RESID = 1, PF_F32_SCALE = 2 };
+enum { PF_BF16 = 0, PF_RESID = 1 };
 
 struct PfGemm {
   const bf16_t* X;   // activations (M x K), row stride ldx
   const bf16_t* W;   // "weights" (N x K), row stride ldw
-  void* C;           // output (M x N), row stride ldc; bf16 (PF_BF16, PF_RESID: in place on the residual) or fp32
+  void* C;           // output (M x N), row stride ldc; bf16 (PF_RESID: in place on the residual), fp32 for the scores
   int M, N, K, ldx, ldw, ldc;
   size_t xb, wb, cb;  // element offsets per batch index z: X + z*xb, W + (z / wgroup)*wb, C + z*cb
   int wgroup;
   float scale;
 };
 
-// Workgroup: 64 rows x 64 features, four waves in a 2 x 2 arrangement of 32 x 32 tiles, each four
-// v_mfma_f32_16x16x32_bf16 per K step of 32.  Operand A of the instruction is the weight tile (lane:
-// feature lane % 16, eight k from (lane / 16) * 8), operand B the activation tile (lane: row lane % 16,
-// same k): the lane then holds four consecutive features of one row.  Fragments go from global memory
-// straight to registers, the next step's loads are issued before this step's instructions.
-template <int EPI>
-__global__ __launch_bounds__(256) void pf_gemm_kernel(const PfGemm p) {
+// Scores (K = head_dim, a few steps only).  Workgroup: 64 rows x 64 features, four waves in a 2 x 2 arrangement
+// of 32 x 32 tiles, each four v_mfma_f32_16x16x32_bf16 per K step of 32.  Operand A of the instruction is the
+// "weight" tile (lane: feature lane % 16, eight k from (lane / 16) * 8), operand B the activation tile (lane: row
+// lane % 16, same k): the lane then holds four consecutive features of one row.  Fragments go from global memory
+// straight to registers.  Output fp32, scaled.
+__global__ __launch_bounds__(256) void pf_scores_kernel(const PfGemm p) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int l16 = lane & 15, kg = lane >> 4;
   const int z = blockIdx.z;
@@ -57,20 +56,15 @@ __global__ __launch_bounds__(256) void pf_gemm_kernel(const PfGemm p) {
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) acc[i][j] = pf_floatx4{0.f, 0.f, 0.f, 0.f};
-  uint4 xa[2], wa[2], xn[2], wn[2];
-#pragma unroll
-  for (int j = 0; j < 2; ++j) { xa[j] = *reinterpret_cast<const uint4*>(xr[j]); wa[j] = *reinterpret_cast<const uint4*>(wr[j]); }
   for (int k = 0; k < p.K; k += 32) {
-    const int kn = (k + 32 < p.K) ? k + 32 : k;  // the last step reloads itself (unused)
+    uint4 xa[2], wa[2];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) { xn[j] = *reinterpret_cast<const uint4*>(xr[j] + kn); wn[j] = *reinterpret_cast<const uint4*>(wr[j] + kn); }
+    for (int j = 0; j < 2; ++j) { xa[j] = *reinterpret_cast<const uint4*>(xr[j] + k); wa[j] = *reinterpret_cast<const uint4*>(wr[j] + k); }
 #pragma unroll
     for (int i = 0; i < 2; ++i)    // feature tile
 #pragma unroll
       for (int j = 0; j < 2; ++j)  // row tile
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf_frag(wa[i]), pf_frag(xa[j]), acc[i][j], 0, 0, 0);
-#pragma unroll
-    for (int j = 0; j < 2; ++j) { xa[j] = xn[j]; wa[j] = wn[j]; }
   }
   // lane holds features n0 + 16 i + 4 kg + r (r = 0..3) of row m0 + 16 j + l16
 #pragma unroll
@@ -80,22 +74,112 @@ __global__ __launch_bounds__(256) void pf_gemm_kernel(const PfGemm p) {
       const int m = m0 + 16 * j + l16, n = n0 + 16 * i + 4 * kg;
       if (m >= p.M || n >= p.N) continue;
       const pf_floatx4 a = acc[i][j];
-      if (EPI == PF_F32_SCALE) {
-        float* c = (float*)p.C + (size_t)z * p.cb + (size_t)m * p.ldc + n;
-        if (n + 3 < p.N) *reinterpret_cast<float4*>(c) = make_float4(a[0] * p.scale, a[1] * p.scale, a[2] * p.scale, a[3] * p.scale);
-        else for (int r = 0; r < 4; ++r) if (n + r < p.N) c[r] = a[r] * p.scale;
-      } else {
-        bf16_t* c = (bf16_t*)p.C + (size_t)z * p.cb + (size_t)m * p.ldc + n;
-        float v[4] = {a[0], a[1], a[2], a[3]};
-        if (EPI == PF_RESID) {  // x = rnd(x + rnd(y)), src/vui/model.py:367, 374
-          const uint2 old = *reinterpret_cast<const uint2*>(c);
-          v[0] = bf_lo(old.x) + bf2f(f2bf(v[0])); v[1] = bf_hi(old.x) + bf2f(f2bf(v[1]));
-          v[2] = bf_lo(old.y) + bf2f(f2bf(v[2])); v[3] = bf_hi(old.y) + bf2f(f2bf(v[3]));
-        }
-        if (n + 3 < p.N) *reinterpret_cast<uint2*>(c) = make_uint2(f2bf2(v[0], v[1]), f2bf2(v[2], v[3]));
-        else for (int r = 0; r < 4; ++r) if (n + r < p.N) c[r] = f2bf(v[r]);
-      }
+      float* c = (float*)p.C + (size_t)z * p.cb + (size_t)m * p.ldc + n;
+      if (n + 3 < p.N) *reinterpret_cast<float4*>(c) = make_float4(a[0] * p.scale, a[1] * p.scale, a[2] * p.scale, a[3] * p.scale);
+      else for (int r = 0; r < 4; ++r) if (n + r < p.N) c[r] = a[r] * p.scale;
     }
+}
+
+// The same product for the projections (K = d_model ... ffn, where 64 x 64 tiles give only 9 x 12 ... 9 x 64
+// workgroups, each a long serial walk over K): a workgroup owns 32 rows x 32 features and its four waves split
+// the K steps between them, so a wave's chain of dependent trips to memory is a quarter as long and four times as
+// many workgroups are in flight.  The four partial tiles meet in LDS and are added in wave order (a fixed order:
+// results do not depend on timing).
+// DUAL: two weight matrices against the same activations, h = rnd(rnd(silu(rnd(a))) * rnd(c)) written once
+// (SwiGLU, src/vui/model.py:282) instead of two products and a pass over both.
+template <int EPI, bool DUAL>
+__global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf16_t* __restrict__ W2, int batch) {
+  constexpr int TILE = 1024;  // floats of one partial tile
+  constexpr int PW = (DUAL ? 2 : 1) * TILE;
+  __shared__ float part[4 * PW];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int l16 = lane & 15, kg = lane >> 4;
+  const int MT = (p.M + 31) >> 5, NT = (p.N + 31) >> 5;
+  const int id = blockIdx.x;
+  const int m0 = (id % MT) * 32, n0 = ((id / MT) % NT) * 32, z = id / (MT * NT);
+  if (z >= batch) return;
+  const bf16_t* X = p.X + (size_t)z * p.xb;
+  const size_t woff = (size_t)(z / p.wgroup) * p.wb;
+  // A step covers 64 values of k: the lane takes 16 consecutive ones (k0 + 16 kg ...), i.e. the four lanes of a
+  // row read one whole 128-byte line with two adjacent loads, and the two instructions of the step use the lower
+  // and the upper eight (any assignment of k to lanes is a valid one as long as both operands share it).
+  const int nsteps = p.K >> 6;
+  const int s0 = nsteps * wave / 4, s1 = nsteps * (wave + 1) / 4;
+  const bf16_t* xr[2];
+  const bf16_t* wr[2];
+  const bf16_t* vr[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    xr[j] = X + (size_t)min(m0 + 16 * j + l16, p.M - 1) * p.ldx + kg * 16;
+    const size_t wo = woff + (size_t)min(n0 + 16 * j + l16, p.N - 1) * p.ldw + kg * 16;
+    wr[j] = p.W + wo;
+    vr[j] = DUAL ? W2 + wo : p.W + wo;
+  }
+  pf_floatx4 acc[2][2], acc2[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) { acc[i][j] = pf_floatx4{0.f, 0.f, 0.f, 0.f}; acc2[i][j] = acc[i][j]; }
+  for (int s = s0; s < s1; ++s) {
+    const int k = s << 6;
+    uint4 xa[2][2], wa[2][2], va[2][2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        xa[j][h] = *reinterpret_cast<const uint4*>(xr[j] + k + 8 * h);
+        wa[j][h] = *reinterpret_cast<const uint4*>(wr[j] + k + 8 * h);
+        if (DUAL) va[j][h] = *reinterpret_cast<const uint4*>(vr[j] + k + 8 * h);
+      }
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf_frag(wa[i][h]), pf_frag(xa[j][h]), acc[i][j], 0, 0, 0);
+          if (DUAL) acc2[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf_frag(va[i][h]), pf_frag(xa[j][h]), acc2[i][j], 0, 0, 0);
+        }
+  }
+  // partial tiles to LDS: [wave][(i, j)][lane] as float4
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      *reinterpret_cast<pf_floatx4*>(&part[wave * PW + ((i * 2 + j) * 64 + lane) * 4]) = acc[i][j];
+      if (DUAL) *reinterpret_cast<pf_floatx4*>(&part[wave * PW + TILE + ((i * 2 + j) * 64 + lane) * 4]) = acc2[i][j];
+    }
+  __syncthreads();
+  // thread: sub-tile (i, j) = its wave's two bits, features n0 + 16 i + 4 kg + r (r = 0..3) of row m0 + 16 j + l16
+  const int i = wave >> 1, j = wave & 1;
+  const int m = m0 + 16 * j + l16, n = n0 + 16 * i + 4 * kg;
+  float v[4], u[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int e = tid * 4 + r;
+    v[r] = ((part[e] + part[PW + e]) + part[2 * PW + e]) + part[3 * PW + e];
+    if (DUAL) u[r] = ((part[TILE + e] + part[PW + TILE + e]) + part[2 * PW + TILE + e]) + part[3 * PW + TILE + e];
+  }
+  if (m >= p.M || n >= p.N) return;
+  bf16_t* c = (bf16_t*)p.C + (size_t)z * p.cb + (size_t)m * p.ldc + n;
+  if (DUAL) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float a = bf2f(f2bf(v[r])), b = bf2f(f2bf(u[r]));
+      v[r] = bf2f(f2bf(a / (1.0f + expf(-a)))) * b;
+    }
+  }
+  if (EPI == PF_RESID) {  // x = rnd(x + rnd(y)), src/vui/model.py:367, 374
+    if (n + 3 < p.N) {
+      const uint2 old = *reinterpret_cast<const uint2*>(c);
+      v[0] = bf_lo(old.x) + bf2f(f2bf(v[0])); v[1] = bf_hi(old.x) + bf2f(f2bf(v[1]));
+      v[2] = bf_lo(old.y) + bf2f(f2bf(v[2])); v[3] = bf_hi(old.y) + bf2f(f2bf(v[3]));
+    } else {
+      for (int r = 0; r < 4; ++r) if (n + r < p.N) v[r] = bf2f(c[r]) + bf2f(f2bf(v[r]));
+    }
+  }
+  if (n + 3 < p.N) *reinterpret_cast<uint2*>(c) = make_uint2(f2bf2(v[0], v[1]), f2bf2(v[2], v[3]));
+  else for (int r = 0; r < 4; ++r) if (n + r < p.N) c[r] = f2bf(v[r]);
 }
 
 // two-rounding RMSNorm of rows (src/vui/model.py:286-297); one wave per row
@@ -188,41 +272,38 @@ __global__ __launch_bounds__(256) void pf_transpose_v_kernel(const bf16_t* vc, b
   }
 }
 
-// h = rnd(rnd(silu(a)) * b) in place on a (src/vui/model.py:282)
-__global__ __launch_bounds__(256) void pf_swiglu_kernel(bf16_t* a, const bf16_t* b, size_t n8) {
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= n8) return;
-  float x[8], y[8], o[8];
-  El<bf16_t>::ld8(a + i * 8, x);
-  El<bf16_t>::ld8(b + i * 8, y);
-#pragma unroll
-  for (int e = 0; e < 8; ++e) o[e] = bf2f(f2bf(x[e] / (1.0f + expf(-x[e])))) * y[e];
-  El<bf16_t>::st8(a + i * 8, o);
-}
-
 __global__ void pf_set_len_kernel(int32_t* seq_lens, int slot, int v) { seq_lens[slot] = v; }
 
-static int pf_gemm(int epi, const PfGemm& g, int batch, hipStream_t st) {
-  if (g.K % 32 || g.M < 1 || g.N < 1) { vui_set_error("prefill GEMM: K=%d must be a multiple of 32", g.K); return VUI_EINVAL; }
+static int pf_scores(const PfGemm& g, int batch, hipStream_t st) {
+  if (g.K % 32 || g.M < 1 || g.N < 1) { vui_set_error("prefill scores: head_dim=%d must be a multiple of 32", g.K); return VUI_EINVAL; }
   dim3 grid((g.M + 63) / 64, (g.N + 63) / 64, batch);
-  if (epi == PF_BF16) hipLaunchKernelGGL(pf_gemm_kernel<PF_BF16>, grid, dim3(256), 0, st, g);
-  else if (epi == PF_RESID) hipLaunchKernelGGL(pf_gemm_kernel<PF_RESID>, grid, dim3(256), 0, st, g);
-  else hipLaunchKernelGGL(pf_gemm_kernel<PF_F32_SCALE>, grid, dim3(256), 0, st, g);
+  hipLaunchKernelGGL(pf_scores_kernel, grid, dim3(256), 0, st, g);
+  HIP_TRY(hipGetLastError());
+  return VUI_OK;
+}
+
+// bf16 out, K split over the waves of a workgroup; W2 != nullptr: the SwiGLU pair
+static int pf_gemm4(int epi, const PfGemm& g, const bf16_t* W2, int batch, hipStream_t st) {
+  if (g.K % 64 || g.M < 1 || g.N < 1 || batch < 1) { vui_set_error("prefill GEMM: K=%d must be a multiple of 64", g.K); return VUI_EINVAL; }
+  const dim3 grid((unsigned)(((g.M + 31) / 32) * ((g.N + 31) / 32) * batch));
+  if (W2) hipLaunchKernelGGL((pf_gemm4_kernel<PF_BF16, true>), grid, dim3(256), 0, st, g, W2, batch);
+  else if (epi == PF_RESID) hipLaunchKernelGGL((pf_gemm4_kernel<PF_RESID, false>), grid, dim3(256), 0, st, g, W2, batch);
+  else hipLaunchKernelGGL((pf_gemm4_kernel<PF_BF16, false>), grid, dim3(256), 0, st, g, W2, batch);
   HIP_TRY(hipGetLastError());
   return VUI_OK;
 }
 
 static size_t pf_align(size_t b) { return (b + 255) & ~(size_t)255; }
 
-// scratch: residual x, normed xn, qkv, attention output, two FFN buffers, scores, probabilities, transposed values
+// scratch: residual x, normed xn, qkv, attention output, FFN buffer, scores, probabilities, transposed values
 size_t prefill_scratch_bytes(const vui_config& c, int T, int L) {
   const size_t d = c.d_model, nq = (size_t)c.n_heads * c.head_dim, nkv = (size_t)c.n_kv_heads * c.head_dim;
-  const size_t Lpad = ((size_t)L + 31) & ~(size_t)31;
+  const size_t Lpad = ((size_t)L + 63) & ~(size_t)63;
   size_t b = 0;
   b += pf_align((size_t)T * d * 2) * 2;
   b += pf_align((size_t)T * (nq + 2 * nkv) * 2);
   b += pf_align((size_t)T * nq * 2);
-  b += pf_align((size_t)T * c.ffn * 2) * 2;
+  b += pf_align((size_t)T * c.ffn * 2);
   b += pf_align((size_t)c.n_heads * T * Lpad * 4);
   b += pf_align((size_t)c.n_heads * T * Lpad * 2);
   b += pf_align(nkv * Lpad * 2);
@@ -233,7 +314,8 @@ bool prefill_supported(const vui_config& c, char* why, size_t why_len) {
   const char* r = nullptr;
   const int nkv = c.n_kv_heads * c.head_dim;
   if (c.dtype != VUI_DTYPE_BF16 || c.int8_backbone) r = "bf16 weights only";
-  else if ((c.d_model % 32) || (c.ffn % 32) || (c.head_dim % 32) || (nkv % 8) || (c.rope_dim & 1)) r = "d_model, ffn and head_dim must be multiples of 32";
+  else if ((c.d_model % 64) || (c.ffn % 64) || ((c.n_heads * c.head_dim) % 64) || (c.head_dim % 32) || (nkv % 8) || (c.rope_dim & 1))
+    r = "d_model, heads x head_dim and ffn must be multiples of 64, head_dim of 32";
   else if (c.n_kv_heads < 1 || c.n_heads % c.n_kv_heads) r = "heads must be a multiple of KV heads";
   if (r && why) snprintf(why, why_len, "%s", r);
   return r == nullptr;
@@ -242,7 +324,7 @@ bool prefill_supported(const vui_config& c, char* why, size_t why_len) {
 int launch_prefill(const vui_config& c, const vui_weights& w, const void* emb, int T, int slot, int pos0, int32_t* seq_lens,
                    void* k_cache, void* v_cache, void* out, void* scratch, size_t scratch_bytes, hipStream_t st) {
   const int d = c.d_model, H = c.n_heads, KV = c.n_kv_heads, hd = c.head_dim, F = c.ffn, S = c.max_seqlen;
-  const int nq = H * hd, nkv = KV * hd, L = pos0 + T, Lpad = (L + 31) & ~31;
+  const int nq = H * hd, nkv = KV * hd, L = pos0 + T, Lpad = (L + 63) & ~63;
   char why[96];
   if (!prefill_supported(c, why, sizeof(why))) { vui_set_error("prefill: %s", why); return VUI_EINVAL; }
   if (T < 1 || pos0 < 0 || L > S) { vui_set_error("prefill: positions %d..%d outside the cache (S=%d)", pos0, L, S); return VUI_EINVAL; }
@@ -255,7 +337,6 @@ int launch_prefill(const vui_config& c, const vui_weights& w, const void* emb, i
   bf16_t* qkv = (bf16_t*)take((size_t)T * (nq + 2 * nkv) * 2);
   bf16_t* att = (bf16_t*)take((size_t)T * nq * 2);
   bf16_t* fa = (bf16_t*)take((size_t)T * F * 2);
-  bf16_t* fb = (bf16_t*)take((size_t)T * F * 2);
   float* scores = (float*)take((size_t)H * T * Lpad * 4);
   bf16_t* P = (bf16_t*)take((size_t)H * T * Lpad * 2);
   bf16_t* vt = (bf16_t*)take((size_t)nkv * Lpad * 2);
@@ -271,7 +352,7 @@ int launch_prefill(const vui_config& c, const vui_weights& w, const void* emb, i
     PfGemm g{};
     g.X = xn; g.W = (const bf16_t*)lw.wqkv; g.C = qkv; g.M = T; g.N = nq + 2 * nkv; g.K = d; g.ldx = d; g.ldw = d; g.ldc = nq + 2 * nkv;
     g.wgroup = 1; g.scale = 1.f;
-    if ((rc = pf_gemm(PF_BF16, g, 1, st))) return rc;
+    if ((rc = pf_gemm4(PF_BF16, g, nullptr, 1, st))) return rc;
     hipLaunchKernelGGL(pf_rope_append_kernel, dim3(T), dim3(256), 0, st, qkv, kc, vc, w.rope_table, T, nq, nkv, hd, c.rope_dim, pos0,
                        slot, S);
     // scores[h] = q_h K_h^T * scale over the L cached positions of this slot
@@ -280,27 +361,23 @@ int launch_prefill(const vui_config& c, const vui_weights& w, const void* emb, i
     PfGemm s{};
     s.X = qkv; s.ldx = nq + 2 * nkv; s.xb = hd; s.W = krow; s.ldw = nkv; s.wb = hd; s.wgroup = H / KV; s.C = scores; s.ldc = Lpad;
     s.cb = (size_t)T * Lpad; s.M = T; s.N = L; s.K = hd; s.scale = scale;
-    if ((rc = pf_gemm(PF_F32_SCALE, s, H, st))) return rc;
+    if ((rc = pf_scores(s, H, st))) return rc;
     hipLaunchKernelGGL(pf_softmax_kernel, dim3(T, H), dim3(256), 0, st, scores, P, T, Lpad, pos0, c.window);
     hipLaunchKernelGGL(pf_transpose_v_kernel, dim3(Lpad / 32, (nkv + 31) / 32), dim3(256), 0, st, vrow, vt, L, Lpad, nkv, hd);
     PfGemm o{};
     o.X = P; o.ldx = Lpad; o.xb = (size_t)T * Lpad; o.W = vt; o.ldw = Lpad; o.wb = (size_t)hd * Lpad; o.wgroup = H / KV; o.C = att;
     o.ldc = nq; o.cb = hd; o.M = T; o.N = hd; o.K = Lpad; o.scale = 1.f;
-    if ((rc = pf_gemm(PF_BF16, o, H, st))) return rc;
+    if ((rc = pf_gemm4(PF_BF16, o, nullptr, H, st))) return rc;
     PfGemm wo{};
     wo.X = att; wo.ldx = nq; wo.W = (const bf16_t*)lw.wo; wo.ldw = nq; wo.C = x; wo.ldc = d; wo.M = T; wo.N = d; wo.K = nq; wo.wgroup = 1;
-    if ((rc = pf_gemm(PF_RESID, wo, 1, st))) return rc;
+    if ((rc = pf_gemm4(PF_RESID, wo, nullptr, 1, st))) return rc;
     hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)lw.mlp_norm, xn, T, d, c.norm_eps);
     PfGemm f1{};
     f1.X = xn; f1.ldx = d; f1.W = (const bf16_t*)lw.w1; f1.ldw = d; f1.C = fa; f1.ldc = F; f1.M = T; f1.N = F; f1.K = d; f1.wgroup = 1;
-    if ((rc = pf_gemm(PF_BF16, f1, 1, st))) return rc;
-    f1.W = (const bf16_t*)lw.w3; f1.C = fb;
-    if ((rc = pf_gemm(PF_BF16, f1, 1, st))) return rc;
-    const size_t n8 = (size_t)T * F / 8;
-    hipLaunchKernelGGL(pf_swiglu_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, st, fa, fb, n8);
+    if ((rc = pf_gemm4(PF_BF16, f1, (const bf16_t*)lw.w3, 1, st))) return rc;
     PfGemm f2{};
     f2.X = fa; f2.ldx = F; f2.W = (const bf16_t*)lw.w2; f2.ldw = F; f2.C = x; f2.ldc = d; f2.M = T; f2.N = d; f2.K = F; f2.wgroup = 1;
-    if ((rc = pf_gemm(PF_RESID, f2, 1, st))) return rc;
+    if ((rc = pf_gemm4(PF_RESID, f2, nullptr, 1, st))) return rc;
   }
   hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)w.final_norm, (bf16_t*)out, T, d, c.norm_eps);
   hipLaunchKernelGGL(pf_set_len_kernel, dim3(1), dim3(1), 0, st, seq_lens, slot, L);

@@ -321,7 +321,7 @@ class Decoder:
     PREFILL_CHUNK = 1024  # positions per pass: bounds the score scratch (heads x chunk x cache length)
 
     def _prefill_available(self) -> bool:
-        """The one-pass form takes bf16 weights and dims that are multiples of 32 (the library decides)."""
+        """The one-pass form takes bf16 weights and dims that are multiples of 64, head_dim of 32 (the library decides)."""
         if self._prefill_ok is None:
             nat = self._model._native
             self._prefill_ok = nat.lib.vui_prefill_scratch_bytes(C.byref(nat.cfg), 1, 1) >= 0
