@@ -50,23 +50,22 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attn_kernel(const AttnArgs
   if (act) El<T>::ld8((const T*)p.q + (size_t)b * p.H * hd + h * hd + l16 * 8, q8);
 
   const size_t rowstride = (size_t)p.KV * hd;
-  const T* kbase = (const T*)p.kc + ((size_t)slot * p.S) * rowstride + kvh * hd + l16 * 8;
-  const T* vbase = (const T*)p.vc + ((size_t)slot * p.S) * rowstride + kvh * hd + l16 * 8;
+  // lanes beyond head_dim read the head's first elements instead (their q is zero and their sums are dropped)
+  const T* kbase = (const T*)p.kc + ((size_t)slot * p.S) * rowstride + kvh * hd + (act ? l16 * 8 : 0);
+  const T* vbase = (const T*)p.vc + ((size_t)slot * p.S) * rowstride + kvh * hd + (act ? l16 * 8 : 0);
 
   float m = -INFINITY, l = 0.f, acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
   for (int j0 = lo + g; j0 < hi; j0 += 4 * ATT_KEYS_PER_ITER) {
+    // Eight loads in flight per lane, none behind a branch (a guarded load is waited for inside its branch, one
+    // at a time): a key beyond the piece reads the piece's last key instead and gets weight exp(-inf) = 0 below.
     float k8[4][8], v8[4][8];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const int j = j0 + u * ATT_KEYS_PER_ITER;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) { k8[u][e] = 0.f; v8[u][e] = 0.f; }
-      if (act && j < hi) {
-        El<T>::ld8(kbase + (size_t)j * rowstride, k8[u]);
-        El<T>::ld8(vbase + (size_t)j * rowstride, v8[u]);
-      }
+      const int j = min(j0 + u * ATT_KEYS_PER_ITER, hi - 1);
+      El<T>::ld8(kbase + (size_t)j * rowstride, k8[u]);
+      El<T>::ld8(vbase + (size_t)j * rowstride, v8[u]);
     }
     float s[4];
     float mn = m;
