@@ -736,6 +736,15 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
       if (tid < hd) put(b_att, h * hd + tid, part[tid]);
     }
     // ---- out_proj, residual with per-channel scale ----
+    // the scales of this thread's channels (tid, tid + 256, ...) are asked for ahead of the waits: fetched when
+    // the sums arrive, their pointer and then their value would be two trips to memory on the critical path
+    float asc_r[6], msc_r[6];  // d_model <= 1536
+#pragma unroll
+    for (int k = 0; k < 6; ++k) {
+      const int i = tid + FR_THREADS * k;
+      asc_r[k] = i < D ? W.asc[i] : 0.f;
+      msc_r[k] = i < D ? W.msc[i] : 0.f;
+    }
     get(b_att, A, xs);
     uint64_t* b_o = take(D);
     tr_compute<1, 4>(xs, A, olo, ohi, rr, [&](int row, float s) { if (lane == 0) put(b_o, row, s); });
@@ -743,7 +752,7 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
     tr_rows(mlp, wg, nwg, glo, ghi);  // channels; rows 2i, 2i + 1 are gate_i, up_i
     glo *= 2; ghi *= 2;
     tr_prefetch<TR_MAXR, 2>(W.Wgu, D, glo, ghi, rr);
-    ll_poll(b_o, D, c, [&](int i, uint32_t v) { x[i] += W.asc[i] * __uint_as_float(v); });
+    ll_poll(b_o, D, c, [&](int i, uint32_t v) { x[i] += asc_r[i / FR_THREADS] * __uint_as_float(v); });
     // ---- gate / up rows interleaved: channel i = silu(gate_i) * up_i ----
     const float r2 = tr_rstd(x, D, a.eps, red);
     uint64_t* b_h = take(mlp);
@@ -772,7 +781,7 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
       tr_rows(L, wg, nwg, plo, phi);
       tr_prefetch<1, 2>(a.Wout, D, plo, phi, rr);
     }
-    ll_poll(b_d, D, c, [&](int i, uint32_t v) { x[i] += W.msc[i] * __uint_as_float(v); });
+    ll_poll(b_d, D, c, [&](int i, uint32_t v) { x[i] += msc_r[i / FR_THREADS] * __uint_as_float(v); });
   }
   // ---- final norm (folded) + output_proj ----
   const float r3 = tr_rstd(x, D, a.eps, red);
