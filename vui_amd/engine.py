@@ -382,12 +382,16 @@ class Engine:
         self.seq_lens[row.idx] = offset
         return offset
 
-    def _prefill_emb(self, row: Row, emb: Tensor) -> Tensor:
+    def _prefill_emb(self, row: Row, emb: Tensor, offset: int | None = None) -> Tensor:
+        """offset: the row's current length when the caller keeps count of it (saves reading it back from
+        the device, a synchronisation)."""
         T = emb.shape[1]
-        if row.offset + T > self.max_seq:
-            raise ValueError(f"prefill of {T} positions at offset {row.offset} exceeds max_seq={self.max_seq}")
-        pos = torch.arange(row.offset, row.offset + T, device=self.device)
-        return self.model.decoder.forward_flash(emb.to(self.dtype), pos, slot_idx=row._slot)
+        off = row.offset if offset is None else offset
+        if off + T > self.max_seq:
+            raise ValueError(f"prefill of {T} positions at offset {off} exceeds max_seq={self.max_seq}")
+        pos = torch.arange(off, off + T, device=self.device)
+        return self.model.decoder.forward_flash(emb.to(self.dtype), pos, slot_idx=row._slot,
+                                                known=(row.idx, off) if offset is not None else None)
 
     def set_conditioning(self, *, sq_scores=None, wps_score: float = 0.0) -> None:
         self.model.set_cond_bias(sq_scores=sq_scores, wps_score=wps_score)
@@ -502,6 +506,9 @@ class Engine:
         one_slot = torch.zeros(1, dtype=torch.int32, device=self.device)
         rq_code0 = torch.zeros(self._buckets[-1], dtype=torch.long, device=self.device)
         rq_out = torch.zeros(self._buckets[-1], self.Q, dtype=torch.long, device=self.device)
+        # the latest frame of every slot (zero beyond nq), so that a step's input is one gather; the host keeps
+        # count of every row's length instead of reading it back
+        last = torch.zeros(self.max_rows + 1, self.Q, dtype=torch.long, device=self.device)
 
         def sample(cb0: Tensor, slots: Tensor, top_k: int, out: Tensor | None = None) -> Tensor:
             B = cb0.shape[0]
@@ -526,16 +533,17 @@ class Engine:
             chunk = info.chunks[info.chunk_idx]
             row = info.row
             info.max_turn_frames = cfg.max_turn_frames(chunk.n_words, row.prompt_wps)
-            hidden = self._prefill_emb(row, chunk.emb)[:, -1]
+            hidden = self._prefill_emb(row, chunk.emb, offset=info.seq_offset)[:, -1]
+            info.seq_offset += chunk.emb.shape[1]
             cb0 = model.codec_head(hidden)
             one_slot.fill_(row.idx)
             code0 = sample(cb0, one_slot, 1 if greedy else 0)
             info.last_codes = depth_head(hidden, code0, 1)[0].clone()
+            last[row.idx, :nq] = info.last_codes
             self._frame_ctr += 1
             frame_bufs[info.request_idx].append(info.last_codes)
             info.frame_count += 1
             info.turn_count = 1
-            info.seq_offset = row.offset
             return True
 
         def backfill() -> None:
@@ -545,36 +553,41 @@ class Engine:
                 row = self.new_row()
                 self._rep_counts[row.idx].zero_()
                 row.prompt_wps = req.prompt_wps
+                off = 0  # new_row starts the slot at length zero
                 if req.prompt_emb is not None and req.prompt_emb.shape[1] > 0:
-                    self._prefill_emb(row, req.prompt_emb)
+                    self._prefill_emb(row, req.prompt_emb, offset=0)
+                    off = req.prompt_emb.shape[1]
                 if not req.chunks:
                     row.close()
                     continue
-                info = _ActiveSlot(row=row, request_idx=req_idx, chunks=req.chunks)
+                info = _ActiveSlot(row=row, request_idx=req_idx, chunks=req.chunks, seq_offset=off)
                 if not advance_slot(info):
                     row.close()
                     continue
                 active[row.idx] = info
 
         backfill()
+        prev_slots: list[int] = []
+        slots_t = slots_l = None
         while active:
             slot_list = sorted(active)
             B_active = len(slot_list)
             B_bucket = _get_bucket(B_active, self._buckets)
-            self._g_seq_inc.zero_()
-            for qi, slot in enumerate(slot_list):
-                info = active[slot]
-                self._gc_codes_in[qi].zero_()
-                self._gc_codes_in[qi, : info.last_codes.shape[0]] = info.last_codes
-            slots_t = torch.tensor(slot_list, dtype=torch.int32, device=self.device)
-            self._g_slot_idx[:B_active] = slots_t
-            self._g_seq_inc[slots_t.long()] = 1
+            if slot_list != prev_slots:  # membership changes only when a request ends or starts
+                slots_t = torch.tensor(slot_list, dtype=torch.int32, device=self.device)
+                slots_l = slots_t.long()
+                self._g_slot_idx[:B_active] = slots_t
+                self._g_seq_inc.zero_()
+                self._g_seq_inc[slots_l] = 1
+                prev_slots = slot_list
+            torch.index_select(last, 0, slots_l, out=self._gc_codes_in[:B_active])
             hidden_all, cb0_all, eos_all = self._bucketed_decode_step(B_active)
             for slot in slot_list:
                 active[slot].seq_offset += 1
             sample(cb0_all, slots_t, cfg.top_k, out=rq_code0[:B_active])
             eos_flags = (torch.sigmoid(eos_all.float()).flatten() > cfg.eos_threshold).cpu()
             frames_all = depth_head(self._gc_hidden_out[:B_bucket], rq_code0, B_bucket)[:B_active].clone()
+            last[slots_l, :nq] = frames_all  # a slot that starts a new chunk below overwrites its row
             self._frame_ctr += 1
             to_remove: list[int] = []
             for qi, slot in enumerate(slot_list):

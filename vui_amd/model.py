@@ -295,7 +295,7 @@ class Decoder:
         return max(1, min(32, 1024 // max(1, B * H)))
 
     def forward_flash(self, x: Tensor, positions: Tensor, per_sample_positions: bool = False,
-                      slot_idx: Tensor | None = None) -> Tensor:
+                      slot_idx: Tensor | None = None, known: "tuple[int, int] | None" = None) -> Tensor:
         """x (B, T, d) appended at seq_lens[slot]; returns the final-norm output (B, T, d) and advances
         seq_lens by T (src/vui/model.py:534-549).  The native step rotates at the position it writes
         to, so `positions` must be the cache positions (seq_lens .. seq_lens+T-1), as in every
@@ -305,7 +305,7 @@ class Decoder:
             raise ValueError(f"batch {B} > {MAX_BATCH}")
         model = self._model
         if B == 1 and T >= self.PREFILL_MIN and self._prefill_available():
-            return self._prefill(x, slot_idx)
+            return self._prefill(x, slot_idx, known)
         out = torch.empty_like(x)
         st = torch.cuda.current_stream().cuda_stream
         ns = self.default_splits(B)
@@ -327,13 +327,17 @@ class Decoder:
             self._prefill_ok = nat.lib.vui_prefill_scratch_bytes(C.byref(nat.cfg), 1, 1) >= 0
         return self._prefill_ok
 
-    def _prefill(self, x: Tensor, slot_idx: Tensor | None) -> Tensor:
-        """One row, T positions: the matrix-core pass of the native library, in chunks."""
+    def _prefill(self, x: Tensor, slot_idx: Tensor | None, known: "tuple[int, int] | None" = None) -> Tensor:
+        """One row, T positions: the matrix-core pass of the native library, in chunks.  known = (slot, length
+        of the slot) from a caller that keeps count: otherwise both are read back from the device."""
         model = self._model
         nat = model._native
         seq_lens = self.flash_kv_caches[0].seq_lens
-        slot = 0 if slot_idx is None else int(slot_idx[0])
-        pos = int(seq_lens[slot])
+        if known is not None:
+            slot, pos = known
+        else:
+            slot = 0 if slot_idx is None else int(slot_idx[0])
+            pos = int(seq_lens[slot])
         T = x.shape[1]
         if pos + T > self._k.shape[2]:
             raise ValueError(f"prefill of {T} positions at offset {pos} exceeds the cache length {self._k.shape[2]}")
