@@ -2,10 +2,10 @@
 //
 //   Decoder.forward_flash / Engine._prefill_emb with T > 1  (src/vui/model.py:534-549, engine.py:674-694)
 //
-// bf16 only.  Per layer: row RMSNorm, QKV GEMM, RoPE + cache append, scores = q K^T (fp32, one
-// GEMM batched over heads against the cache itself), causal softmax (probabilities rounded to
-// bf16), transpose of the values, P V GEMM, out_proj GEMM with the residual add in its epilogue,
-// row RMSNorm, one GEMM over W1 and W3 with the SwiGLU product in its epilogue, W2 GEMM with residual.
+// bf16 only.  Per layer: row RMSNorm, QKV GEMM, RoPE + cache append, transpose of the values, causal attention of
+// the new positions against the cache itself (scores never leave the registers; probabilities rounded to bf16
+// before they meet the values), out_proj GEMM with the residual add in its epilogue, row RMSNorm, one GEMM over
+// W1 and W3 with the SwiGLU product in its epilogue, W2 GEMM with residual: nine launches.
 // Every GEMM is C (M x N) = X (M x K) W^T (N x K), K contiguous in both operands, on the matrix cores.
 //
 // Rounding points are those of the single-position step (one rounding after each linear, two in
@@ -28,57 +28,7 @@ struct PfGemm {
   int M, N, K, ldx, ldw, ldc;
   size_t xb, wb, cb;  // element offsets per batch index z: X + z*xb, W + (z / wgroup)*wb, C + z*cb
   int wgroup;
-  float scale;
 };
-
-// Scores (K = head_dim, a few steps only).  Workgroup: 64 rows x 64 features, four waves in a 2 x 2 arrangement
-// of 32 x 32 tiles, each four v_mfma_f32_16x16x32_bf16 per K step of 32.  Operand A of the instruction is the
-// "weight" tile (lane: feature lane % 16, eight k from (lane / 16) * 8), operand B the activation tile (lane: row
-// lane % 16, same k): the lane then holds four consecutive features of one row.  Fragments go from global memory
-// straight to registers.  Output fp32, scaled.
-__global__ __launch_bounds__(256) void pf_scores_kernel(const PfGemm p) {
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int l16 = lane & 15, kg = lane >> 4;
-  const int z = blockIdx.z;
-  const int m0 = blockIdx.x * 64 + (wave & 1) * 32, n0 = blockIdx.y * 64 + (wave >> 1) * 32;
-  if (m0 >= p.M || n0 >= p.N) return;  // the whole 32 x 32 tile is outside
-  const bf16_t* X = p.X + (size_t)z * p.xb;
-  const bf16_t* W = p.W + (size_t)(z / p.wgroup) * p.wb;
-  const bf16_t* xr[2];
-  const bf16_t* wr[2];
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    xr[j] = X + (size_t)min(m0 + 16 * j + l16, p.M - 1) * p.ldx + kg * 8;
-    wr[j] = W + (size_t)min(n0 + 16 * j + l16, p.N - 1) * p.ldw + kg * 8;
-  }
-  pf_floatx4 acc[2][2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) acc[i][j] = pf_floatx4{0.f, 0.f, 0.f, 0.f};
-  for (int k = 0; k < p.K; k += 32) {
-    uint4 xa[2], wa[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) { xa[j] = *reinterpret_cast<const uint4*>(xr[j] + k); wa[j] = *reinterpret_cast<const uint4*>(wr[j] + k); }
-#pragma unroll
-    for (int i = 0; i < 2; ++i)    // feature tile
-#pragma unroll
-      for (int j = 0; j < 2; ++j)  // row tile
-        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf_frag(wa[i]), pf_frag(xa[j]), acc[i][j], 0, 0, 0);
-  }
-  // lane holds features n0 + 16 i + 4 kg + r (r = 0..3) of row m0 + 16 j + l16
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int m = m0 + 16 * j + l16, n = n0 + 16 * i + 4 * kg;
-      if (m >= p.M || n >= p.N) continue;
-      const pf_floatx4 a = acc[i][j];
-      float* c = (float*)p.C + (size_t)z * p.cb + (size_t)m * p.ldc + n;
-      if (n + 3 < p.N) *reinterpret_cast<float4*>(c) = make_float4(a[0] * p.scale, a[1] * p.scale, a[2] * p.scale, a[3] * p.scale);
-      else for (int r = 0; r < 4; ++r) if (n + r < p.N) c[r] = a[r] * p.scale;
-    }
-}
 
 // The same product for the projections (K = d_model ... ffn, where 64 x 64 tiles give only 9 x 12 ... 9 x 64
 // workgroups, each a long serial walk over K): a workgroup owns 32 rows x 32 features and its four waves split
@@ -231,29 +181,126 @@ __global__ __launch_bounds__(256) void pf_rope_append_kernel(bf16_t* qkv, bf16_t
   }
 }
 
-// causal softmax of one (head, query) row of scores; probabilities rounded to bf16, zero outside the
-// visible range [start, pos0 + t] up to the padded length
-__global__ __launch_bounds__(256) void pf_softmax_kernel(const float* scores, bf16_t* P, int T, int Lpad, int pos0, int window) {
-  const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
-  const float* s = scores + ((size_t)h * T + t) * Lpad;
-  bf16_t* o = P + ((size_t)h * T + t) * Lpad;
-  const int len = pos0 + t + 1;
-  const int start = window > 0 ? max(0, len - 1 - window) : 0;
-  __shared__ float red[8];
-  float m = -INFINITY;
-  for (int j = start + tid; j < len; j += 256) m = fmaxf(m, s[j]);
-  m = wave_max(m);
-  if ((tid & 63) == 0) red[tid >> 6] = m;
+// Attention of the new positions against the row's cache without materialised scores: one workgroup per
+// (16 queries, head), its waves (eight, four for head_dim 128) take 32 keys at a time in turn with a running maximum and sum each and
+// meet in LDS at the end.  Per step: scores^T (keys x queries) = K q^T on the matrix cores, so that a lane holds
+// eight keys of ONE query (its column) and the softmax bookkeeping is per lane plus a fold over the four lane
+// rows; the probabilities, rounded to bf16, are then already in operand layout for out^T (dims x queries) =
+// V^T p^T, with V^T read from the transposed copy in the same key order (any assignment of k to lanes is valid
+// when both operands share it).  HD32 = head_dim / 32.
+#define PF_ATT_WAVES (HD32 <= 3 ? 8 : 4)  // the partial outputs of the waves must fit 64 KiB of LDS
+template <int HD32>
+__global__ __launch_bounds__(64 * PF_ATT_WAVES) void pf_attn_kernel(const bf16_t* __restrict__ qkv, const bf16_t* __restrict__ krow,
+                                                      const bf16_t* __restrict__ vt, bf16_t* __restrict__ att, int T, int L,
+                                                      int Lpad, int nq, int nkv, int gsz, int pos0, int window, float scale) {
+  constexpr int HD = 32 * HD32, DT = 2 * HD32;
+  __shared__ float s_acc[PF_ATT_WAVES][DT * 256];
+  __shared__ float s_m[PF_ATT_WAVES][16], s_l[PF_ATT_WAVES][16];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int l16 = lane & 15, kg = lane >> 4;
+  const int q0 = blockIdx.x * 16, h = blockIdx.y, kvh = h / gsz;
+  const int ldq = nq + 2 * nkv;
+  // this lane's query (column of every product below)
+  const int tq = min(q0 + l16, T - 1);
+  const int qlast = pos0 + tq;                                   // last visible key
+  const int qfirst = window > 0 ? max(0, qlast - window) : 0;   // first visible key
+  uint4 qf[HD32];
+#pragma unroll
+  for (int c = 0; c < HD32; ++c)
+    qf[c] = *reinterpret_cast<const uint4*>(qkv + (size_t)tq * ldq + h * HD + c * 32 + kg * 8);
+  // keys any query of the tile can see
+  const int t_hi = min(q0 + 15, T - 1);
+  const int kend = pos0 + t_hi + 1;
+  const int kbeg = (window > 0 ? max(0, pos0 + q0 - window) : 0) & ~31;
+  const bf16_t* kb = krow + kvh * HD + kg * 8;
+  const bf16_t* vb = vt + (size_t)kvh * HD * Lpad;
+
+  pf_floatx4 acc[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d) acc[d] = pf_floatx4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+  for (int k0 = kbeg + 32 * wave; k0 < kend; k0 += 32 * PF_ATT_WAVES) {
+    // every load of the step goes out before the first product (keys and values alike: the values do not depend
+    // on the scores), so a step is one trip to memory
+    uint4 kf[2][HD32];
+    uint2 vf[DT][2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      const bf16_t* kr = kb + (size_t)min(k0 + 16 * kt + l16, L - 1) * nkv;
+#pragma unroll
+      for (int c = 0; c < HD32; ++c) kf[kt][c] = *reinterpret_cast<const uint4*>(kr + c * 32);
+    }
+#pragma unroll
+    for (int d = 0; d < DT; ++d) {
+      // V^T of dims 16 d + l16: the lane's eight keys k0 + 4 kg + r and k0 + 16 + 4 kg + r, in the order of its scores
+      const bf16_t* vr = vb + (size_t)(16 * d + l16) * Lpad + k0 + 4 * kg;
+      vf[d][0] = *reinterpret_cast<const uint2*>(vr);
+      vf[d][1] = *reinterpret_cast<const uint2*>(vr + 16);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // scores^T of 32 keys: two tiles of 16 keys x 16 queries
+    pf_floatx4 sc[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      sc[kt] = pf_floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < HD32; ++c)
+        sc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf_frag(kf[kt][c]), pf_frag(qf[c]), sc[kt], 0, 0, 0);
+    }
+    // the lane holds keys k0 + 16 kt + 4 kg + r of its query
+    float sv[8], mx = -INFINITY;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int j = k0 + 16 * kt + 4 * kg + r;
+        const float v = (j >= qfirst && j <= qlast) ? sc[kt][r] * scale : -INFINITY;
+        sv[4 * kt + r] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = rows_max(mx);  // over the four lane rows: every key of the step for this query
+    const float m_new = fmaxf(m_run, mx);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // nothing visible yet: every weight below is zero
+    const float alpha = expf(m_run - m_use);                  // 0 on the first visible step (m_run = -inf)
+    float pv[8], ps = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { pv[e] = expf(sv[e] - m_use); ps += pv[e]; }
+    l_run = l_run * alpha + ps;
+    m_run = m_new;
+    uint4 pf;
+    pf.x = f2bf2(pv[0], pv[1]); pf.y = f2bf2(pv[2], pv[3]); pf.z = f2bf2(pv[4], pv[5]); pf.w = f2bf2(pv[6], pv[7]);
+#pragma unroll
+    for (int d = 0; d < DT; ++d) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[d][r] *= alpha;
+      acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf_frag(make_uint4(vf[d][0].x, vf[d][0].y, vf[d][1].x, vf[d][1].y)), pf_frag(pf), acc[d], 0, 0, 0);
+    }
+  }
+  // the waves' parts meet: lane holds dims 16 d + 4 kg + r of query l16
+  l_run = rows_sum(l_run);
+  if (kg == 0) { s_m[wave][l16] = m_run; s_l[wave][l16] = l_run; }
+#pragma unroll
+  for (int d = 0; d < DT; ++d) *reinterpret_cast<pf_floatx4*>(&s_acc[wave][(d * 64 + lane) * 4]) = acc[d];
   __syncthreads();
-  m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-  float sum = 0.f;
-  for (int j = start + tid; j < len; j += 256) sum += expf(s[j] - m);
-  sum = wave_sum(sum);
-  if ((tid & 63) == 0) red[4 + (tid >> 6)] = sum;
-  __syncthreads();
-  sum = (red[4] + red[5]) + (red[6] + red[7]);
-  const float inv = 1.0f / sum;
-  for (int j = tid; j < Lpad; j += 256) o[j] = (j >= start && j < len) ? f2bf(expf(s[j] - m) * inv) : (bf16_t)0;
+  for (int sl = tid; sl < DT * 64; sl += 64 * PF_ATT_WAVES) {
+    const int d = sl >> 6, ln = sl & 63, q = ln & 15, g4 = ln >> 4;
+    const int t = q0 + q;
+    if (t >= T) continue;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < PF_ATT_WAVES; ++w) M = fmaxf(M, s_m[w][q]);
+    float den = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < PF_ATT_WAVES; ++w) {
+      const float f = (s_m[w][q] == -INFINITY) ? 0.f : expf(s_m[w][q] - M);
+      den = fmaf(f, s_l[w][q], den);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[r] = fmaf(f, s_acc[w][sl * 4 + r], o[r]);
+    }
+    const float inv = 1.0f / den;
+    bf16_t* dst = att + (size_t)t * nq + h * HD + 16 * d + 4 * g4;
+    *reinterpret_cast<uint2*>(dst) = make_uint2(f2bf2(o[0] * inv, o[1] * inv), f2bf2(o[2] * inv, o[3] * inv));
+  }
 }
 
 // values of one row's cache slab, (L x KV*hd) -> per KV head (hd x Lpad), zero beyond L
@@ -274,14 +321,6 @@ __global__ __launch_bounds__(256) void pf_transpose_v_kernel(const bf16_t* vc, b
 
 __global__ void pf_set_len_kernel(int32_t* seq_lens, int slot, int v) { seq_lens[slot] = v; }
 
-static int pf_scores(const PfGemm& g, int batch, hipStream_t st) {
-  if (g.K % 32 || g.M < 1 || g.N < 1) { vui_set_error("prefill scores: head_dim=%d must be a multiple of 32", g.K); return VUI_EINVAL; }
-  dim3 grid((g.M + 63) / 64, (g.N + 63) / 64, batch);
-  hipLaunchKernelGGL(pf_scores_kernel, grid, dim3(256), 0, st, g);
-  HIP_TRY(hipGetLastError());
-  return VUI_OK;
-}
-
 // bf16 out, K split over the waves of a workgroup; W2 != nullptr: the SwiGLU pair
 static int pf_gemm4(int epi, const PfGemm& g, const bf16_t* W2, int batch, hipStream_t st) {
   if (g.K % 64 || g.M < 1 || g.N < 1 || batch < 1) { vui_set_error("prefill GEMM: K=%d must be a multiple of 64", g.K); return VUI_EINVAL; }
@@ -295,7 +334,7 @@ static int pf_gemm4(int epi, const PfGemm& g, const bf16_t* W2, int batch, hipSt
 
 static size_t pf_align(size_t b) { return (b + 255) & ~(size_t)255; }
 
-// scratch: residual x, normed xn, qkv, attention output, FFN buffer, scores, probabilities, transposed values
+// scratch: residual x, normed xn, qkv, attention output, FFN buffer, transposed values
 size_t prefill_scratch_bytes(const vui_config& c, int T, int L) {
   const size_t d = c.d_model, nq = (size_t)c.n_heads * c.head_dim, nkv = (size_t)c.n_kv_heads * c.head_dim;
   const size_t Lpad = ((size_t)L + 63) & ~(size_t)63;
@@ -304,8 +343,6 @@ size_t prefill_scratch_bytes(const vui_config& c, int T, int L) {
   b += pf_align((size_t)T * (nq + 2 * nkv) * 2);
   b += pf_align((size_t)T * nq * 2);
   b += pf_align((size_t)T * c.ffn * 2);
-  b += pf_align((size_t)c.n_heads * T * Lpad * 4);
-  b += pf_align((size_t)c.n_heads * T * Lpad * 2);
   b += pf_align(nkv * Lpad * 2);
   return b;
 }
@@ -314,8 +351,8 @@ bool prefill_supported(const vui_config& c, char* why, size_t why_len) {
   const char* r = nullptr;
   const int nkv = c.n_kv_heads * c.head_dim;
   if (c.dtype != VUI_DTYPE_BF16 || c.int8_backbone) r = "bf16 weights only";
-  else if ((c.d_model % 64) || (c.ffn % 64) || ((c.n_heads * c.head_dim) % 64) || (c.head_dim % 32) || (nkv % 8) || (c.rope_dim & 1))
-    r = "d_model, heads x head_dim and ffn must be multiples of 64, head_dim of 32";
+  else if ((c.d_model % 64) || (c.ffn % 64) || ((c.n_heads * c.head_dim) % 64) || (c.head_dim % 32) || c.head_dim > 128 || (nkv % 8) || (c.rope_dim & 1))
+    r = "d_model, heads x head_dim and ffn must be multiples of 64, head_dim a multiple of 32 up to 128";
   else if (c.n_kv_heads < 1 || c.n_heads % c.n_kv_heads) r = "heads must be a multiple of KV heads";
   if (r && why) snprintf(why, why_len, "%s", r);
   return r == nullptr;
@@ -337,8 +374,6 @@ int launch_prefill(const vui_config& c, const vui_weights& w, const void* emb, i
   bf16_t* qkv = (bf16_t*)take((size_t)T * (nq + 2 * nkv) * 2);
   bf16_t* att = (bf16_t*)take((size_t)T * nq * 2);
   bf16_t* fa = (bf16_t*)take((size_t)T * F * 2);
-  float* scores = (float*)take((size_t)H * T * Lpad * 4);
-  bf16_t* P = (bf16_t*)take((size_t)H * T * Lpad * 2);
   bf16_t* vt = (bf16_t*)take((size_t)nkv * Lpad * 2);
   HIP_TRY(hipMemcpyAsync(x, emb, (size_t)T * d * 2, hipMemcpyDeviceToDevice, st));
   const size_t slab = (size_t)c.n_slots * S * nkv;
@@ -351,23 +386,23 @@ int launch_prefill(const vui_config& c, const vui_weights& w, const void* emb, i
     hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)lw.attn_norm, xn, T, d, c.norm_eps);
     PfGemm g{};
     g.X = xn; g.W = (const bf16_t*)lw.wqkv; g.C = qkv; g.M = T; g.N = nq + 2 * nkv; g.K = d; g.ldx = d; g.ldw = d; g.ldc = nq + 2 * nkv;
-    g.wgroup = 1; g.scale = 1.f;
+    g.wgroup = 1;
     if ((rc = pf_gemm4(PF_BF16, g, nullptr, 1, st))) return rc;
     hipLaunchKernelGGL(pf_rope_append_kernel, dim3(T), dim3(256), 0, st, qkv, kc, vc, w.rope_table, T, nq, nkv, hd, c.rope_dim, pos0,
                        slot, S);
-    // scores[h] = q_h K_h^T * scale over the L cached positions of this slot
+    // attention over the L cached positions of this slot
     const bf16_t* krow = kc + (size_t)slot * S * nkv;
     const bf16_t* vrow = vc + (size_t)slot * S * nkv;
-    PfGemm s{};
-    s.X = qkv; s.ldx = nq + 2 * nkv; s.xb = hd; s.W = krow; s.ldw = nkv; s.wb = hd; s.wgroup = H / KV; s.C = scores; s.ldc = Lpad;
-    s.cb = (size_t)T * Lpad; s.M = T; s.N = L; s.K = hd; s.scale = scale;
-    if ((rc = pf_scores(s, H, st))) return rc;
-    hipLaunchKernelGGL(pf_softmax_kernel, dim3(T, H), dim3(256), 0, st, scores, P, T, Lpad, pos0, c.window);
     hipLaunchKernelGGL(pf_transpose_v_kernel, dim3(Lpad / 32, (nkv + 31) / 32), dim3(256), 0, st, vrow, vt, L, Lpad, nkv, hd);
-    PfGemm o{};
-    o.X = P; o.ldx = Lpad; o.xb = (size_t)T * Lpad; o.W = vt; o.ldw = Lpad; o.wb = (size_t)hd * Lpad; o.wgroup = H / KV; o.C = att;
-    o.ldc = nq; o.cb = hd; o.M = T; o.N = hd; o.K = Lpad; o.scale = 1.f;
-    if ((rc = pf_gemm4(PF_BF16, o, nullptr, H, st))) return rc;
+    {
+      const dim3 grid((T + 15) / 16, H);
+      switch (hd / 32) {
+        case 1: hipLaunchKernelGGL(pf_attn_kernel<1>, grid, dim3(512), 0, st, qkv, krow, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, c.window, scale); break;
+        case 2: hipLaunchKernelGGL(pf_attn_kernel<2>, grid, dim3(512), 0, st, qkv, krow, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, c.window, scale); break;
+        case 3: hipLaunchKernelGGL(pf_attn_kernel<3>, grid, dim3(512), 0, st, qkv, krow, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, c.window, scale); break;
+        default: hipLaunchKernelGGL(pf_attn_kernel<4>, grid, dim3(256), 0, st, qkv, krow, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, c.window, scale); break;
+      }
+    }
     PfGemm wo{};
     wo.X = att; wo.ldx = nq; wo.W = (const bf16_t*)lw.wo; wo.ldw = nq; wo.C = x; wo.ldc = d; wo.M = T; wo.N = d; wo.K = nq; wo.wgroup = 1;
     if ((rc = pf_gemm4(PF_RESID, wo, nullptr, 1, st))) return rc;
