@@ -318,7 +318,7 @@ class Decoder:
         return out
 
     PREFILL_MIN = 4      # shorter blocks go position by position through the decode step
-    PREFILL_CHUNK = 1024  # positions per pass: bounds the score scratch (heads x chunk x cache length)
+    PREFILL_CHUNK = 1024  # positions per pass: bounds the activation scratch (about 15 KB per position)
 
     def _prefill_available(self) -> bool:
         """The one-pass form takes bf16 weights and dims that are multiples of 64, head_dim of 32 (the library decides)."""
