@@ -23,33 +23,29 @@ enum { PF_BF16 = 0, PF_RESID = 1 };
 
 struct PfGemm {
   const bf16_t* X;   // activations (M x K), row stride ldx
-  const bf16_t* W;   // "weights" (N x K), row stride ldw
-  void* C;           // output (M x N), row stride ldc; bf16 (PF_RESID: in place on the residual), fp32 for the scores
+  const bf16_t* W;   // weights (N x K), row stride ldw
+  void* C;           // output (M x N) bf16, row stride ldc (PF_RESID: in place on the residual)
   int M, N, K, ldx, ldw, ldc;
-  size_t xb, wb, cb;  // element offsets per batch index z: X + z*xb, W + (z / wgroup)*wb, C + z*cb
-  int wgroup;
 };
 
-// The same product for the projections (K = d_model ... ffn, where 64 x 64 tiles give only 9 x 12 ... 9 x 64
-// workgroups, each a long serial walk over K): a workgroup owns 32 rows x 32 features and its four waves split
+// C = X W^T for the projections (K = d_model ... ffn; 64 x 64 tiles would give only 9 x 12 ... 9 x 64
+// workgroups at 576 positions, each a long serial walk over K): a workgroup owns 32 rows x 32 features and its four waves split
 // the K steps between them, so a wave's chain of dependent trips to memory is a quarter as long and four times as
 // many workgroups are in flight.  The four partial tiles meet in LDS and are added in wave order (a fixed order:
 // results do not depend on timing).
 // DUAL: two weight matrices against the same activations, h = rnd(rnd(silu(rnd(a))) * rnd(c)) written once
 // (SwiGLU, src/vui/model.py:282) instead of two products and a pass over both.
 template <int EPI, bool DUAL>
-__global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf16_t* __restrict__ W2, int batch) {
+__global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf16_t* __restrict__ W2) {
   constexpr int TILE = 1024;  // floats of one partial tile
   constexpr int PW = (DUAL ? 2 : 1) * TILE;
   __shared__ float part[4 * PW];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int l16 = lane & 15, kg = lane >> 4;
-  const int MT = (p.M + 31) >> 5, NT = (p.N + 31) >> 5;
+  const int MT = (p.M + 31) >> 5;
   const int id = blockIdx.x;
-  const int m0 = (id % MT) * 32, n0 = ((id / MT) % NT) * 32, z = id / (MT * NT);
-  if (z >= batch) return;
-  const bf16_t* X = p.X + (size_t)z * p.xb;
-  const size_t woff = (size_t)(z / p.wgroup) * p.wb;
+  const int m0 = (id % MT) * 32, n0 = (id / MT) * 32;
+  const bf16_t* X = p.X;
   // A step covers 64 values of k: the lane takes 16 consecutive ones (k0 + 16 kg ...), i.e. the four lanes of a
   // row read one whole 128-byte line with two adjacent loads, and the two instructions of the step use the lower
   // and the upper eight (any assignment of k to lanes is a valid one as long as both operands share it).
@@ -61,7 +57,7 @@ __global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf1
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     xr[j] = X + (size_t)min(m0 + 16 * j + l16, p.M - 1) * p.ldx + kg * 16;
-    const size_t wo = woff + (size_t)min(n0 + 16 * j + l16, p.N - 1) * p.ldw + kg * 16;
+    const size_t wo = (size_t)min(n0 + 16 * j + l16, p.N - 1) * p.ldw + kg * 16;
     wr[j] = p.W + wo;
     vr[j] = DUAL ? W2 + wo : p.W + wo;
   }
@@ -111,7 +107,7 @@ __global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf1
     if (DUAL) u[r] = ((part[TILE + e] + part[PW + TILE + e]) + part[2 * PW + TILE + e]) + part[3 * PW + TILE + e];
   }
   if (m >= p.M || n >= p.N) return;
-  bf16_t* c = (bf16_t*)p.C + (size_t)z * p.cb + (size_t)m * p.ldc + n;
+  bf16_t* c = (bf16_t*)p.C + (size_t)m * p.ldc + n;
   if (DUAL) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -322,12 +318,12 @@ __global__ __launch_bounds__(256) void pf_transpose_v_kernel(const bf16_t* vc, b
 __global__ void pf_set_len_kernel(int32_t* seq_lens, int slot, int v) { seq_lens[slot] = v; }
 
 // bf16 out, K split over the waves of a workgroup; W2 != nullptr: the SwiGLU pair
-static int pf_gemm4(int epi, const PfGemm& g, const bf16_t* W2, int batch, hipStream_t st) {
-  if (g.K % 64 || g.M < 1 || g.N < 1 || batch < 1) { vui_set_error("prefill GEMM: K=%d must be a multiple of 64", g.K); return VUI_EINVAL; }
-  const dim3 grid((unsigned)(((g.M + 31) / 32) * ((g.N + 31) / 32) * batch));
-  if (W2) hipLaunchKernelGGL((pf_gemm4_kernel<PF_BF16, true>), grid, dim3(256), 0, st, g, W2, batch);
-  else if (epi == PF_RESID) hipLaunchKernelGGL((pf_gemm4_kernel<PF_RESID, false>), grid, dim3(256), 0, st, g, W2, batch);
-  else hipLaunchKernelGGL((pf_gemm4_kernel<PF_BF16, false>), grid, dim3(256), 0, st, g, W2, batch);
+static int pf_gemm4(int epi, const PfGemm& g, const bf16_t* W2, hipStream_t st) {
+  if (g.K % 64 || g.M < 1 || g.N < 1) { vui_set_error("prefill GEMM: K=%d must be a multiple of 64", g.K); return VUI_EINVAL; }
+  const dim3 grid((unsigned)(((g.M + 31) / 32) * ((g.N + 31) / 32)));
+  if (W2) hipLaunchKernelGGL((pf_gemm4_kernel<PF_BF16, true>), grid, dim3(256), 0, st, g, W2);
+  else if (epi == PF_RESID) hipLaunchKernelGGL((pf_gemm4_kernel<PF_RESID, false>), grid, dim3(256), 0, st, g, W2);
+  else hipLaunchKernelGGL((pf_gemm4_kernel<PF_BF16, false>), grid, dim3(256), 0, st, g, W2);
   HIP_TRY(hipGetLastError());
   return VUI_OK;
 }
@@ -386,8 +382,7 @@ int launch_prefill(const vui_config& c, const vui_weights& w, const void* emb, i
     hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)lw.attn_norm, xn, T, d, c.norm_eps);
     PfGemm g{};
     g.X = xn; g.W = (const bf16_t*)lw.wqkv; g.C = qkv; g.M = T; g.N = nq + 2 * nkv; g.K = d; g.ldx = d; g.ldw = d; g.ldc = nq + 2 * nkv;
-    g.wgroup = 1;
-    if ((rc = pf_gemm4(PF_BF16, g, nullptr, 1, st))) return rc;
+    if ((rc = pf_gemm4(PF_BF16, g, nullptr, st))) return rc;
     hipLaunchKernelGGL(pf_rope_append_kernel, dim3(T), dim3(256), 0, st, qkv, kc, vc, w.rope_table, T, nq, nkv, hd, c.rope_dim, pos0,
                        slot, S);
     // attention over the L cached positions of this slot
@@ -404,15 +399,15 @@ int launch_prefill(const vui_config& c, const vui_weights& w, const void* emb, i
       }
     }
     PfGemm wo{};
-    wo.X = att; wo.ldx = nq; wo.W = (const bf16_t*)lw.wo; wo.ldw = nq; wo.C = x; wo.ldc = d; wo.M = T; wo.N = d; wo.K = nq; wo.wgroup = 1;
-    if ((rc = pf_gemm4(PF_RESID, wo, nullptr, 1, st))) return rc;
+    wo.X = att; wo.ldx = nq; wo.W = (const bf16_t*)lw.wo; wo.ldw = nq; wo.C = x; wo.ldc = d; wo.M = T; wo.N = d; wo.K = nq;
+    if ((rc = pf_gemm4(PF_RESID, wo, nullptr, st))) return rc;
     hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)lw.mlp_norm, xn, T, d, c.norm_eps);
     PfGemm f1{};
-    f1.X = xn; f1.ldx = d; f1.W = (const bf16_t*)lw.w1; f1.ldw = d; f1.C = fa; f1.ldc = F; f1.M = T; f1.N = F; f1.K = d; f1.wgroup = 1;
-    if ((rc = pf_gemm4(PF_BF16, f1, (const bf16_t*)lw.w3, 1, st))) return rc;
+    f1.X = xn; f1.ldx = d; f1.W = (const bf16_t*)lw.w1; f1.ldw = d; f1.C = fa; f1.ldc = F; f1.M = T; f1.N = F; f1.K = d;
+    if ((rc = pf_gemm4(PF_BF16, f1, (const bf16_t*)lw.w3, st))) return rc;
     PfGemm f2{};
-    f2.X = fa; f2.ldx = F; f2.W = (const bf16_t*)lw.w2; f2.ldw = F; f2.C = x; f2.ldc = d; f2.M = T; f2.N = d; f2.K = F; f2.wgroup = 1;
-    if ((rc = pf_gemm4(PF_RESID, f2, nullptr, 1, st))) return rc;
+    f2.X = fa; f2.ldx = F; f2.W = (const bf16_t*)lw.w2; f2.ldw = F; f2.C = x; f2.ldc = d; f2.M = T; f2.N = d; f2.K = F;
+    if ((rc = pf_gemm4(PF_RESID, f2, nullptr, st))) return rc;
   }
   hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)w.final_norm, (bf16_t*)out, T, d, c.norm_eps);
   hipLaunchKernelGGL(pf_set_len_kernel, dim3(1), dim3(1), 0, st, seq_lens, slot, L);
