@@ -91,7 +91,9 @@ typedef struct vui_ctx vui_ctx;
 const char* vui_last_error(void);
 int vui_version(void);
 
-/* Bytes of device workspace a context needs for up to max_batch rows. */
+/* Bytes of device workspace a context needs for up to max_batch rows.  For a configuration that has the one-pass
+ * prompt ingestion (vui_prefill) this includes a second copy of the layers' projection weights in the operand
+ * layout of its GEMMs (Vui Nano: 311 MB), written by vui_ctx_init. */
 int64_t vui_workspace_bytes(const vui_config* cfg, int max_batch);
 /* Bytes of ONE of the two (K or V) backbone caches: layers * slots * S * KV * hd elements.
  * Layout (layers, slots, S, KV, hd); layer l's (slots, S, KV, hd) slab is what the reference
@@ -105,7 +107,8 @@ int64_t vui_kv_bytes(const vui_config* cfg);
 int vui_ctx_create(const vui_config* cfg, const vui_weights* w, void* workspace, int64_t workspace_bytes,
                    int max_batch, vui_ctx** out);
 void vui_ctx_destroy(vui_ctx* ctx);
-/* One-time device-side initialisation of the workspace (zeroes counters).  Enqueued on stream. */
+/* One-time device-side initialisation of the workspace (zeroes counters, writes the prefill copy of the
+ * projection weights: the weight tensors must hold their final values).  Enqueued on stream. */
 int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream);
 
 /* The batch-1 bf16 calls below run as one persistent kernel ("fused") when the device can keep

@@ -36,6 +36,7 @@ struct vui_ctx {
   size_t ll_words;
   vui_weights* wdev;
   uint32_t* ctl;  // [0] epoch, [1] arrive, [2] err
+  void* pf_w;     // projection weights of every layer in the prefill GEMMs' operand layout (bf16 contexts)
   int fused_ok, fused_on, nwg, ns;
   size_t lds_bytes;
   char fused_why[96];
@@ -112,6 +113,7 @@ static size_t carve(const vui_config* c, int Bm, vui_ctx* x) {
   TAKE(ll, uint64_t*, ll_words_needed(*c) * 8);
   TAKE(wdev, vui_weights*, sizeof(vui_weights));
   TAKE(ctl, uint32_t*, 256);
+  TAKE(pf_w, void*, prefill_weight_bytes(*c));  // empty when the configuration has no prefill pass
 #undef TAKE
   return cv.off;
 }
@@ -180,6 +182,7 @@ int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream) {
   if ((rc = launch_fill_u32((uint32_t*)ctx->ll, 0u, (int64_t)ctx->ll_words * 2, st))) return rc;
   if ((rc = launch_fill_u32(ctx->ctl, 0u, 64, st))) return rc;
   HIP_TRY(hipMemcpyAsync(ctx->wdev, &ctx->w, sizeof(vui_weights), hipMemcpyHostToDevice, st));
+  if (prefill_weight_bytes(ctx->cfg) && (rc = prefill_tile_weights(ctx->cfg, ctx->w, ctx->pf_w, st))) return rc;
   HIP_TRY(hipStreamSynchronize(st));
   ctx->fused_ok = 0;
   ctx->fused_why[0] = 0;
@@ -263,8 +266,8 @@ int vui_prefill(vui_ctx* ctx, const void* emb_in, int T, int slot, int pos0, int
   if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
   if (!emb_in || !seq_lens || !k_cache || !v_cache || !hidden_out || !scratch) { vui_set_error("vui_prefill: NULL argument"); return VUI_EINVAL; }
   if (((uintptr_t)scratch & 255) || scratch_bytes < 0) { vui_set_error("vui_prefill: scratch must be 256-byte aligned"); return VUI_EINVAL; }
-  return launch_prefill(ctx->cfg, ctx->w, emb_in, T, slot, pos0, seq_lens, k_cache, v_cache, hidden_out, scratch,
-                        (size_t)scratch_bytes, (hipStream_t)stream);
+  return launch_prefill(ctx->cfg, ctx->w, prefill_weight_bytes(ctx->cfg) ? ctx->pf_w : nullptr, emb_in, T, slot, pos0, seq_lens, k_cache,
+                        v_cache, hidden_out, scratch, (size_t)scratch_bytes, (hipStream_t)stream);
 }
 
 int vui_backbone_step(vui_ctx* ctx, const int64_t* codes_in, const void* emb_in, const int32_t* slot_idx,

@@ -201,8 +201,10 @@ int launch_rq_batch(const vui_config& c, const vui_weights* wdev, const void* hi
 // prefill.hip
 size_t prefill_scratch_bytes(const vui_config& c, int T, int L);
 bool prefill_supported(const vui_config& c, char* why, size_t why_len);
-int launch_prefill(const vui_config& c, const vui_weights& w, const void* emb, int T, int slot, int pos0, int32_t* seq_lens,
-                   void* k_cache, void* v_cache, void* out, void* scratch, size_t scratch_bytes, hipStream_t st);
+size_t prefill_weight_bytes(const vui_config& c);  // the projection weights in the GEMMs' operand layout; 0: no pass
+int prefill_tile_weights(const vui_config& c, const vui_weights& w, void* dst, hipStream_t st);
+int launch_prefill(const vui_config& c, const vui_weights& w, const void* tiled_w, const void* emb, int T, int slot, int pos0,
+                   int32_t* seq_lens, void* k_cache, void* v_cache, void* out, void* scratch, size_t scratch_bytes, hipStream_t st);
 
 void vui_set_error(const char* fmt, ...);
 #define HIP_TRY(expr)                                                                  \

@@ -21,12 +21,34 @@ __device__ __forceinline__ pf_bf16x8 pf_frag(const uint4& x) { PfU128 t; t.u = x
 
 enum { PF_BF16 = 0, PF_RESID = 1 };
 
+// Operand layout of the GEMMs ("tiled"): a matrix of R rows x K columns (K a multiple of 64, rows padded to 16) is
+// cut into blocks of 16 rows x 64 columns, block (r / 16, k / 64) at element offset ((r / 16) * (K / 64) + k / 64)
+// * 1024, and inside a block the 8-element piece p = (k % 16) / 8 of lane (r % 16) + 16 * ((k % 64) / 16) sits at
+// p * 512 + lane * 8.  A wave then fetches the operand fragment of a 16 x 64 block with two loads of 1 KiB
+// contiguous each (lane l: 16 bytes at 16 l), where the row-major form makes the 16 lanes of a quarter-wave read
+// 16 different lines - which the address unit serves at about a quarter of the rate (measured on this machine
+// from an L2-sized buffer: 9.6 TB/s over the chip for 16 rows x 64 bytes per instruction, 31 TB/s for 1 KiB
+// contiguous).  Weights are brought into this form once per context, activations are written in it by their
+// producers.
+__host__ __device__ __forceinline__ size_t pf_toff(int r, int k, int K) {
+  return ((size_t)(r >> 4) * (K >> 6) + (k >> 6)) * 1024 + (size_t)(((k & 15) >> 3) * 512 + (((k & 63) >> 4) * 16 + (r & 15)) * 8 + (k & 7));
+}
+
 struct PfGemm {
-  const bf16_t* X;   // activations (M x K), row stride ldx
-  const bf16_t* W;   // weights (N x K), row stride ldw
-  void* C;           // output (M x N) bf16, row stride ldc (PF_RESID: in place on the residual)
-  int M, N, K, ldx, ldw, ldc;
+  const bf16_t* X;   // activations (M x K), tiled
+  const bf16_t* W;   // weights (N x K), tiled
+  void* C;           // output (M x N) bf16: row-major with row stride ldc (PF_RESID: in place on the residual), or tiled
+  int M, N, K, ldc;
 };
+
+// row-major (N x K) -> tiled; one 8-element piece per thread
+__global__ __launch_bounds__(256) void pf_tile_kernel(const bf16_t* __restrict__ src, bf16_t* __restrict__ dst, int N, int K) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const int per_row = K >> 3;
+  if (i >= (size_t)N * per_row) return;
+  const int n = (int)(i / per_row), k = (int)(i % per_row) * 8;
+  *reinterpret_cast<uint4*>(dst + pf_toff(n, k, K)) = *reinterpret_cast<const uint4*>(src + (size_t)n * K + k);
+}
 
 // C = X W^T for the projections (K = d_model ... ffn; 64 x 64 tiles would give only 9 x 12 ... 9 x 64
 // workgroups at 576 positions, each a long serial walk over K): a workgroup owns 32 rows x 32 features and its four waves split
@@ -36,7 +58,7 @@ struct PfGemm {
 // DUAL: two weight matrices against the same activations, h = rnd(rnd(silu(rnd(a))) * rnd(c)) written once
 // (SwiGLU, src/vui/model.py:282) instead of two products and a pass over both.
 template <int EPI, bool DUAL>
-__global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf16_t* __restrict__ W2) {
+__global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf16_t* __restrict__ W2, int c_tiled) {
   constexpr int TILE = 1024;  // floats of one partial tile
   constexpr int PW = (DUAL ? 2 : 1) * TILE;
   __shared__ float part[4 * PW];
@@ -45,19 +67,19 @@ __global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf1
   const int MT = (p.M + 31) >> 5;
   const int id = blockIdx.x;
   const int m0 = (id % MT) * 32, n0 = (id / MT) * 32;
-  const bf16_t* X = p.X;
-  // A step covers 64 values of k: the lane takes 16 consecutive ones (k0 + 16 kg ...), i.e. the four lanes of a
-  // row read one whole 128-byte line with two adjacent loads, and the two instructions of the step use the lower
-  // and the upper eight (any assignment of k to lanes is a valid one as long as both operands share it).
+  // A step covers 64 values of k, one block of the tiled operands per 16 rows: the lane's 16-byte piece of half h
+  // (k = 64 s + 16 kg + 8 h ...; any assignment of k to lanes is valid as long as both operands share it) is at
+  // block + 512 h + 8 lane.
   const int nsteps = p.K >> 6;
   const int s0 = nsteps * wave / 4, s1 = nsteps * (wave + 1) / 4;
+  const int MB = (p.M + 15) >> 4, NB = (p.N + 15) >> 4;  // 16-row blocks; a tile past the end reads the last block again
   const bf16_t* xr[2];
   const bf16_t* wr[2];
   const bf16_t* vr[2];
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
-    xr[j] = X + (size_t)min(m0 + 16 * j + l16, p.M - 1) * p.ldx + kg * 16;
-    const size_t wo = (size_t)min(n0 + 16 * j + l16, p.N - 1) * p.ldw + kg * 16;
+    xr[j] = p.X + (size_t)min((m0 >> 4) + j, MB - 1) * nsteps * 1024 + lane * 8;
+    const size_t wo = (size_t)min((n0 >> 4) + j, NB - 1) * nsteps * 1024 + lane * 8;
     wr[j] = p.W + wo;
     vr[j] = DUAL ? W2 + wo : p.W + wo;
   }
@@ -67,15 +89,15 @@ __global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf1
 #pragma unroll
     for (int j = 0; j < 2; ++j) { acc[i][j] = pf_floatx4{0.f, 0.f, 0.f, 0.f}; acc2[i][j] = acc[i][j]; }
   for (int s = s0; s < s1; ++s) {
-    const int k = s << 6;
+    const int k = s << 10;
     uint4 xa[2][2], wa[2][2], va[2][2];
 #pragma unroll
     for (int h = 0; h < 2; ++h)
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        xa[j][h] = *reinterpret_cast<const uint4*>(xr[j] + k + 8 * h);
-        wa[j][h] = *reinterpret_cast<const uint4*>(wr[j] + k + 8 * h);
-        if (DUAL) va[j][h] = *reinterpret_cast<const uint4*>(vr[j] + k + 8 * h);
+        xa[j][h] = *reinterpret_cast<const uint4*>(xr[j] + k + 512 * h);
+        wa[j][h] = *reinterpret_cast<const uint4*>(wr[j] + k + 512 * h);
+        if (DUAL) va[j][h] = *reinterpret_cast<const uint4*>(vr[j] + k + 512 * h);
       }
 #pragma unroll
     for (int h = 0; h < 2; ++h)
@@ -107,7 +129,7 @@ __global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf1
     if (DUAL) u[r] = ((part[TILE + e] + part[PW + TILE + e]) + part[2 * PW + TILE + e]) + part[3 * PW + TILE + e];
   }
   if (m >= p.M || n >= p.N) return;
-  bf16_t* c = (bf16_t*)p.C + (size_t)m * p.ldc + n;
+  bf16_t* c = (bf16_t*)p.C + (c_tiled ? pf_toff(m, n, p.N) : (size_t)m * p.ldc + n);  // n % 4 == 0: inside one piece
   if (DUAL) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -129,7 +151,7 @@ __global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf1
 }
 
 // two-rounding RMSNorm of rows (src/vui/model.py:286-297); one wave per row
-__global__ __launch_bounds__(256) void pf_rownorm_kernel(const bf16_t* x, const bf16_t* w, bf16_t* y, int M, int K, float eps) {
+__global__ __launch_bounds__(256) void pf_rownorm_kernel(const bf16_t* x, const bf16_t* w, bf16_t* y, int M, int K, float eps, int y_tiled) {
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (row >= M) return;
   const bf16_t* xr = x + (size_t)row * K;
@@ -148,7 +170,7 @@ __global__ __launch_bounds__(256) void pf_rownorm_kernel(const bf16_t* x, const 
     El<bf16_t>::ld8(w + c * 8, g);
 #pragma unroll
     for (int e = 0; e < 8; ++e) o[e] = bf2f(f2bf(v[e] * r)) * g[e];
-    El<bf16_t>::st8(y + (size_t)row * K + c * 8, o);
+    El<bf16_t>::st8(y + (y_tiled ? pf_toff(row, c * 8, K) : (size_t)row * K + c * 8), o);
   }
 }
 
@@ -294,7 +316,7 @@ __global__ __launch_bounds__(64 * PF_ATT_WAVES) void pf_attn_kernel(const bf16_t
       for (int r = 0; r < 4; ++r) o[r] = fmaf(f, s_acc[w][sl * 4 + r], o[r]);
     }
     const float inv = 1.0f / den;
-    bf16_t* dst = att + (size_t)t * nq + h * HD + 16 * d + 4 * g4;
+    bf16_t* dst = att + pf_toff(t, h * HD + 16 * d + 4 * g4, nq);  // tiled: operand of out_proj
     *reinterpret_cast<uint2*>(dst) = make_uint2(f2bf2(o[0] * inv, o[1] * inv), f2bf2(o[2] * inv, o[3] * inv));
   }
 }
@@ -318,12 +340,12 @@ __global__ __launch_bounds__(256) void pf_transpose_v_kernel(const bf16_t* vc, b
 __global__ void pf_set_len_kernel(int32_t* seq_lens, int slot, int v) { seq_lens[slot] = v; }
 
 // bf16 out, K split over the waves of a workgroup; W2 != nullptr: the SwiGLU pair
-static int pf_gemm4(int epi, const PfGemm& g, const bf16_t* W2, hipStream_t st) {
-  if (g.K % 64 || g.M < 1 || g.N < 1) { vui_set_error("prefill GEMM: K=%d must be a multiple of 64", g.K); return VUI_EINVAL; }
+static int pf_gemm4(int epi, const PfGemm& g, const bf16_t* W2, int c_tiled, hipStream_t st) {
+  if (g.K % 64 || g.N % 16 || g.M < 1 || g.N < 1 || (c_tiled && g.N % 64)) { vui_set_error("prefill GEMM: bad shape N=%d K=%d", g.N, g.K); return VUI_EINVAL; }
   const dim3 grid((unsigned)(((g.M + 31) / 32) * ((g.N + 31) / 32)));
-  if (W2) hipLaunchKernelGGL((pf_gemm4_kernel<PF_BF16, true>), grid, dim3(256), 0, st, g, W2);
-  else if (epi == PF_RESID) hipLaunchKernelGGL((pf_gemm4_kernel<PF_RESID, false>), grid, dim3(256), 0, st, g, W2);
-  else hipLaunchKernelGGL((pf_gemm4_kernel<PF_BF16, false>), grid, dim3(256), 0, st, g, W2);
+  if (W2) hipLaunchKernelGGL((pf_gemm4_kernel<PF_BF16, true>), grid, dim3(256), 0, st, g, W2, c_tiled);
+  else if (epi == PF_RESID) hipLaunchKernelGGL((pf_gemm4_kernel<PF_RESID, false>), grid, dim3(256), 0, st, g, W2, c_tiled);
+  else hipLaunchKernelGGL((pf_gemm4_kernel<PF_BF16, false>), grid, dim3(256), 0, st, g, W2, c_tiled);
   HIP_TRY(hipGetLastError());
   return VUI_OK;
 }
@@ -334,13 +356,45 @@ static size_t pf_align(size_t b) { return (b + 255) & ~(size_t)255; }
 size_t prefill_scratch_bytes(const vui_config& c, int T, int L) {
   const size_t d = c.d_model, nq = (size_t)c.n_heads * c.head_dim, nkv = (size_t)c.n_kv_heads * c.head_dim;
   const size_t Lpad = ((size_t)L + 63) & ~(size_t)63;
+  const size_t T16 = ((size_t)T + 15) & ~(size_t)15;  // tiled operands come in blocks of 16 rows
   size_t b = 0;
-  b += pf_align((size_t)T * d * 2) * 2;
+  b += pf_align((size_t)T * d * 2) + pf_align(T16 * d * 2);
   b += pf_align((size_t)T * (nq + 2 * nkv) * 2);
-  b += pf_align((size_t)T * nq * 2);
-  b += pf_align((size_t)T * c.ffn * 2);
+  b += pf_align(T16 * nq * 2);
+  b += pf_align(T16 * c.ffn * 2);
   b += pf_align(nkv * Lpad * 2);
   return b;
+}
+
+// elements of one layer's weights in tiled form (wqkv | wo | w1 | w3 | w2), and of all layers
+static size_t pf_layer_elems(const vui_config& c) {
+  const size_t d = c.d_model, nq = (size_t)c.n_heads * c.head_dim, nkv = (size_t)c.n_kv_heads * c.head_dim, F = c.ffn;
+  return (nq + 2 * nkv) * d + d * nq + 2 * F * d + d * F;
+}
+size_t prefill_weight_bytes(const vui_config& c) {
+  char why[96];
+  return prefill_supported(c, why, sizeof(why)) ? pf_layer_elems(c) * c.n_layers * 2 : 0;
+}
+
+// one-time: the layers' projection weights in the GEMMs' operand layout
+int prefill_tile_weights(const vui_config& c, const vui_weights& w, void* dst, hipStream_t st) {
+  const int d = c.d_model, nq = c.n_heads * c.head_dim, nkv = c.n_kv_heads * c.head_dim, F = c.ffn;
+  bf16_t* o = (bf16_t*)dst;
+  auto tile = [&](const void* src, int N, int K) {
+    const size_t pieces = (size_t)N * (K / 8);
+    hipLaunchKernelGGL(pf_tile_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, st, (const bf16_t*)src, o, N, K);
+    o += (size_t)N * K;
+  };
+  for (int l = 0; l < c.n_layers; ++l) {
+    const vui_layer_weights& lw = w.layers[l];
+    tile(lw.wqkv, nq + 2 * nkv, d);
+    tile(lw.wo, d, nq);
+    tile(lw.w1, F, d);
+    tile(lw.w3, F, d);
+    tile(lw.w2, d, F);
+  }
+  HIP_TRY(hipGetLastError());
+  return VUI_OK;
 }
 
 bool prefill_supported(const vui_config& c, char* why, size_t why_len) {
@@ -354,8 +408,8 @@ bool prefill_supported(const vui_config& c, char* why, size_t why_len) {
   return r == nullptr;
 }
 
-int launch_prefill(const vui_config& c, const vui_weights& w, const void* emb, int T, int slot, int pos0, int32_t* seq_lens,
-                   void* k_cache, void* v_cache, void* out, void* scratch, size_t scratch_bytes, hipStream_t st) {
+int launch_prefill(const vui_config& c, const vui_weights& w, const void* tiled_w, const void* emb, int T, int slot, int pos0,
+                   int32_t* seq_lens, void* k_cache, void* v_cache, void* out, void* scratch, size_t scratch_bytes, hipStream_t st) {
   const int d = c.d_model, H = c.n_heads, KV = c.n_kv_heads, hd = c.head_dim, F = c.ffn, S = c.max_seqlen;
   const int nq = H * hd, nkv = KV * hd, L = pos0 + T, Lpad = (L + 63) & ~63;
   char why[96];
@@ -363,13 +417,15 @@ int launch_prefill(const vui_config& c, const vui_weights& w, const void* emb, i
   if (T < 1 || pos0 < 0 || L > S) { vui_set_error("prefill: positions %d..%d outside the cache (S=%d)", pos0, L, S); return VUI_EINVAL; }
   if (slot < 0 || slot >= c.n_slots) { vui_set_error("prefill: slot %d outside [0,%d)", slot, c.n_slots); return VUI_EINVAL; }
   if (scratch_bytes < prefill_scratch_bytes(c, T, L)) { vui_set_error("prefill: scratch of %zu bytes, %zu needed", scratch_bytes, prefill_scratch_bytes(c, T, L)); return VUI_EINVAL; }
+  if (!tiled_w) { vui_set_error("prefill: the context holds no tiled weights"); return VUI_EINVAL; }
+  const size_t T16 = ((size_t)T + 15) & ~(size_t)15;
   char* sp = (char*)scratch;
   auto take = [&](size_t bytes) { char* r = sp; sp += pf_align(bytes); return r; };
-  bf16_t* x = (bf16_t*)take((size_t)T * d * 2);
-  bf16_t* xn = (bf16_t*)take((size_t)T * d * 2);
-  bf16_t* qkv = (bf16_t*)take((size_t)T * (nq + 2 * nkv) * 2);
-  bf16_t* att = (bf16_t*)take((size_t)T * nq * 2);
-  bf16_t* fa = (bf16_t*)take((size_t)T * F * 2);
+  bf16_t* x = (bf16_t*)take((size_t)T * d * 2);                 // residual stream, row-major
+  bf16_t* xn = (bf16_t*)take(T16 * d * 2);                      // normed rows, tiled (rows past T are never written:
+  bf16_t* qkv = (bf16_t*)take((size_t)T * (nq + 2 * nkv) * 2);  //  what a GEMM reads there only reaches output rows it drops)
+  bf16_t* att = (bf16_t*)take(T16 * nq * 2);                    // attention output, tiled
+  bf16_t* fa = (bf16_t*)take(T16 * F * 2);                      // SwiGLU product, tiled
   bf16_t* vt = (bf16_t*)take((size_t)nkv * Lpad * 2);
   HIP_TRY(hipMemcpyAsync(x, emb, (size_t)T * d * 2, hipMemcpyDeviceToDevice, st));
   const size_t slab = (size_t)c.n_slots * S * nkv;
@@ -377,12 +433,17 @@ int launch_prefill(const vui_config& c, const vui_weights& w, const void* emb, i
   int rc;
   for (int l = 0; l < c.n_layers; ++l) {
     const vui_layer_weights& lw = w.layers[l];
+    const bf16_t* t_qkv = (const bf16_t*)tiled_w + pf_layer_elems(c) * l;
+    const bf16_t* t_o = t_qkv + (size_t)(nq + 2 * nkv) * d;
+    const bf16_t* t_1 = t_o + (size_t)d * nq;
+    const bf16_t* t_3 = t_1 + (size_t)F * d;
+    const bf16_t* t_2 = t_3 + (size_t)F * d;
     bf16_t* kc = (bf16_t*)k_cache + slab * l;
     bf16_t* vc = (bf16_t*)v_cache + slab * l;
-    hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)lw.attn_norm, xn, T, d, c.norm_eps);
+    hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)lw.attn_norm, xn, T, d, c.norm_eps, 1);
     PfGemm g{};
-    g.X = xn; g.W = (const bf16_t*)lw.wqkv; g.C = qkv; g.M = T; g.N = nq + 2 * nkv; g.K = d; g.ldx = d; g.ldw = d; g.ldc = nq + 2 * nkv;
-    if ((rc = pf_gemm4(PF_BF16, g, nullptr, st))) return rc;
+    g.X = xn; g.W = t_qkv; g.C = qkv; g.M = T; g.N = nq + 2 * nkv; g.K = d; g.ldc = nq + 2 * nkv;
+    if ((rc = pf_gemm4(PF_BF16, g, nullptr, 0, st))) return rc;
     hipLaunchKernelGGL(pf_rope_append_kernel, dim3(T), dim3(256), 0, st, qkv, kc, vc, w.rope_table, T, nq, nkv, hd, c.rope_dim, pos0,
                        slot, S);
     // attention over the L cached positions of this slot
@@ -399,17 +460,17 @@ int launch_prefill(const vui_config& c, const vui_weights& w, const void* emb, i
       }
     }
     PfGemm wo{};
-    wo.X = att; wo.ldx = nq; wo.W = (const bf16_t*)lw.wo; wo.ldw = nq; wo.C = x; wo.ldc = d; wo.M = T; wo.N = d; wo.K = nq;
-    if ((rc = pf_gemm4(PF_RESID, wo, nullptr, st))) return rc;
-    hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)lw.mlp_norm, xn, T, d, c.norm_eps);
+    wo.X = att; wo.W = t_o; wo.C = x; wo.ldc = d; wo.M = T; wo.N = d; wo.K = nq;
+    if ((rc = pf_gemm4(PF_RESID, wo, nullptr, 0, st))) return rc;
+    hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)lw.mlp_norm, xn, T, d, c.norm_eps, 1);
     PfGemm f1{};
-    f1.X = xn; f1.ldx = d; f1.W = (const bf16_t*)lw.w1; f1.ldw = d; f1.C = fa; f1.ldc = F; f1.M = T; f1.N = F; f1.K = d;
-    if ((rc = pf_gemm4(PF_BF16, f1, (const bf16_t*)lw.w3, st))) return rc;
+    f1.X = xn; f1.W = t_1; f1.C = fa; f1.ldc = F; f1.M = T; f1.N = F; f1.K = d;
+    if ((rc = pf_gemm4(PF_BF16, f1, t_3, 1, st))) return rc;  // written tiled: operand of W2
     PfGemm f2{};
-    f2.X = fa; f2.ldx = F; f2.W = (const bf16_t*)lw.w2; f2.ldw = F; f2.C = x; f2.ldc = d; f2.M = T; f2.N = d; f2.K = F;
-    if ((rc = pf_gemm4(PF_RESID, f2, nullptr, st))) return rc;
+    f2.X = fa; f2.W = t_2; f2.C = x; f2.ldc = d; f2.M = T; f2.N = d; f2.K = F;
+    if ((rc = pf_gemm4(PF_RESID, f2, nullptr, 0, st))) return rc;
   }
-  hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)w.final_norm, (bf16_t*)out, T, d, c.norm_eps);
+  hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)w.final_norm, (bf16_t*)out, T, d, c.norm_eps, 0);
   hipLaunchKernelGGL(pf_set_len_kernel, dim3(1), dim3(1), 0, st, seq_lens, slot, L);
   HIP_TRY(hipGetLastError());
   return VUI_OK;
