@@ -208,7 +208,7 @@ __global__ __launch_bounds__(256) void pf_rope_append_kernel(bf16_t* qkv, bf16_t
 // when both operands share it).  HD32 = head_dim / 32.
 #define PF_ATT_WAVES (HD32 <= 3 ? 8 : 4)  // the partial outputs of the waves must fit 64 KiB of LDS
 template <int HD32>
-__global__ __launch_bounds__(64 * PF_ATT_WAVES) void pf_attn_kernel(const bf16_t* __restrict__ qkv, const bf16_t* __restrict__ krow,
+__global__ __launch_bounds__(64 * PF_ATT_WAVES) void pf_attn_kernel(const bf16_t* __restrict__ qkv, const bf16_t* __restrict__ kt,
                                                       const bf16_t* __restrict__ vt, bf16_t* __restrict__ att, int T, int L,
                                                       int Lpad, int nq, int nkv, int gsz, int pos0, int window, float scale) {
   constexpr int HD = 32 * HD32, DT = 2 * HD32;
@@ -230,8 +230,9 @@ __global__ __launch_bounds__(64 * PF_ATT_WAVES) void pf_attn_kernel(const bf16_t
   const int t_hi = min(q0 + 15, T - 1);
   const int kend = pos0 + t_hi + 1;
   const int kbeg = (window > 0 ? max(0, pos0 + q0 - window) : 0) & ~31;
-  const bf16_t* kb = krow + kvh * HD + kg * 8;
-  const bf16_t* vb = vt + (size_t)kvh * HD * Lpad;
+  // staged keys / values of this KV head (pf_stage_kv_kernel): a fragment is 16 bytes per lane, 1 KiB contiguous per wave
+  const bf16_t* kb = kt + (size_t)kvh * (Lpad >> 4) * HD32 * 512 + lane * 8;
+  const bf16_t* vb = vt + (size_t)kvh * DT * (Lpad >> 5) * 512 + lane * 8;
 
   pf_floatx4 acc[DT];
 #pragma unroll
@@ -240,21 +241,15 @@ __global__ __launch_bounds__(64 * PF_ATT_WAVES) void pf_attn_kernel(const bf16_t
   for (int k0 = kbeg + 32 * wave; k0 < kend; k0 += 32 * PF_ATT_WAVES) {
     // every load of the step goes out before the first product (keys and values alike: the values do not depend
     // on the scores), so a step is one trip to memory
-    uint4 kf[2][HD32];
-    uint2 vf[DT][2];
+    uint4 kf[2][HD32], vf[DT];
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt) {
-      const bf16_t* kr = kb + (size_t)min(k0 + 16 * kt + l16, L - 1) * nkv;
+    for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int c = 0; c < HD32; ++c) kf[kt][c] = *reinterpret_cast<const uint4*>(kr + c * 32);
-    }
+      for (int c = 0; c < HD32; ++c)
+        kf[kt][c] = *reinterpret_cast<const uint4*>(kb + ((size_t)((k0 >> 4) + kt) * HD32 + c) * 512);
+    // V^T of dims 16 d + l16: the lane's eight keys k0 + 4 kg + r and k0 + 16 + 4 kg + r, in the order of its scores
 #pragma unroll
-    for (int d = 0; d < DT; ++d) {
-      // V^T of dims 16 d + l16: the lane's eight keys k0 + 4 kg + r and k0 + 16 + 4 kg + r, in the order of its scores
-      const bf16_t* vr = vb + (size_t)(16 * d + l16) * Lpad + k0 + 4 * kg;
-      vf[d][0] = *reinterpret_cast<const uint2*>(vr);
-      vf[d][1] = *reinterpret_cast<const uint2*>(vr + 16);
-    }
+    for (int d = 0; d < DT; ++d) vf[d] = *reinterpret_cast<const uint4*>(vb + ((size_t)d * (Lpad >> 5) + (k0 >> 5)) * 512);
     __builtin_amdgcn_sched_barrier(0);
     // scores^T of 32 keys: two tiles of 16 keys x 16 queries
     pf_floatx4 sc[2];
@@ -291,7 +286,7 @@ __global__ __launch_bounds__(64 * PF_ATT_WAVES) void pf_attn_kernel(const bf16_t
     for (int d = 0; d < DT; ++d) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) acc[d][r] *= alpha;
-      acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf_frag(make_uint4(vf[d][0].x, vf[d][0].y, vf[d][1].x, vf[d][1].y)), pf_frag(pf), acc[d], 0, 0, 0);
+      acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf_frag(vf[d]), pf_frag(pf), acc[d], 0, 0, 0);
     }
   }
   // the waves' parts meet: lane holds dims 16 d + 4 kg + r of query l16
@@ -321,19 +316,42 @@ __global__ __launch_bounds__(64 * PF_ATT_WAVES) void pf_attn_kernel(const bf16_t
   }
 }
 
-// values of one row's cache slab, (L x KV*hd) -> per KV head (hd x Lpad), zero beyond L
-__global__ __launch_bounds__(256) void pf_transpose_v_kernel(const bf16_t* vc, bf16_t* vt, int L, int Lpad, int nkv, int hd) {
-  __shared__ bf16_t tile[32][33];
-  const int j0 = blockIdx.x * 32, f0 = blockIdx.y * 32;  // f over nkv (= KV*hd)
-  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
-  for (int r = ty; r < 32; r += 8) {
-    const int j = j0 + r, f = f0 + tx;
-    tile[r][tx] = (j < L && f < nkv) ? vc[(size_t)j * nkv + f] : (bf16_t)0;
+// Keys and values of one row's cache slab in the operand layouts of pf_attn_kernel, zero beyond position L.
+// Keys of KV head g: blocks of 16 keys x 32 dims, block ((g * Lpad / 16 + j / 16) * hd / 32 + dim / 32) of 512
+// elements, lane (j % 16) + 16 * ((dim % 32) / 8) holds its 8 dims at 8 * lane.  Values, transposed: blocks of 16
+// dims x 32 keys, block ((g * hd / 16 + dim / 16) * Lpad / 32 + j / 32), lane (dim % 16) + 16 * ((j % 16) / 4)
+// holds keys j % 4 of both halves (j % 32) / 16 of the step at 8 * lane + 4 * half + j % 4 - the order in which a
+// lane of the attention kernel holds the scores of a step.  One workgroup: 32 keys x 32 features.
+__global__ __launch_bounds__(256) void pf_stage_kv_kernel(const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+                                                          bf16_t* __restrict__ kt, bf16_t* __restrict__ vt, int L, int Lpad,
+                                                          int nkv, int hd) {
+  __shared__ bf16_t tile[32][34];
+  const int j0 = blockIdx.x * 32, f0 = blockIdx.y * 32;  // f over nkv (= KV * hd); hd is a multiple of 32
+  const int tid = threadIdx.x;
+  const int g = f0 / hd, dim0 = f0 % hd;
+  if (tid < 128) {  // keys: 32 keys x four 8-dim pieces
+    const int key = tid >> 2, pc = tid & 3, j = j0 + key;
+    const uint4 v = j < L ? *reinterpret_cast<const uint4*>(kc + (size_t)j * nkv + f0 + pc * 8) : make_uint4(0, 0, 0, 0);
+    const size_t blk = ((size_t)g * (Lpad >> 4) + (j >> 4)) * (hd >> 5) + (dim0 >> 5);
+    *reinterpret_cast<uint4*>(kt + blk * 512 + ((j & 15) + 16 * pc) * 8) = v;
+  }
+  {
+    const int tx = tid & 31, ty = tid >> 5;  // 32 x 8
+    for (int r = ty; r < 32; r += 8) {
+      const int j = j0 + r;
+      tile[r][tx] = j < L ? vc[(size_t)j * nkv + f0 + tx] : (bf16_t)0;
+    }
   }
   __syncthreads();
-  for (int r = ty; r < 32; r += 8) {
-    const int f = f0 + r, j = j0 + tx;
-    if (f < nkv && j < Lpad) vt[(size_t)f * Lpad + j] = tile[tx][r];  // head = f / hd, feature f % hd: rows of hd x Lpad blocks
+  {
+    // thread: dim dl of the 32, piece q = 4 * half + key group: four consecutive keys
+    const int dl = tid >> 3, q = tid & 7, half = q >> 2, kgk = q & 3;
+    const int dim = dim0 + dl;
+    const int jj = half * 16 + kgk * 4;
+    const uint32_t lo = (uint32_t)tile[jj][dl] | ((uint32_t)tile[jj + 1][dl] << 16);
+    const uint32_t hi = (uint32_t)tile[jj + 2][dl] | ((uint32_t)tile[jj + 3][dl] << 16);
+    const size_t blk = ((size_t)g * (hd >> 4) + (dim >> 4)) * (Lpad >> 5) + (j0 >> 5);
+    *reinterpret_cast<uint2*>(vt + blk * 512 + ((dim & 15) + 16 * kgk) * 8 + 4 * half) = make_uint2(lo, hi);
   }
 }
 
@@ -352,7 +370,7 @@ static int pf_gemm4(int epi, const PfGemm& g, const bf16_t* W2, int c_tiled, hip
 
 static size_t pf_align(size_t b) { return (b + 255) & ~(size_t)255; }
 
-// scratch: residual x, normed xn, qkv, attention output, FFN buffer, transposed values
+// scratch: residual x, normed xn, qkv, attention output, FFN buffer, staged keys and values
 size_t prefill_scratch_bytes(const vui_config& c, int T, int L) {
   const size_t d = c.d_model, nq = (size_t)c.n_heads * c.head_dim, nkv = (size_t)c.n_kv_heads * c.head_dim;
   const size_t Lpad = ((size_t)L + 63) & ~(size_t)63;
@@ -362,7 +380,7 @@ size_t prefill_scratch_bytes(const vui_config& c, int T, int L) {
   b += pf_align((size_t)T * (nq + 2 * nkv) * 2);
   b += pf_align(T16 * nq * 2);
   b += pf_align(T16 * c.ffn * 2);
-  b += pf_align(nkv * Lpad * 2);
+  b += pf_align(nkv * Lpad * 2) * 2;
   return b;
 }
 
@@ -426,6 +444,7 @@ int launch_prefill(const vui_config& c, const vui_weights& w, const void* tiled_
   bf16_t* qkv = (bf16_t*)take((size_t)T * (nq + 2 * nkv) * 2);  //  what a GEMM reads there only reaches output rows it drops)
   bf16_t* att = (bf16_t*)take(T16 * nq * 2);                    // attention output, tiled
   bf16_t* fa = (bf16_t*)take(T16 * F * 2);                      // SwiGLU product, tiled
+  bf16_t* kt = (bf16_t*)take((size_t)nkv * Lpad * 2);                // staged keys and values of the slot
   bf16_t* vt = (bf16_t*)take((size_t)nkv * Lpad * 2);
   HIP_TRY(hipMemcpyAsync(x, emb, (size_t)T * d * 2, hipMemcpyDeviceToDevice, st));
   const size_t slab = (size_t)c.n_slots * S * nkv;
@@ -449,14 +468,14 @@ int launch_prefill(const vui_config& c, const vui_weights& w, const void* tiled_
     // attention over the L cached positions of this slot
     const bf16_t* krow = kc + (size_t)slot * S * nkv;
     const bf16_t* vrow = vc + (size_t)slot * S * nkv;
-    hipLaunchKernelGGL(pf_transpose_v_kernel, dim3(Lpad / 32, (nkv + 31) / 32), dim3(256), 0, st, vrow, vt, L, Lpad, nkv, hd);
+    hipLaunchKernelGGL(pf_stage_kv_kernel, dim3(Lpad / 32, nkv / 32), dim3(256), 0, st, krow, vrow, kt, vt, L, Lpad, nkv, hd);
     {
       const dim3 grid((T + 15) / 16, H);
       switch (hd / 32) {
-        case 1: hipLaunchKernelGGL(pf_attn_kernel<1>, grid, dim3(512), 0, st, qkv, krow, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, c.window, scale); break;
-        case 2: hipLaunchKernelGGL(pf_attn_kernel<2>, grid, dim3(512), 0, st, qkv, krow, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, c.window, scale); break;
-        case 3: hipLaunchKernelGGL(pf_attn_kernel<3>, grid, dim3(512), 0, st, qkv, krow, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, c.window, scale); break;
-        default: hipLaunchKernelGGL(pf_attn_kernel<4>, grid, dim3(256), 0, st, qkv, krow, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, c.window, scale); break;
+        case 1: hipLaunchKernelGGL(pf_attn_kernel<1>, grid, dim3(512), 0, st, qkv, kt, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, c.window, scale); break;
+        case 2: hipLaunchKernelGGL(pf_attn_kernel<2>, grid, dim3(512), 0, st, qkv, kt, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, c.window, scale); break;
+        case 3: hipLaunchKernelGGL(pf_attn_kernel<3>, grid, dim3(512), 0, st, qkv, kt, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, c.window, scale); break;
+        default: hipLaunchKernelGGL(pf_attn_kernel<4>, grid, dim3(256), 0, st, qkv, kt, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, c.window, scale); break;
       }
     }
     PfGemm wo{};
