@@ -93,7 +93,8 @@ int vui_version(void);
 
 /* Bytes of device workspace a context needs for up to max_batch rows.  For a configuration that has the one-pass
  * prompt ingestion (vui_prefill) this includes a second copy of the layers' projection weights in the operand
- * layout of its GEMMs (Vui Nano: 311 MB), written by vui_ctx_init. */
+ * layout of its GEMMs (Vui Nano: 311 MB), and for one that has the batched depth-head kernel a copy of the depth
+ * head's matrices in that kernel's layout (58 MB); both are written by vui_ctx_init. */
 int64_t vui_workspace_bytes(const vui_config* cfg, int max_batch);
 /* Bytes of ONE of the two (K or V) backbone caches: layers * slots * S * KV * hd elements.
  * Layout (layers, slots, S, KV, hd); layer l's (slots, S, KV, hd) slab is what the reference

@@ -51,6 +51,8 @@ def test_sizes(lib):
     n1, n16 = lib.vui_workspace_bytes(C.byref(c), 1), lib.vui_workspace_bytes(C.byref(c), 16)
     # the workspace of a bf16 context also holds the layers' projection weights in the prefill pass's operand layout
     tiled = 22 * (2304 * 768 + 768 * 768 + 2 * 2048 * 768 + 768 * 2048) * 2
+    # ... and the depth head's matrices in the batched kernel's layout (4 layers, 15 codebook heads, the projection)
+    tiled += (4 * (4 * 512 * 512 + 3 * 1408 * 512) + 15 * 2048 * 512 + 512 * 768) * 2
     assert 0 < n1 < n16 and tiled < n1 and n16 - tiled < 64 << 20
     assert lib.vui_attn_scratch_bytes(1, 8, 96, 32) >= 8 * 32 * 98 * 4
     assert lib.vui_version() >= 1

@@ -37,6 +37,8 @@ struct vui_ctx {
   vui_weights* wdev;
   uint32_t* ctl;  // [0] epoch, [1] arrive, [2] err
   void* pf_w;     // projection weights of every layer in the prefill GEMMs' operand layout (bf16 contexts)
+  void* rq_tw;    // the depth head's matrices in the batched kernel's operand layout
+  vui_weights* wdev_t;  // device copy of the weight table with those matrices' pointers
   int fused_ok, fused_on, nwg, ns;
   size_t lds_bytes;
   char fused_why[96];
@@ -114,6 +116,8 @@ static size_t carve(const vui_config* c, int Bm, vui_ctx* x) {
   TAKE(wdev, vui_weights*, sizeof(vui_weights));
   TAKE(ctl, uint32_t*, 256);
   TAKE(pf_w, void*, prefill_weight_bytes(*c));  // empty when the configuration has no prefill pass
+  TAKE(rq_tw, void*, rq_batch_weight_bytes(*c, FUSED_NWG));  // empty when the batched depth-head kernel is unavailable
+  TAKE(wdev_t, vui_weights*, sizeof(vui_weights));
 #undef TAKE
   return cv.off;
 }
@@ -183,6 +187,12 @@ int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream) {
   if ((rc = launch_fill_u32(ctx->ctl, 0u, 64, st))) return rc;
   HIP_TRY(hipMemcpyAsync(ctx->wdev, &ctx->w, sizeof(vui_weights), hipMemcpyHostToDevice, st));
   if (prefill_weight_bytes(ctx->cfg) && (rc = prefill_tile_weights(ctx->cfg, ctx->w, ctx->pf_w, st))) return rc;
+  if (rq_batch_weight_bytes(ctx->cfg, FUSED_NWG)) {
+    vui_weights wt;
+    if ((rc = rq_batch_tile_weights(ctx->cfg, ctx->w, ctx->rq_tw, &wt, st))) return rc;
+    HIP_TRY(hipMemcpyAsync(ctx->wdev_t, &wt, sizeof(vui_weights), hipMemcpyHostToDevice, st));
+    HIP_TRY(hipStreamSynchronize(st));  // wt is a local
+  }
   HIP_TRY(hipStreamSynchronize(st));
   ctx->fused_ok = 0;
   ctx->fused_why[0] = 0;
@@ -429,7 +439,7 @@ int vui_rq_generate(vui_ctx* ctx, const void* hidden, const int64_t* code0, cons
     return launch_frame(a, ctx->nwg, ctx->lds_bytes, st);
   }
   if (ctx->rqb_ok && ctx->fused_on && B > 1)
-    return launch_rq_batch(c, ctx->wdev, hidden, code0, logit_bias, n_q, sp->temperature, sp->top_k, sp->seed, sp->frame_ctr,
+    return launch_rq_batch(c, ctx->wdev_t, hidden, code0, logit_bias, n_q, sp->temperature, sp->top_k, sp->seed, sp->frame_ctr,
                            codes_out, codes_stride, zero_pad, B, ctx->ll, ctx->ctl, ctx->nwg, st);
   const int R = c.rq_dim, CS = c.codebook_size;
   const char* pos_emb = (const char*)ctx->w.rq_pos_emb;

@@ -193,6 +193,8 @@ int launch_frame(const FrameArgs& a, int nwg, size_t lds_bytes, hipStream_t st);
 size_t rq_batch_ll_words(const vui_config& c);
 size_t rq_batch_lds_bytes(const vui_config& c);
 bool rq_batch_supported(const vui_config& c, int nwg, char* why, size_t why_len);
+size_t rq_batch_weight_bytes(const vui_config& c, int nwg);  // tiled copies of the depth head's matrices; 0: kernel unavailable
+int rq_batch_tile_weights(const vui_config& c, const vui_weights& w, void* dst, vui_weights* tiled, hipStream_t st);
 int rq_batch_max_resident(size_t lds_bytes);
 int launch_rq_batch(const vui_config& c, const vui_weights* wdev, const void* hidden, const int64_t* code0, const float* logit_bias,
                     int n_q, float temp, int topk, uint64_t seed, const int32_t* frame_ctr, int64_t* codes_out, int codes_stride,

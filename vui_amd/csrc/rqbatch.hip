@@ -41,18 +41,34 @@ struct Tile { int n0, N, K; bool on; };
 template <int MAXS, bool DUAL>
 struct TileW { uint4 a[MAXS]; uint4 b[DUAL ? MAXS : 1]; };
 
+// The matrices this kernel multiplies by are read from a copy in "tiled" form (rb_tile_kernel): inside every band of
+// 16 rows, the block of columns 32 s .. 32 s + 31 is 512 consecutive elements, the 8 elements of lane
+// (row % 16) + 16 * ((col % 32) / 8) at 8 * lane.  A wave's fragment load is then 1 KiB contiguous; from the
+// row-major form the 16 lanes of a quarter-wave would read 16 different lines, which the address unit serves at
+// about a quarter of the rate.  A band starts where it does in the row-major form (16 rows x K elements each).
 template <int MAXS, bool DUAL>
 __device__ __forceinline__ void tile_prefetch(const bf16_t* W, const bf16_t* W2, const Tile& t, TileW<MAXS, DUAL>& r) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l16 = lane & 15, kg = lane >> 4;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   if (!t.on) return;
-  const size_t row = (size_t)min(t.n0 + l16, t.N - 1) * t.K;
+  const size_t band = (size_t)t.n0 * t.K + lane * 8;  // n0 is a multiple of 16, N as well: the band is inside the matrix
 #pragma unroll
   for (int i = 0; i < MAXS; ++i) {
-    const int k = (wave + 4 * i) * 32 + kg * 8;
-    const bool on = k < t.K;
-    r.a[i] = on ? *reinterpret_cast<const uint4*>(W + row + k) : make_uint4(0, 0, 0, 0);
-    if (DUAL) r.b[i] = on ? *reinterpret_cast<const uint4*>(W2 + row + k) : make_uint4(0, 0, 0, 0);
+    const int s = wave + 4 * i;
+    const bool on = s * 32 < t.K;
+    r.a[i] = on ? *reinterpret_cast<const uint4*>(W + band + (size_t)s * 512) : make_uint4(0, 0, 0, 0);
+    if (DUAL) r.b[i] = on ? *reinterpret_cast<const uint4*>(W2 + band + (size_t)s * 512) : make_uint4(0, 0, 0, 0);
   }
+}
+
+// row-major (N x K, N % 16 == 0, K % 32 == 0) -> tiled; one 8-element piece per thread
+__global__ __launch_bounds__(256) void rb_tile_kernel(const bf16_t* __restrict__ src, bf16_t* __restrict__ dst, size_t N, int K) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const int per_row = K >> 3;
+  if (i >= N * per_row) return;
+  const size_t n = i / per_row;
+  const int k = (int)(i % per_row) * 8;
+  const size_t o = (n >> 4) * 16 * (size_t)K + (size_t)(k >> 5) * 512 + ((n & 15) + 16 * ((k & 31) >> 3)) * 8;
+  *reinterpret_cast<uint4*>(dst + o) = *reinterpret_cast<const uint4*>(src + n * K + k);
 }
 
 // xp: activations of the group's rows as packed bf16 pairs (row stride xs words) followed by one zero row that
@@ -600,6 +616,41 @@ bool rq_batch_supported(const vui_config& c, int nwg, char* why, size_t why_len)
   }
   if (r && why) snprintf(why, why_len, "%s", r);
   return r == nullptr;
+}
+
+// elements of the matrices the kernel multiplies by: the layers, the codebook heads, the hidden-state projection
+static size_t rb_weight_elems(const vui_config& c) {
+  const size_t R = c.rq_dim, F = c.rq_ffn, d = c.d_model;
+  return (size_t)c.rq_layers * (3 * R * R + R * R + 3 * F * R) + (size_t)(c.n_quantizers - 1) * c.codebook_size * R + (R != d ? R * d : 0);
+}
+size_t rq_batch_weight_bytes(const vui_config& c, int nwg) {
+  return rq_batch_supported(c, nwg, nullptr, 0) ? rb_weight_elems(c) * 2 : 0;
+}
+// One-time: the tiled copies into dst; *tiled = w with those matrices' pointers replaced by the copies'.
+int rq_batch_tile_weights(const vui_config& c, const vui_weights& w, void* dst, vui_weights* tiled, hipStream_t st) {
+  const size_t R = c.rq_dim, F = c.rq_ffn, d = c.d_model;
+  bf16_t* o = (bf16_t*)dst;
+  *tiled = w;
+  auto tile = [&](const void* src, size_t N, size_t K) -> const void* {
+    const size_t pieces = N * (K / 8);
+    hipLaunchKernelGGL(rb_tile_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, st, (const bf16_t*)src, o, N, (int)K);
+    const void* r = o;
+    o += N * K;
+    return r;
+  };
+  for (int l = 0; l < c.rq_layers; ++l) {
+    const vui_rq_layer_weights& L = w.rq_layers[l];
+    vui_rq_layer_weights& T = tiled->rq_layers[l];
+    T.wqkv = tile(L.wqkv, 3 * R, R);
+    T.wo = tile(L.wo, R, R);
+    T.w1 = tile(L.w1, F, R);
+    T.w3 = tile(L.w3, F, R);
+    T.w2 = tile(L.w2, R, F);
+  }
+  tiled->rq_head_w = tile(w.rq_head_w, (size_t)(c.n_quantizers - 1) * c.codebook_size, R);
+  if (R != d && w.rq_backbone_proj) tiled->rq_backbone_proj = tile(w.rq_backbone_proj, R, d);
+  HIP_TRY(hipGetLastError());
+  return VUI_OK;
 }
 
 int rq_batch_max_resident(size_t lds_bytes) {
