@@ -2,11 +2,12 @@
 //
 //   Decoder.forward_flash / Engine._prefill_emb with T > 1  (src/vui/model.py:534-549, engine.py:674-694)
 //
-// bf16 only.  Per layer: row RMSNorm, QKV GEMM, RoPE + cache append, transpose of the values, causal attention of
-// the new positions against the cache itself (scores never leave the registers; probabilities rounded to bf16
-// before they meet the values), out_proj GEMM with the residual add in its epilogue, row RMSNorm, one GEMM over
-// W1 and W3 with the SwiGLU product in its epilogue, W2 GEMM with residual: nine launches.
-// Every GEMM is C (M x N) = X (M x K) W^T (N x K), K contiguous in both operands, on the matrix cores.
+// bf16 only.  Per layer: row RMSNorm, QKV GEMM, one kernel that rotates the new keys, appends keys and values to the
+// cache and stages the slot's keys / transposed values in operand layout, causal attention of the new positions
+// against them (the same kernel rotates the queries in place; scores never leave the registers; probabilities
+// rounded to bf16 before they meet the values), out_proj GEMM with the residual add in its epilogue, row RMSNorm, one GEMM over
+// W1 and W3 with the SwiGLU product in its epilogue, W2 GEMM with residual: eight launches.
+// Every GEMM is C (M x N) = X (M x K) W^T (N x K) on the matrix cores, both operands in the tiled layout below.
 //
 // Rounding points are those of the single-position step (one rounding after each linear, two in
 // the norm, products of the rotation rounded before their sum, residual sums rounded).
@@ -174,29 +175,20 @@ __global__ __launch_bounds__(256) void pf_rownorm_kernel(const bf16_t* x, const 
   }
 }
 
-// interleaved rotation of q (in place) and k, append of k and v to the cache at positions pos0 + t
-// (src/vui/rope.py:16-77, model.py:234-247)
-__global__ __launch_bounds__(256) void pf_rope_append_kernel(bf16_t* qkv, bf16_t* kc, bf16_t* vc, const float* rope, int T,
-                                                             int nq, int nkv, int hd, int rope_dim, int pos0, int slot, int S) {
-  const int t = blockIdx.x;
-  const int pos = pos0 + t;
-  bf16_t* row = qkv + (size_t)t * (nq + 2 * nkv);
-  for (int pr = threadIdx.x; pr < (nq + 2 * nkv) / 2; pr += blockDim.x) {
-    const int n = 2 * pr;
-    uint32_t v = *reinterpret_cast<const uint32_t*>(row + n);
-    int region, m;
-    if (n < nq) { region = 0; m = n; }
-    else if (n < nq + nkv) { region = 1; m = n - nq; }
-    else { region = 2; m = n - nq - nkv; }
-    const int dd = m % hd;
-    if (region != 2 && dd < rope_dim) {
-      const float4 f = *reinterpret_cast<const float4*>(rope + ((size_t)pos * rope_dim + dd) * 2);  // cos, sin of dd and dd + 1
-      const float a = bf_lo(v), b = bf_hi(v);
-      v = f2bf2(rope_mix(a, f.x, -b, f.y), rope_mix(b, f.z, a, f.w));
+// interleaved rotation (src/vui/rope.py:16-77) of the four pairs of an 8-element piece whose first dim is dd (even)
+// at position pos; pairs at or beyond rope_dim pass through
+__device__ __forceinline__ uint4 pf_rope8(uint4 v, const float* __restrict__ rope, int pos, int rope_dim, int dd) {
+  uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d2 = dd + 2 * i;
+    if (d2 < rope_dim) {
+      const float4 f = *reinterpret_cast<const float4*>(rope + ((size_t)pos * rope_dim + d2) * 2);  // cos, sin of d2 and d2 + 1
+      const float a = bf_lo(w[i]), b = bf_hi(w[i]);
+      w[i] = f2bf2(rope_mix(a, f.x, -b, f.y), rope_mix(b, f.z, a, f.w));
     }
-    if (region == 0) *reinterpret_cast<uint32_t*>(row + n) = v;
-    else *reinterpret_cast<uint32_t*>((region == 1 ? kc : vc) + ((size_t)slot * S + pos) * nkv + m) = v;
   }
+  return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
 // Attention of the new positions against the row's cache without materialised scores: one workgroup per
@@ -316,22 +308,39 @@ __global__ __launch_bounds__(64 * PF_ATT_WAVES) void pf_attn_kernel(const bf16_t
   }
 }
 
-// Keys and values of one row's cache slab in the operand layouts of pf_attn_kernel, zero beyond position L.
+// Keys and values of one row's cache slab in the operand layouts of pf_attn_kernel, zero beyond position L; the new
+// positions pos0 .. L - 1 are taken from the projection output, the keys rotated (src/vui/model.py:234-247), and
+// appended to the cache on the way.
 // Keys of KV head g: blocks of 16 keys x 32 dims, block ((g * Lpad / 16 + j / 16) * hd / 32 + dim / 32) of 512
 // elements, lane (j % 16) + 16 * ((dim % 32) / 8) holds its 8 dims at 8 * lane.  Values, transposed: blocks of 16
 // dims x 32 keys, block ((g * hd / 16 + dim / 16) * Lpad / 32 + j / 32), lane (dim % 16) + 16 * ((j % 16) / 4)
 // holds keys j % 4 of both halves (j % 32) / 16 of the step at 8 * lane + 4 * half + j % 4 - the order in which a
 // lane of the attention kernel holds the scores of a step.  One workgroup: 32 keys x 32 features.
-__global__ __launch_bounds__(256) void pf_stage_kv_kernel(const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
-                                                          bf16_t* __restrict__ kt, bf16_t* __restrict__ vt, int L, int Lpad,
-                                                          int nkv, int hd) {
+__global__ __launch_bounds__(256) void pf_stage_kv_kernel(bf16_t* __restrict__ qkv, bf16_t* __restrict__ kc, bf16_t* __restrict__ vc,
+                                                          bf16_t* __restrict__ kt, bf16_t* __restrict__ vt, const float* __restrict__ rope,
+                                                          int L, int Lpad, int nq, int nkv, int hd, int rope_dim, int pos0) {
   __shared__ bf16_t tile[32][34];
-  const int j0 = blockIdx.x * 32, f0 = blockIdx.y * 32;  // f over nkv (= KV * hd); hd is a multiple of 32
   const int tid = threadIdx.x;
+  const int ldq = nq + 2 * nkv;
+  if ((int)blockIdx.y >= nkv / 32) {
+    // the other workgroups rotate the queries in place: 32 rows x 32 dims each
+    const int t = blockIdx.x * 32 + (tid >> 2), f = ((int)blockIdx.y - nkv / 32) * 32 + (tid & 3) * 8;
+    if (tid < 128 && t < L - pos0) {
+      uint4* q = reinterpret_cast<uint4*>(qkv + (size_t)t * ldq + f);
+      *q = pf_rope8(*q, rope, pos0 + t, rope_dim, f % hd);
+    }
+    return;
+  }
+  const int j0 = blockIdx.x * 32, f0 = blockIdx.y * 32;  // f over nkv (= KV * hd); hd is a multiple of 32
   const int g = f0 / hd, dim0 = f0 % hd;
   if (tid < 128) {  // keys: 32 keys x four 8-dim pieces
     const int key = tid >> 2, pc = tid & 3, j = j0 + key;
-    const uint4 v = j < L ? *reinterpret_cast<const uint4*>(kc + (size_t)j * nkv + f0 + pc * 8) : make_uint4(0, 0, 0, 0);
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (j < pos0) v = *reinterpret_cast<const uint4*>(kc + (size_t)j * nkv + f0 + pc * 8);
+    else if (j < L) {
+      v = pf_rope8(*reinterpret_cast<const uint4*>(qkv + (size_t)(j - pos0) * ldq + nq + f0 + pc * 8), rope, j, rope_dim, dim0 + pc * 8);
+      *reinterpret_cast<uint4*>(kc + (size_t)j * nkv + f0 + pc * 8) = v;
+    }
     const size_t blk = ((size_t)g * (Lpad >> 4) + (j >> 4)) * (hd >> 5) + (dim0 >> 5);
     *reinterpret_cast<uint4*>(kt + blk * 512 + ((j & 15) + 16 * pc) * 8) = v;
   }
@@ -339,7 +348,10 @@ __global__ __launch_bounds__(256) void pf_stage_kv_kernel(const bf16_t* __restri
     const int tx = tid & 31, ty = tid >> 5;  // 32 x 8
     for (int r = ty; r < 32; r += 8) {
       const int j = j0 + r;
-      tile[r][tx] = j < L ? vc[(size_t)j * nkv + f0 + tx] : (bf16_t)0;
+      bf16_t v = (bf16_t)0;
+      if (j < pos0) v = vc[(size_t)j * nkv + f0 + tx];
+      else if (j < L) { v = qkv[(size_t)(j - pos0) * ldq + nq + nkv + f0 + tx]; vc[(size_t)j * nkv + f0 + tx] = v; }
+      tile[r][tx] = v;
     }
   }
   __syncthreads();
@@ -463,12 +475,11 @@ int launch_prefill(const vui_config& c, const vui_weights& w, const void* tiled_
     PfGemm g{};
     g.X = xn; g.W = t_qkv; g.C = qkv; g.M = T; g.N = nq + 2 * nkv; g.K = d; g.ldc = nq + 2 * nkv;
     if ((rc = pf_gemm4(PF_BF16, g, nullptr, 0, st))) return rc;
-    hipLaunchKernelGGL(pf_rope_append_kernel, dim3(T), dim3(256), 0, st, qkv, kc, vc, w.rope_table, T, nq, nkv, hd, c.rope_dim, pos0,
-                       slot, S);
     // attention over the L cached positions of this slot
-    const bf16_t* krow = kc + (size_t)slot * S * nkv;
-    const bf16_t* vrow = vc + (size_t)slot * S * nkv;
-    hipLaunchKernelGGL(pf_stage_kv_kernel, dim3(Lpad / 32, nkv / 32), dim3(256), 0, st, krow, vrow, kt, vt, L, Lpad, nkv, hd);
+    bf16_t* krow = kc + (size_t)slot * S * nkv;
+    bf16_t* vrow = vc + (size_t)slot * S * nkv;
+    hipLaunchKernelGGL(pf_stage_kv_kernel, dim3(Lpad / 32, (nkv + nq) / 32), dim3(256), 0, st, qkv, krow, vrow, kt, vt, w.rope_table, L, Lpad, nq, nkv,
+                       hd, c.rope_dim, pos0);
     {
       const dim3 grid((T + 15) / 16, H);
       switch (hd / 32) {
