@@ -114,3 +114,35 @@ def test_prefill_nano_576_positions():
     assert rel_err(ka, m.decoder._k[:, 0, :576]) <= BF16_TOL
     k0a, k0b = ka[0].float(), m.decoder._k[0, 0, :576].float()  # layer 0 keys: only the summation order differs
     assert float((k0a != k0b).float().mean()) < 0.01
+
+
+@pytest.mark.parametrize("heads,kv,rope_dim", [(4, 2, 64), (2, 1, 64), (2, 2, 128)])
+def test_prefill_other_head_dims(heads, kv, rope_dim):
+    """head_dim 64 and 128 (other instantiations of the attention kernel; 128 runs four waves per workgroup), grouped
+    KV heads, a rotation that covers only part of the head: the pass against the oracle's bf16 regime, and the
+    cache it leaves against the position-by-position path, across a block boundary of the staged keys."""
+    d = O.Dims(d_model=256, n_layers=2, n_heads=heads, n_kv_heads=kv, n_quantizers=4, codebook_size=32, rq_d_model=64,
+               rq_n_layers=1, rq_n_heads=2, vocab_size=50, max_seqlen=192, rope_dim=rope_dim)
+    assert d.head_dim in (64, 128)
+    sd = O.synthetic_state_dict(d, **TINY_SD)
+    sdb = {k: O.rnd(v, BF) for k, v in sd.items()}
+    o = O.OracleModel(d, sdb, BF, n_slots=1, max_seqlen=192)
+    m = make_model(d, sd, BF, max_seqlen=192)
+    m.decoder.allocate_flash_kv_cache(1, m.device, BF)
+    assert m.decoder._prefill_available()
+    m2 = make_model(d, sd, BF, max_seqlen=192)
+    m2.decoder.allocate_flash_kv_cache(1, m2.device, BF)
+    m2.decoder.PREFILL_MIN = 10 ** 9
+    g = torch.Generator().manual_seed(3)
+    pos = 0
+    for T in (45, 83):  # 45 + 83 = 128 positions: the second block starts inside a staged block of 32 keys
+        emb = O.rnd(torch.randn(T, d.d_model, generator=g) * 0.5, BF)
+        ref = o.prefill(emb, slot=0)
+        got = m.decoder.forward_flash(emb[None].to(BF).cuda(), None)[0]
+        want = m2.decoder.forward_flash(emb[None].to(BF).cuda(), None)[0]
+        pos += T
+        assert int(m.decoder.flash_kv_caches[0].seq_lens[0]) == pos
+        assert rel_err(got, ref) <= BF16_TOL, rel_err(got, ref)
+        assert rel_err(got, want) <= BF16_TOL, rel_err(got, want)
+    for mine, theirs in ((m.decoder._k, m2.decoder._k), (m.decoder._v, m2.decoder._v)):
+        assert rel_err(mine[:, 0, :pos], theirs[:, 0, :pos]) <= BF16_TOL
