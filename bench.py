@@ -284,6 +284,33 @@ def copy_line():
             "frac_of_8TBs": round(2 * (1 << 30) / us / 1e3 / HBM_PEAK_GBS, 3)}
 
 
+def loadpat_line():
+    """What an operand fragment costs to fetch: 16-byte-per-lane loads from a 3 MB (L2-sized) buffer under three
+    lane -> address patterns, 4096 workgroups x 384 loads per lane each (vui_debug_load_pattern)."""
+    import torch
+
+    from vui_amd import _lib
+
+    lib = _lib.load()
+    buf = torch.ones(2048 * 1536, dtype=torch.uint8, device="cuda")
+    sink = torch.zeros(16, dtype=torch.uint8, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    grid, iters = 4096, 48
+    out = {"config": "load_pattern_16B_per_lane", "buffer_bytes": buf.numel()}
+    for pat, name in ((0, "rows16_x_64B"), (1, "rows8_x_128B"), (2, "contiguous_1KiB")):
+        best = None
+        for _ in range(5):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            _lib.check(lib.vui_debug_load_pattern(pat, grid, iters, buf.data_ptr(), buf.numel(), sink.data_ptr(), st), "vui_debug_load_pattern")
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1)
+            best = ms if best is None else min(best, ms)
+        out[name + "_TBs"] = round(grid * 256 * iters * 128 / best / 1e9, 2)
+    return out
+
+
 def suite(model, eng, d, sd, preset="A"):
     """Extra lines for the other benchmark configs: backbone step at KV 256/1024/4096, depth head alone,
     16 int8 streams with ragged caches."""
@@ -372,6 +399,7 @@ def suite(model, eng, d, sd, preset="A"):
     lines.append(b16_line(sd, preset))
     lines.append(serve_line(sd, preset))
     lines.append(copy_line())
+    lines.append(loadpat_line())
     return lines
 
 
@@ -417,6 +445,8 @@ def main():
                     help="print only the 16-stream int8 line (the run its rocprofv3 summaries come from)")
     ap.add_argument("--vocoder-only", action="store_true",
                     help="print only the vocoder line (the run rocprofv3 summaries of the vocoder kernels come from)")
+    ap.add_argument("--loadpat-only", action="store_true",
+                    help="print only the load-pattern line (what an operand fragment costs to fetch)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (streams are independent); "
@@ -424,6 +454,9 @@ def main():
         sys.exit(2)
     if args.vocoder_only:
         print(json.dumps(vocoder_line()[1]))
+        return
+    if args.loadpat_only:
+        print(json.dumps(loadpat_line()))
         return
     if args.prefill_only:
         import torch

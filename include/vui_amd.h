@@ -131,6 +131,13 @@ int vui_ctx_status(vui_ctx* ctx);
  * it off.  No counterpart in the reference. */
 int vui_debug_phase_clock(vui_ctx* ctx, uint64_t* buf, int cap, int workgroup);
 
+/* Measurement aid behind the operand layouts of the prompt-ingestion pass: `grid` workgroups of 256 threads each
+ * issue iters x 8 loads of 16 bytes per lane from buf (buf_bytes >= 1536, 16-byte aligned; every address is reduced
+ * modulo the buffer) with lane -> address pattern 0 (16 rows x 64 bytes per instruction: an operand fragment read from
+ * a row-major matrix), 1 (8 rows x 128 bytes) or 2 (1 KiB contiguous); bytes moved = grid * 256 * iters * 128.  sink:
+ * 16 writable bytes.  No counterpart in the reference. */
+int vui_debug_load_pattern(int pattern, int grid, int iters, const void* buf, int64_t buf_bytes, void* sink, vui_stream_t stream);
+
 /* One backbone decode step for B rows (B <= max_batch).
  *   Engine._backbone_decode_body / _backbone_decode_body_b  (engine.py:434-449, 485-502)
  *   Vui._decode_step_inner                                  (model.py:1280-1287)

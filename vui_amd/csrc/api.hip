@@ -236,6 +236,10 @@ int vui_debug_phase_clock(vui_ctx* ctx, uint64_t* buf, int cap, int workgroup) {
   return VUI_OK;
 }
 
+int vui_debug_load_pattern(int pattern, int grid, int iters, const void* buf, int64_t buf_bytes, void* sink, vui_stream_t stream) {
+  return launch_load_pattern(pattern, grid, iters, buf, buf_bytes, sink, (hipStream_t)stream);
+}
+
 int vui_ctx_status(vui_ctx* ctx) {
   if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
   uint32_t h[4] = {0, 0, 0, 0};
