@@ -877,35 +877,40 @@ struct CvFinal {
   const int* ctr;
 };
 
+#define FIN_TW 16  // output columns per workgroup: 120 workgroups per frame, and a window small enough that every
+                   // thread has all its loads in flight at once (64 columns: 30 workgroups, four rounds of loads)
 __global__ __launch_bounds__(256) void cv_final_kernel(const CvFinal p) {
-  extern __shared__ float xs[];  // C x (64 + k - 1) window of the ring | 4 x 64 partial sums | C x k weights
-  const int tid = threadIdx.x, qd = tid >> 6, l = tid & 63;
-  const int t0 = blockIdx.x * 64, W = 64 + p.k - 1;
+  extern __shared__ float xs[];  // C x (FIN_TW + k - 1) window of the ring | 16 x FIN_TW partial sums | C x k weights
+  const int tid = threadIdx.x, qd = tid / FIN_TW, l = tid % FIN_TW;  // 16 channel groups x FIN_TW columns
+  const int t0 = blockIdx.x * FIN_TW, W = FIN_TW + p.k - 1;
   const int n = p.C * W;
-  float* ws = xs + n + 256;
+  float* part = xs + n;
+  float* ws = part + 256;
   for (int i = tid; i < p.C * p.k; i += 256) ws[i] = p.w[i];
   const int f = *p.ctr - 1, base = ring_base(p.in, f);
-  for (int i0 = tid; i0 < n; i0 += 256 * 8) {
-    float v[8];
+  for (int i0 = tid; i0 < n; i0 += 256 * 12) {
+    float v[12];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < 12; ++u) {
       const int i = i0 + 256 * u;
       v[u] = i < n ? *ring_ptr(p.in, base, i / W, t0 + i % W) : 0.f;
     }
 #pragma unroll
-    for (int u = 0; u < 8; ++u) { const int i = i0 + 256 * u; if (i < n) xs[i] = v[u]; }
+    for (int u = 0; u < 12; ++u) { const int i = i0 + 256 * u; if (i < n) xs[i] = v[u]; }
   }
   __syncthreads();
   float a = 0.f;
-  const int c0 = (p.C * qd) / 4, c1 = (p.C * (qd + 1)) / 4;
+  const int c0 = (p.C * qd) / 16, c1 = (p.C * (qd + 1)) / 16;
   for (int c = c0; c < c1; ++c)
     for (int k = 0; k < p.k; ++k) a = fmaf(ws[c * p.k + k], xs[c * W + l + k], a);
-  float* part = xs + n;
-  part[qd * 64 + l] = a;
+  part[qd * FIN_TW + l] = a;
   __syncthreads();
   const int t = t0 + l;
   if (qd == 0 && t < p.T) {
-    const float y = ((part[l] + part[64 + l]) + (part[128 + l] + part[192 + l])) + p.b[0];
+    float y = 0.f;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) y += part[q * FIN_TW + l];  // group order: a fixed order of the sum
+    y += p.b[0];
     p.audio[t] = fminf(1.0f, fmaxf(-1.0f, y));
   }
 }
@@ -992,7 +997,7 @@ static int cv_check(const vui_codec_config* c) {
   for (int v : dims32)
     if (v < 32 || (v % 32)) { vui_set_error("codec: every layer width must be a multiple of 32 (got %d)", v); return VUI_EINVAL; }
   if (c->head_dim > 64 || (c->head_dim & 15) || c->n_heads < 1) { vui_set_error("codec: head_dim=%d unsupported (a multiple of 16, <= 64)", c->head_dim); return VUI_EINVAL; }
-  if ((c->decoder_dim >> c->n_rates) * (64 + 6) * 4 > 60000) { vui_set_error("codec: last stage too wide"); return VUI_EINVAL; }
+  if ((c->decoder_dim >> c->n_rates) * (FIN_TW + 6 + 7) * 4 > 60000) { vui_set_error("codec: last stage too wide"); return VUI_EINVAL; }
   if (c->max_seq < 1 || c->max_seq > 4096) { vui_set_error("codec: max_seq=%d outside [1,4096]", c->max_seq); return VUI_EINVAL; }
   if (c->latent_dim > 256 * DW_MAXC) { vui_set_error("codec: latent_dim=%d above %d", c->latent_dim, 256 * DW_MAXC); return VUI_EINVAL; }
   int dim = c->decoder_dim;
@@ -1483,7 +1488,7 @@ int vui_codec_decode_frame(vui_codec* c, const int64_t* codes, int32_t n_q, floa
   }
   CvFinal fin = c->fin;
   fin.audio = audio_out;
-  hipLaunchKernelGGL(cv_final_kernel, dim3((fin.T + 63) / 64), dim3(256), (size_t)(fin.C * (64 + fin.k - 1) + 256 + fin.C * fin.k) * 4, st, fin);
+  hipLaunchKernelGGL(cv_final_kernel, dim3((fin.T + FIN_TW - 1) / FIN_TW), dim3(256), (size_t)(fin.C * (FIN_TW + fin.k - 1) + 256 + fin.C * fin.k) * 4, st, fin);
   HIP_TRY(hipGetLastError());
   return VUI_OK;
 }
