@@ -234,3 +234,55 @@ def test_batch12_mfma_rows_match_small_batches(dims):
                       for r in range(0, B, 4)])
     agree = (full == part).all(dim=1).float().mean()
     assert agree >= 0.75, agree
+
+
+def test_full_size_streaming_workload_properties():
+    """The headline workload at its real size (Vui Nano dims, bf16, a 512-frame voice prefix + 64 text tokens
+    ingested, then 750 sampled frames through the one-graph frame step), checked through what does not depend on
+    size: a second run from the same seed gives the same 750 x 16 tokens and EOS probabilities, another seed
+    does not; every code is inside its codebook; the cache grew by one position per frame; the rolling
+    repetition counts equal the histogram of the last `window` code-0 values (engine.py:930-934); and the frames
+    the graph logged are the frames it fed back."""
+    from vui_amd.engine import Engine, GenConfig
+    from vui_amd.model import Vui
+    from vui_amd.synthetic import nano_for_cache, synthetic_state_dict
+
+    n_prefix, n_text, n_frames = 512, 64, 750
+    max_seq = 64 * ((n_prefix + n_text + n_frames + 2 + 63) // 64)
+    d = nano_for_cache("A", 64).model
+    sd = synthetic_state_dict(d, seed=0)
+    model = Vui(nano_for_cache("A", max_seq), sd, device="cuda", dtype=BF)
+    eng = Engine(model=model, max_rows=1, max_seq=max_seq)
+    assert model._native.fused(-1), "the one-launch frame kernel must be the path at these dims"
+    g = torch.Generator().manual_seed(0)
+    prefix = torch.randint(0, d.codebook_size, (n_prefix, d.n_quantizers), generator=g).cuda()
+    ids = torch.randint(0, d.vocab_size, (n_text,), generator=g).cuda()
+    row = eng.new_row()
+    row.prefill_emb(model.embed_audio(prefix[None]).to(BF))
+    h = row.prefill_emb(model.token_emb(ids[None]))[:, -1]
+    row.mark_prompt()
+    assert row.offset == n_prefix + n_text
+
+    def run(seed):
+        row.rewind()
+        cfg = GenConfig(seed=seed)  # temperature 0.9, top-k 100, repetition penalty 1.1 over 24 frames
+        frames, eos = eng.generate([row], h, n_frames, cfg)
+        model._native.status()
+        return frames.cpu(), eos.cpu(), eng._rep_counts.cpu().clone(), eng._rep_pos.cpu().clone(), cfg
+
+    f0, e0, counts, pos, cfg = run(0)
+    assert f0.shape == (n_frames, 1, d.n_quantizers)
+    assert int(f0.min()) >= 0 and int(f0.max()) < d.codebook_size
+    assert bool(((e0 >= 0) & (e0 <= 1)).all()) and float(e0[0, 0]) == 0.0
+    assert row.offset == n_prefix + n_text + n_frames - 1  # the last frame is not fed back
+    last = f0[-cfg.rep_window:, 0, 0]
+    assert torch.equal(counts[0], torch.bincount(last, minlength=d.codebook_size).float())
+    assert pos[0].tolist() == [n_frames % cfg.rep_window, cfg.rep_window]
+    # the codes the graph fed back are the codes it logged
+    assert torch.equal(eng._g_codes_in[0, :d.n_quantizers].cpu(), f0[-1, 0])
+    # the sampler uses its whole support: code 0 is not stuck and no codebook column is constant
+    assert all(len(torch.unique(f0[:, 0, q])) > 50 for q in range(d.n_quantizers))
+    f1, e1, *_ = run(0)
+    assert torch.equal(f0, f1) and torch.equal(e0, e1)
+    f2, *_ = run(1)
+    assert not torch.equal(f0, f2)
