@@ -708,6 +708,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
             for (int e = 0; e < 8; ++e) { const int j = tid * E + e; if (e < E && j < a.CS) cn[e] = counts[j]; }
           }
         }
+        const uint32_t rnd0 = philox_u32(a.seed0, frame0, 0u, 0u, 0u);  // ahead of the wait
         poll_words((uint32_t*)lg, rep_rd(lgbuf), a.CS / 2, c);
         float lv[8], raw[8];
         uint32_t key[8];
@@ -728,7 +729,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           }
         }
         TS(20);
-        code0 = block_sample<8>(lv, key, counts ? 0 : 16, a.CS, E, greedy, a.topk0, a.seed0, frame0, 0u, 0u, ssh, (int*)sc);
+        code0 = block_sample<8>(lv, key, counts ? 0 : 16, a.CS, E, greedy, a.topk0, rnd0, 0u, ssh, (int*)sc);
         TS(21);
       }
     }
@@ -973,6 +974,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
         gemv_compute<2, false>(xp, R_hd, wr, red, [&](int gp, float v0, float v1, float, float) {
           rep_st(lgbuf, gp, pack2(v0, v1), ep); });
         TS(42);
+        const uint32_t rnd = philox_u32(a.seed1, frame1, 0u, (uint32_t)t, 0u);  // ahead of the wait
         poll_words((uint32_t*)lg, rep_rd(lgbuf), CS / 2, c);
         TS(43);
         const int E = (CS + FR_THREADS - 1) / FR_THREADS;
@@ -992,7 +994,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
             key[e] = float_key(bias ? lv[e] : raw[e]);
           }
         }
-        prev_code = block_sample<8>(lv, key, bias ? 0 : 16, CS, E, greedy, a.topk1, a.seed1, frame1, 0u, (uint32_t)t, ssh, (int*)sc);
+        prev_code = block_sample<8>(lv, key, bias ? 0 : 16, CS, E, greedy, a.topk1, rnd, (uint32_t)t, ssh, (int*)sc);
         TS(44);
 #ifdef VUI_SAMPLE_CLOCK
         if (prof_on && tid == 0) {

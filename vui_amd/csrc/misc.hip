@@ -109,8 +109,8 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const SampleArgs p
     }
   }
   const uint32_t frame = p.frame_ctr ? (uint32_t)p.frame_ctr[0] : 0u;
-  const int pick = block_sample<EMAX>(l, key, raw_keys ? 16 : 0, CS, E, greedy, p.top_k, p.seed, frame, (uint32_t)sb,
-                                      (uint32_t)p.codebook, sh, hist);
+  const uint32_t rnd = philox_u32(p.seed, frame, (uint32_t)sb, (uint32_t)p.codebook, 0u);
+  const int pick = block_sample<EMAX>(l, key, raw_keys ? 16 : 0, CS, E, greedy, p.top_k, rnd, (uint32_t)p.codebook, sh, hist);
 
   if (tid == 0) {
     p.out[(size_t)b * p.out_stride + p.out_col] = (int64_t)pick;

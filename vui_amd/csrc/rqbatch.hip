@@ -518,6 +518,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
         const int b = b0 + wl;
         // the row's logits pass through the first words of the staging area
         uint32_t* lgw = xp;
+        const uint32_t rnd = philox_u32(a.seed, frame, (uint32_t)b, (uint32_t)t, 0u);  // ahead of the wait
         __syncthreads();
         ll_poll(lgb + (size_t)b * (CS / 2), CS / 2, c, [&](int i, uint32_t v) { lgw[i] = v; });
         __syncthreads();
@@ -540,8 +541,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
         }
         __syncthreads();  // every thread holds its logits: the staging words go back to zero (the spare row must
         for (int i = tid; i < CS / 2; i += FR_THREADS) lgw[i] = 0u;  // read as zero, the others are rewritten by the next norm)
-        const int code = block_sample<8>(lv, key, bias ? 0 : 16, CS, E, greedy, a.topk, a.seed, frame, (uint32_t)b, (uint32_t)t, ssh,
-                                         (int*)red);
+        const int code = block_sample<8>(lv, key, bias ? 0 : 16, CS, E, greedy, a.topk, rnd, (uint32_t)t, ssh, (int*)red);
         if (tid == 0) {
           ll_st(cb + b, (uint32_t)code, ep);
           a.codes_out[(size_t)b * a.codes_stride + t] = code;

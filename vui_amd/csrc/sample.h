@@ -30,8 +30,7 @@ struct SampleShared {
   int ired[SAMP_THREADS / WAVE];
   float wsum[SAMP_THREADS / WAVE];
   int cnt[2][3 * SAMP_THREADS / WAVE];
-  int pick;
-  int sel[4][2];   // key search, per 8-bit round: chosen digit, count of keys above it
+  int pick[2];     // slot codebook % 2: consecutive draws of a workgroup alternate, so a draw needs no barrier after its last read
 #ifdef VUI_SAMPLE_CLOCK
   unsigned long long ts[8];
 #endif
@@ -41,22 +40,16 @@ struct SampleShared {
 #else
 #define SAMP_TS(k) do { } while (0)
 #endif
-// The 8-bit digit histogram of the 16-bit key search can be kept in HIST_COPIES copies (thread t adds
-// to copy t % HIST_COPIES) against serialised additions to one LDS word; measured, one copy is fastest.
-#define HIST_COPIES 1
-#define HIST_WORDS (HIST_COPIES * 256)
+// Scratch of the digit search: one 256-bin histogram per 8-bit round (two rounds for keys that come from bf16
+// values, four for fp32 keys), so that no round has to wait for the bins of an earlier one to be cleared.
+#define HIST_WORDS (4 * 256)
 
-// Wave 0 finds, in the 256-bin histogram (hist: HIST_WORDS ints of LDS), the largest digit whose suffix count (keys with digit >= it)
-// reaches `need`, stores {digit, keys above it} and clears the bins for the next round.
-__device__ __forceinline__ void hist_select(int* hist, int need, int* out) {
+// Every wave calls this after the barrier that completes the round's histogram and finds, for itself, the largest
+// digit whose suffix count (keys with digit >= it) reaches `need` and the number of keys above that digit: the
+// four waves arrive at the same answer without a word passing between them.
+__device__ __forceinline__ void hist_select(const int* hist, int need, int& digit_out, int& over_out) {
   const int lane = threadIdx.x & 63;
-  int4 b = make_int4(0, 0, 0, 0);  // bins 4*lane .. 4*lane+3, summed over the copies
-#pragma unroll
-  for (int c = 0; c < HIST_COPIES; ++c) {
-    const int4 t = *reinterpret_cast<const int4*>(&hist[c * 256 + 4 * lane]);
-    *reinterpret_cast<int4*>(&hist[c * 256 + 4 * lane]) = make_int4(0, 0, 0, 0);
-    b.x += t.x; b.y += t.y; b.z += t.z; b.w += t.w;
-  }
+  const int4 b = *reinterpret_cast<const int4*>(&hist[4 * lane]);  // bins 4*lane .. 4*lane+3
   const int s3 = b.w, s2 = s3 + b.z, s1 = s2 + b.y, s0 = s1 + b.x;  // suffix sums inside the lane
   // exclusive suffix over the lanes: keys in the bins of higher lanes
   int v = s0;
@@ -76,14 +69,20 @@ __device__ __forceinline__ void hist_select(int* hist, int need, int* out) {
   else if (above + s2 >= need && above + s3 < need) { digit = 4 * lane + 2; over = above + s3; }
   else if (above + s1 >= need && above + s2 < need) { digit = 4 * lane + 1; over = above + s2; }
   else if (above + s0 >= need && above + s1 < need) { digit = 4 * lane; over = above + s1; }
-  if (digit >= 0) { out[0] = digit; out[1] = over; }
+  // exactly one lane holds the answer when the round's keys number at least `need` (they do: need <= top_k < CS)
+  const unsigned long long found = __ballot(digit >= 0);
+  const int src = found ? (int)__builtin_ctzll(found) : 0;
+  digit_out = max(__builtin_amdgcn_readlane(digit, src), 0);
+  over_out = __builtin_amdgcn_readlane(over, src);
 }
 
 // One draw from the values l[e] (element index tid*E + e, -inf beyond CS) held by a 256-thread
 // block.  RQ rule (src/vui/model.py:955-962): drop l < k-th largest, softmax, draw.  code-0 rule
 // (src/vui/engine.py:855-863): softmax, keep the top-k probabilities, renormalise, draw.  Both
 // are: keep {l >= k-th largest l}, weights exp(l - max), inverse CDF in index order with one
-// uniform.  greedy: the lowest index of the maximum.  Every thread returns the same pick.
+// uniform (rnd: philox_u32(seed, frame, row, codebook, 0), computed by the caller ahead of its last wait; codebook
+// also picks the slot of the shared result, see SampleShared).  greedy: the lowest index of the maximum.  Every
+// thread returns the same pick.
 // hist: HIST_WORDS ints of LDS scratch (16-byte aligned) for the digit histograms.
 //
 // key[e] orders the elements for the top-k cut (any order-preserving image of l[e]); bits below
@@ -92,11 +91,10 @@ __device__ __forceinline__ void hist_select(int* hist, int need, int* out) {
 // stopping as soon as exactly top_k keys lie above the candidate.
 template <int EMAX>
 __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32_t (&key)[EMAX], int low_bit, int CS,
-                                            int E, bool greedy, int top_k, uint64_t seed, uint32_t frame,
-                                            uint32_t row, uint32_t codebook, SampleShared& sh, int* hist) {
+                                            int E, bool greedy, int top_k, uint32_t rnd, uint32_t codebook,
+                                            SampleShared& sh, int* hist) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   SAMP_TS(0);
-  const uint32_t rnd = philox_u32(seed, frame, row, codebook, 0u);  // ahead of the first wait
   const bool digits = top_k > 0 && top_k < CS && (low_bit == 16 || low_bit == 0) && !greedy;
   float m = -INFINITY; int mi = 0x7fffffff;
 #pragma unroll
@@ -108,11 +106,13 @@ __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32
     const int cand = wave_min_i((m == wm) ? mi : 0x7fffffff);
     if (lane == 0) { sh.sred[wave] = wm; sh.ired[wave] = cand; }
   }
+  const int rounds = (32 - low_bit) / 8;
+  int* pick_slot = &sh.pick[codebook & 1];
+  if (tid == 0) *pick_slot = -1;
   if (digits) {
 #pragma unroll
-    for (int i = 0; i < HIST_WORDS / SAMP_THREADS; ++i) hist[tid + SAMP_THREADS * i] = 0;
+    for (int i = 0; i < 4; ++i) if (i < rounds) hist[tid + SAMP_THREADS * i] = 0;
   }
-  if (tid == 0) sh.pick = -1;
   __syncthreads();
   float M = sh.sred[0]; int Mi = sh.ired[0];
 #pragma unroll
@@ -128,22 +128,22 @@ __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32
   if (digits) {
     // one byte per round from the top, each among the keys that share the bytes chosen so far
     int need = top_k;
-    const int rounds = (32 - low_bit) / 8;
 #pragma unroll
     for (int round = 0; round < 4; ++round) {
       if (round >= rounds) break;
       const int shift = 24 - 8 * round;
+      int* bins = hist + 256 * round;
 #pragma unroll
       for (int e = 0; e < EMAX; ++e)
         if (e < E && tid * E + e < CS && (round == 0 || (key[e] >> (shift + 8)) == (thr >> (shift + 8))))
-          atomicAdd(&hist[(tid & (HIST_COPIES - 1)) * 256 + ((key[e] >> shift) & 255)], 1);
+          atomicAdd(&bins[(key[e] >> shift) & 255], 1);
       __syncthreads();
       SAMP_TS(2 + 2 * round);
-      if (wave == 0) hist_select(hist, need, sh.sel[round]);
-      __syncthreads();
+      int digit, over;
+      hist_select(bins, need, digit, over);
       SAMP_TS(3 + 2 * round);
-      thr |= (uint32_t)sh.sel[round][0] << shift;
-      need -= sh.sel[round][1];
+      thr |= (uint32_t)digit << shift;
+      need -= over;
     }
   } else if (top_k > 0 && top_k < CS) {
     int it = 0;
@@ -215,12 +215,14 @@ __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32
 #pragma unroll
       for (int e = 0; e < EMAX; ++e) if (e < E && pw[e] > 0.f) j = tid * E + e;
     }
-    if (j >= 0) atomicMax(&sh.pick, j);
+    if (j >= 0) atomicMax(pick_slot, j);
   }
   __syncthreads();
-  const int pick = (sh.pick >= 0) ? sh.pick : Mi;
+  const int got = *pick_slot;
+  const int pick = (got >= 0) ? got : Mi;
   SAMP_TS(7);
-  __syncthreads();  // the next draw may rewrite the shared state
+  // no barrier here: the next draw of this workgroup (codebook + 1) uses the other slot, and every other word of the
+  // shared state is next written behind a barrier of that draw which this read precedes
   return pick;
 }
 
