@@ -73,8 +73,11 @@ __device__ __forceinline__ void stage_x(const GemvArgs& p, float* xs, int nb) {
 }
 
 template <typename T, typename WT, int NB, int MAXC, bool DUAL>
-__global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs p, const int b0, const int nb_rt) {
+__global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs p, const int b0_in, const int nb_in) {
   extern __shared__ float xs[];
+  // N == 0: only the extra outputs are wanted (the matrix cores did the rest); one row per workgroup then,
+  // instead of one workgroup walking through eight rows
+  const int b0 = p.N == 0 ? (int)blockIdx.x : b0_in, nb_rt = p.N == 0 ? 1 : nb_in;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int nch = p.K >> 3;
   const int nmain = (p.N + 2 * RPW - 1) / (2 * RPW);
@@ -197,7 +200,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs p, co
 template <typename T, typename WT, int NB, int MAXC, bool DUAL>
 static int launch_one(const GemvArgs& a, int b0, int nb, hipStream_t st) {
   const int nmain = (a.N + 2 * RPW - 1) / (2 * RPW);
-  const int grid = nmain + ((a.Wx && b0 >= 0) ? 1 : 0);
+  const int grid = a.N == 0 ? a.B : nmain + ((a.Wx && b0 >= 0) ? 1 : 0);
   const size_t lds = (size_t)nb * a.K * sizeof(float);
   hipLaunchKernelGGL((gemv_kernel<T, WT, NB, MAXC, DUAL>), dim3(grid), dim3(GEMV_THREADS), lds, st, a, b0, nb);
   HIP_TRY(hipGetLastError());
@@ -239,11 +242,7 @@ int launch_gemv(const GemvArgs& a, hipStream_t st) {
     if (rc || !a.Wx) return rc;
     GemvArgs x = a;
     x.N = 0;
-    for (int b0 = 0; b0 < a.B; b0 += 8) {
-      const int nb = (a.B - b0 < 8) ? a.B - b0 : 8;
-      if ((rc = pick_nb<bf16_t, bf16_t, false>(x, b0, nb, st))) return rc;
-    }
-    return VUI_OK;
+    return pick_nb<bf16_t, bf16_t, false>(x, 0, 1, st);
   }
   // batch tile: at most 8 rows and at most 64 KiB of LDS
   int tile = 8;
