@@ -65,6 +65,110 @@ template <> struct W16<int8_t> {
   }
 };
 
+// ---- epilogue of four consecutive features of one row (the lane's share of the 16 x 16 tile) ----
+// Same arithmetic and rounding points as epilogue() of gemv_epi.h, for the forms the batch step uses, with what it
+// reads fetched ahead (epi_prefetch) and one 8-byte store instead of four 2-byte ones.
+struct EpiPre {
+  uint2 sc, sc2, res;  // four bf16 each: scales of the two matrices, residual values
+  float4 f0, f1;       // (cos, sin) of dims dd, dd + 1 and dd + 2, dd + 3
+  int slot, pos;
+};
+__device__ __forceinline__ bool epi_fast(const GemvArgs& p) {
+  if ((p.N & 3) || (p.ldy & 3)) return false;
+  if (p.epi == EPI_STORE || p.epi == EPI_RESID || p.epi == EPI_SWIGLU) return true;
+  return p.epi == EPI_QKV && !((p.nq | p.nkv | p.hd | p.rope_dim) & 3) && p.rope_dim >= 4;  // a group of four rotates as a whole or not at all
+}
+// region of feature n of the fused projection: 0 q, 1 k, 2 v; m = index inside the region
+__device__ __forceinline__ int qkv_region(const GemvArgs& p, int n, int& m) {
+  if (n < p.nq) { m = n; return 0; }
+  if (n < p.nq + p.nkv) { m = n - p.nq; return 1; }
+  m = n - p.nq - p.nkv;
+  return 2;
+}
+template <bool DUAL>
+__device__ __forceinline__ void epi_prefetch(const GemvArgs& p, bool fast, int eb, int en, EpiPre& e) {
+  e.sc = e.sc2 = e.res = make_uint2(0, 0);
+  e.f0 = e.f1 = make_float4(1.f, 0.f, 1.f, 0.f);
+  e.slot = eb; e.pos = 0;
+  if (!fast) return;  // uniform
+  if (p.w_int8) {
+    e.sc = *reinterpret_cast<const uint2*>((const bf16_t*)p.sc + en);
+    if (DUAL) e.sc2 = *reinterpret_cast<const uint2*>((const bf16_t*)p.sc2 + en);
+  }
+  if (p.epi == EPI_RESID) e.res = *reinterpret_cast<const uint2*>((const bf16_t*)p.resid + (size_t)eb * p.ldy + en);
+  if (p.epi == EPI_QKV) {
+    // slot and position of every row through uniform addresses (the scalar unit fetches them, beside the queue of
+    // vector loads and in no order with it), then this lane's pair by selection
+    int sl[16], ps[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sl[i] = min(i, p.B - 1);
+    if (p.slot_idx) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sl[i] = p.slot_idx[sl[i]];
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) ps[i] = p.seq_lens[sl[i]];
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      if (eb == i) { e.slot = sl[i]; e.pos = ps[i]; }
+    int m;
+    qkv_region(p, en, m);
+    const int dd = min(m % p.hd, p.rope_dim - 4);           // clamped: unused where the dims are not rotated
+    const int pc = min(max(e.pos, 0), p.S - 1);
+    const float* f = p.rope + ((size_t)pc * p.rope_dim + dd) * 2;
+    e.f0 = *reinterpret_cast<const float4*>(f);
+    e.f1 = *reinterpret_cast<const float4*>(f + 4);
+  }
+}
+template <bool DUAL>
+__device__ __forceinline__ void epi_fast4(const GemvArgs& p, const EpiPre& e, int b, int n, const float* v, const float* v2) {
+  float a[4], a2[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) { a[r] = v[r]; a2[r] = DUAL ? v2[r] : 0.f; }
+  if (p.w_int8) {
+    a[0] *= bf_lo(e.sc.x); a[1] *= bf_hi(e.sc.x); a[2] *= bf_lo(e.sc.y); a[3] *= bf_hi(e.sc.y);
+    if (DUAL) { a2[0] *= bf_lo(e.sc2.x); a2[1] *= bf_hi(e.sc2.x); a2[2] *= bf_lo(e.sc2.y); a2[3] *= bf_hi(e.sc2.y); }
+  }
+  bf16_t* y = (bf16_t*)p.y;
+  float o[4];
+  bf16_t* dst = y + (size_t)b * p.ldy + n;
+  if (p.epi == EPI_STORE) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) o[r] = a[r];
+  } else if (p.epi == EPI_RESID) {
+    const float rs[4] = {bf_lo(e.res.x), bf_hi(e.res.x), bf_lo(e.res.y), bf_hi(e.res.y)};
+#pragma unroll
+    for (int r = 0; r < 4; ++r) o[r] = rs[r] + El<bf16_t>::rnd(a[r]);
+  } else if (p.epi == EPI_SWIGLU) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float g = El<bf16_t>::rnd(a[r]), c = El<bf16_t>::rnd(a2[r]);
+      o[r] = El<bf16_t>::rnd(g / (1.0f + expf(-g))) * c;
+    }
+  } else {  // EPI_QKV
+    int m;
+    const int region = qkv_region(p, n, m);
+    const int dd = m % p.hd;
+    const bool in_cache = e.pos >= 0 && e.pos < p.S;
+    const float cs[4] = {e.f0.x, e.f0.z, e.f1.x, e.f1.z}, sn[4] = {e.f0.y, e.f0.w, e.f1.y, e.f1.w};
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float val = El<bf16_t>::rnd(a[r]);
+      if (region != 2 && dd + r < p.rope_dim && in_cache) {
+        const float partner = El<bf16_t>::rnd(a[r ^ 1]);
+        val = rope_mix(val, cs[r], (r & 1) ? partner : -partner, sn[r]);
+      }
+      o[r] = val;
+    }
+    if (region == 0) dst = y + (size_t)b * p.ldy + m;
+    else {
+      if (!in_cache) return;
+      dst = (bf16_t*)(region == 1 ? p.kc : p.vc) + ((size_t)e.slot * p.S + e.pos) * p.nkv + m;
+    }
+  }
+  *reinterpret_cast<uint2*>(dst) = make_uint2(f2bf2(o[0], o[1]), f2bf2(o[2], o[3]));
+}
+
 template <typename WT, bool DUAL>
 __global__ __launch_bounds__(G16_THREADS) void gemm16_kernel(const GemvArgs p) {
   extern __shared__ __align__(16) unsigned char smem16[];
@@ -89,6 +193,15 @@ __global__ __launch_bounds__(G16_THREADS) void gemm16_kernel(const GemvArgs p) {
     if (DUAL) wr2[i] = on ? W16<WT>::load(wrow2 + k) : W16<WT>::zero();
   }
 
+  // What the epilogue of this lane will need (row f16, features n0 + 4 kg ... + 3) is requested now, behind the
+  // weights: scales, the residual values, the row's position and its rotation factors.  Written as part of the
+  // epilogue they were a chain of small dependent loads, each waited for in turn, after everything else was done.
+  // Every wave runs this (only wave 0 uses it): no branch, so the loads go out together with the rest (the call
+  // sits below, between the requests for the activations and their use).
+  const bool fast = epi_fast(p);
+  const int eb = min(f16, p.B - 1), en = fast ? min(n0 + 4 * kg, p.N - 4) : 0;
+  EpiPre pre;
+
   // activations -> LDS (bf16), rows >= B are zero.  A wave stages rows wave, wave+4, ...: all their
   // 16-byte chunks (and the norm weights) are requested first, then normalised and written.
   {
@@ -106,6 +219,7 @@ __global__ __launch_bounds__(G16_THREADS) void gemm16_kernel(const GemvArgs p) {
         xr[j][i] = (b < p.B && c < nch) ? *reinterpret_cast<const uint4*>(x + (size_t)b * K + c * 8) : make_uint4(0, 0, 0, 0);
       }
     }
+    epi_prefetch<DUAL>(p, fast, eb, en, pre);  // behind the weights and activations in the queue
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int b = wave + 4 * j;
@@ -188,6 +302,10 @@ __global__ __launch_bounds__(G16_THREADS) void gemm16_kernel(const GemvArgs p) {
   // lane holds features n0 + 4 * kg + r (r = 0..3) of activation row f16
   const int b = f16;
   if (b >= p.B) return;
+  if (fast) {
+    if (n0 + 4 * kg < p.N) epi_fast4<DUAL>(p, pre, b, n0 + 4 * kg, v, v2);
+    return;
+  }
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int n = n0 + 4 * kg + r;
