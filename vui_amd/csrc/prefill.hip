@@ -89,6 +89,13 @@ __global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf1
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) { acc[i][j] = pf_floatx4{0.f, 0.f, 0.f, 0.f}; acc2[i][j] = acc[i][j]; }
+  // the residual values this thread will add to (its four outputs, see the epilogue) are requested with the first
+  // operands instead of after the last product; clamped to the matrix, unused where the thread has no output
+  uint2 old = make_uint2(0, 0);
+  if (EPI == PF_RESID) {
+    const int em = min(m0 + 16 * (wave & 1) + l16, p.M - 1), en = min(n0 + 16 * (wave >> 1) + 4 * kg, p.N - 4);
+    old = *reinterpret_cast<const uint2*>((const bf16_t*)p.C + (c_tiled ? pf_toff(em, en, p.N) : (size_t)em * p.ldc + en));
+  }
   for (int s = s0; s < s1; ++s) {
     const int k = s << 10;
     uint4 xa[2][2], wa[2][2], va[2][2];
@@ -140,7 +147,6 @@ __global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf1
   }
   if (EPI == PF_RESID) {  // x = rnd(x + rnd(y)), src/vui/model.py:367, 374
     if (n + 3 < p.N) {
-      const uint2 old = *reinterpret_cast<const uint2*>(c);
       v[0] = bf_lo(old.x) + bf2f(f2bf(v[0])); v[1] = bf_hi(old.x) + bf2f(f2bf(v[1]));
       v[2] = bf_lo(old.y) + bf2f(f2bf(v[2])); v[3] = bf_hi(old.y) + bf2f(f2bf(v[3]));
     } else {
@@ -178,15 +184,18 @@ __global__ __launch_bounds__(256) void pf_rownorm_kernel(const bf16_t* x, const 
 // interleaved rotation (src/vui/rope.py:16-77) of the four pairs of an 8-element piece whose first dim is dd (even)
 // at position pos; pairs at or beyond rope_dim pass through
 __device__ __forceinline__ uint4 pf_rope8(uint4 v, const float* __restrict__ rope, int pos, int rope_dim, int dd) {
+  if (rope_dim < 2) return v;  // uniform
   uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  // the four factor loads go out together (a pair beyond rope_dim reads the last rotated pair's and ignores it):
+  // behind a branch each, every load would be waited for before the next is issued
+  float4 f[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f[i] = *reinterpret_cast<const float4*>(rope + ((size_t)pos * rope_dim + min(dd + 2 * i, rope_dim - 2)) * 2);
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int d2 = dd + 2 * i;
-    if (d2 < rope_dim) {
-      const float4 f = *reinterpret_cast<const float4*>(rope + ((size_t)pos * rope_dim + d2) * 2);  // cos, sin of d2 and d2 + 1
-      const float a = bf_lo(w[i]), b = bf_hi(w[i]);
-      w[i] = f2bf2(rope_mix(a, f.x, -b, f.y), rope_mix(b, f.z, a, f.w));
-    }
+    const float a = bf_lo(w[i]), b = bf_hi(w[i]);  // cos, sin of d2 and d2 + 1
+    const uint32_t r = f2bf2(rope_mix(a, f[i].x, -b, f[i].y), rope_mix(b, f[i].z, a, f[i].w));
+    w[i] = (dd + 2 * i < rope_dim) ? r : w[i];
   }
   return make_uint4(w[0], w[1], w[2], w[3]);
 }
