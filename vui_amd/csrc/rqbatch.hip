@@ -18,7 +18,8 @@
 //               of each matrix that follows an RMSNorm (QKV, W1/W3, logits head; projection of position 0)
 //   attention   workgroup 63 - task, task = local row * heads + head: that row's head, its keys/values of
 //               all layers and positions in LDS
-//   out tiles   workgroup 63 - tile, tile < R/16: out_proj and W2
+//   out tiles   workgroup 63 - tile - (R/16) * half: out_proj and W2 of tile < R/16 for one half of the group's rows
+//               (all rows when R/16 > 32)
 //   sampler     workgroup r < rows of the group draws row r's code
 // Rounding points are those of the kernel sequence (gemv_epi.h, attn.hip, sample.h).
 #include "common.h"
@@ -232,7 +233,13 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
   const int back = RB_NWL - 1 - wl;
   const bool att_on = active && back < Bg * a.rqH;
   const int att_lr = back / a.rqH, att_h = back % a.rqH;
-  const bool out_on = active && back < nO;
+  // out_proj / W2 tiles: with twice as many workgroups as tiles the rows of the group are split in two halves, so
+  // a workgroup waits for half as many exchanged words (the wait, not the product, is what these phases cost)
+  const bool out_split = 2 * nO <= RB_NWL;
+  const int out_tile = out_split ? back % nO : back;
+  const int out_r0 = out_split ? (back / nO) * (RB_RG / 2) : 0;                     // first local row
+  const int out_nr = out_split ? max(0, min(Bg - out_r0, RB_RG / 2)) : Bg;          // rows taken
+  const bool out_on = active && out_nr > 0 && back < (out_split ? 2 * nO : nO);
   const uint32_t inv_r2 = 0xFFFFFFFFu / (uint32_t)(R / 2) + 1u, inv_f2 = 0xFFFFFFFFu / (uint32_t)(a.rqF / 2) + 1u;
 
   for (int i = tid; i < (RB_RG + 1) * xs; i += FR_THREADS) xp[i] = 0u;
@@ -423,17 +430,17 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
       uint64_t* ob = llp;
       llp += (size_t)B * (R / 2);
       if (out_on) {
-        const Tile to = {16 * back, R, R, true};
+        const Tile to = {16 * out_tile, R, R, true};
         TileW<8, false> wr;
         tile_prefetch<8, false>((const bf16_t*)Lw.wo, nullptr, to, wr);
         __syncthreads();
-        ll_poll(attb + (size_t)b0 * (R / 2), Bg * (R / 2), c, [&](int i, uint32_t v) {
+        ll_poll(attb + (size_t)(b0 + out_r0) * (R / 2), out_nr * (R / 2), c, [&](int i, uint32_t v) {
           const int lr = div_small(i, inv_r2), j = i - lr * (R / 2);
           xp[(size_t)lr * xs + j] = v;
         });
         __syncthreads();
-        tile_compute<8, false>(xp, xs, to, wr, red, Bg, [&](int n, int lr, const float* v, const float*) {
-          uint64_t* dst = ob + (size_t)(b0 + lr) * (R / 2) + n / 2;
+        tile_compute<8, false>(xp, xs, to, wr, red, out_nr, [&](int n, int lr, const float* v, const float*) {
+          uint64_t* dst = ob + (size_t)(b0 + out_r0 + lr) * (R / 2) + n / 2;
           ll_st(dst, f2bf2(v[0], v[1]), ep);
           ll_st(dst + 1, f2bf2(v[2], v[3]), ep);
         });
@@ -471,17 +478,17 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
       uint64_t* yb = llp;
       llp += (size_t)B * (R / 2);
       if (out_on) {
-        const Tile tw = {16 * back, R, a.rqF, true};
+        const Tile tw = {16 * out_tile, R, a.rqF, true};
         TileW<16, false> wr;
         tile_prefetch<16, false>((const bf16_t*)Lw.w2, nullptr, tw, wr);
         __syncthreads();
-        ll_poll(hb + (size_t)b0 * (a.rqF / 2), Bg * (a.rqF / 2), c, [&](int i, uint32_t v) {
+        ll_poll(hb + (size_t)(b0 + out_r0) * (a.rqF / 2), out_nr * (a.rqF / 2), c, [&](int i, uint32_t v) {
           const int lr = div_small(i, inv_f2), j = i - lr * (a.rqF / 2);
           xp[(size_t)lr * xs + j] = v;
         });
         __syncthreads();
-        tile_compute<16, false>(xp, xs, tw, wr, red, Bg, [&](int n, int lr, const float* v, const float*) {
-          uint64_t* dst = yb + (size_t)(b0 + lr) * (R / 2) + n / 2;
+        tile_compute<16, false>(xp, xs, tw, wr, red, out_nr, [&](int n, int lr, const float* v, const float*) {
+          uint64_t* dst = yb + (size_t)(b0 + out_r0 + lr) * (R / 2) + n / 2;
           ll_st(dst, f2bf2(v[0], v[1]), ep);
           ll_st(dst + 1, f2bf2(v[2], v[3]), ep);
         });
