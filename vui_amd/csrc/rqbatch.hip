@@ -109,6 +109,53 @@ __device__ __forceinline__ void tile_compute(const uint32_t* xp, int xs, const T
   }
 }
 
+// Two tiles of the same matrix against the same activations in one pass: one read of every activation fragment, one
+// barrier, and the two epilogues side by side in waves 0 and 1 (as two calls of tile_compute they were a second
+// barrier and a second epilogue behind the first).  red: twice the floats of tile_compute.
+template <int MAXS, bool DUAL, typename Epi>
+__device__ __forceinline__ void tile_compute2(const uint32_t* xp, int xs, const Tile& t0, const TileW<MAXS, DUAL>& r0, const Tile& t1,
+                                              const TileW<MAXS, DUAL>& r1, float* red, int B, Epi&& epi) {
+  if (!t0.on) return;  // uniform over the workgroup; t1 is never on without t0
+  if (!t1.on) { tile_compute<MAXS, DUAL>(xp, xs, t0, r0, red, B, epi); return; }
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l16 = lane & 15, kg = lane >> 4;
+  rb_floatx4 a0 = {0.f, 0.f, 0.f, 0.f}, a0b = a0, a1 = a0, a1b = a0;
+#pragma unroll
+  for (int i = 0; i < MAXS; ++i) {
+    const int s = wave + 4 * i;
+    if (s * 32 < t0.K) {
+      const uint4 x = *reinterpret_cast<const uint4*>(xp + (size_t)min(l16, RB_RG) * xs + s * 16 + kg * 4);
+      a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rb_frag(r0.a[i]), rb_frag(x), a0, 0, 0, 0);
+      a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rb_frag(r1.a[i]), rb_frag(x), a1, 0, 0, 0);
+      if (DUAL) {
+        a0b = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rb_frag(r0.b[i]), rb_frag(x), a0b, 0, 0, 0);
+        a1b = __builtin_amdgcn_mfma_f32_16x16x32_bf16(rb_frag(r1.b[i]), rb_frag(x), a1b, 0, 0, 0);
+      }
+    }
+  }
+  const int per = DUAL ? 8 : 4, half = 4 * 64 * per;
+  float* mine = red + ((size_t)wave * 64 + lane) * per;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    mine[q] = a0[q]; mine[half + q] = a1[q];
+    if (DUAL) { mine[4 + q] = a0b[q]; mine[half + 4 + q] = a1b[q]; }
+  }
+  __syncthreads();
+  if (wave < 2) {
+    const float* src = red + (wave ? half : 0);
+    const Tile& t = wave ? t1 : t0;
+    float v[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < 4; ++w)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        v[q] += src[((size_t)w * 64 + lane) * per + q];
+        if (DUAL) u[q] += src[((size_t)w * 64 + lane) * per + 4 + q];
+      }
+    const int n = t.n0 + 4 * kg;
+    if (l16 < B && n < t.N) epi(n, l16, v, u);
+  }
+}
+
 struct NormRegs { uint4 w[2]; };  // norm weights of chunks lane, lane + 64 (R <= 1024)
 __device__ __forceinline__ NormRegs load_norm(const bf16_t* nw, int R) {
   NormRegs r;
@@ -199,7 +246,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
   extern __shared__ __align__(16) unsigned char smem[];
   float* xres = (float*)smem;                             // [RB_RG][R]
   uint32_t* xp = (uint32_t*)(smem + a.off_xp);            // [RB_RG + 1][xs], the last row stays zero
-  float* red = (float*)(smem + a.off_red);                // 4 x 64 x 8 floats; the sampler's histogram
+  float* red = (float*)(smem + a.off_red);                // 2 x 4 x 64 x 8 floats; the sampler's histogram
   int* codes_s = (int*)(smem + a.off_misc);               // codes of the group's rows at the current position
   SampleShared& ssh = *(SampleShared*)(smem + a.off_misc + 64);
   uint32_t* aq = (uint32_t*)(smem + a.off_att);           // attention role: q (packed), softmax weights
@@ -349,9 +396,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
           ll_st(dst, f2bf2(v[0], v[1]), ep);
           ll_st(dst + 1, f2bf2(v[2], v[3]), ep);
         };
-        tile_compute<8, false>(xp, xs, t0, w0, red, Bg, epi);
-        if (t1.on) __syncthreads();
-        tile_compute<8, false>(xp, xs, t1, w1, red, Bg, epi);
+        tile_compute2<8, false>(xp, xs, t0, w0, t1, w1, red, Bg, epi);
       }
       RB_TS();
       const bool kv_only = (t == 0 && l == a.rqL - 1);  // position 0 only feeds later keys/values
@@ -469,9 +514,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
           ll_st(dst, f2bf2(h[0], h[1]), ep);
           ll_st(dst + 1, f2bf2(h[2], h[3]), ep);
         };
-        tile_compute<8, true>(xp, xs, t0, w0, red, Bg, epi);
-        if (t1.on) __syncthreads();
-        tile_compute<8, true>(xp, xs, t1, w1, red, Bg, epi);
+        tile_compute2<8, true>(xp, xs, t0, w0, t1, w1, red, Bg, epi);
       }
       RB_TS();
       // ---- E: W2
@@ -517,9 +560,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
           ll_st(dst, f2bf2(v[0], v[1]), ep);
           ll_st(dst + 1, f2bf2(v[2], v[3]), ep);
         };
-        tile_compute<8, false>(xp, xs, t0, w0, red, Bg, epi);
-        if (t1.on) __syncthreads();
-        tile_compute<8, false>(xp, xs, t1, w1, red, Bg, epi);
+        tile_compute2<8, false>(xp, xs, t0, w0, t1, w1, red, Bg, epi);
       }
       if (active && wl < Bg) {
         const int b = b0 + wl;
@@ -584,7 +625,7 @@ static RbLayout rb_layout(const vui_config& c) {
   RbLayout l;
   size_t off = (size_t)RB_RG * c.rq_dim * 4;
   l.xp = off; off += (size_t)(RB_RG + 1) * rb_xs(c) * 4;
-  l.red = off; off += 4 * 64 * 8 * 4;
+  l.red = off; off += 2 * 4 * 64 * 8 * 4;  // two tiles' partial sums
   l.misc = off; off += 64 + 512;
   l.att = off; off += 512 + 256;
   l.kv = off;
