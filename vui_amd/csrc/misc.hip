@@ -12,10 +12,18 @@ __global__ void embed_kernel(const int64_t* codes, const T* table, T* x, int Q, 
   const int k = blockIdx.x * blockDim.x + threadIdx.x;
   if (k >= d) return;
   float s = 0.f;
-  for (int q = 0; q < Q; ++q) {
-    int64_t c = codes[(size_t)b * Q + q];
-    c = c < 0 ? 0 : (c >= CS ? CS - 1 : c);
-    s += El<T>::ld(table + ((size_t)(c + (int64_t)q * CS)) * d + k);
+  for (int q0 = 0; q0 < Q; q0 += 16) {  // 16 codes, then their 16 rows, are requested together; summed in codebook order
+    int64_t c[16];
+    float v[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) c[u] = codes[(size_t)b * Q + min(q0 + u, Q - 1)];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int64_t cc = c[u] < 0 ? 0 : (c[u] >= CS ? CS - 1 : c[u]);
+      v[u] = El<T>::ld(table + ((size_t)(cc + (int64_t)min(q0 + u, Q - 1) * CS)) * d + k);
+    }
+#pragma unroll
+    for (int u = 0; u < 16; ++u) if (q0 + u < Q) s += v[u];
   }
   El<T>::st(x + (size_t)b * d + k, s);
 }
