@@ -454,6 +454,8 @@ def main():
                     help="print only the prompt-ingestion line, one-pass path only (the run its rocprofv3 summary comes from)")
     ap.add_argument("--b16-only", action="store_true",
                     help="print only the 16-stream int8 line (the run its rocprofv3 summaries come from)")
+    ap.add_argument("--serve-only", action="store_true",
+                    help="print only the continuous-batching line (32 requests through 16 rows, wall clock)")
     ap.add_argument("--vocoder-only", action="store_true",
                     help="print only the vocoder line (the run rocprofv3 summaries of the vocoder kernels come from)")
     ap.add_argument("--loadpat-only", action="store_true",
@@ -480,6 +482,11 @@ def main():
         model2 = Vui(nano_for_cache(args.preset, 1024), sd, device="cuda", dtype=torch.bfloat16)
         eng2 = Engine(model=model2, max_rows=1, max_seq=1024)
         print(json.dumps(prefill_line(model2, eng2, torch.Generator().manual_seed(0), loop_too=False, reps=20)))
+        return
+    if args.serve_only:
+        from vui_amd.synthetic import nano_for_cache, synthetic_state_dict
+
+        print(json.dumps(serve_line(synthetic_state_dict(nano_for_cache(args.preset, 64).model, seed=0), args.preset)))
         return
     if args.b16_only:
         from vui_amd.synthetic import nano_for_cache, synthetic_state_dict

@@ -526,27 +526,38 @@ class Engine:
                        "vui_rq_generate")
             return rq_out[:B, :nq]
 
-        def advance_slot(info: _ActiveSlot) -> bool:
-            """Write the next chunk's text, draw its first frame; False when no chunk is left."""
-            if info.chunk_idx >= len(info.chunks):
-                return False
-            chunk = info.chunks[info.chunk_idx]
-            row = info.row
-            info.max_turn_frames = cfg.max_turn_frames(chunk.n_words, row.prompt_wps)
-            hidden = self._prefill_emb(row, chunk.emb, offset=info.seq_offset)[:, -1]
-            info.seq_offset += chunk.emb.shape[1]
+        def advance_slots(infos: "list[_ActiveSlot]") -> "list[bool]":
+            """Write the next chunk's text of every given slot and draw its first frame; False where no chunk is
+            left.  The slots that advance in the same step share one codec-head call, one code-0 draw and one
+            depth-head call (rows are independent: a burst of sixteen costs one batched depth head instead of
+            sixteen single ones)."""
+            ok = [info.chunk_idx < len(info.chunks) for info in infos]
+            ready = [info for info, k in zip(infos, ok) if k]
+            if not ready:
+                return ok
+            hiddens = []
+            for info in ready:
+                chunk = info.chunks[info.chunk_idx]
+                info.max_turn_frames = cfg.max_turn_frames(chunk.n_words, info.row.prompt_wps)
+                hiddens.append(self._prefill_emb(info.row, chunk.emb, offset=info.seq_offset)[:, -1])
+                info.seq_offset += chunk.emb.shape[1]
+            n = len(ready)
+            hidden = hiddens[0] if n == 1 else torch.cat(hiddens, dim=0)
             cb0 = model.codec_head(hidden)
-            one_slot.fill_(row.idx)
-            code0 = sample(cb0, one_slot, 1 if greedy else 0)
-            info.last_codes = depth_head(hidden, code0, 1)[0].clone()
-            last[row.idx, :nq] = info.last_codes
+            slots = torch.tensor([info.row.idx for info in ready], dtype=torch.int32, device=self.device)
+            code0 = sample(cb0, slots, 1 if greedy else 0)
+            frames = depth_head(hidden, code0, n)[:n].clone()
+            last[slots.long(), :nq] = frames
             self._frame_ctr += 1
-            frame_bufs[info.request_idx].append(info.last_codes)
-            info.frame_count += 1
-            info.turn_count = 1
-            return True
+            for i, info in enumerate(ready):
+                info.last_codes = frames[i]
+                frame_bufs[info.request_idx].append(info.last_codes)
+                info.frame_count += 1
+                info.turn_count = 1
+            return ok
 
         def backfill() -> None:
+            admitted: "list[_ActiveSlot]" = []
             while pending and self._free:
                 req_idx = pending.pop(0)
                 req = requests[req_idx]
@@ -560,11 +571,12 @@ class Engine:
                 if not req.chunks:
                     row.close()
                     continue
-                info = _ActiveSlot(row=row, request_idx=req_idx, chunks=req.chunks, seq_offset=off)
-                if not advance_slot(info):
-                    row.close()
-                    continue
-                active[row.idx] = info
+                admitted.append(_ActiveSlot(row=row, request_idx=req_idx, chunks=req.chunks, seq_offset=off))
+            for info, k in zip(admitted, advance_slots(admitted)):
+                if k:
+                    active[info.row.idx] = info
+                else:
+                    info.row.close()
 
         backfill()
         prev_slots: list[int] = []
@@ -590,6 +602,7 @@ class Engine:
             last[slots_l, :nq] = frames_all  # a slot that starts a new chunk below overwrites its row
             self._frame_ctr += 1
             to_remove: list[int] = []
+            turning: "list[_ActiveSlot]" = []  # slots whose chunk ended with this step
             for qi, slot in enumerate(slot_list):
                 info = active[slot]
                 if info.frame_count >= max_frames or info.seq_offset >= max_seq:
@@ -598,13 +611,15 @@ class Engine:
                 turn_n = info.turn_count
                 if (turn_n >= min_frames and bool(eos_flags[qi])) or turn_n >= info.max_turn_frames:
                     info.chunk_idx += 1
-                    if not advance_slot(info):
-                        to_remove.append(slot)
+                    turning.append(info)
                     continue
                 info.last_codes = frames_all[qi]
                 frame_bufs[info.request_idx].append(info.last_codes)
                 info.frame_count += 1
                 info.turn_count += 1
+            for info, k in zip(turning, advance_slots(turning)):
+                if not k:
+                    to_remove.append(info.row.idx)
             for slot in to_remove:
                 active.pop(slot).row.close()
             backfill()
