@@ -150,3 +150,43 @@ def test_engine_render_continuous_sampled_bf16():
     st = torch.cat(out)
     assert st.shape[1] == d.n_quantizers and int(st.min()) >= 0 and int(st.max()) < d.codebook_size
     assert len(eng._free) == 4
+
+
+@pytest.mark.gpu
+def test_ingestion_lanes_do_not_change_results():
+    """Blocks of different rows are ingested on side streams at once (Engine.prefill_lanes); the frames must not
+    depend on it: bf16, sampled, five requests with prompts through three rows, one lane against four, and a
+    queue of requests without chunks must drain."""
+    import torch
+
+    from oracle import vui_oracle as O
+    from tests.util import TINY_SD, make_model, tiny_dims
+    from vui_amd.engine import Chunk, Engine, GenConfig, RenderRequest
+
+    # dims the one-pass ingestion accepts (multiples of 64, head_dim 32)
+    d = O.Dims(d_model=128, n_layers=3, n_heads=4, n_kv_heads=2, n_quantizers=4, codebook_size=32, rq_d_model=64,
+               rq_n_layers=1, rq_n_heads=2, vocab_size=50, max_seqlen=256)
+    sd = O.synthetic_state_dict(d, **TINY_SD)
+    g = torch.Generator().manual_seed(3)
+
+    def emb(n):
+        return (torch.randn(1, n, d.d_model, generator=g) * 0.3).to(torch.bfloat16).cuda()
+
+    reqs = [RenderRequest(chunks=[Chunk(emb=emb(5 + i), n_words=2), Chunk(emb=emb(4), n_words=1)], prompt_emb=emb(9 + 2 * i))
+            for i in range(5)]
+    cfg = GenConfig(temperature=0.9, top_k=8, rq_top_k=8, eos_threshold=2.0, max_secs=2.0, seed=5)
+    outs = {}
+    for lanes in (1, 4):
+        m = make_model(d, sd, torch.bfloat16, max_seqlen=d.max_seqlen)
+        eng = Engine(model=m, max_rows=3, max_seq=d.max_seqlen)
+        assert m.decoder._prefill_available()
+        eng.prefill_lanes = lanes
+        outs[lanes] = [o.cpu() for o in eng.render_continuous(reqs, cfg)]
+        m._native.status()
+        assert len(eng._free) == 3
+        # requests that only carry a prompt: more of them than rows, every one admitted and released
+        empty = eng.render_continuous([RenderRequest(chunks=[], prompt_emb=emb(6)) for _ in range(7)], cfg)
+        assert all(o.shape[0] == 0 for o in empty) and len(eng._free) == 3
+    assert all(o.shape[0] > 0 for o in outs[1])
+    for a, b in zip(outs[1], outs[4]):
+        assert torch.equal(a, b)

@@ -212,6 +212,7 @@ class Engine:
         self._free: set[int] = set(range(max_rows))
         self._rows: dict[int, Row] = {}
         self._frame_graphs: dict = {}
+        self._lane_streams: list = []
 
     # ------------------------------------------------------------------ setup
     def _setup_graphs(self) -> None:
@@ -382,16 +383,44 @@ class Engine:
         self.seq_lens[row.idx] = offset
         return offset
 
-    def _prefill_emb(self, row: Row, emb: Tensor, offset: int | None = None) -> Tensor:
+    def _prefill_emb(self, row: Row, emb: Tensor, offset: int | None = None, lane: int = 0) -> Tensor:
         """offset: the row's current length when the caller keeps count of it (saves reading it back from
-        the device, a synchronisation)."""
+        the device, a synchronisation).  lane: see Decoder._prefill."""
         T = emb.shape[1]
         off = row.offset if offset is None else offset
         if off + T > self.max_seq:
             raise ValueError(f"prefill of {T} positions at offset {off} exceeds max_seq={self.max_seq}")
         pos = torch.arange(off, off + T, device=self.device)
         return self.model.decoder.forward_flash(emb.to(self.dtype), pos, slot_idx=row._slot,
-                                                known=(row.idx, off) if offset is not None else None)
+                                                known=(row.idx, off) if offset is not None else None, lane=lane)
+
+    prefill_lanes = 4  # streams that ingest the blocks of different rows at once (1: one after the other)
+
+    def _prefill_many(self, jobs: "list[tuple[Row, Tensor, int]]") -> "list[Tensor]":
+        """Blocks (row, embeddings, the row's length) of different rows through the prompt-ingestion pass.  Rows
+        share nothing but read-only weights, and a short block's kernels fill a fraction of the GPU, so several
+        blocks go out on side streams (default priority, a scratch buffer each) and the calling stream waits for
+        all of them.  The results do not depend on how many lanes there are."""
+        dec = self.model.decoder
+        lanes = min(self.prefill_lanes, len(jobs))
+        if lanes < 2 or not dec._prefill_available() or any(e.shape[1] < dec.PREFILL_MIN for _, e, _ in jobs):
+            return [self._prefill_emb(r, e, offset=o) for r, e, o in jobs]
+        main = torch.cuda.current_stream()
+        if len(self._lane_streams) < lanes:
+            self._lane_streams += [torch.cuda.Stream(device=self.device) for _ in range(lanes - len(self._lane_streams))]
+        used = self._lane_streams[:lanes]
+        start = main.record_event()
+        for s in used:
+            s.wait_event(start)
+        outs = []
+        for i, (r, e, o) in enumerate(jobs):
+            with torch.cuda.stream(used[i % lanes]):
+                h = self._prefill_emb(r, e, offset=o, lane=1 + i % lanes)
+                h.record_stream(main)
+            outs.append(h)
+        for s in used:
+            main.wait_stream(s)
+        return outs
 
     def set_conditioning(self, *, sq_scores=None, wps_score: float = 0.0) -> None:
         self.model.set_cond_bias(sq_scores=sq_scores, wps_score=wps_score)
@@ -535,12 +564,13 @@ class Engine:
             ready = [info for info, k in zip(infos, ok) if k]
             if not ready:
                 return ok
-            hiddens = []
+            jobs = []
             for info in ready:
                 chunk = info.chunks[info.chunk_idx]
                 info.max_turn_frames = cfg.max_turn_frames(chunk.n_words, info.row.prompt_wps)
-                hiddens.append(self._prefill_emb(info.row, chunk.emb, offset=info.seq_offset)[:, -1])
+                jobs.append((info.row, chunk.emb, info.seq_offset))
                 info.seq_offset += chunk.emb.shape[1]
+            hiddens = [h[:, -1] for h in self._prefill_many(jobs)]
             n = len(ready)
             hidden = hiddens[0] if n == 1 else torch.cat(hiddens, dim=0)
             cb0 = model.codec_head(hidden)
@@ -557,26 +587,31 @@ class Engine:
             return ok
 
         def backfill() -> None:
-            admitted: "list[_ActiveSlot]" = []
-            while pending and self._free:
-                req_idx = pending.pop(0)
-                req = requests[req_idx]
-                row = self.new_row()
-                self._rep_counts[row.idx].zero_()
-                row.prompt_wps = req.prompt_wps
-                off = 0  # new_row starts the slot at length zero
-                if req.prompt_emb is not None and req.prompt_emb.shape[1] > 0:
-                    self._prefill_emb(row, req.prompt_emb, offset=0)
-                    off = req.prompt_emb.shape[1]
-                if not req.chunks:
-                    row.close()
-                    continue
-                admitted.append(_ActiveSlot(row=row, request_idx=req_idx, chunks=req.chunks, seq_offset=off))
-            for info, k in zip(admitted, advance_slots(admitted)):
-                if k:
-                    active[info.row.idx] = info
-                else:
-                    info.row.close()
+            while pending and self._free:  # again while rows closed below leave room for waiting requests
+                prompts, taken = [], []
+                while pending and self._free:
+                    req_idx = pending.pop(0)
+                    req = requests[req_idx]
+                    row = self.new_row()
+                    self._rep_counts[row.idx].zero_()
+                    row.prompt_wps = req.prompt_wps
+                    off = 0  # new_row starts the slot at length zero
+                    if req.prompt_emb is not None and req.prompt_emb.shape[1] > 0:
+                        prompts.append((row, req.prompt_emb, 0))
+                        off = req.prompt_emb.shape[1]
+                    taken.append((row, req_idx, req, off))
+                self._prefill_many(prompts)
+                admitted: "list[_ActiveSlot]" = []
+                for row, req_idx, req, off in taken:
+                    if not req.chunks:
+                        row.close()
+                        continue
+                    admitted.append(_ActiveSlot(row=row, request_idx=req_idx, chunks=req.chunks, seq_offset=off))
+                for info, k in zip(admitted, advance_slots(admitted)):
+                    if k:
+                        active[info.row.idx] = info
+                    else:
+                        info.row.close()
 
         backfill()
         prev_slots: list[int] = []

@@ -252,7 +252,7 @@ class Decoder:
                                               m.rope_theta_rescale_factor).to(model.device)
         self.flash_kv_caches: list[FlashKVCache] | None = None
         self._k = self._v = None
-        self._prefill_scratch: Tensor | None = None
+        self._prefill_scratch: dict[int, Tensor] = {}  # one buffer per lane (stream) that ingests prompts
         self._prefill_ok: bool | None = None
 
     def allocate_flash_kv_cache(self, batch_size: int, device, dtype=torch.bfloat16, max_seqlen: int | None = None):
@@ -295,7 +295,7 @@ class Decoder:
         return max(1, min(32, 1024 // max(1, B * H)))
 
     def forward_flash(self, x: Tensor, positions: Tensor, per_sample_positions: bool = False,
-                      slot_idx: Tensor | None = None, known: "tuple[int, int] | None" = None) -> Tensor:
+                      slot_idx: Tensor | None = None, known: "tuple[int, int] | None" = None, lane: int = 0) -> Tensor:
         """x (B, T, d) appended at seq_lens[slot]; returns the final-norm output (B, T, d) and advances
         seq_lens by T (src/vui/model.py:534-549).  The native step rotates at the position it writes
         to, so `positions` must be the cache positions (seq_lens .. seq_lens+T-1), as in every
@@ -305,7 +305,7 @@ class Decoder:
             raise ValueError(f"batch {B} > {MAX_BATCH}")
         model = self._model
         if B == 1 and T >= self.PREFILL_MIN and self._prefill_available():
-            return self._prefill(x, slot_idx, known)
+            return self._prefill(x, slot_idx, known, lane)
         out = torch.empty_like(x)
         st = torch.cuda.current_stream().cuda_stream
         ns = self.default_splits(B)
@@ -327,9 +327,10 @@ class Decoder:
             self._prefill_ok = nat.lib.vui_prefill_scratch_bytes(C.byref(nat.cfg), 1, 1) >= 0
         return self._prefill_ok
 
-    def _prefill(self, x: Tensor, slot_idx: Tensor | None, known: "tuple[int, int] | None" = None) -> Tensor:
+    def _prefill(self, x: Tensor, slot_idx: Tensor | None, known: "tuple[int, int] | None" = None, lane: int = 0) -> Tensor:
         """One row, T positions: the matrix-core pass of the native library, in chunks.  known = (slot, length
-        of the slot) from a caller that keeps count: otherwise both are read back from the device."""
+        of the slot) from a caller that keeps count: otherwise both are read back from the device.  lane: which
+        scratch buffer to use; passes of different rows that run on different streams at once take different lanes."""
         model = self._model
         nat = model._native
         seq_lens = self.flash_kv_caches[0].seq_lens
@@ -348,9 +349,10 @@ class Decoder:
             need = nat.lib.vui_prefill_scratch_bytes(C.byref(nat.cfg), n, pos + n)
             if need < 0:
                 raise RuntimeError(f"vui_prefill_scratch_bytes failed: {_lib.last_error()}")
-            if self._prefill_scratch is None or self._prefill_scratch.numel() < need + 256:
-                self._prefill_scratch = torch.empty(need + 256, dtype=torch.uint8, device=x.device)
-            base = (self._prefill_scratch.data_ptr() + 255) & ~255
+            buf = self._prefill_scratch.get(lane)
+            if buf is None or buf.numel() < need + 256:
+                buf = self._prefill_scratch[lane] = torch.empty(need + 256, dtype=torch.uint8, device=x.device)
+            base = (buf.data_ptr() + 255) & ~255
             xc = x[0, t0:t0 + n].contiguous()
             _lib.check(nat.lib.vui_prefill(nat.handle, xc.data_ptr(), n, slot, pos, seq_lens.data_ptr(), self._k.data_ptr(),
                                            self._v.data_ptr(), out[0, t0:t0 + n].data_ptr(), base, need, st), "vui_prefill")
