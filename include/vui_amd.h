@@ -196,7 +196,8 @@ int vui_rq_generate(vui_ctx* ctx, const void* hidden, const int64_t* code0, cons
  * pos0 + T) bytes, 256-byte aligned; the library allocates nothing.  vui_prefill_scratch_bytes returns
  * VUI_EINVAL for a configuration the pass does not take (fp32 or int8 weights, d_model / heads x head_dim /
  * ffn not multiples of 64, head_dim not a multiple of 32): such prompts go position by position through
- * vui_backbone_step. */
+ * vui_backbone_step.  Calls for different slots may be in flight on different streams at once if each has a
+ * scratch buffer of its own: beyond the caller's buffers a call touches only read-only weights. */
 int64_t vui_prefill_scratch_bytes(const vui_config* cfg, int T, int L);
 int vui_prefill(vui_ctx* ctx, const void* emb_in, int T, int slot, int pos0, int32_t* seq_lens, void* k_cache,
                 void* v_cache, void* hidden_out, void* scratch, int64_t scratch_bytes, vui_stream_t stream);
