@@ -202,6 +202,80 @@ __device__ __forceinline__ void norm_rows(const float* xres, const NormRegs& nw,
   }
 }
 
+// Residual add of an exchanged vector and the norm that follows it, row by row inside one wave: wave w waits for the
+// words of rows w, w + 4, ... (a lane for the four words of chunk lane, and of chunk lane + 64), adds them to the
+// residual stream (x = rnd(x + y), written back), and normalises the row at once - the row never leaves the wave, so
+// no barrier stands between the wait, the add and the norm.  buf: the group's rows, R/2 words each.
+__device__ __forceinline__ void poll_add_norm_rows(const uint64_t* buf, Ctl& c, float* xres, const NormRegs& nw, float eps, int R,
+                                                   int B, uint32_t* xp, int xs) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int nch = R / 8;
+  const int NI = nch > WAVE ? 2 : 1;  // chunks per lane
+  for (int b = wave; b < B; b += 4) {
+    const uint64_t* row = buf + (size_t)b * (R / 2);
+    float* x = xres + (size_t)b * R;
+    uint64_t v[2][4] = {};
+    int spins = 0;
+    while (true) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        if (i >= NI) break;                            // uniform
+        const int ch = min(lane + WAVE * i, nch - 1);  // a chunk past the row repeats the last one and is dropped below
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[i][k] = ll_ld(row + 4 * ch + k);
+      }
+      bool all = true;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) all = all && (i >= NI || (uint32_t)(v[i][k] >> 32) == c.epoch);
+      if (all || c.dead) break;
+      if (++spins > SPIN_LIMIT) {
+        c.dead = 1;
+        __hip_atomic_store(c.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    float q[2][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      if (i >= NI) break;
+      const int ch = min(lane + WAVE * i, nch - 1);
+      const float4 o0 = *reinterpret_cast<const float4*>(x + ch * 8), o1 = *reinterpret_cast<const float4*>(x + ch * 8 + 4);
+      const float old[8] = {o0.x, o0.y, o0.z, o0.w, o1.x, o1.y, o1.z, o1.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t y = (uint32_t)v[i][k];
+        const uint32_t pk = f2bf2(old[2 * k] + bf_lo(y), old[2 * k + 1] + bf_hi(y));
+        q[i][2 * k] = bf_lo(pk); q[i][2 * k + 1] = bf_hi(pk);
+      }
+      const float t = (q[i][0] * q[i][0] + q[i][1] * q[i][1]) + (q[i][2] * q[i][2] + q[i][3] * q[i][3]) +
+                      (q[i][4] * q[i][4] + q[i][5] * q[i][5]) + (q[i][6] * q[i][6] + q[i][7] * q[i][7]);
+      if (lane + WAVE * i < nch) {
+        ss += t;
+        *reinterpret_cast<float4*>(x + ch * 8) = make_float4(q[i][0], q[i][1], q[i][2], q[i][3]);
+        *reinterpret_cast<float4*>(x + ch * 8 + 4) = make_float4(q[i][4], q[i][5], q[i][6], q[i][7]);
+      }
+    }
+    ss = wave_sum_v(ss);
+    const float r = 1.0f / sqrtf(ss / (float)R + eps);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int ch = lane + WAVE * i;
+      if (ch < nch) {
+        const uint4 g = nw.w[i];
+        uint4 o;
+        uint32_t t;
+        t = f2bf2(q[i][0] * r, q[i][1] * r); o.x = f2bf2(bf_lo(t) * bf_lo(g.x), bf_hi(t) * bf_hi(g.x));
+        t = f2bf2(q[i][2] * r, q[i][3] * r); o.y = f2bf2(bf_lo(t) * bf_lo(g.y), bf_hi(t) * bf_hi(g.y));
+        t = f2bf2(q[i][4] * r, q[i][5] * r); o.z = f2bf2(bf_lo(t) * bf_lo(g.z), bf_hi(t) * bf_hi(g.z));
+        t = f2bf2(q[i][6] * r, q[i][7] * r); o.w = f2bf2(bf_lo(t) * bf_lo(g.w), bf_hi(t) * bf_hi(g.w));
+        *reinterpret_cast<uint4*>(xp + (size_t)b * xs + ch * 4) = o;
+      }
+    }
+  }
+}
+
 // i / nw for i < 65536 with inv = ceil(2^32 / nw)
 __device__ __forceinline__ int div_small(int i, uint32_t inv) { return (int)__umulhi((uint32_t)i, inv); }
 
@@ -227,20 +301,6 @@ struct RqBatchArgs {
 };
 
 struct RbLayer { const bf16_t *attn_norm, *wqkv, *wo, *mlp_norm, *w1, *w3, *w2; };
-
-// residual add of an exchanged vector: x = rnd(x + y) for the group's rows
-#define RB_POLL_ADD(buf, nwords)                                                                      \
-  do {                                                                                                \
-    __syncthreads();                                                                                  \
-    ll_poll((buf) + (size_t)b0 * (nwords), Bg * (nwords), c, [&](int i, uint32_t v) {                \
-      const int lr = div_small(i, inv_r2), j = i - lr * (R / 2);                                      \
-      float2* px = reinterpret_cast<float2*>(xres + (size_t)lr * R + 2 * j);                          \
-      const float2 o = *px;                                                                           \
-      const uint32_t pk = f2bf2(o.x + bf_lo(v), o.y + bf_hi(v));                                      \
-      *px = make_float2(bf_lo(pk), bf_hi(pk));                                                        \
-    });                                                                                               \
-    __syncthreads();                                                                                  \
-  } while (0)
 
 __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -388,8 +448,8 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
         tile_prefetch<8, false>((const bf16_t*)Lw.wqkv, nullptr, t0, w0);
         tile_prefetch<8, false>((const bf16_t*)Lw.wqkv, nullptr, t1, w1);
         const NormRegs nw = load_norm((const bf16_t*)Lw.attn_norm, R);
-        if (ybuf) RB_POLL_ADD(ybuf, R / 2);
-        norm_rows(xres, nw, a.rq_eps, R, Bg, xp, xs);
+        if (ybuf) poll_add_norm_rows(ybuf + (size_t)b0 * (R / 2), c, xres, nw, a.rq_eps, R, Bg, xp, xs);
+        else norm_rows(xres, nw, a.rq_eps, R, Bg, xp, xs);
         __syncthreads();
         auto epi = [&](int n, int lr, const float* v, const float*) {
           uint64_t* dst = qkvb + (size_t)(b0 + lr) * (3 * R / 2) + n / 2;
@@ -500,8 +560,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
         tile_prefetch<8, true>((const bf16_t*)Lw.w1, (const bf16_t*)Lw.w3, t0, w0);
         tile_prefetch<8, true>((const bf16_t*)Lw.w1, (const bf16_t*)Lw.w3, t1, w1);
         const NormRegs nw = load_norm((const bf16_t*)Lw.mlp_norm, R);
-        RB_POLL_ADD(ob, R / 2);
-        norm_rows(xres, nw, a.rq_eps, R, Bg, xp, xs);
+        poll_add_norm_rows(ob + (size_t)b0 * (R / 2), c, xres, nw, a.rq_eps, R, Bg, xp, xs);
         __syncthreads();
         auto epi = [&](int n, int lr, const float* v, const float* u) {
           float h[4];
@@ -552,8 +611,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
         tile_prefetch<8, false>(hw_, nullptr, t0, w0);
         tile_prefetch<8, false>(hw_, nullptr, t1, w1);
         const NormRegs nw = load_norm(g_norm, R);
-        RB_POLL_ADD(ybuf, R / 2);
-        norm_rows(xres, nw, a.rq_eps, R, Bg, xp, xs);
+        poll_add_norm_rows(ybuf + (size_t)b0 * (R / 2), c, xres, nw, a.rq_eps, R, Bg, xp, xs);
         __syncthreads();
         auto epi = [&](int n, int lr, const float* v, const float*) {
           uint64_t* dst = lgb + (size_t)(b0 + lr) * (CS / 2) + n / 2;
