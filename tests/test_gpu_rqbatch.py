@@ -32,10 +32,17 @@ def _small_dims():
                   rq_n_layers=2, rq_n_heads=4, vocab_size=50, max_seqlen=64)
 
 
-@pytest.mark.parametrize("dims", ["small", "nano"])
+def _wide_dims():
+    # a 640-d depth head: 80 chunks of 8 (a lane of the fused wait + norm holds a second, partly filled chunk) and
+    # 40 out_proj / W2 tiles (more than half of a row group's workgroups: every tile takes all rows)
+    return O.Dims(d_model=128, n_layers=1, n_heads=4, n_kv_heads=4, n_quantizers=5, codebook_size=64, rq_d_model=640,
+                  rq_n_layers=2, rq_n_heads=8, vocab_size=50, max_seqlen=64)
+
+
+@pytest.mark.parametrize("dims", ["small", "wide", "nano"])
 def test_batched_depth_head_vs_oracle_and_sequence(dims):
-    if dims == "small":
-        d, sd = _small_dims(), None
+    if dims in ("small", "wide"):
+        d = _small_dims() if dims == "small" else _wide_dims()
         sd = O.synthetic_state_dict(d, **TINY_SD)
     else:
         d = O.Dims()
