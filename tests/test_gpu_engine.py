@@ -286,3 +286,26 @@ def test_full_size_streaming_workload_properties():
     assert torch.equal(f0, f1) and torch.equal(e0, e1)
     f2, *_ = run(1)
     assert not torch.equal(f0, f2)
+
+
+def test_backbone_alone_in_one_launch_when_depth_head_cache_does_not_fit():
+    """A depth head whose 16-position cache exceeds LDS (768 wide, 5 layers: 245 KB) cannot run inside the one-launch
+    frame kernel; the backbone step still does, and the frames equal those of the kernel sequence."""
+    from vui_amd.engine import GenConfig
+
+    d = O.Dims(d_model=128, n_layers=2, n_heads=4, n_kv_heads=4, n_quantizers=16, codebook_size=64, rq_d_model=768,
+               rq_n_layers=5, rq_n_heads=8, vocab_size=50, max_seqlen=64)
+    sd = O.synthetic_state_dict(d, **TINY_SD)
+    cfg = GenConfig(temperature=0.9, top_k=10, rq_top_k=10, rep_penalty=1.2, rep_window=4, seed=3)
+    ids = torch.tensor([4, 9, 2, 7])
+    out = {}
+    for fused in (1, 0):
+        m, eng = _engine(d, sd, BF)
+        assert m._native.fused(fused) is False  # the whole frame never fits
+        row = eng.new_row()
+        h = row.prefill_emb(m.token_emb(ids.cuda()[None]))[:, -1]
+        frames, eos = eng.generate([row], h, 8, cfg)
+        m._native.status()
+        out[fused] = (frames.cpu(), eos.cpu())
+    assert torch.equal(out[0][0], out[1][0])
+    np.testing.assert_allclose(out[0][1].numpy(), out[1][1].numpy(), rtol=0, atol=0)

@@ -40,7 +40,8 @@ struct vui_ctx {
   void* rq_tw;    // the depth head's matrices in the batched kernel's operand layout
   vui_weights* wdev_t;  // device copy of the weight table with those matrices' pointers
   int fused_ok, fused_on, nwg, ns;
-  size_t lds_bytes;
+  int fused_bb_ok;      // the backbone step alone can run as the one-launch kernel (its LDS need is smaller)
+  size_t lds_bytes, lds_bb;
   char fused_why[96];
   uint64_t* prof;
   int prof_cap, prof_wg;
@@ -200,11 +201,20 @@ int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream) {
   ctx->lds_bytes = frame_lds_bytes(ctx->cfg);
   int n_cu = 0;
   ctx->nwg = FUSED_NWG;
-  if (frame_supported(ctx->cfg, ctx->nwg, ctx->ns, ctx->fused_why, sizeof(ctx->fused_why))) {
+  if (frame_supported(ctx->cfg, ctx->nwg, ctx->ns, true, ctx->fused_why, sizeof(ctx->fused_why))) {
     const int cap = frame_max_resident(ctx->lds_bytes, &n_cu);
     if (cap < 0) return cap;
     if (cap >= ctx->nwg) ctx->fused_ok = 1;
     else snprintf(ctx->fused_why, sizeof(ctx->fused_why), "only %d workgroups can be resident (%d CUs), %d needed", cap, n_cu, ctx->nwg);
+  }
+  // a depth head whose keys/values do not fit in LDS still leaves the backbone step to the one-launch kernel
+  ctx->fused_bb_ok = ctx->fused_ok;
+  ctx->lds_bb = ctx->lds_bytes;
+  if (!ctx->fused_ok && frame_supported(ctx->cfg, ctx->nwg, ctx->ns, false, nullptr, 0)) {
+    ctx->lds_bb = frame_lds_bytes_backbone(ctx->cfg);
+    const int cap = frame_max_resident(ctx->lds_bb, &n_cu);
+    if (cap < 0) return cap;
+    if (cap >= ctx->nwg) ctx->fused_bb_ok = 1;
   }
   ctx->rqb_ok = 0;
   ctx->rqb_why[0] = 0;
@@ -293,7 +303,7 @@ int vui_backbone_step(vui_ctx* ctx, const int64_t* codes_in, const void* emb_in,
   if (!seq_lens || !k_cache || !v_cache) { vui_set_error("seq_lens and the KV caches are required"); return VUI_EINVAL; }
   const vui_config& c = ctx->cfg;
   hipStream_t st = (hipStream_t)stream;
-  if (use_fused(ctx, B)) {
+  if (ctx->fused_bb_ok && ctx->fused_on && B == 1) {
     FrameArgs a;
     fused_base(ctx, a);
     a.mode = FR_BACKBONE;
@@ -302,7 +312,8 @@ int vui_backbone_step(vui_ctx* ctx, const int64_t* codes_in, const void* emb_in,
     a.hidden_out = (uint16_t*)(hidden_out ? hidden_out : ctx->hidden);
     a.cb0_out = (uint16_t*)(cb0_out ? cb0_out : ctx->cb0);
     a.eos_out = (uint16_t*)(eos_out ? eos_out : ctx->eos);
-    return launch_frame(a, ctx->nwg, ctx->lds_bytes, st);
+    if (!ctx->fused_ok) a.lds_kv_off = (int)ctx->lds_bb;  // no depth-head cache in this launch
+    return launch_frame(a, ctx->nwg, ctx->fused_ok ? ctx->lds_bytes : ctx->lds_bb, st);
   }
   const int d = c.d_model, H = c.n_heads, KV = c.n_kv_heads, hd = c.head_dim;
   if (codes_in) rc = launch_embed(c.dtype, codes_in, ctx->w.audio_emb, ctx->x, B, c.n_quantizers, c.codebook_size, d, st);

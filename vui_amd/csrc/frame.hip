@@ -1079,8 +1079,11 @@ size_t frame_rq_cache_bytes(const vui_config& c) {
 size_t frame_lds_bytes(const vui_config& c) {
   return (size_t)LDS_FIXED + frame_ptr_bytes(c) + frame_rq_cache_bytes(c);
 }
+// launches that stop after the backbone step need no room for the depth head's keys and values
+size_t frame_lds_bytes_backbone(const vui_config& c) { return (size_t)LDS_FIXED + frame_ptr_bytes(c); }
 
-bool frame_supported(const vui_config& c, int nwg, int ns, char* why, size_t why_len) {
+// with_rq false: only what a backbone-step launch (mode FR_BACKBONE alone) needs
+bool frame_supported(const vui_config& c, int nwg, int ns, bool with_rq, char* why, size_t why_len) {
   const char* r = nullptr;
   if (c.dtype != VUI_DTYPE_BF16) r = "bf16 only";
   else if (c.int8_backbone) r = "int8 weights use the per-kernel path";
@@ -1090,7 +1093,7 @@ bool frame_supported(const vui_config& c, int nwg, int ns, char* why, size_t why
   else if ((c.head_dim & 7) || c.head_dim > 128) r = "head_dim";
   else if ((c.rq_dim / c.rq_heads) % 2 || c.rq_dim / c.rq_heads > 128) r = "depth-head head_dim must be even, at most 128";
   else if ((c.d_model | c.ffn | c.rq_dim | c.rq_ffn) & 7) r = "vector lengths must be multiples of 8";
-  else if (frame_lds_bytes(c) > 160 * 1024) r = "depth-head keys/values do not fit in LDS";
+  else if (with_rq && frame_lds_bytes(c) > 160 * 1024) r = "depth-head keys/values do not fit in LDS";
   else if (c.rq_layers < 1) r = "no depth head";
   else {
     const int np_max = (c.n_heads + 2 * c.n_kv_heads) * c.head_dim / 2;

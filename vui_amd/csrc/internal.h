@@ -186,7 +186,8 @@ enum { FR_BACKBONE = 1, FR_CB0 = 2, FR_RQ = 4, FR_FINISH = 8 };
 size_t frame_ll_words(const vui_config& c, int ns);
 size_t frame_lds_bytes(const vui_config& c);
 size_t frame_rq_cache_bytes(const vui_config& c);
-bool frame_supported(const vui_config& c, int nwg, int ns, char* why, size_t why_len);
+size_t frame_lds_bytes_backbone(const vui_config& c);
+bool frame_supported(const vui_config& c, int nwg, int ns, bool with_rq, char* why, size_t why_len);
 int frame_max_resident(size_t lds_bytes, int* n_cu);
 int launch_frame(const FrameArgs& a, int nwg, size_t lds_bytes, hipStream_t st);
 
