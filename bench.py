@@ -116,6 +116,9 @@ def gpu_bench(args):
 # HBM traffic of one frame_kernel launch on the default workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch) scaled by what the same counters read for a plain copy of known size;
 # see profiles/frame_kernel_e2e_b1.txt.  None until measured.
+# MFMA busy cycles / busy cycles of the 16-stream step's matrix-core kernels, from rocprofv3 --pmc
+# SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CYCLES; see profiles/e2e_b16_int8_step_kernels.txt.
+MEASURED_B16_MFMA_BUSY = {"gemm16_kernel": [0.08, 0.16], "rq_batch_kernel": 0.30}
 MEASURED_TRAFFIC_BYTES = 517_680_951  # at cache length 596..651 (algorithmic 414.6 MB there): 1.25 x
 
 
@@ -238,8 +241,10 @@ def b16_line(sd, preset="A", n=100):
     us = e0.elapsed_time(e1) * 1e3 / n
     kv_bytes = float((lens.float() + 3 + n / 2 + 1).sum()) * 2 * m.kv_heads * m.head_dim * 2 * m.n_layers
     wbytes = frame_bytes(m, 0, 1)["backbone"] - (m.n_quantizers * m.d_model + 2 * m.kv_heads * m.head_dim * 2 * m.n_layers)
+    gbs = (kv_bytes + wbytes) / us / 1e3
     return {"config": "e2e_b16_int8_ragged", "us_per_frame_step": round(us, 1), "aggregate_frames_per_s": round(16e6 / us, 1),
-            "kv_bytes": int(kv_bytes), "int8_weight_bytes": int(wbytes), "achieved_GBs": round((kv_bytes + wbytes) / us / 1e3, 1)}
+            "rtf": round(16e6 / us / 12.5, 1), "steps": n, "kv_bytes": int(kv_bytes), "int8_weight_bytes": int(wbytes),
+            "achieved_GBs": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "mfma_busy_frac": MEASURED_B16_MFMA_BUSY}
 
 
 def serve_line(sd, preset="A", n_requests=32, max_rows=16):
@@ -293,33 +298,6 @@ def copy_line():
     us = e0.elapsed_time(e1) * 1e3 / 10
     return {"config": "device_copy_1GiB", "us": round(us, 1), "read_plus_write_GBs": round(2 * (1 << 30) / us / 1e3, 1),
             "frac_of_8TBs": round(2 * (1 << 30) / us / 1e3 / HBM_PEAK_GBS, 3)}
-
-
-def loadpat_line():
-    """What an operand fragment costs to fetch: 16-byte-per-lane loads from a 3 MB (L2-sized) buffer under three
-    lane -> address patterns, 4096 workgroups x 384 loads per lane each (vui_debug_load_pattern)."""
-    import torch
-
-    from vui_amd import _lib
-
-    lib = _lib.load()
-    buf = torch.ones(2048 * 1536, dtype=torch.uint8, device="cuda")
-    sink = torch.zeros(16, dtype=torch.uint8, device="cuda")
-    st = torch.cuda.current_stream().cuda_stream
-    grid, iters = 4096, 48
-    out = {"config": "load_pattern_16B_per_lane", "buffer_bytes": buf.numel()}
-    for pat, name in ((0, "rows16_x_64B"), (1, "rows8_x_128B"), (2, "contiguous_1KiB")):
-        best = None
-        for _ in range(5):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            _lib.check(lib.vui_debug_load_pattern(pat, grid, iters, buf.data_ptr(), buf.numel(), sink.data_ptr(), st), "vui_debug_load_pattern")
-            e1.record()
-            torch.cuda.synchronize()
-            ms = e0.elapsed_time(e1)
-            best = ms if best is None else min(best, ms)
-        out[name + "_TBs"] = round(grid * 256 * iters * 128 / best / 1e9, 2)
-    return out
 
 
 def suite(model, eng, d, sd, preset="A"):
@@ -410,33 +388,62 @@ def suite(model, eng, d, sd, preset="A"):
     lines.append(b16_line(sd, preset))
     lines.append(serve_line(sd, preset))
     lines.append(copy_line())
-    lines.append(loadpat_line())
     return lines
 
 
-def cpu_baseline(preset, n_frames: int = 150, n_ctx: int = 576):
-    """The CPU oracle (a port of the reference's fp32 CPU path) on a bounded sample of the same
-    workload (about 10 s of CPU work): the 576-position context, then n_frames sampled frames; host cores of this box."""
+def cpu_baseline(preset, n_frames: int = 40, n_frames_bf16: int = 16, n_prefix: int = 512, n_text: int = 64):
+    """The CPU oracle (a port of the reference's CPU path) on a bounded sample of the same workload, on this
+    box's host cores: the headline context (512 prefix frames through the audio embedding + 64 text ids, seed 0)
+    is ingested once, then n_frames frames (backbone step + depth head, greedy as the baseline plan asks) are
+    timed three times after one warm-up and the median is reported; the same in the oracle's bf16 regime on a
+    shorter sample.  Threads: the box's CPU share (OMP_NUM_THREADS where the box sets it, else every CPU)."""
+    import platform
+
     import torch
 
     from oracle import vui_oracle as O
 
-    threads = min(16, os.cpu_count() or 1)
+    host_cpus = os.cpu_count() or 1
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or host_cpus
+    threads = max(1, min(threads, host_cpus))
     torch.set_num_threads(threads)
     d = O.Dims() if preset == "A" else O.Dims(rq_d_model=768, rq_n_layers=5, rq_n_heads=8, vocab_size=50534)
     sd = O.synthetic_state_dict(d, seed=0)
-    o = O.OracleModel(d, sd, torch.float32, max_seqlen=n_ctx + n_frames + 8)
     g = torch.Generator().manual_seed(0)
-    ids = torch.randint(0, d.vocab_size, (n_ctx,), generator=g)
-    with torch.inference_mode():
-        h = o.prefill(o.embed_text(ids))[-1:]
-        o.generate_frames(h, 2, temperature=0.9, top_k=100, rep_penalty=1.1, rep_window=24)  # warm
-        t0 = time.perf_counter()
-        o.generate_frames(h, n_frames, temperature=0.9, top_k=100, rep_penalty=1.1, rep_window=24)
-        dt = time.perf_counter() - t0
-    return {"value": round(n_frames / dt, 3), "unit": "frames/s", "cores": threads, "kind": "port",
-            "sample": f"fp32 oracle, {n_ctx}-position prefill then {n_frames} frames (backbone step + depth head), "
-                      f"torch CPU ops with {threads} threads"}
+    prefix = torch.randint(0, d.codebook_size, (n_prefix, d.n_quantizers), generator=g)
+    ids = torch.randint(0, d.vocab_size, (n_text,), generator=g)
+    cpu_model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for ln in f:
+                if ln.startswith("model name"):
+                    cpu_model = ln.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        cpu_model = platform.processor()
+
+    def run(dt, n):
+        o = O.OracleModel(d, sd, dt, max_seqlen=n_prefix + n_text + n + 8)
+        with torch.inference_mode():
+            ctx = torch.cat([o.embed_audio(prefix), o.embed_text(ids)], 0)
+            h = o.prefill(ctx)[-1:]
+            L0 = int(o.seq_lens[0])
+            times = []
+            for rep in range(4):  # one warm-up, then three timed passes from the same cache state
+                o.seq_lens[0] = L0
+                t0 = time.perf_counter()
+                o.generate_frames(h, n, temperature=1.0, top_k=1)
+                times.append(time.perf_counter() - t0)
+        return n / sorted(times[1:])[1]
+
+    f32 = run(torch.float32, n_frames)
+    bf16 = run(torch.bfloat16, n_frames_bf16)
+    return {"value": round(f32, 3), "unit": "frames/s", "cores": threads, "kind": "port",
+            "value_bf16_regime": round(bf16, 3), "rtf": round(f32 / 12.5, 3), "ms_per_frame": round(1e3 / f32, 2),
+            "host_cpus": host_cpus, "cpu_model": cpu_model,
+            "sample": f"fp32 oracle: {n_prefix} prefix frames + {n_text} text ids ingested, then {n_frames} greedy frames "
+                      f"(backbone step + depth head), median of 3 after 1 warm-up; bf16 regime: {n_frames_bf16} frames; "
+                      f"torch CPU ops, {threads} threads of {host_cpus} CPUs"}
 
 
 def main():
@@ -447,6 +454,7 @@ def main():
     ap.add_argument("--preset", default="A", choices=["A", "B"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--no-b16", action="store_true", help="skip the 16-stream int8 leg of the default line")
     ap.add_argument("--suite", action="store_true", help="also print one JSON line per further benchmark config")
     ap.add_argument("--calib", action="store_true",
                     help="end with three plain 512 MiB device copies (reference points for hardware counters)")
@@ -458,8 +466,6 @@ def main():
                     help="print only the continuous-batching line (32 requests through 16 rows, wall clock)")
     ap.add_argument("--vocoder-only", action="store_true",
                     help="print only the vocoder line (the run rocprofv3 summaries of the vocoder kernels come from)")
-    ap.add_argument("--loadpat-only", action="store_true",
-                    help="print only the load-pattern line (what an operand fragment costs to fetch)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (streams are independent); "
@@ -467,9 +473,6 @@ def main():
         sys.exit(2)
     if args.vocoder_only:
         print(json.dumps(vocoder_line()[1]))
-        return
-    if args.loadpat_only:
-        print(json.dumps(loadpat_line()))
         return
     if args.prefill_only:
         import torch
@@ -497,6 +500,10 @@ def main():
     out, (model, eng, d, sd) = gpu_bench(args)
     if not args.no_roofline:
         out["roofline"] = kernel_roofline(out, out["frame_bytes"])
+    if not args.no_b16 and not args.suite:
+        # batch 16 (benchmark configuration 5) beside the batch-1 figure, after its timed region: 16 int8 streams
+        # with ragged caches, a bounded number of replays of the captured step
+        out["b16"] = b16_line(sd, args.preset, n=60)
     extra = suite(model, eng, d, sd, args.preset) if args.suite else []
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.preset)

@@ -5,9 +5,18 @@
  * surface of src/vui/model.py and src/vui/engine.py, whose GPU arithmetic is delegated to
  * torch/cuBLAS, flash_attn_with_kvcache and torch.cuda.CUDAGraph.  Each entry point below
  * names the reference call it stands in for.  All pointers marked "device" are HIP device
- * pointers; the library never allocates, frees or synchronises: buffers (weights, KV caches,
- * workspace, outputs) are owned by the caller, work is enqueued on the given stream, and
- * every call may be recorded into a HIP graph.
+ * pointers; the library never allocates or frees device memory: buffers (weights, KV caches,
+ * workspace, outputs) are owned by the caller.  Work is enqueued on the given stream without
+ * waiting for it, and the per-step calls may be recorded into a HIP graph; the exceptions are
+ * vui_ctx_init and vui_ctx_status, which wait for the stream / the device (said at each).
+ *
+ * Persistent kernels: the batch-1 frame kernel, the batched depth head and the vocoder's trunk
+ * kernel keep one workgroup resident on every compute unit and hand values to each other
+ * while they run.  While such a launch is in flight NO other kernel may run on the device
+ * (another stream, another context, another process): a workgroup kept off its compute unit
+ * makes the others wait until a bounded spin gives up, the launch then commits nothing (no
+ * position update, no repetition state, no codes), raises the context's error word, and
+ * vui_ctx_status reports VUI_EHIP until the context is initialised again with vui_ctx_init.
  *
  * Return value: 0 on success, a negative VUI_E* code on failure; vui_last_error() returns a
  * human-readable description of the last failure on the calling thread.
@@ -108,8 +117,10 @@ int64_t vui_kv_bytes(const vui_config* cfg);
 int vui_ctx_create(const vui_config* cfg, const vui_weights* w, void* workspace, int64_t workspace_bytes,
                    int max_batch, vui_ctx** out);
 void vui_ctx_destroy(vui_ctx* ctx);
-/* One-time device-side initialisation of the workspace (zeroes counters, writes the prefill copy of the
- * projection weights: the weight tensors must hold their final values).  Enqueued on stream. */
+/* Device-side initialisation of the workspace (zeroes counters, exchange words and the error word, writes
+ * the prefill copy of the projection weights: the weight tensors must hold their final values).  Enqueues
+ * on stream AND waits for the stream before it returns (it copies from host locals and then asks the
+ * runtime how many workgroups can be resident).  May be called again to clear a raised error word. */
 int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream);
 
 /* The batch-1 bf16 calls below run as one persistent kernel ("fused") when the device can keep
@@ -123,7 +134,10 @@ int vui_ctx_fused(vui_ctx* ctx, int enable);
 /* 1 when the depth head of 2..16 rows runs as one persistent kernel (bf16, enough resident workgroups, the
  * fused form switched on), else 0 and vui_last_error() says why.  No counterpart in the reference. */
 int vui_ctx_rq_batch(vui_ctx* ctx);
-/* Synchronous health check: VUI_EHIP if a fused launch gave up waiting for another workgroup. */
+/* Synchronous health check (a blocking 16-byte device-to-host copy): VUI_EHIP if a persistent launch gave up
+ * waiting for another workgroup, or if the 32-bit launch count of the context has wrapped (after 2^32 - 1
+ * persistent launches; the launch that would wrap does nothing).  Either way nothing was committed by the
+ * failing launch and the context stays unusable until vui_ctx_init is called again. */
 int vui_ctx_status(vui_ctx* ctx);
 
 /* Profiling aid: fused launches made after this call let four workgroups (`workgroup`, +1, +8, +131;
@@ -132,13 +146,6 @@ int vui_ctx_status(vui_ctx* ctx);
  * receives the count in its low 32 bits and the launch's shader cycles above.  buf = NULL switches
  * it off.  No counterpart in the reference. */
 int vui_debug_phase_clock(vui_ctx* ctx, uint64_t* buf, int cap, int workgroup);
-
-/* Measurement aid behind the operand layouts of the prompt-ingestion pass: `grid` workgroups of 256 threads each
- * issue iters x 8 loads of 16 bytes per lane from buf (buf_bytes >= 1536, 16-byte aligned; every address is reduced
- * modulo the buffer) with lane -> address pattern 0 (16 rows x 64 bytes per instruction: an operand fragment read from
- * a row-major matrix), 1 (8 rows x 128 bytes) or 2 (1 KiB contiguous); bytes moved = grid * 256 * iters * 128.  sink:
- * 16 writable bytes.  No counterpart in the reference. */
-int vui_debug_load_pattern(int pattern, int grid, int iters, const void* buf, int64_t buf_bytes, void* sink, vui_stream_t stream);
 
 /* One backbone decode step for B rows (B <= max_batch).
  *   Engine._backbone_decode_body / _backbone_decode_body_b  (engine.py:434-449, 485-502)
@@ -209,7 +216,8 @@ int vui_prefill(vui_ctx* ctx, const void* emb_in, int T, int slot, int pos0, int
  *   Engine._stream_row / _render_rows loop body (engine.py:1450-1485, 1011-1044)
  * frames_out: optional device (max_frames, B, Q) int64 log; the frame goes to row *frame_ctr.
  * eos_prob_out fp32 device, may be NULL: sigmoid(eos logit) (engine.py:1468-1471); (B) values, or,
- *   when frames_out is given, a (max_frames, B) log whose row *frame_ctr is written.
+ *   when frames_out is given, a (max_frames, B) log whose row *frame_ctr is written.  A batch-1 step whose
+ *   persistent launch failed (see vui_ctx_status) writes -1 there and commits nothing else.
  * frame_ctr (device int32) is incremented at the end of the step. */
 int vui_frame_step(vui_ctx* ctx, int64_t* codes_io, const int32_t* slot_idx, int32_t* seq_lens,
                    const int32_t* seq_inc, int B, void* k_cache, void* v_cache, float* rep_counts,

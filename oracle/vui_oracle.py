@@ -21,8 +21,9 @@ How each function is pinned (see tests/test_oracle_golden.py, tests/test_oracle_
   golden vectors written from the reference's own classes by tests/golden/make_golden.py.
 * attention: additionally brute force against an explicit softmax on tiny sizes.
 * philox4x32_10: Random123 known-answer vectors.
-* sample_rq / sample_cb0 selection rule: exhaustive small cases + chi-square against the
-  analytic top-k softmax; the *random stream* itself has no counterpart in the reference
+* sample_rq / sample_cb0 selection rule: exhaustive small cases (ties at the k-th place kept
+  by the depth-head rule, cut to exactly k in index order by the code-0 rule) + chi-square against
+  the analytic top-k softmax; the *random stream* itself has no counterpart in the reference
   (torch.multinomial's CUDA generator is third-party) -> "parity unpinned" for the
   drawn token under sampling, pinned for greedy.
 * rep_penalty: closed form + ring-buffer invariant (counts == histogram of the window).
@@ -258,14 +259,16 @@ def rep_penalise(logits: Tensor, counts: Tensor, penalty: float) -> Tensor:
 def cb0_probs(logits: Tensor, temperature: float, top_k: int) -> np.ndarray:
     """Kept weights of the code-0 sampler.  Reference: engine.py:855-863, 1456-1464.
 
-    softmax(logits/T) in fp32, then the top-k probabilities are kept and renormalised.  Kept
-    set = {p >= k-th largest p}: identical to the reference's exact-k scatter unless several
-    probabilities tie at the k-th place (torch.topk's choice among ties is unspecified).
+    softmax(logits/T) in fp32, then exactly top_k probabilities are kept (topk + scatter) and
+    renormalised.  Where several probabilities tie at the k-th place torch.topk's choice among
+    them is unspecified; here, and on the device, the lowest indices among the tied are kept.
     """
     p = torch.softmax(logits.float() / temperature, dim=-1)
-    if top_k is not None and top_k > 0:
-        kth = torch.topk(p, min(top_k, p.numel())).values[-1]
-        p = torch.where(p >= kth, p, torch.zeros_like(p))
+    if top_k is not None and 0 < top_k < p.numel():
+        order = torch.sort(p, descending=True, stable=True).indices[:top_k]  # stable: ties in index order
+        kept = torch.zeros_like(p)
+        kept[order] = p[order]
+        p = kept
     return p.numpy()
 
 

@@ -252,6 +252,7 @@ def test_sampler_16bit_key_search_equals_32bit(lib, CS, top_k):
     _lib.check(lib.vui_ctx_create(C.byref(cfgc), C.byref(w), (ws.data_ptr() + 255) & ~255, n, 16, C.byref(h)), "ctx")
     ld = lg.cuda()
     counts = torch.zeros(B, CS, dtype=torch.float32, device="cuda")
+    n_match = n_all = 0
     for frame in range(20):
         ctr = torch.tensor([frame], dtype=torch.int32, device="cuda")
         sp = _lib.SampleParamsC()
@@ -264,6 +265,11 @@ def test_sampler_16bit_key_search_equals_32bit(lib, CS, top_k):
                                       stream()), "b")
         assert torch.equal(a, b), frame
         for r in range(B):
+            # the code-0 rule keeps exactly top_k entries: of row 2's ties only the lowest indices survive
             kept = O.cb0_probs(lg[r].float(), 0.9, top_k)
+            assert (kept > 0).sum() == min(top_k, CS)
             assert kept[int(a[r])] > 0
+            n_match += int(a[r]) == O.sample_cb0(lg[r].float(), torch.zeros(CS), 1.0, 0.9, top_k, O.uniform01(99, frame, r, 0))
+            n_all += 1
+    assert n_match >= 0.99 * n_all, (n_match, n_all)
     lib.vui_ctx_destroy(h)

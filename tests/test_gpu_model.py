@@ -123,8 +123,9 @@ BF16_TOL = 2.0 ** -5  # stated bf16 tolerance: 8 bf16 ulps of the largest logit
 
 @pytest.mark.parametrize("fused", [0, 1])
 def test_nano_backbone_bf16_vs_oracle(fused):
-    """One decode step at Vui Nano dims in bf16 at several cache lengths, as a sequence of kernels
-    (fused=0) and as the one persistent kernel (fused=1).
+    """One decode step at Vui Nano dims in bf16 at cache lengths 0, 255, 1023 and 4095, as a sequence of
+    kernels (fused=0) and as the one persistent kernel (fused=1, whose attention split and merge phases are
+    code of their own).
 
     With an empty cache the native step equals the oracle's bf16 regime bit for bit (same
     roundings, same per-row summation).  With a filled cache the attention sums run in another
@@ -133,13 +134,13 @@ def test_nano_backbone_bf16_vs_oracle(fused):
     evaluation of the same bf16 weights.  Checked: (a) within BF16_TOL of the oracle's bf16
     regime, (b) no further from the fp32 evaluation than the oracle's bf16 regime is (x1.3),
     (c) same argmax wherever the oracle's top-2 margin exceeds the tolerance."""
-    S = 1100
+    S = 4608  # cache lengths up to the longest of the benchmark's backbone configurations (4096 keys)
     d, sd, m, o = _nano_models(BF, S=S)
     of = O.OracleModel(d, {k: O.rnd(v, BF) for k, v in sd.items()}, F32, max_seqlen=S)
     m.decoder.allocate_flash_kv_cache(1, m.device, BF, max_seqlen=S)
     assert m._native.fused(fused) == bool(fused), "the fused kernel must be available on an MI355X"
     g = torch.Generator().manual_seed(3)
-    for L in (0, 255, 1023):
+    for L in (0, 255, 1023, 4095):
         kc = O.rnd(torch.randn(d.n_layers, 1, S, d.n_kv_heads, d.head_dim, generator=g), BF)
         vc = O.rnd(torch.randn(d.n_layers, 1, S, d.n_kv_heads, d.head_dim, generator=g), BF)
         for om in (o, of):

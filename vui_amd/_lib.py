@@ -72,7 +72,6 @@ SIGNATURES = {
     "vui_ctx_status": (_I, [_P]),
     "vui_ctx_rq_batch": (_I, [_P]),
     "vui_debug_phase_clock": (_I, [_P, _P, _I, _I]),
-    "vui_debug_load_pattern": (_I, [_I, _I, _I, _P, C.c_int64, _P, _P]),
     "vui_prefill_scratch_bytes": (_L, [C.POINTER(VuiConfigC), _I, _I]),
     "vui_prefill": (_I, [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _L, _P]),
     "vui_codec_hop": (C.c_int32, [C.POINTER(CodecConfigC)]),

@@ -81,7 +81,7 @@ static int check_cfg(const vui_config* c, int max_batch) {
   if (c->rope_dim < 0 || c->rope_dim > c->head_dim || (c->rope_dim & 1)) { vui_set_error("bad rope_dim %d", c->rope_dim); return VUI_EINVAL; }
   if (c->n_quantizers < 2 || c->n_quantizers > 64 || c->codebook_size < 2 || c->codebook_size > 8192) {
     vui_set_error("n_quantizers in [2,64], codebook_size in [2,8192] required"); return VUI_EINVAL; }
-  if (c->rq_layers > 0 && (c->rq_heads < 1 || c->rq_dim % c->rq_heads || (c->rq_dim & 7) || (c->rq_ffn & 7) ||
+  if (c->rq_layers > 0 && (c->rq_heads < 1 || c->rq_dim < 8 || c->rq_dim % c->rq_heads || (c->rq_dim & 7) || (c->rq_ffn & 7) ||
                            c->rq_dim / c->rq_heads > 128)) {
     vui_set_error("bad depth-head layout R=%d heads=%d ffn=%d", c->rq_dim, c->rq_heads, c->rq_ffn); return VUI_EINVAL; }
   if (c->max_seqlen < 1 || c->n_slots < 1) { vui_set_error("max_seqlen and n_slots must be positive"); return VUI_EINVAL; }
@@ -246,15 +246,12 @@ int vui_debug_phase_clock(vui_ctx* ctx, uint64_t* buf, int cap, int workgroup) {
   return VUI_OK;
 }
 
-int vui_debug_load_pattern(int pattern, int grid, int iters, const void* buf, int64_t buf_bytes, void* sink, vui_stream_t stream) {
-  return launch_load_pattern(pattern, grid, iters, buf, buf_bytes, sink, (hipStream_t)stream);
-}
-
 int vui_ctx_status(vui_ctx* ctx) {
   if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
   uint32_t h[4] = {0, 0, 0, 0};
   HIP_TRY(hipMemcpy(h, ctx->ctl, sizeof(h), hipMemcpyDeviceToHost));
-  if (h[2]) { vui_set_error("fused frame kernel: an exchange wait timed out (epoch %u)", h[0]); return VUI_EHIP; }
+  if (h[2] == 2) { vui_set_error("persistent kernel: the launch count wrapped (epoch %u); call vui_ctx_init again", h[0]); return VUI_EHIP; }
+  if (h[2]) { vui_set_error("persistent kernel: an exchange wait timed out (epoch %u); was another kernel running on the device? call vui_ctx_init again", h[0]); return VUI_EHIP; }
   return VUI_OK;
 }
 
@@ -390,7 +387,7 @@ int vui_sample_cb0(vui_ctx* ctx, const void* logits, float* rep_counts, int32_t*
   if (window > 0 && rep_counts && penalty > 1.0f && (!rep_hist || !rep_pos)) { vui_set_error("a repetition window needs rep_hist and rep_pos"); return VUI_EINVAL; }
   SampleArgs s = sample_base(sp);
   s.dtype = ctx->cfg.dtype; s.logits = logits; s.rep_counts = rep_counts; s.rep_hist = rep_hist; s.rep_pos = rep_pos;
-  s.penalty = penalty; s.window = window; s.codebook = 0; s.CS = ctx->cfg.codebook_size; s.B = B;
+  s.penalty = penalty; s.window = window; s.codebook = 0; s.exact_k = 1; s.CS = ctx->cfg.codebook_size; s.B = B;
   s.out = code0_out; s.out_stride = 1; s.out_col = 0;
   return launch_sample(s, (hipStream_t)stream);
 }
@@ -534,7 +531,7 @@ int vui_frame_step(vui_ctx* ctx, int64_t* codes_io, const int32_t* slot_idx, int
   if (window > 0 && rep_counts && penalty > 1.0f && (!rep_hist || !rep_pos)) { vui_set_error("a repetition window needs rep_hist and rep_pos"); return VUI_EINVAL; }
   SampleArgs s = sample_base(sp_cb0);
   s.dtype = c.dtype; s.logits = cb0; s.rep_counts = rep_counts; s.rep_hist = rep_hist; s.rep_pos = rep_pos;
-  s.penalty = penalty; s.window = window; s.codebook = 0; s.CS = c.codebook_size; s.B = B;
+  s.penalty = penalty; s.window = window; s.codebook = 0; s.exact_k = 1; s.CS = c.codebook_size; s.B = B;
   s.out = ctx->code0; s.out_stride = 1; s.out_col = 0;
   s.eos_logit = ctx->eos; s.eos_prob = ctx->eos_prob;
   if ((rc = launch_sample(s, st))) return rc;

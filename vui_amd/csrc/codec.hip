@@ -528,9 +528,7 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
   float* red = part + 4 * 64;
   const int wg = blockIdx.x, nwg = gridDim.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   Ctl c;
-  c.epoch = __hip_atomic_load(a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
-  c.err = a.lerr;
-  c.dead = 0;
+  ctl_begin(c, a.epoch, a.lerr);
   const uint32_t ep = c.epoch;
   int f = *a.ctr;
   const bool over = f >= a.max_seq;
@@ -805,10 +803,7 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
   }
   if (wg == 0 && tid == 0) {
     // every workgroup has read the epoch and the frame counter before they may change
-    int spins = 0;
-    while (__hip_atomic_load(a.arrive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (uint32_t)nwg && ++spins < SPIN_LIMIT) {}
-    __hip_atomic_store(a.arrive, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(a.epoch, ep, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    ctl_finish(c, a.epoch, a.arrive, (uint32_t)nwg);
     if (over) *a.err = 2;
     *a.ctr = f + 1;
   }
@@ -1496,8 +1491,15 @@ int vui_codec_decode_frame(vui_codec* c, const int64_t* codes, int32_t n_q, floa
 int64_t vui_codec_status(vui_codec* c, vui_stream_t stream) {
   if (!c) { vui_set_error("NULL codec"); return VUI_EINVAL; }
   int h[2] = {0, 0};
+  uint32_t lerr = 0;
   HIP_TRY(hipMemcpyAsync(h, c->ctr, sizeof(h), hipMemcpyDeviceToHost, (hipStream_t)stream));
+  if (c->trunk.lerr) HIP_TRY(hipMemcpyAsync(&lerr, c->trunk.lerr, sizeof(lerr), hipMemcpyDeviceToHost, (hipStream_t)stream));
   HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+  if (lerr) {
+    vui_set_error(lerr == 2 ? "codec: the persistent kernel's launch count wrapped; create the decoder again"
+                            : "codec: an exchange wait of the persistent kernel timed out (is another kernel running on the device?)");
+    return VUI_EHIP;
+  }
   if (h[1] == 1) { vui_set_error("codec: a code outside [0, %d) was clamped", c->cfg.codebook_size); return VUI_EINVAL; }
   if (h[1] == 2) { vui_set_error("codec: more than max_seq=%d frames since the last reset", c->cfg.max_seq); return VUI_EINVAL; }
   return h[0];

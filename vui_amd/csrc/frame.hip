@@ -286,9 +286,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
 
   const int wg = blockIdx.x, nwg = gridDim.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   Ctl c;
-  c.epoch = __hip_atomic_load(a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
-  c.err = a.err;
-  c.dead = 0;
+  ctl_begin(c, a.epoch, a.err);
   const uint32_t ep = c.epoch;
   uint64_t* llp = a.ll;
   const vui_weights& W = *a.w;
@@ -729,7 +727,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           }
         }
         TS(20);
-        code0 = block_sample<8>(lv, key, counts ? 0 : 16, a.CS, E, greedy, a.topk0, rnd0, 0u, ssh, (int*)sc);
+        code0 = block_sample<8>(lv, key, counts ? 0 : 16, a.CS, E, greedy, a.topk0, rnd0, 0u, ssh, (int*)sc, true);
         TS(21);
       }
     }
@@ -1020,6 +1018,10 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
     out[a.prof_cap] = (uint64_t)n | (((uint64_t)clock64() - cyc_first) << 32);  // count | shader cycles of the launch
   }
   if (wg == 0) {
+    // Nothing is committed (positions, repetition state, codes, frame log) by a launch in which this workgroup gave
+    // up a wait, or on a context whose error word is already raised: the caller sees the failure through
+    // vui_ctx_status instead of consuming unwritten words as if they were results.
+    if (!__syncthreads_or(c.dead | (int)ctl_failed(c))) {
     if ((a.mode & FR_CB0) && tid == 0) {
       if (a.code0_out) a.code0_out[0] = code0;
       if (a.rep_counts && a.penalty > 1.0f) rep_push(a.rep_counts, a.rep_hist, a.rep_pos, a.rep_window, code0);
@@ -1044,14 +1046,14 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       __syncthreads();
       if (tid == 0) a.frame_ctr[0] = f + 1;
     }
-    if (tid == 0) {
-      // every workgroup has read the epoch before it may change
-      int spins = 0;
-      while (__hip_atomic_load(a.arrive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (uint32_t)nwg && ++spins < SPIN_LIMIT)
-        if (POLL_SLEEP) __builtin_amdgcn_s_sleep(POLL_SLEEP);
-      __hip_atomic_store(a.arrive, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(a.epoch, ep, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else if ((a.mode & FR_FINISH) && a.eos_prob_out && tid == 0) {
+      // a failed step marks its EOS probability with -1, so a caller that reads that value every frame
+      // learns of the failure from the same read
+      const int f = a.frame_ctr[0];
+      if (!a.frames_out) a.eos_prob_out[0] = -1.0f;
+      else if (f >= 0 && f < a.max_frames) a.eos_prob_out[f] = -1.0f;
     }
+    if (tid == 0) ctl_finish(c, a.epoch, a.arrive, (uint32_t)nwg);
   }
 }
 
@@ -1091,10 +1093,10 @@ bool frame_supported(const vui_config& c, int nwg, int ns, bool with_rq, char* w
   else if (c.codebook_size > 2048 || (c.codebook_size & 1)) r = "codebook_size > 2048";
   else if (c.n_quantizers > 64) r = "too many codebooks";
   else if ((c.head_dim & 7) || c.head_dim > 128) r = "head_dim";
+  else if (c.rq_layers < 1 || c.rq_heads < 1) r = "no depth head";
   else if ((c.rq_dim / c.rq_heads) % 2 || c.rq_dim / c.rq_heads > 128) r = "depth-head head_dim must be even, at most 128";
   else if ((c.d_model | c.ffn | c.rq_dim | c.rq_ffn) & 7) r = "vector lengths must be multiples of 8";
   else if (with_rq && frame_lds_bytes(c) > 160 * 1024) r = "depth-head keys/values do not fit in LDS";
-  else if (c.rq_layers < 1) r = "no depth head";
   else {
     const int np_max = (c.n_heads + 2 * c.n_kv_heads) * c.head_dim / 2;
     int m = np_max;

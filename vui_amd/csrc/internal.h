@@ -102,6 +102,7 @@ struct SampleArgs {
   const int32_t* frame_ctr;
   const int32_t* state_rows;  // (B) or nullptr: repetition state / random-stream row of row b
   int codebook;  // Philox counter word 2
+  int exact_k;   // code-0 rule: exactly top_k entries kept, ties at the k-th place cut in index order
   int CS, B;
   int64_t* out;  // out[b * out_stride + out_col]
   int out_stride, out_col;
@@ -128,7 +129,6 @@ int launch_frame_finish(const int64_t* codes, int64_t* frames_out, int n, int ma
                         const float* eos_in, float* eos_out, int B, hipStream_t st);
 int launch_add_rows(int dtype, const void* a, const void* vec, void* out, int B, int R, hipStream_t st);
 int launch_fill_u32(uint32_t* p, uint32_t v, int64_t n, hipStream_t st);
-int launch_load_pattern(int pattern, int grid, int iters, const void* buf, int64_t buf_bytes, void* sink, hipStream_t st);
 
 // ---- fused frame kernel (frame.hip) ----
 struct FrameArgs {

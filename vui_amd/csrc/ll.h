@@ -40,6 +40,41 @@ struct Ctl {
   int dead;
 };
 
+// Launch handshake of a persistent kernel over three control words: the epoch of the last finished launch, the
+// number of workgroups of the running launch that have read it, and a sticky error word.
+// A launch uses epoch + 1.  Epoch 0 means "never written" in every exchange word, so when the 32-bit count
+// wraps the launch raises the error word (value 2) instead of running: the host re-initialises the context
+// (which zeroes the words) and goes on.
+__device__ __forceinline__ void ctl_begin(Ctl& c, const uint32_t* epoch, uint32_t* err) {
+  c.epoch = __hip_atomic_load(epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+  c.err = err;
+  c.dead = 0;
+  if (c.epoch == 0u) {
+    c.dead = 1;
+    if (threadIdx.x == 0) __hip_atomic_store(err, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+// A non-zero error word (this launch or an earlier one): results must not be committed.
+__device__ __forceinline__ bool ctl_failed(const Ctl& c) {
+  return __hip_atomic_load(c.err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+}
+// One thread of workgroup 0, last thing in the launch: every workgroup has read the epoch before it may change.
+// If some workgroup never arrives the error word is raised and the words are left as they are; the context is
+// then unusable until it is re-initialised (a late arrival would otherwise be counted into the next launch).
+__device__ __forceinline__ void ctl_finish(const Ctl& c, uint32_t* epoch, uint32_t* arrive, uint32_t nwg) {
+  int spins = 0;
+  while (__hip_atomic_load(arrive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < nwg) {
+    if (++spins >= SPIN_LIMIT) {
+      __hip_atomic_store(c.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return;
+    }
+    if (POLL_SLEEP) __builtin_amdgcn_s_sleep(POLL_SLEEP);
+  }
+  if (ctl_failed(c)) return;
+  __hip_atomic_store(arrive, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(epoch, c.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // Wait until words [0, n) of buf carry the current epoch; sink(i, payload) once per word.
 // Threads take words tid, tid+256, ...  A thread that exceeds the spin limit raises the error
 // word and stops waiting for the rest of the launch, so every wave always reaches the end.

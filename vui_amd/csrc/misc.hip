@@ -118,7 +118,7 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const SampleArgs p
   }
   const uint32_t frame = p.frame_ctr ? (uint32_t)p.frame_ctr[0] : 0u;
   const uint32_t rnd = philox_u32(p.seed, frame, (uint32_t)sb, (uint32_t)p.codebook, 0u);
-  const int pick = block_sample<EMAX>(l, key, raw_keys ? 16 : 0, CS, E, greedy, p.top_k, rnd, (uint32_t)p.codebook, sh, hist);
+  const int pick = block_sample<EMAX>(l, key, raw_keys ? 16 : 0, CS, E, greedy, p.top_k, rnd, (uint32_t)p.codebook, sh, hist, p.exact_k != 0);
 
   if (tid == 0) {
     p.out[(size_t)b * p.out_stride + p.out_col] = (int64_t)pick;
@@ -210,40 +210,6 @@ int launch_frame_finish(const int64_t* codes, int64_t* frames_out, int n, int ma
                         const float* eos_in, float* eos_out, int B, hipStream_t st) {
   hipLaunchKernelGGL(frame_finish_kernel, dim3(1), dim3(256), 0, st, codes, frames_out, n, max_frames, ctr, eos_in,
                      eos_out, B);
-  HIP_TRY(hipGetLastError());
-  return VUI_OK;
-}
-
-// Measurement aid: 16-byte-per-lane loads from `buf` under three lane -> address patterns (0: an operand fragment
-// read straight from a row-major matrix, 16 rows x 64 bytes per instruction; 1: 8 rows x 128 bytes, whole lines;
-// 2: 1 KiB contiguous).  Rows are 1536 bytes; every address is reduced modulo the buffer.
-template <int PAT>
-__global__ __launch_bounds__(256) void load_pattern_kernel(const uint4* __restrict__ buf, uint4* sink, int iters, int rows) {
-  const int lane = threadIdx.x & 63, wid = blockIdx.x * 4 + (threadIdx.x >> 6);
-  uint4 acc = make_uint4(0, 0, 0, 0);
-  for (int it = 0; it < iters; ++it) {
-    uint4 v[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int step = it * 8 + u;
-      size_t off;
-      if (PAT == 0) off = (size_t)((wid * 16 + (lane & 15)) % rows) * 1536 + (size_t)(step % 24) * 64 + (lane >> 4) * 16;
-      else if (PAT == 1) off = (size_t)((wid * 16 + (lane >> 3) + 8 * (step & 1)) % rows) * 1536 + (size_t)((step >> 1) % 12) * 128 + (lane & 7) * 16;
-      else off = ((size_t)wid * 24576 + (size_t)(step % 24) * 1024 + lane * 16) % ((size_t)rows * 1536);
-      v[u] = buf[off >> 4];
-    }
-#pragma unroll
-    for (int u = 0; u < 8; ++u) { acc.x ^= v[u].x; acc.y ^= v[u].y; acc.z ^= v[u].z; acc.w ^= v[u].w; }
-  }
-  if (acc.x == 0x12345678u && acc.y == 0x9abcdef0u) sink[0] = acc;  // keeps the loads alive
-}
-int launch_load_pattern(int pattern, int grid, int iters, const void* buf, int64_t buf_bytes, void* sink, hipStream_t st) {
-  const int rows = (int)(buf_bytes / 1536);
-  if (pattern < 0 || pattern > 2 || grid < 1 || iters < 1 || !buf || !sink || rows < 1 || ((uintptr_t)buf & 15)) {
-    vui_set_error("load pattern: bad arguments"); return VUI_EINVAL; }
-  if (pattern == 0) hipLaunchKernelGGL(load_pattern_kernel<0>, dim3(grid), dim3(256), 0, st, (const uint4*)buf, (uint4*)sink, iters, rows);
-  else if (pattern == 1) hipLaunchKernelGGL(load_pattern_kernel<1>, dim3(grid), dim3(256), 0, st, (const uint4*)buf, (uint4*)sink, iters, rows);
-  else hipLaunchKernelGGL(load_pattern_kernel<2>, dim3(grid), dim3(256), 0, st, (const uint4*)buf, (uint4*)sink, iters, rows);
   HIP_TRY(hipGetLastError());
   return VUI_OK;
 }

@@ -318,9 +318,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
   const int B = a.B, R = a.R, d = a.d, CS = a.CS, Q = a.Q, xs = a.xs;
   const int rhd = R / a.rqH, QP8 = (Q + 7) & ~7;
   Ctl c;
-  c.epoch = __hip_atomic_load(a.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
-  c.err = a.err;
-  c.dead = 0;
+  ctl_begin(c, a.epoch, a.err);
   const uint32_t ep = c.epoch;
   const vui_weights& W = *a.w;
   const bf16_t* g_proj = (const bf16_t*)W.rq_backbone_proj;
@@ -663,12 +661,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
   __syncthreads();
   if (active && wl < Bg && a.zero_pad)
     for (int q = a.n_q + tid; q < a.codes_stride; q += FR_THREADS) a.codes_out[(size_t)(b0 + wl) * a.codes_stride + q] = 0;
-  if (wg == 0 && tid == 0) {
-    int spins = 0;
-    while (__hip_atomic_load(a.arrive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (uint32_t)nwg && ++spins < SPIN_LIMIT) {}
-    __hip_atomic_store(a.arrive, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(a.epoch, ep, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
+  if (wg == 0 && tid == 0) ctl_finish(c, a.epoch, a.arrive, (uint32_t)nwg);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -31,6 +31,7 @@ struct SampleShared {
   float wsum[SAMP_THREADS / WAVE];
   int cnt[2][3 * SAMP_THREADS / WAVE];
   int pick[2];     // slot codebook % 2: consecutive draws of a workgroup alternate, so a draw needs no barrier after its last read
+  int tie[SAMP_THREADS / WAVE];  // per wave: keys above the threshold | keys equal to it << 16 (exact-k cut)
 #ifdef VUI_SAMPLE_CLOCK
   unsigned long long ts[8];
 #endif
@@ -79,7 +80,7 @@ __device__ __forceinline__ void hist_select(const int* hist, int need, int& digi
 // One draw from the values l[e] (element index tid*E + e, -inf beyond CS) held by a 256-thread
 // block.  RQ rule (src/vui/model.py:955-962): drop l < k-th largest, softmax, draw.  code-0 rule
 // (src/vui/engine.py:855-863): softmax, keep the top-k probabilities, renormalise, draw.  Both
-// are: keep {l >= k-th largest l}, weights exp(l - max), inverse CDF in index order with one
+// are: keep {l >= k-th largest l} (code 0: cut to exactly k, see exact_k), weights exp(l - max), inverse CDF in index order with one
 // uniform (rnd: philox_u32(seed, frame, row, codebook, 0), computed by the caller ahead of its last wait; codebook
 // also picks the slot of the shared result, see SampleShared).  greedy: the lowest index of the maximum.  Every
 // thread returns the same pick.
@@ -89,10 +90,14 @@ __device__ __forceinline__ void hist_select(const int* hist, int need, int& digi
 // low_bit are known to carry no information (16 when the keys come from bf16 values).  low_bit 16 or 0:
 // two or four rounds of an 8-bit digit histogram; otherwise two bits per barrier over bits 31..low_bit,
 // stopping as soon as exactly top_k keys lie above the candidate.
+//
+// exact_k (the code-0 rule: topk + scatter keeps exactly top_k entries): of the keys that tie with the k-th largest
+// only as many as fill the quota are kept, lowest indices first (torch.topk leaves the choice among equal values
+// open); without it every tie is kept (the depth-head rule drops only l < k-th).
 template <int EMAX>
 __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32_t (&key)[EMAX], int low_bit, int CS,
                                             int E, bool greedy, int top_k, uint32_t rnd, uint32_t codebook,
-                                            SampleShared& sh, int* hist) {
+                                            SampleShared& sh, int* hist, bool exact_k = false) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   SAMP_TS(0);
   const bool digits = top_k > 0 && top_k < CS && (low_bit == 16 || low_bit == 0) && !greedy;
@@ -176,14 +181,49 @@ __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32
       if (tsel == top_k) break;  // exactly k keys are >= thr: the kept set is final
     }
   }
+  // exact-k: how many of this thread's ties with the threshold are kept (all of them otherwise)
+  int tie_keep = EMAX;
+  if (exact_k && top_k > 0 && top_k < CS) {
+    const uint32_t tt = thr >> low_bit;
+    int gt = 0, eq = 0;
+#pragma unroll
+    for (int e = 0; e < EMAX; ++e)
+      if (e < E && tid * E + e < CS) { gt += (key[e] >> low_bit) > tt; eq += (key[e] >> low_bit) == tt; }
+    const int mine = gt | (eq << 16);  // both counts stay below 2^14 (CS <= 8192)
+    int incl = mine;
+    incl += dpp_i<0x111>(incl);  // row_shr:1 .. 8: inclusive scan inside each row of 16 lanes
+    incl += dpp_i<0x112>(incl);
+    incl += dpp_i<0x114>(incl);
+    incl += dpp_i<0x118>(incl);
+    {
+      const int t0 = __builtin_amdgcn_readlane(incl, 15), t1 = __builtin_amdgcn_readlane(incl, 31), t2 = __builtin_amdgcn_readlane(incl, 47);
+      const int row = lane >> 4;
+      incl += (row >= 1 ? t0 : 0) + (row >= 2 ? t1 : 0) + (row >= 3 ? t2 : 0);
+    }
+    if (lane == WAVE - 1) sh.tie[wave] = incl;
+    __syncthreads();
+    int before = incl - mine, total = 0;
+#pragma unroll
+    for (int w = 0; w < SAMP_THREADS / WAVE; ++w) { if (w < wave) before += sh.tie[w]; total += sh.tie[w]; }
+    const int quota = top_k - (total & 0xffff);  // ties to keep over the whole block, >= 1
+    tie_keep = max(0, min(eq, quota - (before >> 16)));
+  }
   // weights, their total, and the inverse CDF in index order
   float wloc = 0.f;
   float pw[EMAX];
+  {
+    const uint32_t tt = thr >> low_bit;
+    int ties_seen = 0;
 #pragma unroll
-  for (int e = 0; e < EMAX; ++e) {
-    pw[e] = 0.f;
-    if (e < E && tid * E + e < CS && key[e] >= thr) pw[e] = __expf(l[e] - M);
-    wloc += pw[e];
+    for (int e = 0; e < EMAX; ++e) {
+      pw[e] = 0.f;
+      if (e < E && tid * E + e < CS && key[e] >= thr) {
+        bool keep = true;
+        if (exact_k && (key[e] >> low_bit) == tt) keep = ties_seen++ < tie_keep;
+        if (keep) pw[e] = __expf(l[e] - M);
+      }
+      wloc += pw[e];
+    }
   }
   // inclusive scan over the wave: shifts inside each row of 16 lanes, then the row totals
   float incl = wloc;

@@ -503,6 +503,7 @@ class Engine:
             if sync_every and f % sync_every == 0:
                 torch.cuda.current_stream().synchronize()
         torch.cuda.current_stream().synchronize()
+        nat.status()  # a persistent launch that gave up a wait committed nothing: raise instead of returning stale frames
         return frames[:n_frames, :, :nq].clone(), eos[:n_frames].clone()
 
     # ------------------------------------------------------------------ continuous batching
@@ -633,6 +634,7 @@ class Engine:
                 active[slot].seq_offset += 1
             sample(cb0_all, slots_t, cfg.top_k, out=rq_code0[:B_active])
             eos_flags = (torch.sigmoid(eos_all.float()).flatten() > cfg.eos_threshold).cpu()
+            nat.status()  # the stream is idle here: the steps so far (persistent depth head included) are complete
             frames_all = depth_head(self._gc_hidden_out[:B_bucket], rq_code0, B_bucket)[:B_active].clone()
             last[slots_l, :nq] = frames_all  # a slot that starts a new chunk below overwrites its row
             self._frame_ctr += 1
@@ -767,7 +769,11 @@ class Engine:
                         e, p1 = entropy_top1(self._penalised_probs(self._g_cb0_out[0:1], cnt, cfg, cur_temp))
                         entropies.append(e)
                         top1s.append(p1)
-                    if step >= min_frames and eos_now[0, 0].item() > cfg.eos_threshold:
+                    p_eos = eos_now[0, 0].item()
+                    if p_eos < 0.0:  # the step's persistent launch failed and committed nothing
+                        nat.status()
+                        raise RuntimeError("frame step failed without a raised error word")
+                    if step >= min_frames and p_eos > cfg.eos_threshold:
                         for hc in held:
                             yield hc
                             total_frames += 1
