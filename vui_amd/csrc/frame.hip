@@ -1021,7 +1021,14 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
     // Nothing is committed (positions, repetition state, codes, frame log) by a launch in which this workgroup gave
     // up a wait, or on a context whose error word is already raised: the caller sees the failure through
     // vui_ctx_status instead of consuming unwritten words as if they were results.
-    if (!__syncthreads_or(c.dead | (int)ctl_failed(c))) {
+    // (the flag goes through a word of the dynamic LDS: a block-wide vote would add static LDS to a kernel whose
+    // dynamic part already fills the CU's)
+    int* bad = (int*)(red + 48);
+    if (tid == 0) *bad = ctl_failed(c) ? 1 : 0;
+    __syncthreads();
+    if (c.dead) *bad = 1;
+    __syncthreads();
+    if (!*bad) {
     if ((a.mode & FR_CB0) && tid == 0) {
       if (a.code0_out) a.code0_out[0] = code0;
       if (a.rep_counts && a.penalty > 1.0f) rep_push(a.rep_counts, a.rep_hist, a.rep_pos, a.rep_window, code0);
