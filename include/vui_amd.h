@@ -254,6 +254,18 @@ int64_t vui_attn_scratch_bytes(int B, int H, int hd, int n_splits);
 int vui_decode_attn(int dtype, const void* q, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
                     const int32_t* seq_lens, const int32_t* slot_idx, void* out, int B, int H, int KV, int hd,
                     int S, int window, int n_splits, void* scratch, vui_stream_t stream);
+/* vui_decode_attn for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): same arguments without `scratch`, same kernels, same results.  It has
+ * no counterpart in the reference.  The pieces of the key-range splits and their arrival counters live in a
+ * fixed array inside the library's code object (4 MiB + 8 KiB per GPU, held until the process ends), so
+ * B * H <= 2048 and B * H * n_splits * (hd + 2) * 4 <= 4 MiB; anything larger returns VUI_EINVAL and belongs to
+ * vui_decode_attn.  The call allocates and frees nothing (the array's address is looked up once per device, at
+ * vui_ctx_init or on the first call there, so make one of those before a graph capture); the counters are
+ * cleared by a small fill kernel at the start of every call.  All calls on one GPU share the one array: calls
+ * that overlap there (two streams, two threads, two replays in flight) race; serialise them. */
+int vui_decode_attn_noalloc(int dtype, const void* q, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
+                            const int32_t* seq_lens, const int32_t* slot_idx, void* out, int B, int H, int KV, int hd,
+                            int S, int window, int n_splits, vui_stream_t stream);
 /* One draw per row from logits (B, CS) fp32 with the RQ-head rule (model.py:955-962). */
 int vui_sample_logits(const float* logits, const float* bias, int CS, const vui_sample_params* sp, int codebook,
                       int64_t* out, int B, vui_stream_t stream);

@@ -96,6 +96,7 @@ SIGNATURES = {
     "vui_rope": (_I, [_I, _P, _P, _P, _I, _I, _I, _I, _P]),
     "vui_attn_scratch_bytes": (_L, [_I, _I, _I, _I]),
     "vui_decode_attn": (_I, [_I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P]),
+    "vui_decode_attn_noalloc": (_I, [_I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
     "vui_sample_logits": (_I, [_P, _P, _I, C.POINTER(SampleParamsC), _I, _P, _I, _P]),
 }
 

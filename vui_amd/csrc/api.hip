@@ -3,6 +3,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
 #include <new>
 
 #include "internal.h"
@@ -17,6 +18,32 @@ void vui_set_error(const char* fmt, ...) {
 }
 
 #define MAX_SPLITS 64
+
+// ---- scratch of the entry point that allocates nothing (vui_decode_attn_noalloc) ----
+// One array per GPU, part of the code object: [arrival counters: NOALLOC_MAX_ROWS_HEADS words][pieces].  In host
+// code the array's name stands for the symbol, not for device memory: its address on the current device comes
+// from hipGetSymbolAddress, once per device, and only that pointer is handed to kernels.
+#define NOALLOC_MAX_ROWS_HEADS 2048
+#define NOALLOC_PIECE_BYTES (4 << 20)
+#define NOALLOC_MAX_DEVICES 64
+static __device__ __align__(256) unsigned char scratch[NOALLOC_MAX_ROWS_HEADS * 4 + NOALLOC_PIECE_BYTES];
+static std::mutex g_noalloc_mu;
+static unsigned char* g_noalloc_ptr[NOALLOC_MAX_DEVICES];
+
+static int noalloc_scratch(unsigned char** out) {
+  int dev = -1;
+  HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) { vui_set_error("device ordinal %d outside [0, %d)", dev, NOALLOC_MAX_DEVICES); return VUI_EINVAL; }
+  std::lock_guard<std::mutex> lock(g_noalloc_mu);
+  if (!g_noalloc_ptr[dev]) {
+    void* p = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) { vui_set_error("hipGetSymbolAddress returned no address for the built-in scratch"); return VUI_EHIP; }
+    g_noalloc_ptr[dev] = (unsigned char*)p;
+  }
+  *out = g_noalloc_ptr[dev];
+  return VUI_OK;
+}
 
 struct vui_ctx {
   vui_config cfg;
@@ -180,8 +207,10 @@ void vui_ctx_destroy(vui_ctx* ctx) { delete ctx; }
 int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream) {
   if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
   hipStream_t st = (hipStream_t)stream;
-  int rc = launch_fill_u32(ctx->counter, 0u, (int64_t)ctx->max_batch * ctx->cfg.n_heads, st);
+  unsigned char* builtin = nullptr;
+  int rc = noalloc_scratch(&builtin);  // the built-in scratch's address on this device, so that no later call has to ask
   if (rc) return rc;
+  if ((rc = launch_fill_u32(ctx->counter, 0u, (int64_t)ctx->max_batch * ctx->cfg.n_heads, st))) return rc;
   // fused frame kernel: exchange words and control words start at zero (epoch 0 = "never written")
   ctx->ll_words = ll_words_needed(ctx->cfg);
   if ((rc = launch_fill_u32((uint32_t*)ctx->ll, 0u, (int64_t)ctx->ll_words * 2, st))) return rc;
@@ -616,6 +645,36 @@ int vui_decode_attn(int dtype, const void* q, const void* k_new, const void* v_n
   a.counter = (uint32_t*)scratch;
   a.part = (float*)((char*)scratch + (size_t)B * H * 256);
   return launch_decode_attn(a, (hipStream_t)stream);
+}
+
+int vui_decode_attn_noalloc(int dtype, const void* q, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
+                            const int32_t* seq_lens, const int32_t* slot_idx, void* out, int B, int H, int KV, int hd, int S,
+                            int window, int n_splits, vui_stream_t stream) {
+  if (!q || !k_cache || !v_cache || !seq_lens || !out) { vui_set_error("NULL argument"); return VUI_EINVAL; }
+  if (B < 1 || H < 1 || n_splits < 1 || hd < 8) { vui_set_error("decode_attn_noalloc: bad shape B=%d H=%d hd=%d splits=%d", B, H, hd, n_splits); return VUI_EINVAL; }
+  const int64_t bh = (int64_t)B * H, pieces = bh * n_splits * (hd + 2) * 4;
+  if (bh > NOALLOC_MAX_ROWS_HEADS || pieces > (int64_t)NOALLOC_PIECE_BYTES) {
+    vui_set_error("decode_attn_noalloc: B*H=%lld (limit %d) with %d splits needs %lld bytes of pieces (limit %d): beyond the "
+                  "built-in scratch, use vui_decode_attn with a scratch buffer of the caller",
+                  (long long)bh, NOALLOC_MAX_ROWS_HEADS, n_splits, (long long)pieces, NOALLOC_PIECE_BYTES);
+    return VUI_EINVAL;
+  }
+  unsigned char* sp = nullptr;
+  int rc = noalloc_scratch(&sp);
+  if (rc) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  // the array keeps what the last call left: the arrival counters must start at zero (a fill kernel, so that the
+  // call can be recorded into a graph)
+  if (n_splits > 1 && (rc = launch_fill_u32((uint32_t*)sp, 0u, bh, st))) return rc;
+  if (k_new && v_new)
+    if ((rc = launch_kv_append(dtype, k_new, v_new, k_cache, v_cache, seq_lens, slot_idx, B, KV, hd, S, st))) return rc;
+  AttnArgs a;
+  memset(&a, 0, sizeof(a));
+  a.dtype = dtype; a.q = q; a.kc = k_cache; a.vc = v_cache; a.seq_lens = seq_lens; a.slot_idx = slot_idx; a.out = out;
+  a.B = B; a.H = H; a.KV = KV; a.hd = hd; a.S = S; a.window = window; a.n_splits = n_splits;
+  a.counter = (uint32_t*)sp;
+  a.part = (float*)(sp + (size_t)NOALLOC_MAX_ROWS_HEADS * 4);
+  return launch_decode_attn(a, st);
 }
 
 int vui_sample_logits(const float* logits, const float* bias, int CS, const vui_sample_params* sp, int codebook,
