@@ -59,6 +59,12 @@ typedef struct vui_config {
   float norm_eps;         /* backbone RMSNorm eps (model.py:391) */
   float rq_norm_eps;      /* RQ RMSNorm eps (model.py:287) */
   int32_t int8_backbone;  /* 1: backbone linears are int8 weight-only with per-row scales */
+  /* Global-attention layers (Decoder's window_size / global_every / global_rope_*, model.py:396-468): bit l set =
+   * layer l attends over the whole cache whatever `window` says and, when vui_weights.rope_table_global is given,
+   * rotates with that table over its first global_rope_dim features.  0 = every layer as configured above. */
+  uint64_t global_layers;
+  int32_t global_rope_dim; /* rotated features of the global table (<= head_dim, even); used with rope_table_global */
+  int32_t reserved;
 } vui_config;
 
 /* One backbone block (src/vui/model.py:300-340).  nn.Linear layout (out, in), row-major. */
@@ -93,6 +99,8 @@ typedef struct vui_weights {
   const void* rq_head_w;        /* (Q-1, CS, R) */
   const void* rq_norm;          /* (R) */
   vui_rq_layer_weights rq_layers[VUI_MAX_RQ_LAYERS];
+  const float* rope_table_global; /* (max_seqlen, global_rope_dim, 2) fp32 cos/sin of the global layers' own
+                                     table (Decoder.freqs_cis_global, model.py:449-468), or NULL: they use rope_table */
 } vui_weights;
 
 typedef struct vui_ctx vui_ctx;
@@ -175,7 +183,27 @@ typedef struct vui_sample_params {
   const int32_t* state_rows; /* device (B) int32 or NULL: row b of a code-0 call uses the repetition state and the
                                 random-stream row of state_rows[b] (continuous batching: the physical slot,
                                 Engine._rep_apply_slots / _rep_push_slots, engine.py:594-616) */
+  int32_t keep_ties;      /* code-0 sampler only.  0: Engine._sample_cb0's rule, exactly top_k probabilities kept
+                             (topk + scatter, engine.py:855-863; ties at the k-th place go to the lowest indices).
+                             1: sampling.sample_top_k's rule used by inference.stream_frames, everything >= the
+                             k-th largest kept (sampling.py:14-20).  The depth head always keeps ties (model.py:955-962). */
+  int32_t reserved;
 } vui_sample_params;
+
+/* Device-side end-of-turn test of a streamed turn (Engine._stream_row's `step >= min_frames and sigmoid(eos) >
+ * eos_threshold`, engine.py:1468-1471) so that the host need not wait for every frame before it enqueues the next.
+ * state: device int32[2] = {stopped, step}; the host writes {0, 1} when a chunk's first frame has been drawn.
+ * A frame step given this struct (batch 1 only) does nothing at all while stopped != 0; otherwise it runs, then sets
+ * stopped = 1 if step >= min_frames and its EOS probability exceeds threshold, and increments step.  The step that
+ * sets the flag is the reference's last one (a step whose persistent launch failed sets it to 2 instead): its frame is to be dropped by the caller, its position and repetition
+ * push stay.  Only the one-launch form skips stopped steps; the kernel-sequence form maintains the flag but runs
+ * every step it is given (vui_ctx_fused tells which form a context uses), so there the caller reads the flag
+ * before it enqueues the next step.  No counterpart in the reference (its loop reads the logit with .item()). */
+typedef struct vui_eos_stop {
+  float threshold;
+  int32_t min_frames;
+  int32_t* state;
+} vui_eos_stop;
 
 /* Code-0 sampler with repetition penalty for B rows:
  *   Engine._rep_apply / _sample_cb0 / _rep_push  (engine.py:571-590, 855-863, 1451-1466)
@@ -218,13 +246,14 @@ int vui_prefill(vui_ctx* ctx, const void* emb_in, int T, int slot, int pos0, int
  * eos_prob_out fp32 device, may be NULL: sigmoid(eos logit) (engine.py:1468-1471); (B) values, or,
  *   when frames_out is given, a (max_frames, B) log whose row *frame_ctr is written.  A batch-1 step whose
  *   persistent launch failed (see vui_ctx_status) writes -1 there and commits nothing else.
- * frame_ctr (device int32) is incremented at the end of the step. */
+ * frame_ctr (device int32) is incremented at the end of the step.
+ * stop: NULL, or the device-side end-of-turn test described at vui_eos_stop (B == 1). */
 int vui_frame_step(vui_ctx* ctx, int64_t* codes_io, const int32_t* slot_idx, int32_t* seq_lens,
                    const int32_t* seq_inc, int B, void* k_cache, void* v_cache, float* rep_counts,
                    int32_t* rep_hist, int32_t* rep_pos, float penalty, int window,
                    const vui_sample_params* sp_cb0, const vui_sample_params* sp_rq, const float* logit_bias,
                    int n_q, void* hidden_out, void* cb0_out, float* eos_prob_out, int64_t* frames_out,
-                   int max_frames, int32_t* frame_ctr, int n_splits, vui_stream_t stream);
+                   int max_frames, int32_t* frame_ctr, int n_splits, const vui_eos_stop* stop, vui_stream_t stream);
 
 /* HIP graph helpers (stand in for torch.cuda.CUDAGraph capture/replay, model.py:873-876,
  * 1254-1256; engine.py:465-468).  begin/end bracket any sequence of the calls above issued

@@ -67,6 +67,38 @@ class Dims:
     rope_theta_rescale_factor: float = 1.0
     norm_eps: float = 1e-5  # Decoder default, model.py:391
     rq_norm_eps: float = 1e-6  # RMSNorm default used by RQBlock, model.py:287,583
+    # sliding window and global-attention layers (config.py:36-41, model.py:396-468)
+    window_size: int | None = None
+    global_every: int | None = None
+    global_rope_dim: int | None = None
+    global_rope_theta: float | None = None
+    trained_max_seqlen: int | None = None  # Decoder.max_seqlen, the length the global base is derived from
+
+    def block_is_global(self) -> list[bool]:
+        """model.py:406-418: without a window every layer is global; with one, the last layer and every
+        global_every-th are."""
+        def g(idx: int) -> bool:
+            if self.window_size is None:
+                return True
+            if self.global_every is not None:
+                if idx == self.n_layers - 1 or (idx + 1) % self.global_every == 0:
+                    return True
+            return False
+        return [g(i) for i in range(self.n_layers)]
+
+    def global_rope(self, max_seqlen: int):
+        """(dim, theta) of the global layers' own table or None when they share the common one (model.py:449-468)."""
+        rope_dim = self.rope_dim or self.head_dim
+        g_dim = self.global_rope_dim or rope_dim
+        if self.global_rope_theta is not None:
+            g_theta = self.global_rope_theta
+        elif self.window_size is not None and any(self.block_is_global()):
+            g_theta = self.rope_theta * (max_seqlen / self.window_size)
+        else:
+            g_theta = self.rope_theta
+        if g_dim != rope_dim or g_theta != self.rope_theta:
+            return g_dim, g_theta
+        return None
 
     @property
     def head_dim(self) -> int:
@@ -329,14 +361,22 @@ class OracleModel:
     """
 
     def __init__(self, dims: Dims, sd: dict[str, Tensor], dt: torch.dtype = torch.float32,
-                 n_slots: int = 1, max_seqlen: int | None = None, int8: bool = False):
+                 n_slots: int = 1, max_seqlen: int | None = None, int8: bool = False, apply_window: bool = True):
+        """apply_window=False restates the reference's CPU path (SDPA + KVCache, model.py:146-202), which ignores
+        window_size; True the engine's path, where flash-attn applies it per layer (model.py:242-257)."""
         self.dims = dims
+        self.apply_window = apply_window
         self.dt = dt
         self.sd = {k: rnd(v, dt) if v.is_floating_point() else v for k, v in sd.items()}
         self.S = max_seqlen or dims.max_seqlen
         d = dims
         rope_dim = d.rope_dim or d.head_dim
         self.freqs = precompute_freqs_cis(rope_dim, self.S, d.rope_theta, d.rope_theta_rescale_factor)
+        # per-layer window and rotation table (Decoder._get_freqs model.py:504-509; MHA.forward_flash's window, :256)
+        self.is_global = d.block_is_global()
+        gr = d.global_rope(d.trained_max_seqlen or d.max_seqlen)
+        self.freqs_global = (precompute_freqs_cis(gr[0], self.S, gr[1], d.rope_theta_rescale_factor)
+                             if gr is not None else None)
         # FlashKVCache layout (slots, S, KV, hd); one seq_lens shared by all layers (model.py:71-99,492-495)
         self.k_cache = torch.zeros(d.n_layers, n_slots, self.S, d.n_kv_heads, d.head_dim)
         self.v_cache = torch.zeros_like(self.k_cache)
@@ -371,9 +411,11 @@ class OracleModel:
         x = rnd(x, dt)
         start = self.seq_lens[slots.long()].long()  # (B,)
         pos = start[:, None] + torch.arange(T)[None, :]  # (B, T)
-        fr = self.freqs[pos]  # (B, T, rot, 2)
         for li in range(d.n_layers):
             p = f"decoder.blocks.{li}."
+            table = self.freqs_global if (self.freqs_global is not None and self.is_global[li]) else self.freqs
+            fr = table[pos]  # (B, T, rot, 2)
+            win = None if (self.is_global[li] or not self.apply_window) else d.window_size  # (w, 0): keys i-w .. i
             h = rmsnorm(x, sd[p + "attn_norm.weight"], d.norm_eps, dt)
             qkv = self._lin(h, p + "attn.Wqkv.weight")
             q, k, v = torch.split(qkv, [H * hd, KV * hd, KV * hd], dim=-1)
@@ -394,7 +436,10 @@ class OracleModel:
                     kk = kk.repeat_interleave(H // KV, dim=0)
                     vv = vv.repeat_interleave(H // KV, dim=0)
                 qq = q[b].transpose(0, 1)  # (H, T, hd)
-                mask = (torch.arange(L)[None, :] <= (st + torch.arange(T))[:, None])  # (T, L)
+                qpos = (st + torch.arange(T))[:, None]
+                mask = torch.arange(L)[None, :] <= qpos  # (T, L)
+                if win:
+                    mask = mask & (torch.arange(L)[None, :] >= qpos - win)
                 o = attention(qq, kk, vv, hd ** -0.5, dt, mask[None])
                 outs.append(o.transpose(0, 1).reshape(T, H * hd))
             a = torch.stack(outs)
@@ -726,6 +771,193 @@ def stream_row(model: "OracleModel", chunks, *, temperature: float = 0.9, top_k:
                 continue
             out.extend(held)
             break
+    return out
+
+
+def render_rows(model: "OracleModel", chunk_lists, *, temperature: float = 0.9, top_k: int = 100, rq_top_k: int = 100,
+                rep_penalty: float = 1.1, rep_window: int = 24, eos_threshold: float = 0.45, min_secs: float = 0.5,
+                max_turn_secs: float = 15.0, max_secs: float = 30.0, n_codebooks: int = 0, max_turn_wps: float = 0.0,
+                seed: int = 0, prompt_wps: float = 0.0, max_seq: int | None = None, log: list | None = None):
+    """Restatement of Engine._render_rows (engine.py:865-1087) on the oracle model: row r of chunk_lists (a list of
+    (emb (T, d), n_words) per row) renders in cache slot r, all rows in lock step.  Returns {row: (T, Q') codes}.
+
+    The frame counter of the random stream advances once per chunk start and once per decode step (the
+    device's frame step draws before the end-of-turn test); a chunk start draws code 0 (no top-k cut unless
+    greedy) with the repetition state of its own row.  A chunk that ends (EOS or its cap) with fewer than two
+    frames per word is rewound and redone colder: 0.5, then 0.3 (engine.py:952-983), which resets every row's
+    repetition state as the reference does.  log: ("retry", row, chunk, temp) / ("eos", row, chunk) events."""
+    d = model.dims
+    N = len(chunk_lists)
+    max_frames = int(max_secs * FRAME_RATE)
+    min_frames = int(min_secs * FRAME_RATE)
+    max_seq = (max_seq if max_seq is not None else d.max_seqlen) - 10
+    nq = n_codebooks if n_codebooks > 0 else d.n_quantizers
+    greedy = top_k == 1
+    rq_k = rq_top_k if not greedy else 1
+    reps = [RepState(d.codebook_size, rep_window) for _ in range(N)]
+    chunk_idx = [0] * N
+    frames: list[list[Tensor]] = [[] for _ in range(N)]
+    turn_count = [0] * N
+    max_turn = [max_turn_frames(0, prompt_wps, max_turn_secs, max_turn_wps)] * N
+    chunk_offset = [0] * N
+    retry_idx = [0] * N
+    active = [True] * N
+    last: list[Tensor | None] = [None] * N
+    fctr = 0
+
+    def advance_turn(r: int, temp: float | None = None) -> bool:
+        nonlocal fctr
+        ci = chunk_idx[r]
+        if ci >= len(chunk_lists[r]) or len(frames[r]) >= max_frames:
+            return False
+        emb, n_words = chunk_lists[r][ci]
+        max_turn[r] = max_turn_frames(n_words, prompt_wps, max_turn_secs, max_turn_wps)
+        chunk_offset[r] = int(model.seq_lens[r])
+        t = temp or temperature
+        hidden = model.prefill(emb, r)[-1:]
+        cb0, _ = model.heads(hidden)
+        c0 = sample_cb0(cb0[0], reps[r].counts, rep_penalty, t, 1 if greedy else 0, uniform01(seed, fctr, r, 0))
+        if rep_penalty > 1.0:
+            reps[r].push(c0)
+        frame = model.rq_generate(hidden, torch.tensor([c0]), t, rq_k, None, n_codebooks, seed, fctr)[0]
+        fctr += 1
+        last[r] = frame
+        frames[r].append(frame)
+        turn_count[r] = 1
+        return True
+
+    def retry_chunk(r: int) -> bool:
+        nonlocal reps
+        n_words = chunk_lists[r][chunk_idx[r]][1]
+        fpw = turn_count[r] / n_words if n_words > 0 else 999
+        if fpw >= 2.0:
+            retry_idx[r] = 0
+            return False
+        ri = retry_idx[r]
+        if ri >= len(GATE_RETRY_TEMPS):
+            retry_idx[r] = 0
+            return False
+        retry_idx[r] = ri + 1
+        if log is not None:
+            log.append(("retry", r, chunk_idx[r], GATE_RETRY_TEMPS[ri]))
+        model.seq_lens[r] = chunk_offset[r]
+        del frames[r][len(frames[r]) - turn_count[r]:]
+        reps = [RepState(d.codebook_size, rep_window) for _ in range(N)]
+        advance_turn(r, GATE_RETRY_TEMPS[ri])
+        return True
+
+    def next_chunk(r: int) -> None:
+        if retry_chunk(r):
+            return
+        retry_idx[r] = 0
+        chunk_idx[r] += 1
+        if not advance_turn(r):
+            active[r] = False
+
+    for r in range(N):
+        if not advance_turn(r):
+            active[r] = False
+    steps = 0
+    while any(active) and steps < max_frames:
+        for r in range(N):
+            if active[r] and turn_count[r] >= max_turn[r]:
+                next_chunk(r)
+        if not any(active):
+            break
+        # every slot steps (the batched graph covers all rows); rows that are over keep feeding their last frame
+        rows = list(range(N))
+        slots = torch.tensor(rows)
+        codes = torch.zeros(N, d.n_quantizers, dtype=torch.long)
+        for r in rows:
+            if last[r] is not None:
+                codes[r, :nq] = last[r]
+        hidden, cb0, eos = model.decode_step(codes, slots)
+        c0s = []
+        for i, r in enumerate(rows):
+            c = sample_cb0(cb0[i], reps[r].counts, rep_penalty, temperature, top_k, uniform01(seed, fctr, r, 0))
+            if rep_penalty > 1.0:
+                reps[r].push(c)
+            c0s.append(c)
+        new = model.rq_generate(hidden, torch.tensor(c0s), temperature, rq_k, None, n_codebooks, seed, fctr)
+        fctr += 1
+        steps += 1
+        hit = []
+        for i, r in enumerate(rows):
+            if not active[r]:
+                continue
+            if int(model.seq_lens[r]) >= max_seq or len(frames[r]) >= max_frames:
+                active[r] = False
+                continue
+            if turn_count[r] >= min_frames and float(torch.sigmoid(eos[i, 0].float())) > eos_threshold:
+                if log is not None:
+                    log.append(("eos", r, chunk_idx[r]))
+                hit.append(r)
+                continue
+            last[r] = new[i]
+            frames[r].append(new[i])
+            turn_count[r] += 1
+        for r in hit:
+            next_chunk(r)
+    return {r: torch.stack(frames[r]) for r in range(N) if frames[r]}
+
+
+def stream_frames(model: "OracleModel", chunks, *, temperature: float = 0.9, top_k: int = 100, rq_top_k: int = 100,
+                  rep_penalty: float = 1.0, rep_window: int = 0, max_secs: float = 120.0, max_turn_secs: float = 15.0,
+                  eos_threshold: float = 0.45, min_turn_secs: float = 0.5, seed: int = 0, max_seq: int | None = None):
+    """Restatement of inference.stream_frames (inference.py:507-734) on the oracle model, from position 0 of
+    slot 0.  chunks: list of emb (T, d).  Returns [(frame, turn_end)] with turn_end the chunk index on a turn's
+    last frame, else None.  Code 0 is drawn by sampling.sample_top_k's rule (everything >= the k-th largest kept,
+    sampling.py:14-20) on every frame; the depth head runs before the end-of-turn test (inference.py:708-720), so
+    each rq_sample call consumes one frame number of the random stream."""
+    d = model.dims
+    max_frames = int(max_secs * FRAME_RATE)
+    max_per_turn = int(max_turn_secs * FRAME_RATE)
+    min_frames = int(min_turn_secs * FRAME_RATE)
+    max_seq = (max_seq if max_seq is not None else d.max_seqlen) - 10
+    rep = RepState(d.codebook_size, rep_window)
+    s0 = torch.tensor([0])
+    out = []
+    fctr = 0
+    total = 0
+    rq_k = rq_top_k if top_k != 1 else 1
+
+    def rq_sample(cb0: Tensor, hidden: Tensor) -> Tensor:
+        nonlocal fctr
+        l = rep_penalise(cb0, rep.counts, rep_penalty)
+        u = uniform01(seed, fctr, 0, 0)
+        if top_k == 1 or temperature <= 0:
+            c0 = int(torch.argmax(l))
+        else:
+            c0 = _inverse_cdf(topk_threshold_probs(l, temperature, top_k if top_k else 0), u)
+        if rep_penalty > 1.0:
+            rep.push(c0)
+        frame = model.rq_generate(hidden, torch.tensor([c0]), temperature, rq_k, None, 0, seed, fctr)[0]
+        fctr += 1
+        return frame
+
+    model.seq_lens[0] = 0
+    for ti, emb in enumerate(chunks):
+        if int(model.seq_lens[0]) >= max_seq or total >= max_frames:
+            break
+        if int(model.seq_lens[0]) + emb.shape[0] >= max_seq:
+            break
+        hidden = model.prefill(emb, 0)[-1:]
+        cb0, _ = model.heads(hidden)
+        pending = rq_sample(cb0[0], hidden)
+        total += 1
+        codes_in = pending
+        for step in range(1, max_per_turn):
+            if int(model.seq_lens[0]) >= max_seq or total >= max_frames:
+                break
+            hidden, cb0, eos = model.decode_step(codes_in[None], s0)
+            nxt = rq_sample(cb0[0], hidden)
+            if step >= min_frames and float(torch.sigmoid(eos[0, 0].float())) > eos_threshold:
+                break
+            out.append((pending, None))
+            pending = nxt
+            total += 1
+            codes_in = nxt
+        out.append((pending, ti))
     return out
 
 

@@ -12,6 +12,8 @@ Fixtures:
   rope.npz        precompute_freqs_cis (plain and rescaled/partial) + apply_rotary_emb
   pieces.npz      RMSNorm, AudioEmbedding (incl. Q' < Q), sample_top_k support/histogram
   tiny_backbone_{mha,gqa}.npz   Decoder.forward (SDPA + KVCache): prefill T=5, then 4 decode steps
+  tiny_backbone_global_{a,b,c}.npz   Decoder.forward with window_size / global_every / global_rope_* set: which
+                  layers are global, their own rotation table, prefill T=9 and 4 decode steps
   tiny_rq.npz     RQTransformer.forward logits, generate(top_k=1) codes, top-k sampling histogram
   tiny_bf16.npz   the same tiny decoder and RQ head run in bfloat16 on CPU
   nano_grid.npz   the full-size greedy 64x16 token grid with fp32 weights N(0,0.02), seed 0
@@ -44,7 +46,8 @@ def build_reference(d: Dims, sd, max_seqlen: int, dtype=torch.float32):
     dec = M.Decoder(n_layers=d.n_layers, d_model=d.d_model, n_heads=d.n_heads, n_kv_heads=d.n_kv_heads,
                     bias=False, dropout=0.0, max_seqlen=max_seqlen, rope_dim=d.rope_dim,
                     rope_theta=d.rope_theta, rope_theta_rescale_factor=d.rope_theta_rescale_factor,
-                    intermediate_size=d.intermediate_size)
+                    intermediate_size=d.intermediate_size, window_size=d.window_size, global_every=d.global_every,
+                    global_rope_dim=d.global_rope_dim, global_rope_theta=d.global_rope_theta)
     dec.load_state_dict(sub(sd, "decoder."), strict=True)
     aemb = M.AudioEmbedding(d.n_quantizers, d.codebook_size, d.d_model)
     aemb.load_state_dict(sub(sd, "audio_emb."), strict=True)
@@ -162,6 +165,32 @@ def make_tiny_backbone(kv, name):
 
 
 @torch.inference_mode()
+def make_tiny_backbone_global():
+    """Decoder with a window, global-attention layers and their own rotation table (model.py:396-468, 504-509):
+    which layers are global, the derived table, and forward outputs.  The reference's CPU path (SDPA + KVCache)
+    applies no window (only flash-attn does, model.py:256), so these vectors pin which table rotates which layer."""
+    for name, kw in (("a", dict(n_layers=3, window_size=6, global_every=2, global_rope_dim=8)),
+                     ("b", dict(n_layers=4, window_size=8, global_every=3)),
+                     ("c", dict(n_layers=2, global_rope_theta=500.0))):
+        d = tiny_dims(2)
+        for k, v in kw.items():
+            setattr(d, k, v)
+        sd = synthetic_state_dict(d, **TINY_SD)
+        mods = build_reference(d, sd, d.max_seqlen)
+        dec = mods["dec"]
+        g = torch.Generator().manual_seed(21)
+        ids = torch.randint(0, d.vocab_size, (9,), generator=g)
+        codes_seq = torch.randint(0, d.codebook_size, (4, d.n_quantizers), generator=g)
+        h_pre, h, cb0, eos = run_backbone(mods, d, ids, codes_seq)
+        out = dict(ids=ids.numpy(), codes=codes_seq.numpy(), h_prefill=h_pre.numpy(), hidden=h.numpy(), cb0=cb0.numpy(),
+                   is_global=np.array(dec.block_is_global), kw_keys=np.array(sorted(kw)),
+                   kw_vals=np.array([float(kw[k]) for k in sorted(kw)]))
+        if dec.freqs_cis_global is not None:
+            out["freqs_global"] = dec.freqs_cis_global.numpy()
+        np.savez_compressed(os.path.join(HERE, f"tiny_backbone_global_{name}.npz"), **out)
+
+
+@torch.inference_mode()
 def make_tiny_rq():
     d = tiny_dims(4)
     sd = synthetic_state_dict(d, **TINY_SD)
@@ -254,12 +283,17 @@ def make_nano_grid(n_frames=64, n_text=32):
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--skip-nano", action="store_true")
+    ap.add_argument("--only-global", action="store_true", help="write only the global-attention-layer fixtures")
     a = ap.parse_args()
     torch.set_num_threads(8)
+    if a.only_global:
+        make_tiny_backbone_global()
+        sys.exit(0)
     make_rope()
     make_pieces()
     make_tiny_backbone(4, "tiny_backbone_mha.npz")
     make_tiny_backbone(2, "tiny_backbone_gqa.npz")
+    make_tiny_backbone_global()
     make_tiny_rq()
     make_tiny_bf16()
     print("small fixtures written", flush=True)

@@ -46,6 +46,73 @@ def test_tiny_backbone_golden_fp32(kv, name):
     np.testing.assert_allclose(v1, g["v_layer1"], rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("name", ["a", "c"])
+def test_global_layer_rope_golden_fp32(name):
+    """Global-attention layers with a rotation table of their own against the reference's Decoder (whose CPU path
+    applies no window: the native step is given the same layer pattern and tables with the window switched off)."""
+    g = np.load(os.path.join(GOLDEN, f"tiny_backbone_global_{name}.npz"))
+    d = tiny_dims(2)
+    for k, v in zip(g["kw_keys"], g["kw_vals"]):
+        setattr(d, str(k), float(v) if str(k) == "global_rope_theta" else int(v))
+    sd = O.synthetic_state_dict(d, **TINY_SD)
+    m = make_model(d, sd, F32)
+    assert m.decoder.block_is_global == [bool(x) for x in g["is_global"]]
+    if "freqs_global" in g.files:
+        np.testing.assert_allclose(m.decoder.freqs_cis_global.cpu().numpy(), g["freqs_global"], rtol=1e-6, atol=1e-6)
+    # the reference's CPU path applies no window: the context made by the allocation below gets the layer pattern
+    # and tables computed above and window 0 (the window itself is checked against the oracle in the next test)
+    m.config.model.window_size = None
+    m.decoder.allocate_flash_kv_cache(1, m.device, F32)
+    ids, codes = T(g["ids"]).cuda(), T(g["codes"]).cuda()
+    h_pre = m.decoder.forward_flash(m.token_emb(ids[None]), torch.arange(9, device="cuda"))
+    np.testing.assert_allclose(h_pre[0].cpu().numpy(), g["h_prefill"], rtol=1e-4, atol=1e-4)
+    hid = torch.empty(1, d.d_model, dtype=F32, device="cuda")
+    cb0 = torch.empty(1, d.codebook_size, dtype=F32, device="cuda")
+    for i in range(codes.shape[0]):
+        m.decoder._step(codes=codes[i][None].contiguous(), emb=None, slot_idx=None, seq_inc=None, B=1, hidden_out=hid,
+                        cb0_out=cb0, eos_out=None, n_splits=2, stream=torch.cuda.current_stream().cuda_stream)
+        np.testing.assert_allclose(hid[0].cpu().numpy(), g["hidden"][i], rtol=1e-4, atol=1e-4)
+        np.testing.assert_allclose(cb0[0].cpu().numpy(), g["cb0"][i], rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("dt,fused,wide", [(F32, 0, False), (BF, 0, False), (BF, 1, False), (BF, 1, True)])
+def test_windowed_and_global_layers_vs_oracle(dt, fused, wide):
+    """Local layers attend over a sliding window, global layers over the whole cache with their own rotation table
+    (src/vui/model.py:396-468, 504-509, 242-257): prompt ingestion and decode steps against the oracle, as a kernel
+    sequence, as the one-launch kernel, and (wide: head_dim 32) through the one-pass prompt ingestion."""
+    kw = dict(n_layers=3, window_size=6, global_every=2, global_rope_dim=8, max_seqlen=64)
+    if wide:
+        kw.update(d_model=128, n_heads=4, n_kv_heads=2, rq_d_model=64, global_rope_dim=16)
+    d = tiny_dims(2, **kw)
+    sd = O.synthetic_state_dict(d, **TINY_SD)
+    m = make_model(d, sd, dt)
+    o = O.OracleModel(d, sd, dt)
+    assert m.decoder.block_is_global == [False, True, True] and m.decoder.freqs_cis_global is not None
+    m.decoder.allocate_flash_kv_cache(1, m.device, dt)
+    if dt == BF:
+        assert m._native.fused(fused) == bool(fused)
+    g = torch.Generator().manual_seed(31)
+    ids = torch.randint(0, d.vocab_size, (20,), generator=g)
+    tol = 1e-4 if dt == F32 else BF16_TOL
+    h_pre = m.decoder.forward_flash(m.token_emb(ids.cuda()[None]), torch.arange(20, device="cuda"))
+    ref = o.prefill(o.embed_text(ids))
+    assert rel_err(h_pre[0], ref) <= tol, rel_err(h_pre[0], ref)
+    hid = torch.empty(1, d.d_model, dtype=dt, device="cuda")
+    cb0 = torch.empty(1, d.codebook_size, dtype=dt, device="cuda")
+    for i in range(12):  # well past the window of 6
+        codes = torch.randint(0, d.codebook_size, (1, d.n_quantizers), generator=g)
+        h_ref, cb_ref, _ = o.decode_step(codes)
+        m.decoder._step(codes=codes.cuda(), emb=None, slot_idx=None, seq_inc=None, B=1, hidden_out=hid, cb0_out=cb0,
+                        eos_out=None, n_splits=4, stream=torch.cuda.current_stream().cuda_stream)
+        assert rel_err(hid, h_ref) <= tol and rel_err(cb0, cb_ref) <= tol, (i, rel_err(hid, h_ref), rel_err(cb0, cb_ref))
+    # the window matters: an oracle without it is further away than the tolerance
+    d_full = tiny_dims(2, **{**kw, "window_size": None, "global_every": None})
+    o_full = O.OracleModel(d_full, sd, dt)
+    assert rel_err(o_full.prefill(o_full.embed_text(ids)), ref) > 10 * tol
+    m._native.status()
+    m._native.fused(1)
+
+
 def test_tiny_rq_golden_fp32():
     g = np.load(os.path.join(GOLDEN, "tiny_rq.npz"))
     d = tiny_dims(4)

@@ -87,6 +87,66 @@ def test_tiny_backbone(kv, name):
     np.testing.assert_allclose(m.v_cache[1, 0, :9].transpose(0, 1).numpy(), g["v_layer1"], rtol=2e-5, atol=2e-5)
 
 
+@pytest.mark.parametrize("name", ["a", "b", "c"])
+def test_tiny_backbone_global_layers(name):
+    """Which layers are global, their own rotation table (width and derived base) and which table rotates which
+    layer, against the reference's Decoder (its CPU path applies no window, so neither does the oracle here)."""
+    g = load(f"tiny_backbone_global_{name}.npz")
+    d = tiny_dims(2)
+    for k, v in zip(g["kw_keys"], g["kw_vals"]):
+        setattr(d, str(k), float(v) if str(k) == "global_rope_theta" else int(v))
+    assert d.block_is_global() == [bool(x) for x in g["is_global"]]
+    m = O.OracleModel(d, O.synthetic_state_dict(d, **TINY_SD), torch.float32, apply_window=False)
+    if "freqs_global" in g.files:
+        np.testing.assert_allclose(m.freqs_global.numpy(), g["freqs_global"], rtol=1e-6, atol=1e-6)
+    else:
+        assert m.freqs_global is None
+    ids, codes = T(g["ids"]), T(g["codes"])
+    np.testing.assert_allclose(m.prefill(m.embed_text(ids)).numpy(), g["h_prefill"], rtol=2e-5, atol=2e-5)
+    for i in range(codes.shape[0]):
+        h, cb0, _ = m.decode_step(codes[i][None])
+        np.testing.assert_allclose(h[0].numpy(), g["hidden"][i], rtol=2e-5, atol=2e-5)
+        np.testing.assert_allclose(cb0[0].numpy(), g["cb0"][i], rtol=2e-5, atol=2e-5)
+    # a plausible mistake must fail: the common table on the global layers gives other hidden states
+    d2 = tiny_dims(2)
+    d2.n_layers = d.n_layers
+    m2 = O.OracleModel(d2, O.synthetic_state_dict(d, **TINY_SD), torch.float32)
+    assert float((m2.prefill(m2.embed_text(ids)) - T(g["h_prefill"])).abs().max()) > 1e-3
+
+
+def test_window_mask_of_local_layers():
+    """flash-attn's window (w, 0) on the local layers only: a query at position i sees keys i-w .. i
+    (MHA.forward_flash model.py:242-257).  One layer, window 3, against the textbook attention over the last 4 keys."""
+    d = tiny_dims(2)
+    d.n_layers, d.window_size = 1, 3
+    sd = O.synthetic_state_dict(d, **TINY_SD)
+    assert d.block_is_global() == [False]
+    m = O.OracleModel(d, sd, torch.float32)
+    d_full = tiny_dims(2)
+    d_full.n_layers = 1
+    full = O.OracleModel(d_full, sd, torch.float32)
+    g_ = torch.Generator().manual_seed(1)
+    emb = torch.randn(9, d.d_model, generator=g_) * 0.5
+    a, b = m.prefill(emb), full.prefill(emb)
+    assert torch.allclose(a[:4], b[:4], atol=1e-6)  # positions 0..3 see at most 4 keys either way
+    assert float((a[4:] - b[4:]).abs().max()) > 1e-4  # from position 4 on the window cuts keys off
+    # position 8 from scratch: keys 5..8 only
+    H, KV, hd = d.n_heads, d.n_kv_heads, d.head_dim
+    p = "decoder.blocks.0."
+    x = emb[8:9]
+    h = O.rmsnorm(x, sd[p + "attn_norm.weight"], d.norm_eps, torch.float32)
+    q = O.linear(h, sd[p + "attn.Wqkv.weight"], torch.float32)[:, :H * hd].view(1, H, hd)
+    q = O.apply_rotary_emb(m.freqs[8][None, None], q, torch.float32)
+    kk = m.k_cache[0, 0, 5:9].transpose(0, 1).repeat_interleave(H // KV, 0)
+    vv = m.v_cache[0, 0, 5:9].transpose(0, 1).repeat_interleave(H // KV, 0)
+    att = O.attention(q.transpose(0, 1), kk, vv, hd ** -0.5, torch.float32).transpose(0, 1).reshape(1, H * hd)
+    x1 = x + O.linear(att, sd[p + "attn.out_proj.weight"], torch.float32)
+    h2 = O.rmsnorm(x1, sd[p + "mlp_norm.weight"], d.norm_eps, torch.float32)
+    x2 = x1 + O.swiglu(h2, sd[p + "mlp.w1.weight"], sd[p + "mlp.w3.weight"], sd[p + "mlp.w2.weight"], torch.float32)
+    want = O.rmsnorm(x2, sd["decoder.norm.weight"], d.norm_eps, torch.float32)
+    assert torch.allclose(a[8:9], want, atol=2e-5)
+
+
 def test_tiny_rq_forward_and_greedy():
     g = load("tiny_rq.npz")
     d = tiny_dims(4)

@@ -11,7 +11,9 @@ def dims_to_config(d: O.Dims, max_seqlen: int | None = None):
                   intermediate_size=d.intermediate_size, n_quantizers=d.n_quantizers, codebook_size=d.codebook_size,
                   use_rq_transformer=True, rq_d_model=d.rq_d_model, rq_n_layers=d.rq_n_layers,
                   rq_n_heads=d.rq_n_heads, rope_dim=d.rope_dim, rope_theta=d.rope_theta,
-                  rope_theta_rescale_factor=d.rope_theta_rescale_factor, vocab_size=d.vocab_size)
+                  rope_theta_rescale_factor=d.rope_theta_rescale_factor, vocab_size=d.vocab_size,
+                  window_size=d.window_size, global_every=d.global_every, global_rope_dim=d.global_rope_dim,
+                  global_rope_theta=d.global_rope_theta)
     cfg = Config(model=m, data=DataConfig(max_secs=0))
     # decoder.max_seqlen = max_text_tokens + max_audio_tokens + Q when data.max_secs gives 0 (model.py:1069-1073,1127)
     S = max_seqlen or d.max_seqlen

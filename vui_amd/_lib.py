@@ -21,7 +21,8 @@ class VuiConfigC(C.Structure):
     _fields_ = [(n, C.c_int32) for n in (
         "dtype", "d_model", "n_layers", "n_heads", "n_kv_heads", "head_dim", "ffn", "n_quantizers",
         "codebook_size", "rq_dim", "rq_layers", "rq_heads", "rq_ffn", "rope_dim", "max_seqlen", "n_slots",
-        "window")] + [("norm_eps", C.c_float), ("rq_norm_eps", C.c_float), ("int8_backbone", C.c_int32)]
+        "window")] + [("norm_eps", C.c_float), ("rq_norm_eps", C.c_float), ("int8_backbone", C.c_int32),
+                      ("global_layers", C.c_uint64), ("global_rope_dim", C.c_int32), ("reserved", C.c_int32)]
 
 
 class LayerWeightsC(C.Structure):
@@ -41,12 +42,18 @@ class WeightsC(C.Structure):
         ("rq_backbone_proj", C.c_void_p), ("rq_code_emb", C.c_void_p), ("rq_pos_emb", C.c_void_p),
         ("rq_head_w", C.c_void_p), ("rq_norm", C.c_void_p),
         ("rq_layers", RqLayerWeightsC * VUI_MAX_RQ_LAYERS),
+        ("rope_table_global", C.c_void_p),
     ]
 
 
 class SampleParamsC(C.Structure):
     _fields_ = [("temperature", C.c_float), ("top_k", C.c_int32), ("seed", C.c_uint64),
-                ("frame_ctr", C.c_void_p), ("state_rows", C.c_void_p)]
+                ("frame_ctr", C.c_void_p), ("state_rows", C.c_void_p), ("keep_ties", C.c_int32), ("reserved", C.c_int32)]
+
+
+class EosStopC(C.Structure):
+    """vui_eos_stop (include/vui_amd.h)."""
+    _fields_ = [("threshold", C.c_float), ("min_frames", C.c_int32), ("state", C.c_void_p)]
 
 
 class CodecConfigC(C.Structure):
@@ -87,7 +94,7 @@ SIGNATURES = {
     "vui_sample_cb0": (_I, [_P, _P, _P, _P, _P, _F, _I, C.POINTER(SampleParamsC), _P, _I, _P]),
     "vui_rq_generate": (_I, [_P, _P, _P, _P, _I, C.POINTER(SampleParamsC), _P, _I, _I, _I, _P]),
     "vui_frame_step": (_I, [_P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _F, _I, C.POINTER(SampleParamsC),
-                            C.POINTER(SampleParamsC), _P, _I, _P, _P, _P, _P, _I, _P, _I, _P]),
+                            C.POINTER(SampleParamsC), _P, _I, _P, _P, _P, _P, _I, _P, _I, C.POINTER(EosStopC), _P]),
     "vui_graph_begin": (_I, [_P]),
     "vui_graph_end": (_I, [_P, C.POINTER(_P)]),
     "vui_graph_launch": (_I, [_P, _P]),

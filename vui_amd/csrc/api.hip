@@ -113,6 +113,8 @@ static int check_cfg(const vui_config* c, int max_batch) {
     vui_set_error("bad depth-head layout R=%d heads=%d ffn=%d", c->rq_dim, c->rq_heads, c->rq_ffn); return VUI_EINVAL; }
   if (c->max_seqlen < 1 || c->n_slots < 1) { vui_set_error("max_seqlen and n_slots must be positive"); return VUI_EINVAL; }
   if (c->int8_backbone && c->dtype != VUI_DTYPE_BF16) { vui_set_error("int8 weights need bf16 activations"); return VUI_EINVAL; }
+  if (c->global_rope_dim < 0 || c->global_rope_dim > c->head_dim || (c->global_rope_dim & 1)) { vui_set_error("bad global_rope_dim %d", c->global_rope_dim); return VUI_EINVAL; }
+  if (c->n_layers < 64 && (c->global_layers >> c->n_layers)) { vui_set_error("global_layers names layers beyond n_layers"); return VUI_EINVAL; }
   return VUI_OK;
 }
 
@@ -175,6 +177,7 @@ int vui_ctx_create(const vui_config* cfg, const vui_weights* w, void* workspace,
   if (((uintptr_t)workspace) & 255) { vui_set_error("workspace must be 256-byte aligned"); return VUI_EINVAL; }
   if (!w->audio_emb || !w->final_norm || !w->codec_head || !w->eos_w || !w->eos_b || (cfg->rope_dim && !w->rope_table)) {
     vui_set_error("missing backbone weight pointer"); return VUI_EINVAL; }
+  if (w->rope_table_global && cfg->global_rope_dim < 2) { vui_set_error("rope_table_global needs global_rope_dim >= 2"); return VUI_EINVAL; }
   for (int l = 0; l < cfg->n_layers; ++l) {
     const vui_layer_weights& L = w->layers[l];
     if (!L.attn_norm || !L.wqkv || !L.wo || !L.mlp_norm || !L.w1 || !L.w3 || !L.w2) { vui_set_error("missing weights of layer %d", l); return VUI_EINVAL; }
@@ -291,6 +294,7 @@ static void fused_base(vui_ctx* ctx, FrameArgs& a) {
   a.Q = c.n_quantizers; a.CS = c.codebook_size; a.R = c.rq_dim; a.rqL = c.rq_layers; a.rqH = c.rq_heads; a.rqF = c.rq_ffn;
   a.rope_dim = c.rope_dim; a.S = c.max_seqlen; a.window = c.window; a.eps = c.norm_eps; a.rq_eps = c.rq_norm_eps;
   a.w = ctx->wdev; a.n_slots = c.n_slots;
+  a.global_layers = c.global_layers; a.global_rope_dim = c.global_rope_dim;
   a.ll = ctx->ll; a.epoch = ctx->ctl; a.arrive = ctx->ctl + 1; a.err = ctx->ctl + 2;
   a.prof = ctx->prof; a.prof_cap = ctx->prof_cap; a.prof_wg = ctx->prof_wg;
   a.ns = ctx->ns; a.lds_kv_off = (int)(ctx->lds_bytes - frame_rq_cache_bytes(c));
@@ -356,14 +360,14 @@ int vui_backbone_step(vui_ctx* ctx, const int64_t* codes_in, const void* emb_in,
     g.x = ctx->x; g.norm_w = L.attn_norm; g.eps = c.norm_eps;
     g.W = L.wqkv; g.sc = L.s_qkv; g.y = ctx->q; g.ldy = H * hd;
     g.B = B; g.N = (H + 2 * KV) * hd; g.K = d; g.epi = EPI_QKV;
-    g.rope = ctx->w.rope_table; g.rope_dim = c.rope_dim; g.hd = hd; g.nq = H * hd; g.nkv = KV * hd;
+    g.rope = layer_rope(c, ctx->w, l, &g.rope_dim); g.hd = hd; g.nq = H * hd; g.nkv = KV * hd;
     g.kc = kc; g.vc = vc; g.seq_lens = seq_lens; g.slot_idx = slot_idx; g.S = c.max_seqlen;
     if ((rc = launch_gemv(g, st))) return rc;
 
     AttnArgs a;
     memset(&a, 0, sizeof(a));
     a.dtype = c.dtype; a.q = ctx->q; a.kc = kc; a.vc = vc; a.seq_lens = seq_lens; a.slot_idx = slot_idx;
-    a.out = ctx->att; a.B = B; a.H = H; a.KV = KV; a.hd = hd; a.S = c.max_seqlen; a.window = c.window;
+    a.out = ctx->att; a.B = B; a.H = H; a.KV = KV; a.hd = hd; a.S = c.max_seqlen; a.window = layer_window(c, l);
     a.n_splits = n_splits; a.part = ctx->part; a.counter = ctx->counter;
     if ((rc = launch_decode_attn(a, st))) return rc;
 
@@ -416,7 +420,7 @@ int vui_sample_cb0(vui_ctx* ctx, const void* logits, float* rep_counts, int32_t*
   if (window > 0 && rep_counts && penalty > 1.0f && (!rep_hist || !rep_pos)) { vui_set_error("a repetition window needs rep_hist and rep_pos"); return VUI_EINVAL; }
   SampleArgs s = sample_base(sp);
   s.dtype = ctx->cfg.dtype; s.logits = logits; s.rep_counts = rep_counts; s.rep_hist = rep_hist; s.rep_pos = rep_pos;
-  s.penalty = penalty; s.window = window; s.codebook = 0; s.exact_k = 1; s.CS = ctx->cfg.codebook_size; s.B = B;
+  s.penalty = penalty; s.window = window; s.codebook = 0; s.exact_k = sp->keep_ties ? 0 : 1; s.CS = ctx->cfg.codebook_size; s.B = B;
   s.out = code0_out; s.out_stride = 1; s.out_col = 0;
   return launch_sample(s, (hipStream_t)stream);
 }
@@ -528,10 +532,12 @@ int vui_frame_step(vui_ctx* ctx, int64_t* codes_io, const int32_t* slot_idx, int
                    int B, void* k_cache, void* v_cache, float* rep_counts, int32_t* rep_hist, int32_t* rep_pos,
                    float penalty, int window, const vui_sample_params* sp_cb0, const vui_sample_params* sp_rq,
                    const float* logit_bias, int n_q, void* hidden_out, void* cb0_out, float* eos_prob_out,
-                   int64_t* frames_out, int max_frames, int32_t* frame_ctr, int n_splits, vui_stream_t stream) {
+                   int64_t* frames_out, int max_frames, int32_t* frame_ctr, int n_splits, const vui_eos_stop* stop,
+                   vui_stream_t stream) {
   int rc = check_batch(ctx, B, n_splits);
   if (rc) return rc;
   if (!codes_io || !sp_cb0 || !sp_rq || !frame_ctr) { vui_set_error("NULL argument"); return VUI_EINVAL; }
+  if (stop && (B != 1 || !stop->state)) { vui_set_error("the device-side end-of-turn test takes one row and a state pointer"); return VUI_EINVAL; }
   const vui_config& c = ctx->cfg;
   hipStream_t st = (hipStream_t)stream;
   void* hid = hidden_out ? hidden_out : ctx->hidden;
@@ -552,6 +558,8 @@ int vui_frame_step(vui_ctx* ctx, int64_t* codes_io, const int32_t* slot_idx, int
     a.code0_out = ctx->code0; a.logit_bias = logit_bias; a.n_q = n_q;
     a.codes_out = codes_io; a.codes_stride = c.n_quantizers; a.zero_pad = 1;
     a.frames_out = frames_out; a.eos_prob_out = eos_prob_out; a.max_frames = max_frames; a.frame_ctr = frame_ctr;
+    a.exact0 = sp_cb0->keep_ties ? 0 : 1;
+    if (stop) { a.stop_state = stop->state; a.stop_thr = stop->threshold; a.stop_min = stop->min_frames; }
     return launch_frame(a, ctx->nwg, ctx->lds_bytes, st);
   }
   if ((rc = vui_backbone_step(ctx, codes_io, nullptr, slot_idx, seq_lens, seq_inc, B, k_cache, v_cache, hid, cb0,
@@ -560,14 +568,15 @@ int vui_frame_step(vui_ctx* ctx, int64_t* codes_io, const int32_t* slot_idx, int
   if (window > 0 && rep_counts && penalty > 1.0f && (!rep_hist || !rep_pos)) { vui_set_error("a repetition window needs rep_hist and rep_pos"); return VUI_EINVAL; }
   SampleArgs s = sample_base(sp_cb0);
   s.dtype = c.dtype; s.logits = cb0; s.rep_counts = rep_counts; s.rep_hist = rep_hist; s.rep_pos = rep_pos;
-  s.penalty = penalty; s.window = window; s.codebook = 0; s.exact_k = 1; s.CS = c.codebook_size; s.B = B;
+  s.penalty = penalty; s.window = window; s.codebook = 0; s.exact_k = sp_cb0->keep_ties ? 0 : 1; s.CS = c.codebook_size; s.B = B;
   s.out = ctx->code0; s.out_stride = 1; s.out_col = 0;
   s.eos_logit = ctx->eos; s.eos_prob = ctx->eos_prob;
   if ((rc = launch_sample(s, st))) return rc;
   if ((rc = vui_rq_generate(ctx, hid, ctx->code0, logit_bias, n_q, sp_rq, codes_io, c.n_quantizers, 1, B, stream)))
     return rc;
   return launch_frame_finish(codes_io, frames_out, B * c.n_quantizers, max_frames, frame_ctr, ctx->eos_prob,
-                             eos_prob_out, B, st);
+                             eos_prob_out, B, stop ? stop->state : nullptr, stop ? stop->threshold : 0.f,
+                             stop ? stop->min_frames : 0, st);
 }
 
 // ---- HIP graphs ----

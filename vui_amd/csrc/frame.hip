@@ -285,6 +285,9 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
   bf16_t* rqkv = (bf16_t*)(smem + a.lds_kv_off);
 
   const int wg = blockIdx.x, nwg = gridDim.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  // a streamed turn that has met its end-of-turn test: steps enqueued ahead of the host's knowledge do nothing
+  // (the flag was written by an earlier launch or by the host, so every workgroup reads the same value)
+  if (a.stop_state && a.stop_state[0] != 0) return;
   Ctl c;
   ctl_begin(c, a.epoch, a.err);
   const uint32_t ep = c.epoch;
@@ -328,6 +331,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
   const bf16_t* g_eos_w = (const bf16_t*)W.eos_w;
   const bf16_t* g_eos_b = (const bf16_t*)W.eos_b;
   const float* g_rope = W.rope_table;
+  const float* g_rope_global = W.rope_table_global;
   const bf16_t* g_rq_proj = (const bf16_t*)W.rq_backbone_proj;
   const bf16_t* g_rq_emb = (const bf16_t*)W.rq_code_emb;
   const bf16_t* pos_emb = (const bf16_t*)W.rq_pos_emb;
@@ -384,7 +388,8 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
     const int np_qkv = (nq + 2 * nkv) / 2;
     const int n_qkv = pairs_of(np_qkv, wg, nwg), n_o = pairs_of(d / 2, wg, nwg), n_sw = pairs_of(a.F / 2, wg, nwg);
     const Plan P_qkv = plan_of(n_qkv, d, wg, nwg, wave);
-    // QKV epilogue constants of this wave's pairs: region, index in region, rotation factors
+    // QKV epilogue constants of this wave's pairs: region, index in region, rotation factors (the layers' common
+    // table; a global-attention layer with a table of its own fetches its factors at the top of the layer)
     int q_region[2], q_m[2];
     float4 q_rot[2];
 #pragma unroll
@@ -402,19 +407,10 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       else q_region[s] |= 4;  // no rotation
     }
     const uint64_t* ybuf = nullptr;  // previous layer's MLP output, still to be added to xres
-    // attention split geometry (identical in every workgroup)
     const int len = pos + 1;
-    const int start = (a.window > 0) ? max(0, len - 1 - a.window) : 0;
-    const int nkeys = len - start;
     const int NS = a.ns;
-    int ns_eff = (nkeys + 31) / 32;
-    ns_eff = max(1, min(ns_eff, NS));
-    int chunk = (nkeys + ns_eff - 1) / ns_eff;
-    chunk = (chunk + 15) / 16 * 16;
     const size_t slab = (size_t)a.n_slots * a.S * nkv;
     const int att_h = wg % a.H, att_s = wg / a.H;
-    const bool att_on = att_s < ns_eff && wg < a.H * NS;
-    const int att_lo = start + att_s * chunk, att_hi = min(att_lo + chunk, len);
     const int kvh = att_h / (a.H / a.KV);
     const int cpd = (hd + 15) / 16;
     const bool mrg_on = wg < a.H * cpd;
@@ -423,6 +419,32 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       const LayerP Lw = lp[l];
       bf16_t* kcl = a.kc + slab * l;
       bf16_t* vcl = a.vc + slab * l;
+      // this layer's window and rotation (src/vui/model.py:406-418, 504-509): a global layer sees the whole cache
+      const bool glob = (a.global_layers >> l) & 1ull;
+      const int win_l = glob ? 0 : a.window;
+      int l_region[2] = {q_region[0], q_region[1]};
+      float4 l_rot[2] = {q_rot[0], q_rot[1]};
+      if (glob && g_rope_global) {  // uniform over the grid
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+          const int region = q_region[s] & 3, dd = q_m[s] % hd;
+          l_region[s] = region | 4;
+          l_rot[s] = make_float4(1.f, 0.f, 1.f, 0.f);
+          if (s < P_qkv.nslots && region != 2 && dd < a.global_rope_dim) {
+            l_rot[s] = *reinterpret_cast<const float4*>(g_rope_global + ((size_t)pos * a.global_rope_dim + dd) * 2);
+            l_region[s] = region;
+          }
+        }
+      }
+      // attention split geometry of the layer (identical in every workgroup)
+      const int start = (win_l > 0) ? max(0, len - 1 - win_l) : 0;
+      const int nkeys = len - start;
+      int ns_eff = (nkeys + 31) / 32;
+      ns_eff = max(1, min(ns_eff, NS));
+      int chunk = (nkeys + ns_eff - 1) / ns_eff;
+      chunk = (chunk + 15) / 16 * 16;
+      const bool att_on = att_s < ns_eff && wg < a.H * NS;
+      const int att_lo = start + att_s * chunk, att_hi = min(att_lo + chunk, len);
       // ---- QKV + RoPE + cache append ----
       WRegs<2, false> wr;
       const Plan P_qkv = plan_of(n_qkv, d, wg, nwg, wave);
@@ -439,10 +461,10 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       gemv_compute<2, false>(xp, P_qkv, wr, red, [&](int gp, float v0, float v1, float, float) {
         const bool s0 = (gp == P_qkv.gp[0]);
         float o0 = bf2f(f2bf(v0)), o1 = bf2f(f2bf(v1));
-        const int rg = s0 ? q_region[0] : q_region[1];
+        const int rg = s0 ? l_region[0] : l_region[1];
         const int region = rg & 3, m = s0 ? q_m[0] : q_m[1];
         if (!(rg & 4)) {
-          const float4 f = s0 ? q_rot[0] : q_rot[1];
+          const float4 f = s0 ? l_rot[0] : l_rot[1];
           const float r0 = rope_mix(o0, f.x, -o1, f.y);
           const float r1 = rope_mix(o1, f.z, o0, f.w);
           o0 = r0; o1 = r1;
@@ -727,7 +749,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           }
         }
         TS(20);
-        code0 = block_sample<8>(lv, key, counts ? 0 : 16, a.CS, E, greedy, a.topk0, rnd0, 0u, ssh, (int*)sc, true);
+        code0 = block_sample<8>(lv, key, counts ? 0 : 16, a.CS, E, greedy, a.topk0, rnd0, 0u, ssh, (int*)sc, a.exact0 != 0);
         TS(21);
       }
     }
@@ -1048,17 +1070,27 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       const bool in_range = f >= 0 && f < a.max_frames;
       if (a.frames_out && in_range)
         for (int t = tid; t < a.Q; t += FR_THREADS) a.frames_out[(size_t)f * a.Q + t] = (t < a.n_q) ? codes_l[t] : 0;
-      if (a.eos_prob_out && tid == 0 && (in_range || !a.frames_out))
-        a.eos_prob_out[a.frames_out ? f : 0] = 1.0f / (1.0f + expf(-eos_logit));
+      const float p_eos = 1.0f / (1.0f + expf(-eos_logit));
+      if (a.eos_prob_out && tid == 0 && (in_range || !a.frames_out)) a.eos_prob_out[a.frames_out ? f : 0] = p_eos;
       __syncthreads();
-      if (tid == 0) a.frame_ctr[0] = f + 1;
+      if (tid == 0) {
+        a.frame_ctr[0] = f + 1;
+        if (a.stop_state) {  // src/vui/engine.py:1468-1471, decided here instead of on the host
+          const int step = a.stop_state[1];
+          if (step >= a.stop_min && p_eos > a.stop_thr) a.stop_state[0] = 1;
+          a.stop_state[1] = step + 1;
+        }
+      }
     }
-    } else if ((a.mode & FR_FINISH) && a.eos_prob_out && tid == 0) {
-      // a failed step marks its EOS probability with -1, so a caller that reads that value every frame
-      // learns of the failure from the same read
+    } else if ((a.mode & FR_FINISH) && tid == 0) {
+      // a failed step marks its EOS probability with -1 and the end-of-turn flag with 2, so a caller that reads
+      // one of them every frame learns of the failure from the same read (and steps enqueued behind it do nothing)
       const int f = a.frame_ctr[0];
-      if (!a.frames_out) a.eos_prob_out[0] = -1.0f;
-      else if (f >= 0 && f < a.max_frames) a.eos_prob_out[f] = -1.0f;
+      if (a.eos_prob_out) {
+        if (!a.frames_out) a.eos_prob_out[0] = -1.0f;
+        else if (f >= 0 && f < a.max_frames) a.eos_prob_out[f] = -1.0f;
+      }
+      if (a.stop_state) a.stop_state[0] = 2;
     }
     if (tid == 0) ctl_finish(c, a.epoch, a.arrive, (uint32_t)nwg);
   }

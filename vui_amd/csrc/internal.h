@@ -15,6 +15,15 @@ enum {
   EPI_RQ_QKV = 5,  // split into q | k | v without rotation, k/v into the depth-head cache
 };
 
+// per-layer attention window and rotation table (global-attention layers, vui_config.global_layers)
+static inline bool layer_is_global(const vui_config& c, int l) { return (c.global_layers >> l) & 1ull; }
+static inline int layer_window(const vui_config& c, int l) { return layer_is_global(c, l) ? 0 : c.window; }
+static inline const float* layer_rope(const vui_config& c, const vui_weights& w, int l, int* rope_dim) {
+  if (layer_is_global(c, l) && w.rope_table_global) { *rope_dim = c.global_rope_dim; return w.rope_table_global; }
+  *rope_dim = c.rope_dim;
+  return w.rope_table;
+}
+
 struct GemvArgs {
   int dtype;      // VUI_DTYPE_*
   int w_int8;     // weights are int8 with per-row scales
@@ -126,7 +135,8 @@ int launch_rq_token(int dtype, const int64_t* code, int64_t off, const void* emb
 // frames_out[*ctr] = codes (B*Q) if ctr < max_frames; *ctr += 1
 // and eos_out[(frames_out ? *ctr : 0) * B + b] = eos_in[b]
 int launch_frame_finish(const int64_t* codes, int64_t* frames_out, int n, int max_frames, int32_t* ctr,
-                        const float* eos_in, float* eos_out, int B, hipStream_t st);
+                        const float* eos_in, float* eos_out, int B, int32_t* stop_state, float stop_thr, int stop_min,
+                        hipStream_t st);
 int launch_add_rows(int dtype, const void* a, const void* vec, void* out, int B, int R, hipStream_t st);
 int launch_fill_u32(uint32_t* p, uint32_t v, int64_t n, hipStream_t st);
 
@@ -142,6 +152,8 @@ struct FrameArgs {
   int32_t* seq_lens;
   const int32_t* seq_inc;
   int n_slots;
+  unsigned long long global_layers;  // bit l: layer l attends over the whole cache and uses the global rotation table
+  int global_rope_dim;
   uint16_t *kc, *vc;
   uint16_t *hidden_out, *cb0_out, *eos_out;
   // code-0 sampling
@@ -168,6 +180,10 @@ struct FrameArgs {
   float* eos_prob_out;
   int max_frames;
   int32_t* frame_ctr;
+  int32_t* stop_state;  // {stopped, step} or nullptr (vui_eos_stop)
+  float stop_thr;
+  int stop_min;
+  int exact0;           // code-0 cut keeps exactly top_k entries
   // exchange
   uint64_t* ll;
   uint32_t* epoch;

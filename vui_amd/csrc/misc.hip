@@ -196,8 +196,14 @@ int launch_add_rows(int dtype, const void* a, const void* vec, void* out, int B,
 }
 
 __global__ void frame_finish_kernel(const int64_t* codes, int64_t* frames_out, int n, int max_frames, int32_t* ctr,
-                                    const float* eos_in, float* eos_out, int B) {
+                                    const float* eos_in, float* eos_out, int B, int32_t* stop_state, float stop_thr,
+                                    int stop_min) {
   const int f = ctr[0];
+  if (stop_state && threadIdx.x == 0) {  // end-of-turn test on the device (row 0; the caller passes B == 1)
+    const int step = stop_state[1];
+    if (step >= stop_min && eos_in[0] > stop_thr) stop_state[0] = 1;
+    stop_state[1] = step + 1;
+  }
   const bool in_range = f >= 0 && f < max_frames;
   if (frames_out && in_range)
     for (int i = threadIdx.x; i < n; i += blockDim.x) frames_out[(size_t)f * n + i] = codes[i];
@@ -207,9 +213,10 @@ __global__ void frame_finish_kernel(const int64_t* codes, int64_t* frames_out, i
   if (threadIdx.x == 0) ctr[0] = f + 1;
 }
 int launch_frame_finish(const int64_t* codes, int64_t* frames_out, int n, int max_frames, int32_t* ctr,
-                        const float* eos_in, float* eos_out, int B, hipStream_t st) {
+                        const float* eos_in, float* eos_out, int B, int32_t* stop_state, float stop_thr, int stop_min,
+                        hipStream_t st) {
   hipLaunchKernelGGL(frame_finish_kernel, dim3(1), dim3(256), 0, st, codes, frames_out, n, max_frames, ctr, eos_in,
-                     eos_out, B);
+                     eos_out, B, stop_state, stop_thr, stop_min);
   HIP_TRY(hipGetLastError());
   return VUI_OK;
 }

@@ -487,15 +487,18 @@ int launch_prefill(const vui_config& c, const vui_weights& w, const void* tiled_
     // attention over the L cached positions of this slot
     bf16_t* krow = kc + (size_t)slot * S * nkv;
     bf16_t* vrow = vc + (size_t)slot * S * nkv;
-    hipLaunchKernelGGL(pf_stage_kv_kernel, dim3(Lpad / 32, (nkv + nq) / 32), dim3(256), 0, st, qkv, krow, vrow, kt, vt, w.rope_table, L, Lpad, nq, nkv,
-                       hd, c.rope_dim, pos0);
+    int rope_dim_l;
+    const float* rope_l = layer_rope(c, w, l, &rope_dim_l);
+    const int window_l = layer_window(c, l);
+    hipLaunchKernelGGL(pf_stage_kv_kernel, dim3(Lpad / 32, (nkv + nq) / 32), dim3(256), 0, st, qkv, krow, vrow, kt, vt, rope_l, L, Lpad, nq, nkv,
+                       hd, rope_dim_l, pos0);
     {
       const dim3 grid((T + 15) / 16, H);
       switch (hd / 32) {
-        case 1: hipLaunchKernelGGL(pf_attn_kernel<1>, grid, dim3(512), 0, st, qkv, kt, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, c.window, scale); break;
-        case 2: hipLaunchKernelGGL(pf_attn_kernel<2>, grid, dim3(512), 0, st, qkv, kt, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, c.window, scale); break;
-        case 3: hipLaunchKernelGGL(pf_attn_kernel<3>, grid, dim3(512), 0, st, qkv, kt, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, c.window, scale); break;
-        default: hipLaunchKernelGGL(pf_attn_kernel<4>, grid, dim3(256), 0, st, qkv, kt, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, c.window, scale); break;
+        case 1: hipLaunchKernelGGL(pf_attn_kernel<1>, grid, dim3(512), 0, st, qkv, kt, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, window_l, scale); break;
+        case 2: hipLaunchKernelGGL(pf_attn_kernel<2>, grid, dim3(512), 0, st, qkv, kt, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, window_l, scale); break;
+        case 3: hipLaunchKernelGGL(pf_attn_kernel<3>, grid, dim3(512), 0, st, qkv, kt, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, window_l, scale); break;
+        default: hipLaunchKernelGGL(pf_attn_kernel<4>, grid, dim3(256), 0, st, qkv, kt, vt, att, T, L, Lpad, nq, nkv, H / KV, pos0, window_l, scale); break;
       }
     }
     PfGemm wo{};

@@ -57,6 +57,17 @@ class GenConfig:
         return min(int(secs * FRAME_RATE), ceil)
 
 
+@dataclass(frozen=True)
+class Segment:
+    """One voice-reference unit: a transcript and its codec codes (Segment, src/vui/engine.py:48-58).
+    Tokenising is the caller's: `text_emb` (1, T, d) holds the embeddings of the cleaned, tokenised text
+    (model.token_emb of its ids); `text` is kept for the words-per-second estimate.  Either part may be missing."""
+
+    text: str = ""
+    codes: Tensor | None = None  # (T, Q) long
+    text_emb: Tensor | None = None
+
+
 @dataclass
 class Chunk:
     """One text chunk of a turn as the decode loop needs it: the embeddings of `[spk] text` (with
@@ -118,6 +129,9 @@ class Row:
         self._engine = engine
         self._idx = idx
         self._prompt_offset = 0
+        self._spk_token: Tensor | None = None
+        self._spk_token_2: Tensor | None = None  # optional second speaker
+        self._active_speaker = 0  # flipped on chunks flagged as speaker changes
         self._closed = False
         self.prompt_wps: float = 0.0
         self._slot = torch.tensor([idx], dtype=torch.int32, device=engine.device)
@@ -140,6 +154,23 @@ class Row:
         """Write a (1, T, d) embedding block at the row's offset; returns the final-norm output
         (1, T, d).  Engine._prefill_emb, src/vui/engine.py:674-694."""
         return self._engine._prefill_emb(self, emb)
+
+    def prefill(self, segments: "list[Segment]", spk_emb: Tensor | None = None,
+                segments_2: "list[Segment] | None" = None, spk_emb_2: Tensor | None = None) -> int:
+        """Prefill `[spk] text_i codes_i` for every segment, both speakers in order (Row.prefill,
+        src/vui/engine.py:186-202); sets the rewind point and the words-per-second estimate."""
+        return self._engine._prefill_row(self, segments, spk_emb, segments_2, spk_emb_2)
+
+    def add_user(self, text_emb: Tensor | None = None, codes: Tensor | None = None, *, final: bool = True) -> int:
+        """Write a user turn chunk: text ([SC] when final) codes (Row.add_user, src/vui/engine.py:204-208;
+        the text arrives embedded)."""
+        return self._engine._add_user(self, text_emb, codes, final=final)
+
+    def render(self, chunks: "list[Chunk]", cfg: GenConfig = GenConfig()) -> "tuple[Tensor, Tensor | None]":
+        """A whole turn without streaming: (codes (T, Q) on the CPU, audio (1, 1, S) or None without a vocoder)
+        (Row.render, src/vui/engine.py:246-250)."""
+        codes = self._engine._render_row(self, chunks, cfg)
+        return codes, self._engine._decode_full(codes)
 
     def stream(self, chunks: "list[Chunk]", cfg: GenConfig = GenConfig(), cancel=None, *, reset_rep: bool = True,
                final_turn: bool = False) -> Iterator[Tensor]:
@@ -188,7 +219,7 @@ class Engine:
     """Streaming (B=1) and batched (B=N) decode over one flash-style KV cache."""
 
     def __init__(self, name: str | None = None, *, model: Vui | None = None, codec=None, max_rows: int = 1,
-                 max_seq: int | None = None):
+                 max_seq: int | None = None, sc_token_id: int | None = None):
         if model is None:
             if name is None:
                 raise ValueError("pass model= or a local checkpoint path")
@@ -207,6 +238,11 @@ class Engine:
         if self.max_seq > trained:
             raise ValueError(f"max_seq={self.max_seq} exceeds trained ceiling {trained}")
         self._cond_bias = model._cond_bias
+        # embedding of the speaker-change token (src/vui/engine.py:320-324 looks its id up in the tokenizer, which
+        # is not part of this package: the caller passes the id; without it no [SC] position is written)
+        self._sc_emb = None
+        if sc_token_id is not None:
+            self._sc_emb = model.token_emb(torch.tensor([[sc_token_id]], device=self.device)).to(self.dtype)
         self._setup_graphs()
         self._setup_rep_state()
         self._free: set[int] = set(range(max_rows))
@@ -243,6 +279,10 @@ class Engine:
         # fused frame state
         self._frame_ctr = torch.zeros(1, dtype=torch.int32, device=dev)
         self._code0 = torch.zeros(N, dtype=torch.long, device=dev)
+        # device-side end-of-turn test of a streamed turn: {stopped, step}, and what a chunk start resets it to
+        self._stop_state = torch.zeros(2, dtype=torch.int32, device=dev)
+        self._stop_init = torch.tensor([0, 1], dtype=torch.int32, device=dev)
+        self._stop_host = [torch.zeros(1, dtype=torch.int32).pin_memory() for _ in range(2)]
 
     def _splits(self, B: int) -> int:
         return self.model.decoder.default_splits(B)
@@ -394,6 +434,7 @@ class Engine:
         return self.model.decoder.forward_flash(emb.to(self.dtype), pos, slot_idx=row._slot,
                                                 known=(row.idx, off) if offset is not None else None, lane=lane)
 
+    max_frame_graphs = 32  # captured frame graphs kept (oldest dropped first)
     prefill_lanes = 4  # streams that ingest the blocks of different rows at once (1: one after the other)
 
     def _prefill_many(self, jobs: "list[tuple[Row, Tensor, int]]") -> "list[Tensor]":
@@ -427,14 +468,17 @@ class Engine:
         self._cond_bias = self.model._cond_bias
 
     # ------------------------------------------------------------------ fused frame loop
-    def _frame_graph(self, B: int, cfg: GenConfig, slot_idx: Tensor | None, max_frames: int):
+    def _frame_graph(self, B: int, cfg: GenConfig, slot_idx: Tensor | None, max_frames: int,
+                     stop: "tuple[float, int] | None" = None):
         """One HIP graph holding a whole frame: backbone step on the previous frame, code-0
-        sampling with repetition penalty, the depth head, frame log, counters."""
+        sampling with repetition penalty, the depth head, frame log, counters.  stop = (eos_threshold,
+        min_frames): the step also runs the end-of-turn test on the device (self._stop_state)."""
         nq = cfg.n_codebooks if cfg.n_codebooks > 0 else self.Q
         key = (B, nq, cfg.temperature, cfg.top_k, cfg.rq_top_k, cfg.rep_penalty, cfg.rep_window, cfg.seed,
-               None if slot_idx is None else tuple(slot_idx.tolist()), max_frames)
+               None if slot_idx is None else tuple(slot_idx.tolist()), max_frames, stop)
         hit = self._frame_graphs.get(key)
         if hit is not None:
+            self._frame_graphs[key] = self._frame_graphs.pop(key)  # most recently used last
             return hit
         nat = self.model._native
         dec = self.model.decoder
@@ -447,6 +491,10 @@ class Engine:
         win = cfg.rep_window if (use_rep and self._rep_history is not None) else 0
         codes_io = self._gc_codes_in if slot_idx is not None else self._g_codes_in
         ns = self._splits(B)
+        stop_c = None
+        if stop is not None:
+            stop_c = _lib.EosStopC()
+            stop_c.threshold, stop_c.min_frames, stop_c.state = float(stop[0]), int(stop[1]), self._stop_state.data_ptr()
 
         def body(st):
             _lib.check(nat.lib.vui_frame_step(
@@ -455,11 +503,13 @@ class Engine:
                 _lib.ptr(self._rep_history) if win else None, self._rep_pos.data_ptr() if win else None,
                 float(cfg.rep_penalty), win, C.byref(sp0), C.byref(sp1), None, nq, self._g_hidden_out.data_ptr(),
                 self._g_cb0_out.data_ptr(), eos.data_ptr(), _lib.ptr(frames), max_frames,
-                self._frame_ctr.data_ptr(), ns, st), "vui_frame_step")
+                self._frame_ctr.data_ptr(), ns, C.byref(stop_c) if stop_c is not None else None, st), "vui_frame_step")
 
         # captured without a warm-up run: the step mutates seq_lens, the rep state and the counter
         g = Graph(self.model, body, warmup=0)
-        entry = (g, frames, eos, (sp0, sp1, slot_idx))
+        entry = (g, frames, eos, (sp0, sp1, slot_idx, stop_c))
+        if len(self._frame_graphs) >= self.max_frame_graphs:  # a serving loop with ever new seeds must not grow without bound
+            self._frame_graphs.pop(next(iter(self._frame_graphs)))
         self._frame_graphs[key] = entry
         return entry
 
@@ -505,6 +555,257 @@ class Engine:
         torch.cuda.current_stream().synchronize()
         nat.status()  # a persistent launch that gave up a wait committed nothing: raise instead of returning stale frames
         return frames[:n_frames, :, :nq].clone(), eos[:n_frames].clone()
+
+    # ------------------------------------------------------------------ prompt, user turn
+    def _audio_emb(self, codes: Tensor) -> Tensor:
+        pc = codes.to(self.device)
+        if pc.dim() == 2:
+            pc = pc.unsqueeze(0)
+        return self.model.embed_audio(pc).to(self.dtype)
+
+    def _embed_speaker(self, spk_emb: Tensor | None) -> Tensor | None:
+        if spk_emb is None or self.model.spk_proj is None:
+            return None
+        return self.model.embed_speaker(spk_emb).to(self.dtype)
+
+    def _prefill_speaker_segments(self, row: Row, segments: "list[Segment]", spk_token: Tensor | None, *,
+                                  final: bool = False) -> None:
+        """src/vui/engine.py:725-741: `[spk] text_i ([SC] before the last audio) codes_i` per segment."""
+        last = len(segments) - 1
+        for i, seg in enumerate(segments):
+            if spk_token is not None:
+                self._prefill_emb(row, spk_token)
+            if seg.text_emb is not None and seg.text_emb.shape[1] > 0:
+                self._prefill_emb(row, seg.text_emb.to(self.device, self.dtype))  # prompt text carries no cond_bias
+            if final and i == last and self._sc_emb is not None:
+                self._prefill_emb(row, self._sc_emb)
+            if seg.codes is not None:
+                self._prefill_emb(row, self._audio_emb(seg.codes))
+
+    @torch.inference_mode()
+    def _prefill_row(self, row: Row, segments: "list[Segment]", spk_emb: Tensor | None,
+                     segments_2: "list[Segment] | None" = None, spk_emb_2: Tensor | None = None) -> int:
+        """Engine._prefill_row, src/vui/engine.py:743-796."""
+        row._spk_token = self._embed_speaker(spk_emb)
+        row._spk_token_2 = self._embed_speaker(spk_emb_2)
+        row._active_speaker = 0
+        all_segs = list(segments) + (list(segments_2) if segments_2 else [])
+        all_codes = [seg.codes for seg in all_segs if seg.codes is not None]
+        if all_codes and row._codec_ctx is not None:  # seed the row's vocoder context with every prompt code
+            row._codec_ctx.set_prompt(torch.cat([c.to(self.device) for c in all_codes], dim=0).T.unsqueeze(0))
+        self._prefill_speaker_segments(row, segments, row._spk_token, final=True)
+        if segments_2 is not None:
+            self._prefill_speaker_segments(row, segments_2, row._spk_token_2, final=True)
+        row._prompt_offset = row.offset
+        total_words = sum(len(seg.text.split()) for seg in all_segs if seg.text)
+        total_frames = sum(seg.codes.shape[0] for seg in all_segs if seg.codes is not None)
+        if total_frames > 0 and total_words > 0:
+            row.prompt_wps = total_words / (total_frames / FRAME_RATE)
+        return row._prompt_offset
+
+    @torch.inference_mode()
+    def _add_user(self, row: Row, text_emb: Tensor | None, codes: Tensor | None, *, final: bool = True) -> int:
+        """Engine._add_user, src/vui/engine.py:798-826: text ([SC] when final) codes.  The text arrives embedded
+        (the reference adds model.noisy_emb to user text; the caller folds it in)."""
+        if text_emb is not None and text_emb.shape[1] > 0:
+            self._prefill_emb(row, text_emb.to(self.device, self.dtype))
+        if final and self._sc_emb is not None:
+            self._prefill_emb(row, self._sc_emb)
+        if codes is not None:
+            self._prefill_emb(row, self._audio_emb(codes))
+            if row._codec_ctx is not None:
+                row._codec_ctx.add(codes.T.unsqueeze(0).to(self.device))
+        return row.offset
+
+    def _decode_full(self, codes: Tensor) -> Tensor | None:
+        """(T, Q) codes -> (1, 1, S) audio through the vocoder's offline pass (Engine._decode_full); None when
+        the engine has no vocoder."""
+        if self.codec is None:
+            return None
+        if codes.shape[0] == 0:
+            return torch.zeros(1, 1, 0, device=self.device)
+        return self.codec(codes.to(self.device).T.unsqueeze(0))
+
+    # ------------------------------------------------------------------ batched offline render
+    @torch.inference_mode()
+    def _render_rows(self, rows: "list[Row]", chunk_lists: "list[list[Chunk]]", cfg: GenConfig) -> "dict[int, Tensor]":
+        """Core batched decode loop of render()/render_all() (Engine._render_rows, src/vui/engine.py:865-1087):
+        {row.idx: (T, Q) codes on the CPU}.  Every row has been prefilled; per chunk the agent text is written and
+        the first frame drawn without a top-k cut, then all max_rows slots step together (one batched backbone
+        step, code 0 with each row's rolling repetition state, EOS flags read on the host, one batched depth-head
+        call) until every row has used its chunks, max_secs, or the cache.  A chunk that ends with fewer than two
+        frames per word is rewound and drawn again colder (0.5, then 0.3).
+
+        Where this differs from the reference, by necessity: texts arrive as chunks of embeddings; draws come from
+        the counter-based generator, one counter step per chunk start and per decode step; a chunk start uses the
+        repetition state of its own row (the reference broadcasts one row's logits against all rows' counts there,
+        which only works for max_rows == 1 or without a penalty).  With max_rows == 1 the step is the one-launch
+        frame graph and the frames equal what Row.stream yields for the same chunks (the invariant the reference
+        states at engine.py:1001-1008) as long as neither the stream's gate nor this loop's retry fires."""
+        model, nat = self.model, self.model._native
+        N = self.max_rows
+        max_frames = int(cfg.max_secs * FRAME_RATE)
+        min_frames = int(cfg.min_secs * FRAME_RATE)
+        max_seq = self.max_seq - 10
+        nq = cfg.n_codebooks if cfg.n_codebooks > 0 else self.Q
+        greedy = cfg.top_k == 1
+        use_rep = cfg.rep_penalty > 1.0
+        stream = torch.cuda.current_stream()
+        row_chunks = {r.idx: list(ch) for r, ch in zip(rows, chunk_lists)}
+        row_chunk_idx = {r.idx: 0 for r in rows}
+        row_frame_count = {r.idx: 0 for r in rows}
+        row_turn_count = {r.idx: 0 for r in rows}
+        row_max_turn = {r.idx: cfg.max_turn_frames(0, r.prompt_wps) for r in rows}
+        row_offset = {r.idx: r.offset for r in rows}  # host-side count of every row's cache length
+        row_chunk_offset: dict[int, int] = {}
+        row_retry_idx = {r.idx: 0 for r in rows}
+        frame_buf = torch.zeros(N, max(max_frames, 1), self.Q, device=self.device, dtype=torch.long)
+        active = {r.idx: True for r in rows}
+        self._rep_reset(cfg.rep_penalty, cfg.rep_window)
+        self._frame_ctr.zero_()
+        MIN_FPW = 2.0
+        RETRY_TEMPS = (0.5, 0.3)
+        single = N == 1 and nat.fused(-1)  # one row on the one-launch form: the frame graph is the step
+        rq_out = torch.zeros(N, self.Q, dtype=torch.long, device=self.device)
+
+        def advance_turn(row: Row, temp: float | None = None) -> bool:
+            """Write the next chunk's text and draw its first frame (engine.py:909-950); False without a chunk."""
+            ci = row_chunk_idx[row.idx]
+            chunks = row_chunks[row.idx]
+            if ci >= len(chunks) or row_frame_count[row.idx] >= max_frames:
+                return False
+            chunk = chunks[ci]
+            if chunk.sc and row._spk_token_2 is not None:
+                row._active_speaker = 1 - row._active_speaker
+            row_max_turn[row.idx] = cfg.max_turn_frames(chunk.n_words, row.prompt_wps)
+            row_chunk_offset[row.idx] = row_offset[row.idx]
+            t = temp or cfg.temperature
+            hidden = self._prefill_emb(row, chunk.emb, offset=row_offset[row.idx])[:, -1]
+            row_offset[row.idx] += chunk.emb.shape[1]
+            cb0 = model.codec_head(hidden)
+            sp0 = make_sample_params(t, 1 if greedy else 0, cfg.seed, self._frame_ctr, state_rows=row._slot)
+            code0 = torch.empty(1, dtype=torch.long, device=self.device)
+            win = cfg.rep_window if (use_rep and self._rep_history is not None) else 0
+            _lib.check(nat.lib.vui_sample_cb0(
+                nat.handle, cb0.contiguous().data_ptr(), self._rep_counts.data_ptr() if use_rep else None,
+                _lib.ptr(self._rep_history) if win else None, self._rep_pos.data_ptr() if win else None,
+                float(cfg.rep_penalty), win, C.byref(sp0), code0.data_ptr(), 1, stream.cuda_stream), "vui_sample_cb0")
+            sp1 = make_sample_params(t, cfg.rq_top_k if not greedy else 1, cfg.seed, self._frame_ctr, state_rows=None)
+            _lib.check(nat.lib.vui_rq_generate(nat.handle, hidden.contiguous().data_ptr(), code0.data_ptr(), None, nq,
+                                               C.byref(sp1), rq_out.data_ptr(), self.Q, 1, 1, stream.cuda_stream),
+                       "vui_rq_generate")
+            self._frame_ctr += 1
+            self._g_codes_in[row.idx] = rq_out[0]
+            frame_buf[row.idx, row_frame_count[row.idx]] = rq_out[0]
+            row_frame_count[row.idx] += 1
+            row_turn_count[row.idx] = 1
+            return True
+
+        def retry_chunk(row: Row) -> bool:
+            """engine.py:952-983: fewer than two frames per word -> rewind the chunk and draw it again colder."""
+            ci = row_chunk_idx[row.idx]
+            n_words = row_chunks[row.idx][ci].n_words
+            turn_n = row_turn_count[row.idx]
+            fpw = turn_n / n_words if n_words > 0 else 999
+            if fpw >= MIN_FPW:
+                row_retry_idx[row.idx] = 0
+                return False
+            ri = row_retry_idx[row.idx]
+            if ri >= len(RETRY_TEMPS):
+                row_retry_idx[row.idx] = 0
+                return False
+            row_retry_idx[row.idx] = ri + 1
+            self.seq_lens[row.idx] = row_chunk_offset[row.idx]
+            row_offset[row.idx] = row_chunk_offset[row.idx]
+            row_frame_count[row.idx] -= turn_n
+            self._rep_reset(cfg.rep_penalty, cfg.rep_window)
+            advance_turn(row, temp=RETRY_TEMPS[ri])
+            return True
+
+        def next_chunk(row: Row) -> None:
+            if retry_chunk(row):
+                return
+            row_retry_idx[row.idx] = 0
+            row_chunk_idx[row.idx] += 1
+            if not advance_turn(row):
+                active[row.idx] = False
+
+        for r in rows:
+            if not advance_turn(r):
+                active[r.idx] = False
+        g1 = eos1 = None
+        if single:
+            g1, _, eos1, _ = self._frame_graph(1, cfg, None, 0)
+        sp_rq = make_sample_params(cfg.temperature, cfg.rq_top_k if not greedy else 1, cfg.seed, self._frame_ctr)
+        total_steps = 0
+        while any(active.values()) and total_steps < max_frames:
+            # a row whose chunk reached its frame cap moves on before the step (engine.py:1001-1019)
+            for r in rows:
+                if active[r.idx] and row_turn_count[r.idx] >= row_max_turn[r.idx]:
+                    next_chunk(r)
+            if not any(active.values()):
+                break
+            if single:
+                g1.replay()  # backbone step, code 0 (+ push), depth head; the new frame is in _g_codes_in
+                p0 = eos1[0, 0].item()
+                if p0 < 0.0:
+                    nat.status()
+                    raise RuntimeError("frame step failed without a raised error word")
+                eos_cpu = [p0]
+                frames_all = self._g_codes_in
+            else:
+                hidden_all, cb0_all, eos_all = self._decode_step()
+                code0s = self._sample_cb0(cb0_all, cfg)
+                eos_cpu = torch.sigmoid(eos_all.float()).flatten().cpu().tolist()
+                nat.status()
+                _lib.check(nat.lib.vui_rq_generate(nat.handle, hidden_all.data_ptr(), code0s.data_ptr(), None, nq,
+                                                   C.byref(sp_rq), rq_out.data_ptr(), self.Q, 1, N, stream.cuda_stream),
+                           "vui_rq_generate")
+                self._frame_ctr += 1
+                frames_all = rq_out
+            total_steps += 1
+            for r in rows:
+                row_offset[r.idx] += 1  # every slot of the batched step advances
+            hit = []
+            for r in rows:
+                if not active[r.idx]:
+                    continue
+                if row_offset[r.idx] >= max_seq or row_frame_count[r.idx] >= max_frames:
+                    active[r.idx] = False
+                    continue
+                turn_n = row_turn_count[r.idx]
+                if turn_n >= min_frames and eos_cpu[r.idx] > cfg.eos_threshold:
+                    hit.append(r)
+                    continue
+                frame_buf[r.idx, row_frame_count[r.idx]] = frames_all[r.idx]
+                if not single:
+                    self._g_codes_in[r.idx] = frames_all[r.idx]
+                row_frame_count[r.idx] += 1
+                row_turn_count[r.idx] += 1
+            for r in hit:
+                next_chunk(r)
+        result: dict[int, Tensor] = {}
+        for r in rows:
+            n = row_frame_count[r.idx]
+            if n > 0:
+                result[r.idx] = frame_buf[r.idx, :n, :nq].cpu()
+        return result
+
+    def _render_row(self, row: Row, chunks: "list[Chunk]", cfg: GenConfig) -> Tensor:
+        """Engine._render_row, src/vui/engine.py:1089-1092."""
+        nq = cfg.n_codebooks if cfg.n_codebooks > 0 else self.Q
+        return self._render_rows([row], [chunks], cfg).get(row.idx, torch.zeros(0, nq, dtype=torch.long))
+
+    def render_all(self, rows: "list[Row]", chunk_lists: "list[list[Chunk]]", cfg: GenConfig = GenConfig()) -> list:
+        """Batched non-streaming render (Engine.render_all, src/vui/engine.py:1094-1106): one audio tensor per row
+        when the engine has a vocoder, else the (T, Q) codes of every row."""
+        results = self._render_rows(rows, chunk_lists, cfg)
+        nq = cfg.n_codebooks if cfg.n_codebooks > 0 else self.Q
+        out = []
+        for r in rows:
+            codes = results.get(r.idx, torch.zeros(0, nq, dtype=torch.long))
+            out.append(self._decode_full(codes) if self.codec is not None else codes)
+        return out
 
     # ------------------------------------------------------------------ continuous batching
     @torch.inference_mode()
@@ -684,7 +985,9 @@ class Engine:
         frames of the first chunk, and on high mean entropy rewinds the cache to the chunk start and
         retries colder.  A frame step here is one graph replay that also runs the depth head; when
         the EOS test then ends the chunk, that frame is dropped (the reference tests before its depth
-        head runs: same frames out)."""
+        head runs: same frames out).  The EOS test itself runs on the device (vui_eos_stop), the host reads
+        its flag one frame late; after a cancel the cache may hold one position more than the reference's
+        (a step already in flight), callers rewind after a cancel."""
         if not chunks:
             return
         max_frames = int(cfg.max_secs * FRAME_RATE)
@@ -750,51 +1053,86 @@ class Engine:
                 else:
                     yield frame
                     total_frames += 1
-                g, _, eos_now, _ = self._frame_graph(1, cfg_t, slot_idx, 0)
+                # Frames 1.. of the chunk: one graph replay each (backbone step on the previous frame, code-0 draw
+                # + push, depth head, and the end-of-turn test of src/vui/engine.py:1468-1471 on the device).  The
+                # one-launch form does nothing once the test has fired, so the next step is enqueued before this
+                # step's flag is read (one frame late: the GPU never waits for the host between frames); the
+                # kernel-sequence form, and the gate while it gathers (it reads every step's logits), go one
+                # step at a time.
+                g, _, _, _ = self._frame_graph(1, cfg_t, slot_idx, 0, stop=(cfg.eos_threshold, min_frames))
+                self._stop_state.copy_(self._stop_init)
+                ahead = nat.fused(-1)
                 retry_triggered = False
-                for step in range(1, max_per_turn):
-                    if total_frames >= max_frames or offset >= max_seq:
-                        for hc in held:
-                            yield hc
-                            total_frames += 1
-                        return
-                    if cancelled():
-                        return
-                    gathering = use_gate and len(held) < gate_target
-                    counts_before = self._rep_counts[row.idx:row.idx + 1].clone() if (gathering and use_rep) else None
-                    g.replay()  # backbone step on the previous frame, code-0 draw + push, depth head
-                    offset += 1
-                    if gathering:
-                        cnt = counts_before if counts_before is not None else self._rep_counts[row.idx:row.idx + 1]
-                        e, p1 = entropy_top1(self._penalised_probs(self._g_cb0_out[0:1], cnt, cfg, cur_temp))
-                        entropies.append(e)
-                        top1s.append(p1)
-                    p_eos = eos_now[0, 0].item()
-                    if p_eos < 0.0:  # the step's persistent launch failed and committed nothing
-                        nat.status()
-                        raise RuntimeError("frame step failed without a raised error word")
-                    if step >= min_frames and p_eos > cfg.eos_threshold:
-                        for hc in held:
-                            yield hc
-                            total_frames += 1
-                        held = []
-                        break
-                    frame = codes_io[0, :nq].clone()
-                    if gathering:
-                        held.append(frame)
-                        if len(held) == gate_target:
-                            avg_e = sum(entropies) / len(entropies)
-                            if avg_e > cfg.gate_entropy_max and retry_idx < cfg.gate_retries:
-                                retry_triggered = True
-                                break
+                pending = None  # (frame, event, pinned flag, gathering) of the step whose flag is still unread
+                step = 1
+                while True:
+                    launched = None
+                    reason = None
+                    if pending is None or (ahead and not use_gate):
+                        # the reference's tests at the top of an iteration, in its order (engine.py:1441-1449); a
+                        # step in flight counts as kept (if it turns out to be the last, the loop ends anyway)
+                        counted = total_frames + (1 if pending is not None else 0)
+                        if step >= max_per_turn:
+                            reason = "cap"
+                        elif counted >= max_frames or offset >= max_seq:
+                            reason = "limit"
+                        elif cancelled():
+                            return  # a step already in flight is dropped: no frame is yielded after a cancel
+                        else:
+                            gathering = use_gate and len(held) < gate_target
+                            counts_before = self._rep_counts[row.idx:row.idx + 1].clone() if (gathering and use_rep) else None
+                            g.replay()
+                            offset += 1
+                            if gathering:
+                                cnt = counts_before if counts_before is not None else self._rep_counts[row.idx:row.idx + 1]
+                                e, p1 = entropy_top1(self._penalised_probs(self._g_cb0_out[0:1], cnt, cfg, cur_temp))
+                                entropies.append(e)
+                                top1s.append(p1)
+                            flag_t = self._stop_host[step & 1]
+                            flag_t.copy_(self._stop_state[:1], non_blocking=True)
+                            ev = torch.cuda.Event()
+                            ev.record(stream)
+                            launched = (codes_io[0, :nq].clone(), ev, flag_t, gathering)
+                            step += 1
+                    if pending is not None:
+                        frame, ev, flag_t, was_gathering = pending
+                        pending = None
+                        ev.synchronize()
+                        flag = int(flag_t[0])
+                        if flag == 2:  # the step's persistent launch failed and committed nothing
+                            nat.status()
+                            raise RuntimeError("frame step failed without a raised error word")
+                        if flag == 1:  # end of turn: this frame is dropped; a step enqueued behind it did nothing
+                            if launched is not None:
+                                offset -= 1
                             for hc in held:
                                 yield hc
                                 total_frames += 1
                             held = []
-                            use_gate = False
-                    else:
-                        yield frame
-                        total_frames += 1
+                            break
+                        if was_gathering:
+                            held.append(frame)
+                            if len(held) == gate_target:
+                                avg_e = sum(entropies) / len(entropies)
+                                if avg_e > cfg.gate_entropy_max and retry_idx < cfg.gate_retries:
+                                    retry_triggered = True
+                                    break
+                                for hc in held:
+                                    yield hc
+                                    total_frames += 1
+                                held = []
+                                use_gate = False
+                        else:
+                            yield frame
+                            total_frames += 1
+                    pending = launched
+                    if pending is None and reason is not None:
+                        if reason == "cap":  # the chunk's step cap: on to the next chunk
+                            break
+                        for hc in held:  # max_secs or the cache limit: the turn is over
+                            yield hc
+                            total_frames += 1
+                        return
                 if retry_triggered:
                     retry_idx += 1
                     continue

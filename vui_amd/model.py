@@ -118,6 +118,9 @@ class _Native:
         c.rope_dim = (m.rope_dim or m.head_dim) if m.use_rotary_emb else 0
         c.max_seqlen, c.n_slots = max_seqlen, n_slots
         c.window = m.window_size or 0
+        dec = model.decoder
+        c.global_layers = sum(1 << i for i, g in enumerate(dec.block_is_global) if g)
+        c.global_rope_dim = dec.global_rope_dim if (dec.freqs_cis_global is not None and m.use_rotary_emb) else 0
         c.norm_eps, c.rq_norm_eps = 1e-5, 1e-6  # Decoder default / RMSNorm default, model.py:391,287
         c.int8_backbone = 1 if model.int8 else 0
         self.cfg = c
@@ -129,6 +132,8 @@ class _Native:
         w.eos_w = sd["eos_head.weight"].data_ptr()
         w.eos_b = sd["eos_head.bias"].data_ptr()
         w.rope_table = model.decoder.freqs_cis.data_ptr()
+        if dec.freqs_cis_global is not None and m.use_rotary_emb:
+            w.rope_table_global = dec.freqs_cis_global.data_ptr()
         for i in range(m.n_layers):
             p = f"decoder.blocks.{i}."
             L = w.layers[i]
@@ -223,8 +228,9 @@ class Graph:
 
 
 def make_sample_params(temperature: float, top_k: int | None, seed: int, frame_ctr: Tensor | None,
-                       state_rows: Tensor | None = None):
+                       state_rows: Tensor | None = None, keep_ties: bool = False):
     sp = _lib.SampleParamsC()
+    sp.keep_ties = 1 if keep_ties else 0
     sp.state_rows = state_rows.data_ptr() if state_rows is not None else None
     sp.temperature = float(temperature)
     sp.top_k = int(top_k) if top_k is not None else 0
@@ -245,11 +251,36 @@ class Decoder:
         self.n_kv_heads = m.kv_heads
         self.head_dim = m.head_dim
         self.n_layers = m.n_layers
-        if m.global_every is not None or m.global_rope_dim is not None or m.global_rope_theta is not None:
-            raise NotImplementedError("separate global-attention layers are not supported by the native step")
         rope_dim = m.rope_dim or m.head_dim
         self.freqs_cis = precompute_freqs_cis(rope_dim, max_seqlen, m.rope_theta,
                                               m.rope_theta_rescale_factor).to(model.device)
+
+        # Global-attention layers (src/vui/model.py:406-468): without a window every layer is global; with one,
+        # the last layer and every global_every-th are.  Global layers attend over the whole cache and may rotate
+        # with a table of their own (other width and/or base; the base defaults to theta * max_seqlen / window).
+        def _is_global(idx: int) -> bool:
+            if m.window_size is None:
+                return True
+            if m.global_every is not None:
+                if idx == m.n_layers - 1 or (idx + 1) % m.global_every == 0:
+                    return True
+            return False
+
+        self.block_is_global = [_is_global(i) for i in range(m.n_layers)]
+        g_dim = m.global_rope_dim or rope_dim
+        if m.global_rope_theta is not None:
+            g_theta = m.global_rope_theta
+        elif m.window_size is not None and any(self.block_is_global):
+            g_theta = m.rope_theta * (max_seqlen / m.window_size)
+        else:
+            g_theta = m.rope_theta
+        self.global_rope_dim = g_dim
+        self.freqs_cis_global = None
+        if g_dim != rope_dim or g_theta != m.rope_theta:
+            if g_dim > m.head_dim:
+                raise ValueError(f"global_rope_dim={g_dim} exceeds head_dim={m.head_dim}")
+            self.freqs_cis_global = precompute_freqs_cis(g_dim, max_seqlen, g_theta,
+                                                         m.rope_theta_rescale_factor).to(model.device)
         self.flash_kv_caches: list[FlashKVCache] | None = None
         self._k = self._v = None
         self._prefill_scratch: dict[int, Tensor] = {}  # one buffer per lane (stream) that ingests prompts
@@ -430,7 +461,7 @@ class RQTransformer:
         self._gkv_logit_bias.zero_()
         if logit_bias is not None:
             self._gkv_logit_bias[: logit_bias.size(0)].copy_(logit_bias)
-        key = (B, Q, float(temperature))
+        key = (B, Q, float(temperature), int(self.seed), self._gkv_top_k)  # everything a captured launch bakes in
         g = self._gkv_graphs.get(key)
         if g is None:
             sp = make_sample_params(temperature, self._gkv_top_k, self.seed, self._ctr)
