@@ -66,6 +66,7 @@ struct vui_ctx {
   void* pf_w;     // projection weights of every layer in the prefill GEMMs' operand layout (bf16 contexts)
   void* rq_tw;    // the depth head's matrices in the batched kernel's operand layout
   vui_weights* wdev_t;  // device copy of the weight table with those matrices' pointers
+  void* rq_ks;          // depth-head keys of the one-launch kernel when they do not fit in LDS (a region per workgroup)
   int fused_ok, fused_on, nwg, ns;
   int fused_bb_ok;      // the backbone step alone can run as the one-launch kernel (its LDS need is smaller)
   size_t lds_bytes, lds_bb;
@@ -148,6 +149,7 @@ static size_t carve(const vui_config* c, int Bm, vui_ctx* x) {
   TAKE(pf_w, void*, prefill_weight_bytes(*c));  // empty when the configuration has no prefill pass
   TAKE(rq_tw, void*, rq_batch_weight_bytes(*c, FUSED_NWG));  // empty when the batched depth-head kernel is unavailable
   TAKE(wdev_t, vui_weights*, sizeof(vui_weights));
+  TAKE(rq_ks, void*, frame_rq_key_scratch_bytes(*c, FUSED_NWG));
 #undef TAKE
   return cv.off;
 }
@@ -297,7 +299,8 @@ static void fused_base(vui_ctx* ctx, FrameArgs& a) {
   a.global_layers = c.global_layers; a.global_rope_dim = c.global_rope_dim;
   a.ll = ctx->ll; a.epoch = ctx->ctl; a.arrive = ctx->ctl + 1; a.err = ctx->ctl + 2;
   a.prof = ctx->prof; a.prof_cap = ctx->prof_cap; a.prof_wg = ctx->prof_wg;
-  a.ns = ctx->ns; a.lds_kv_off = (int)(ctx->lds_bytes - frame_rq_cache_bytes(c));
+  a.ns = ctx->ns; a.lds_kv_off = (int)(ctx->lds_bytes - frame_rq_lds_cache_bytes(c));
+  a.rq_kg = frame_rq_keys_global(c); a.rq_kscratch = (uint16_t*)ctx->rq_ks;
 }
 static bool use_fused(vui_ctx* ctx, int B) { return ctx->fused_ok && ctx->fused_on && B == 1; }
 

@@ -102,7 +102,7 @@ __device__ __forceinline__ void gemv_prefetch(const bf16_t* W, const bf16_t* W2,
 template <int MAXC, bool DUAL, typename Epi>
 __device__ __forceinline__ void gemv_compute(const uint32_t* xp, const Plan& p, const WRegs<MAXC, DUAL>& r, float* red,
                                              Epi&& epi) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;  // the wave index as a scalar
   float res[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
   uint4 x[MAXC];
   if (p.nslots > 0) {
@@ -197,19 +197,19 @@ __device__ __forceinline__ void stage_norm(const float* src, const NormW& nw, fl
 // workgroup barriers that separate them from earlier readers and later users of dst.
 __device__ __forceinline__ void poll_words(uint32_t* dst, const uint64_t* buf, int nwords, Ctl& c) {
   __syncthreads();
-  ll_poll(buf, nwords, c, [&](int i, uint32_t v) { dst[i] = v; });
+  ll_poll_auto(buf, nwords, c, [&](int i, uint32_t v) { dst[i] = v; });
   __syncthreads();
 }
 __device__ __forceinline__ void poll_set(float* dst, const uint64_t* buf, int nwords, Ctl& c) {
   __syncthreads();
-  ll_poll(buf, nwords, c, [&](int i, uint32_t v) {
+  ll_poll_auto(buf, nwords, c, [&](int i, uint32_t v) {
     *reinterpret_cast<float2*>(dst + 2 * i) = make_float2(bf_lo(v), bf_hi(v)); });
   __syncthreads();
 }
 // dst = rnd(dst + incoming): the residual add (src/vui/model.py:367, 374)
 __device__ __forceinline__ void poll_add(float* dst, const uint64_t* buf, int nwords, Ctl& c) {
   __syncthreads();
-  ll_poll(buf, nwords, c, [&](int i, uint32_t v) {
+  ll_poll_auto(buf, nwords, c, [&](int i, uint32_t v) {
     const float2 o = *reinterpret_cast<const float2*>(dst + 2 * i);
     const uint32_t pk = f2bf2(o.x + bf_lo(v), o.y + bf_hi(v));
     *reinterpret_cast<float2*>(dst + 2 * i) = make_float2(bf_lo(pk), bf_hi(pk)); });
@@ -269,6 +269,9 @@ __device__ __forceinline__ void load_logits8(const uint32_t* lgw, int E, int CS,
 
 struct LayerP { const bf16_t *attn_norm, *wqkv, *wo, *mlp_norm, *w1, *w3, *w2; };
 
+// KG: the depth head's keys live in a per-workgroup global scratch area instead of LDS (see below); a compile-time
+// switch, so that the common form pays nothing for it.
+template <bool KG>
 __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   float* xres = (float*)(smem + LDS_XRES);
@@ -284,7 +287,8 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
   LayerP* lp = (LayerP*)(smem + LDS_FIXED);          // backbone layers, then depth-head layers
   bf16_t* rqkv = (bf16_t*)(smem + a.lds_kv_off);
 
-  const int wg = blockIdx.x, nwg = gridDim.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  // the wave index as a scalar: what depends on it alone (row plans, roles) is then scalar work and scalar branches
+  const int wg = blockIdx.x, nwg = gridDim.x, tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   // a streamed turn that has met its end-of-turn test: steps enqueued ahead of the host's knowledge do nothing
   // (the flag was written by an earlier launch or by the host, so every workgroup reads the same value)
   if (a.stop_state && a.stop_state[0] != 0) return;
@@ -774,7 +778,15 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
     // attention lane layout: QP key slots x PP feature parts per wave
     const int QP8 = (Q + 7) & ~7;
     // values of positions not yet written this frame are multiplied by weight zero: they must be finite
-    for (int i = tid; i < (a.rqL * 2 * R * QP8) / 8; i += FR_THREADS) reinterpret_cast<uint4*>(rqkv)[i] = make_uint4(0, 0, 0, 0);
+    // Keys in global memory (kg): a depth head whose keys AND values do not fit beside the rest in LDS keeps the
+    // values there (they are read once per position and feature by every lane) and the keys of earlier positions in
+    // a global scratch area of this workgroup alone (written and read by the same CU, so plain stores and loads);
+    // the key of the running position stays in a small LDS buffer.
+    constexpr bool kg = KG;
+    const int lds_cache_elems = kg ? a.rqL * R * QP8 + R : a.rqL * 2 * R * QP8;
+    for (int i = tid; i < lds_cache_elems / 8; i += FR_THREADS) reinterpret_cast<uint4*>(rqkv)[i] = make_uint4(0, 0, 0, 0);
+    bf16_t* knew = rqkv + (size_t)a.rqL * R * QP8;  // kg only: the running position's key, chunk-major [R/8][8]
+    bf16_t* kglob = a.rq_kscratch + (size_t)wg * a.rqL * R * QP8;
     int PP = Q <= 16 ? 4 : (Q <= 32 ? 2 : 1);
     while (PP > 1 && ((rhd % PP) || ((rhd / PP) & 1))) PP >>= 1;
     const int fpp = rhd / PP;  // features per part, even
@@ -817,8 +829,9 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
         // depth-head cache of this layer in LDS, QP8 = Q rounded up to 8 positions:
         //   keys    [R/8 chunks][QP8 positions][8 features]   (a lane group reads one position per lane: no bank conflicts)
         //   values  [R features][QP8 positions]               (one feature's values over the positions are contiguous)
-        bf16_t* kcache = rqkv + (size_t)l * 2 * R * QP8;
-        bf16_t* vcache = kcache + (size_t)R * QP8;
+        bf16_t* kcache = rqkv + (size_t)l * 2 * R * QP8;  // LDS form
+        bf16_t* vcache = kg ? rqkv + (size_t)l * R * QP8 : kcache + (size_t)R * QP8;
+        bf16_t* kcache_g = kglob + (size_t)l * R * QP8;   // global form, same [R/8][QP8][8] layout
         // ---- A: QKV ----
         const RepBuf qkvb = rep_alloc(llp, 3 * R / 2);
         {
@@ -843,12 +856,17 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           const Plan R_o = plan_of(m_o, R, wg, nwg, wave);
           if (!kv_only) gemv_prefetch<2, false>(Lw.wo, nullptr, R, R_o, wr);
           __syncthreads();  // xn (A's input) fully consumed before q overwrites it
-          ll_poll(rep_rd(qkvb), 3 * R / 2, c, [&](int i, uint32_t v) {
+          ll_poll_auto(rep_rd(qkvb), 3 * R / 2, c, [&](int i, uint32_t v) {
             const int n = 2 * i;
             if (n < R) xp[i] = v;  // q, packed
             else if (n < 2 * R) {   // new key: features n-R, n-R+1 of position t
               const int f = n - R;
-              *reinterpret_cast<uint32_t*>(kcache + ((size_t)(f >> 3) * QP8 + t) * 8 + (f & 7)) = v;
+              if (kg) {
+                *reinterpret_cast<uint32_t*>(knew + f) = v;  // [f >> 3][f & 7] = f
+                *reinterpret_cast<uint32_t*>(kcache_g + ((size_t)(f >> 3) * QP8 + t) * 8 + (f & 7)) = v;
+              } else {
+                *reinterpret_cast<uint32_t*>(kcache + ((size_t)(f >> 3) * QP8 + t) * 8 + (f & 7)) = v;
+              }
             } else {                // new value
               const int f = n - 2 * R;
               vcache[(size_t)f * QP8 + t] = (bf16_t)(v & 0xffff);
@@ -878,7 +896,9 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
                   const int f0 = hs[h] * rhd + part * fpp + 8 * i;
-                  kr[h] = *reinterpret_cast<const uint4*>(kcache + ((size_t)(f0 >> 3) * QP8 + kk) * 8);
+                  if (!kg) kr[h] = *reinterpret_cast<const uint4*>(kcache + ((size_t)(f0 >> 3) * QP8 + kk) * 8);
+                  else if (kk == t) kr[h] = *reinterpret_cast<const uint4*>(knew + f0);
+                  else kr[h] = *reinterpret_cast<const uint4*>(kcache_g + ((size_t)(f0 >> 3) * QP8 + kk) * 8);
                   qr[h] = *reinterpret_cast<const uint4*>(xp + f0 / 2);
                 }
 #pragma unroll
@@ -889,7 +909,10 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
                   const int f = hs[h] * rhd + part * fpp + 2 * i;
-                  dsum[h] = dot2_bf(*reinterpret_cast<const uint32_t*>(kcache + ((size_t)(f >> 3) * QP8 + kk) * 8 + (f & 7)), xp[f / 2], dsum[h]);
+                  const uint32_t kw = !kg ? *reinterpret_cast<const uint32_t*>(kcache + ((size_t)(f >> 3) * QP8 + kk) * 8 + (f & 7))
+                                      : (kk == t ? *reinterpret_cast<const uint32_t*>(knew + f)
+                                                 : *reinterpret_cast<const uint32_t*>(kcache_g + ((size_t)(f >> 3) * QP8 + kk) * 8 + (f & 7)));
+                  dsum[h] = dot2_bf(kw, xp[f / 2], dsum[h]);
                 }
             }
             float pw[2], Ls[2];
@@ -1110,6 +1133,7 @@ size_t frame_ll_words(const vui_config& c, int ns) {
   return total + 64;
 }
 
+size_t frame_prof_lds_bytes();
 static size_t frame_ptr_bytes(const vui_config& c) {
   return (((size_t)(c.n_layers + c.rq_layers) * sizeof(LayerP)) + 15) & ~(size_t)15;
 }
@@ -1117,8 +1141,22 @@ static size_t frame_ptr_bytes(const vui_config& c) {
 size_t frame_rq_cache_bytes(const vui_config& c) {
   return (size_t)c.rq_layers * ((c.n_quantizers + 7) & ~7) * 2 * c.rq_dim * 2;
 }
+// 1 when the keys of the depth head live in a per-workgroup global scratch area (its keys and values together do not
+// fit in LDS beside the rest, the values and one position's key do)
+int frame_rq_keys_global(const vui_config& c) {
+  return (size_t)LDS_FIXED + frame_ptr_bytes(c) + frame_rq_cache_bytes(c) + frame_prof_lds_bytes() > 160 * 1024 ? 1 : 0;
+}
+// the part of the depth-head cache kept in LDS
+size_t frame_rq_lds_cache_bytes(const vui_config& c) {
+  if (!frame_rq_keys_global(c)) return frame_rq_cache_bytes(c);
+  return (frame_rq_cache_bytes(c) / 2 + (size_t)c.rq_dim * 2 + 15) & ~(size_t)15;
+}
+size_t frame_rq_key_scratch_bytes(const vui_config& c, int nwg) {
+  if (c.dtype != VUI_DTYPE_BF16 || c.rq_layers < 1 || !frame_rq_keys_global(c)) return 0;
+  return (size_t)nwg * frame_rq_cache_bytes(c) / 2;
+}
 size_t frame_lds_bytes(const vui_config& c) {
-  return (size_t)LDS_FIXED + frame_ptr_bytes(c) + frame_rq_cache_bytes(c);
+  return (size_t)LDS_FIXED + frame_ptr_bytes(c) + frame_rq_lds_cache_bytes(c);
 }
 // launches that stop after the backbone step need no room for the depth head's keys and values
 size_t frame_lds_bytes_backbone(const vui_config& c) { return (size_t)LDS_FIXED + frame_ptr_bytes(c); }
@@ -1135,7 +1173,7 @@ bool frame_supported(const vui_config& c, int nwg, int ns, bool with_rq, char* w
   else if (c.rq_layers < 1 || c.rq_heads < 1) r = "no depth head";
   else if ((c.rq_dim / c.rq_heads) % 2 || c.rq_dim / c.rq_heads > 128) r = "depth-head head_dim must be even, at most 128";
   else if ((c.d_model | c.ffn | c.rq_dim | c.rq_ffn) & 7) r = "vector lengths must be multiples of 8";
-  else if (with_rq && frame_lds_bytes(c) > 160 * 1024) r = "depth-head keys/values do not fit in LDS";
+  else if (with_rq && frame_lds_bytes(c) > 160 * 1024) r = "depth-head values do not fit in LDS";
   else {
     const int np_max = (c.n_heads + 2 * c.n_kv_heads) * c.head_dim / 2;
     int m = np_max;
@@ -1163,11 +1201,12 @@ int frame_max_resident(size_t lds_bytes, int* n_cu) {
   if (lds_bytes > lds_attr) {
     // room for the optional phase-clock buffer where it fits
     const size_t want = lds_bytes + frame_prof_lds_bytes() <= 160 * 1024 ? lds_bytes + frame_prof_lds_bytes() : lds_bytes;
-    HIP_TRY(hipFuncSetAttribute((const void*)frame_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)want));
+    HIP_TRY(hipFuncSetAttribute((const void*)frame_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)want));
+    HIP_TRY(hipFuncSetAttribute((const void*)frame_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)want));
     lds_attr = lds_bytes;
   }
   int occ = 0;
-  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, frame_kernel, FR_THREADS, lds_bytes));
+  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, frame_kernel<true>, FR_THREADS, lds_bytes));
   if (n_cu) *n_cu = prop.multiProcessorCount;
   return occ * prop.multiProcessorCount;
 }
@@ -1179,7 +1218,8 @@ int launch_frame(const FrameArgs& a_in, int nwg, size_t lds_bytes, hipStream_t s
     if (lds_bytes + frame_prof_lds_bytes() > 160 * 1024) { vui_set_error("no LDS left for the phase clock"); return VUI_EINVAL; }
     lds_bytes += frame_prof_lds_bytes();
   }
-  hipLaunchKernelGGL(frame_kernel, dim3(nwg), dim3(FR_THREADS), lds_bytes, st, a);
+  if (a.rq_kg) hipLaunchKernelGGL(frame_kernel<true>, dim3(nwg), dim3(FR_THREADS), lds_bytes, st, a);
+  else hipLaunchKernelGGL(frame_kernel<false>, dim3(nwg), dim3(FR_THREADS), lds_bytes, st, a);
   HIP_TRY(hipGetLastError());
   return VUI_OK;
 }

@@ -192,6 +192,8 @@ struct FrameArgs {
   int ns;    // attention key splits per head
   int mode;  // FR_* bits
   int lds_kv_off;  // byte offset of the depth-head K/V store in LDS
+  int rq_kg;       // 1: depth-head keys in rq_kscratch (a region per workgroup), values in LDS
+  uint16_t* rq_kscratch;
   uint64_t* prof;  // optional (prof_cap + 1) words: (clock << 8 | tag) per phase point, count in the last word
   int prof_cap, prof_wg;
   int lds_prof_off;  // set by launch_frame: LDS offset of the stamp buffer
@@ -202,6 +204,9 @@ enum { FR_BACKBONE = 1, FR_CB0 = 2, FR_RQ = 4, FR_FINISH = 8 };
 size_t frame_ll_words(const vui_config& c, int ns);
 size_t frame_lds_bytes(const vui_config& c);
 size_t frame_rq_cache_bytes(const vui_config& c);
+size_t frame_rq_lds_cache_bytes(const vui_config& c);
+int frame_rq_keys_global(const vui_config& c);
+size_t frame_rq_key_scratch_bytes(const vui_config& c, int nwg);
 size_t frame_lds_bytes_backbone(const vui_config& c);
 bool frame_supported(const vui_config& c, int nwg, int ns, bool with_rq, char* why, size_t why_len);
 int frame_max_resident(size_t lds_bytes, int* n_cu);

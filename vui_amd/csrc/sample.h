@@ -98,7 +98,7 @@ template <int EMAX>
 __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32_t (&key)[EMAX], int low_bit, int CS,
                                             int E, bool greedy, int top_k, uint32_t rnd, uint32_t codebook,
                                             SampleShared& sh, int* hist, bool exact_k = false) {
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   SAMP_TS(0);
   const bool digits = top_k > 0 && top_k < CS && (low_bit == 16 || low_bit == 0) && !greedy;
   float m = -INFINITY; int mi = 0x7fffffff;
