@@ -28,7 +28,7 @@ __global__ __launch_bounds__(ATT_THREADS) void decode_attn_kernel(const AttnArgs
   __shared__ int s_last;
 
   const int b = blockIdx.z, h = blockIdx.y, sp = blockIdx.x;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, grp = lane >> 4, l16 = lane & 15;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, grp = lane >> 4, l16 = lane & 15;
   const int g = wave * 4 + grp;  // 0..15 key lane-group inside the workgroup
   const int hd = p.hd;
   const int slot = p.slot_idx ? p.slot_idx[b] : b;

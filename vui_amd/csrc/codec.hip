@@ -83,7 +83,7 @@ template <int TT, bool DB>
 __device__ __forceinline__ void cv_gemm_tile(const CvGemm& p, const int m0, const int t0, float* red,
                                              const int tile, const int part_idx) {
   constexpr int NU = Nu<TT, DB>::N;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int r16 = lane & 15, g = lane >> 4;
   const int G = p.Cin >> 5, Uall = p.taps * G;
   const int M = p.M, Cin = p.Cin;
@@ -336,7 +336,7 @@ __global__ __launch_bounds__(256) void cv_attn_kernel(const CvAttn p) {
   float* sc = q + p.hd;
   float* part = sc + p.max_seq;
   float* red = part + 4 * p.hd;
-  const int h = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int h = blockIdx.x, tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int hd = p.hd, half = hd >> 1, A = p.H * hd;
   const int pos = *p.ctr - 1;
   float* kh = p.kc + (size_t)h * p.max_seq * hd;
@@ -453,7 +453,7 @@ struct TrRows { float4 w[TR_MAXR][TR_MAXC]; };
 // rows r_lo + wave, r_lo + wave + 4, ... below r_hi of W (M x K): request them
 template <int MAXR, int MAXC>
 __device__ __forceinline__ void tr_prefetch(const float* W, int K, int r_lo, int r_hi, TrRows& rr) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
 #pragma unroll
   for (int i = 0; i < MAXR; ++i) {
     const int row = r_lo + wave + 4 * i;
@@ -468,7 +468,7 @@ __device__ __forceinline__ void tr_prefetch(const float* W, int K, int r_lo, int
 // dot products of those rows with xs (K floats in LDS); epi(row, sum) runs in every lane of the wave
 template <int MAXR, int MAXC, typename F>
 __device__ __forceinline__ void tr_compute(const float* xs, int K, int r_lo, int r_hi, const TrRows& rr, F&& epi) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
 #pragma unroll
   for (int i = 0; i < MAXR; ++i) {
     const int row = r_lo + wave + 4 * i;
@@ -507,7 +507,7 @@ __device__ __forceinline__ void tr_rows_qkv(int M, int wg, int nwg, int H, int& 
 }
 
 __device__ __forceinline__ float tr_rstd(const float* x, int n, float eps, float* red) {
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   float ss = 0.f;
   for (int i = tid; i < n; i += FR_THREADS) ss = fmaf(x[i], x[i], ss);
   ss = wave_sum(ss);
@@ -526,7 +526,7 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
   float* sc = q + 64;  // max_seq + 192: scores, and before them the raw q | k | v of the head
   float* part = sc + a.max_seq + 192;
   float* red = part + 4 * 64;
-  const int wg = blockIdx.x, nwg = gridDim.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int wg = blockIdx.x, nwg = gridDim.x, tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   Ctl c;
   ctl_begin(c, a.epoch, a.lerr);
   const uint32_t ep = c.epoch;
@@ -826,7 +826,7 @@ struct CvDwLn {
 
 __global__ __launch_bounds__(256) void cv_dwln_kernel(const CvDwLn p) {
   __shared__ float red[8];
-  const int t = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int t = blockIdx.x, tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int f = *p.ctr - 1, base = ring_base(p.in, f);
   float v[DW_MAXC];
   float s = 0.f;

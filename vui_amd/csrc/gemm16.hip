@@ -175,7 +175,7 @@ __global__ __launch_bounds__(G16_THREADS) void gemm16_kernel(const GemvArgs p) {
   const int K = p.K, KP = K + 8;
   bf16_t* xs = (bf16_t*)smem16;                       // 16 x KP
   float* red = (float*)(smem16 + (size_t)16 * KP * 2);  // 4 waves x 64 lanes x (4 | 8)
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int f16 = lane & 15, kg = lane >> 4;
   const int n0 = (int)blockIdx.x * 16;
   const int row = min(n0 + f16, p.N - 1);

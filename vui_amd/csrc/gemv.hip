@@ -52,7 +52,7 @@ template <> struct WL<int8_t> {
 // activations (B, K) -> LDS fp32, with the two-rounding RMSNorm when norm_w is given
 template <typename T>
 __device__ __forceinline__ void stage_x(const GemvArgs& p, float* xs, int nb) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, nw = blockDim.x >> 6;
   const T* x = (const T*)p.x;
   const T* nw_ = (const T*)p.norm_w;
   for (int b = wave; b < nb; b += nw) {
@@ -78,7 +78,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(const GemvArgs p, co
   // N == 0: only the extra outputs are wanted (the matrix cores did the rest); one row per workgroup then,
   // instead of one workgroup walking through eight rows
   const int b0 = p.N == 0 ? (int)blockIdx.x : b0_in, nb_rt = p.N == 0 ? 1 : nb_in;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int nch = p.K >> 3;
   const int nmain = (p.N + 2 * RPW - 1) / (2 * RPW);
   GemvArgs q = p;  // batch tile view

@@ -63,7 +63,7 @@ __global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf1
   constexpr int TILE = 1024;  // floats of one partial tile
   constexpr int PW = (DUAL ? 2 : 1) * TILE;
   __shared__ float part[4 * PW];
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int l16 = lane & 15, kg = lane >> 4;
   const int MT = (p.M + 31) >> 5;
   const int id = blockIdx.x;
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(64 * PF_ATT_WAVES) void pf_attn_kernel(const bf16_t
   constexpr int HD = 32 * HD32, DT = 2 * HD32;
   __shared__ float s_acc[PF_ATT_WAVES][DT * 256];
   __shared__ float s_m[PF_ATT_WAVES][16], s_l[PF_ATT_WAVES][16];
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int l16 = lane & 15, kg = lane >> 4;
   const int q0 = blockIdx.x * 16, h = blockIdx.y, kvh = h / gsz;
   const int ldq = nq + 2 * nkv;

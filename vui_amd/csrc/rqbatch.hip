@@ -49,7 +49,7 @@ struct TileW { uint4 a[MAXS]; uint4 b[DUAL ? MAXS : 1]; };
 // about a quarter of the rate.  A band starts where it does in the row-major form (16 rows x K elements each).
 template <int MAXS, bool DUAL>
 __device__ __forceinline__ void tile_prefetch(const bf16_t* W, const bf16_t* W2, const Tile& t, TileW<MAXS, DUAL>& r) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (!t.on) return;
   const size_t band = (size_t)t.n0 * t.K + lane * 8;  // n0 is a multiple of 16, N as well: the band is inside the matrix
 #pragma unroll
@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void rb_tile_kernel(const bf16_t* __restrict__
 template <int MAXS, bool DUAL, typename Epi>
 __device__ __forceinline__ void tile_compute(const uint32_t* xp, int xs, const Tile& t, const TileW<MAXS, DUAL>& r, float* red,
                                              int B, Epi&& epi) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l16 = lane & 15, kg = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, l16 = lane & 15, kg = lane >> 4;
   if (!t.on) return;  // uniform over the workgroup
   rb_floatx4 acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -117,7 +117,7 @@ __device__ __forceinline__ void tile_compute2(const uint32_t* xp, int xs, const 
                                               const TileW<MAXS, DUAL>& r1, float* red, int B, Epi&& epi) {
   if (!t0.on) return;  // uniform over the workgroup; t1 is never on without t0
   if (!t1.on) { tile_compute<MAXS, DUAL>(xp, xs, t0, r0, red, B, epi); return; }
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l16 = lane & 15, kg = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, l16 = lane & 15, kg = lane >> 4;
   rb_floatx4 a0 = {0.f, 0.f, 0.f, 0.f}, a0b = a0, a1 = a0, a1b = a0;
 #pragma unroll
   for (int i = 0; i < MAXS; ++i) {
@@ -169,7 +169,7 @@ __device__ __forceinline__ NormRegs load_norm(const bf16_t* nw, int R) {
 }
 // two-rounding RMSNorm of the B rows of xres (fp32, row stride R) into xp (packed bf16); wave w takes rows w, w+4, ...
 __device__ __forceinline__ void norm_rows(const float* xres, const NormRegs& nw, float eps, int R, int B, uint32_t* xp, int xs) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   for (int b = wave; b < B; b += 4) {
     const float* x = xres + (size_t)b * R;
     float4 q[2][2];
@@ -208,7 +208,7 @@ __device__ __forceinline__ void norm_rows(const float* xres, const NormRegs& nw,
 // no barrier stands between the wait, the add and the norm.  buf: the group's rows, R/2 words each.
 __device__ __forceinline__ void poll_add_norm_rows(const uint64_t* buf, Ctl& c, float* xres, const NormRegs& nw, float eps, int R,
                                                    int B, uint32_t* xp, int xs) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int nch = R / 8;
   const int NI = nch > WAVE ? 2 : 1;  // chunks per lane
   for (int b = wave; b < B; b += 4) {
@@ -314,7 +314,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
   bf16_t* pw_lo = pw_hi + 64;
   bf16_t* kvbase = (bf16_t*)(smem + a.off_kv);
 
-  const int wg = blockIdx.x, nwg = gridDim.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int wg = blockIdx.x, nwg = gridDim.x, tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int B = a.B, R = a.R, d = a.d, CS = a.CS, Q = a.Q, xs = a.xs;
   const int rhd = R / a.rqH, QP8 = (Q + 7) & ~7;
   Ctl c;
