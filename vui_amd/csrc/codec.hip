@@ -541,7 +541,7 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
   auto take = [&](int n) { uint64_t* p = ll; ll += n; return p; };
   auto put = [&](uint64_t* buf, int i, float v) { ll_st(buf + i, __float_as_uint(v), ep); };
   auto get = [&](const uint64_t* buf, int n, float* dst) {
-    ll_poll(buf, n, c, [&](int i, uint32_t v) { dst[i] = __uint_as_float(v); });
+    ll_poll_auto(buf, n, c, [&](int i, uint32_t v) { dst[i] = __uint_as_float(v); });
     __syncthreads();
   };
   TrRows rr;
@@ -589,7 +589,7 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
   }
   __syncthreads();  // xs is free again
   for (int i = tid; i < 2 * V; i += FR_THREADS) xs[i] = *ring_ptr(a.pre_in, pbase, i % V, i / V);
-  ll_poll(b_y1, V, c, [&](int i, uint32_t v) { xs[2 * V + i] = __uint_as_float(v); });
+  ll_poll_auto(b_y1, V, c, [&](int i, uint32_t v) { xs[2 * V + i] = __uint_as_float(v); });
   __syncthreads();
   uint64_t* b_pre = take(L);
   tr_compute<1, TR_MAXC>(xs, 3 * V, lo, hi, rr, [&](int row, float s) { if (lane == 0) put(b_pre, row, s + a.bpre[row]); });
@@ -750,7 +750,7 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
     tr_rows(mlp, wg, nwg, glo, ghi);  // channels; rows 2i, 2i + 1 are gate_i, up_i
     glo *= 2; ghi *= 2;
     tr_prefetch<TR_MAXR, 2>(W.Wgu, D, glo, ghi, rr);
-    ll_poll(b_o, D, c, [&](int i, uint32_t v) { x[i] += asc_r[i / FR_THREADS] * __uint_as_float(v); });
+    ll_poll_auto(b_o, D, c, [&](int i, uint32_t v) { x[i] += asc_r[i / FR_THREADS] * __uint_as_float(v); });
     // ---- gate / up rows interleaved: channel i = silu(gate_i) * up_i ----
     const float r2 = tr_rstd(x, D, a.eps, red);
     uint64_t* b_h = take(mlp);
@@ -779,7 +779,7 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
       tr_rows(L, wg, nwg, plo, phi);
       tr_prefetch<1, 2>(a.Wout, D, plo, phi, rr);
     }
-    ll_poll(b_d, D, c, [&](int i, uint32_t v) { x[i] += msc_r[i / FR_THREADS] * __uint_as_float(v); });
+    ll_poll_auto(b_d, D, c, [&](int i, uint32_t v) { x[i] += msc_r[i / FR_THREADS] * __uint_as_float(v); });
   }
   // ---- final norm (folded) + output_proj ----
   const float r3 = tr_rstd(x, D, a.eps, red);

@@ -390,7 +390,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
       });
       if (active) {
         __syncthreads();
-        ll_poll(x0 + (size_t)b0 * (R / 2), Bg * (R / 2), c, [&](int i, uint32_t v) {
+        ll_poll_auto(x0 + (size_t)b0 * (R / 2), Bg * (R / 2), c, [&](int i, uint32_t v) {
           const int lr = div_small(i, inv_r2), j = i - lr * (R / 2);
           *reinterpret_cast<float2*>(xres + (size_t)lr * R + 2 * j) = make_float2(bf_lo(v), bf_hi(v));
         });
@@ -419,7 +419,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
       if (t == 1) {
         if (tid < Bg) { int64_t cc = a.code0[b0 + tid]; codes_s[tid] = (int)(cc < 0 ? 0 : (cc >= CS ? CS - 1 : cc)); }
       } else {
-        ll_poll(codebuf + b0, Bg, c, [&](int i, uint32_t v) { codes_s[i] = (int)v; });
+        ll_poll_auto(codebuf + b0, Bg, c, [&](int i, uint32_t v) { codes_s[i] = (int)v; });
       }
       __syncthreads();
       for (int i = tid; i < Bg * (R / 8); i += FR_THREADS) {
@@ -537,7 +537,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
         TileW<8, false> wr;
         tile_prefetch<8, false>((const bf16_t*)Lw.wo, nullptr, to, wr);
         __syncthreads();
-        ll_poll(attb + (size_t)(b0 + out_r0) * (R / 2), out_nr * (R / 2), c, [&](int i, uint32_t v) {
+        ll_poll_auto(attb + (size_t)(b0 + out_r0) * (R / 2), out_nr * (R / 2), c, [&](int i, uint32_t v) {
           const int lr = div_small(i, inv_r2), j = i - lr * (R / 2);
           xp[(size_t)lr * xs + j] = v;
         });
@@ -582,7 +582,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
         TileW<16, false> wr;
         tile_prefetch<16, false>((const bf16_t*)Lw.w2, nullptr, tw, wr);
         __syncthreads();
-        ll_poll(hb + (size_t)(b0 + out_r0) * (a.rqF / 2), out_nr * (a.rqF / 2), c, [&](int i, uint32_t v) {
+        ll_poll_auto(hb + (size_t)(b0 + out_r0) * (a.rqF / 2), out_nr * (a.rqF / 2), c, [&](int i, uint32_t v) {
           const int lr = div_small(i, inv_f2), j = i - lr * (a.rqF / 2);
           xp[(size_t)lr * xs + j] = v;
         });
@@ -624,7 +624,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
         uint32_t* lgw = xp;
         const uint32_t rnd = philox_u32(a.seed, frame, (uint32_t)b, (uint32_t)t, 0u);  // ahead of the wait
         __syncthreads();
-        ll_poll(lgb + (size_t)b * (CS / 2), CS / 2, c, [&](int i, uint32_t v) { lgw[i] = v; });
+        ll_poll_auto(lgb + (size_t)b * (CS / 2), CS / 2, c, [&](int i, uint32_t v) { lgw[i] = v; });
         __syncthreads();
         const int E = (CS + FR_THREADS - 1) / FR_THREADS;
         const bool greedy = (a.topk == 1) || !(a.temp > 0.f);
