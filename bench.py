@@ -118,8 +118,8 @@ def gpu_bench(args):
 # see profiles/frame_kernel_e2e_b1.txt.  None until measured.
 # MFMA busy cycles / busy cycles of the 16-stream step's matrix-core kernels, from rocprofv3 --pmc
 # SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CYCLES; see profiles/e2e_b16_int8_step_kernels.txt.
-MEASURED_B16_MFMA_BUSY = {"gemm16_kernel": [0.08, 0.16], "rq_batch_kernel": 0.30}
-MEASURED_TRAFFIC_BYTES = 517_680_951  # at cache length 596..651 (algorithmic 414.6 MB there): 1.25 x
+MEASURED_B16_MFMA_BUSY = {"gemm16_kernel": [0.08, 0.16], "rq_batch_kernel": 0.49}
+MEASURED_TRAFFIC_BYTES = 522_142_720  # at cache length 577..682 (algorithmic 413.7 MB there): 1.26 x
 
 
 def kernel_roofline(out, fb):

@@ -136,8 +136,9 @@ int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream);
  * or int8 weights, as a sequence of kernels.  vui_ctx_fused(ctx, enable): enable = 1/0 switches the
  * fused form on/off, -1 only queries; returns 1 when the fused form will be used, else 0 (then
  * vui_last_error() says why it is unavailable).  The answer is about a whole frame (vui_frame_step,
- * vui_rq_generate): when only the depth head's keys and values are too large for the fused form,
- * vui_backbone_step alone still takes it, under the same switch.  No counterpart in the reference. */
+ * vui_rq_generate).  A depth head whose keys and values for one frame do not both fit in a compute unit's
+ * local memory keeps its keys in the workspace and is still fused; when even its values alone do not fit,
+ * vui_backbone_step alone still takes the fused form, under the same switch.  No counterpart in the reference. */
 int vui_ctx_fused(vui_ctx* ctx, int enable);
 /* 1 when the depth head of 2..16 rows runs as one persistent kernel (bf16, enough resident workgroups, the
  * fused form switched on), else 0 and vui_last_error() says why.  No counterpart in the reference. */
