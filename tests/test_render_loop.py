@@ -302,7 +302,10 @@ def test_prefill_segments_and_user_turn_layout():
 
 
 @pytest.mark.gpu
-def test_stream_frames_equals_oracle():
+@pytest.mark.parametrize("compile_rq", [False, True])
+def test_stream_frames_equals_oracle(compile_rq):
+    """compile_rq: the depth head through generate_kv_compilable (the entry the reference compiles) instead of the
+    captured graphs; same kernels, same frames."""
     from vui_amd.engine import Chunk
     from vui_amd.inference import InferenceState, render_codes_stream, stream_frames
 
@@ -317,7 +320,8 @@ def test_stream_frames_equals_oracle():
     from tests.util import make_model
 
     model = make_model(d, sd, torch.float32, max_seqlen=400)
-    state = InferenceState(model, rq_top_k=1)  # the depth-head graphs bake their top-k in; 1 = greedy, as the oracle run
+    # the depth-head graphs bake their top-k in; 1 = greedy, as the oracle run
+    state = InferenceState(model, rq_top_k=1, compile_rq=compile_rq, chunk_frames=7, ctx_frames=3, codec_graphs=True)
     chunks = [Chunk(emb=e[None].cuda(), n_words=w) for e, w in ch]
     got = [(f.cpu(), t) for f, t in stream_frames(state, chunks, eos_threshold=thr, **kw)]
     assert len(got) == len(ref)

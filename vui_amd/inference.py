@@ -31,9 +31,17 @@ class InferenceState:
     """Graphs and the position pointer of one stream (InferenceState, src/vui/inference.py:140-345).  The
     vocoder part of the reference's class (codec chunk graphs) lives in vui_amd.codec."""
 
-    def __init__(self, model: Vui, codec=None, sq_scores=None, wps_score: float = 1.0, rq_top_k: int = 100):
+    def __init__(self, model: Vui, codec=None, chunk_frames: int = 7, ctx_frames: int = 3, sq_scores=None,
+                 wps_score: float = 1.0, codec_graphs: bool = True, compile_rq: bool = False, rq_top_k: int = 100):
+        """Same arguments as the reference's (inference.py:143-166).  chunk_frames / ctx_frames / codec_graphs
+        belong to its chunked vocoder graphs and are kept for callers that pass them (the vocoder here streams
+        frame by frame); compile_rq selects generate_kv_compilable, which runs the same kernels."""
         self.model = model
         self.codec = codec
+        self.chunk_frames = chunk_frames
+        self.ctx_frames = ctx_frames
+        self._codec_graphs = codec_graphs
+        self._compile_rq = compile_rq
         self.device = model.device
         self.dtype = model.dtype
         self.offset = 0
@@ -47,8 +55,14 @@ class InferenceState:
     def _setup_graphs(self) -> None:
         """src/vui/inference.py:169-197: the one-slot backbone step graph and the depth-head graphs."""
         self.model.setup_decode_graph()
-        self.model.rq_transformer.setup_cuda_graph_kv(self.device, self.dtype, top_k=self._rq_top_k)
-        self._rq_generate = self.model.rq_transformer.generate_cuda_graph_kv
+        rq = self.model.rq_transformer
+        rq.setup_cuda_graph_kv(self.device, self.dtype, top_k=self._rq_top_k)
+        if self._compile_rq:
+            top_k = self._rq_top_k
+            self._rq_generate = lambda hidden, code0, temperature, bias: rq.generate_kv_compilable(
+                hidden, code0, temperature, bias, top_k)
+        else:
+            self._rq_generate = rq.generate_cuda_graph_kv
 
     def reset(self) -> None:
         self.rewind(0)

@@ -432,6 +432,15 @@ class RQTransformer:
             self._ctr.add_(1)  # a new draw index per call (and per 16-row chunk of a large batch)
         return out
 
+    def generate_kv_compilable(self, backbone_hidden: Tensor, code_0: Tensor, temperature, logit_bias: Tensor,
+                               top_k: int = 100) -> Tensor:
+        """The entry the reference hands to torch.compile (src/vui/model.py:730-811; temperature as a tensor,
+        logit_bias always given, top_k a Python int).  There is no compiler here: it is the eager form on the same
+        kernels, and a temperature tensor is read on the host (one synchronisation per distinct call site; callers
+        in a loop pass a float, as InferenceState's wrapper does)."""
+        t = float(temperature.item()) if isinstance(temperature, Tensor) else float(temperature)
+        return self.generate(backbone_hidden, code_0, t, top_k, logit_bias)
+
     def setup_cuda_graph_kv(self, device, dtype=torch.bfloat16, top_k: int = 100, pool=None,
                             batch_sizes: tuple[int, ...] = (1,)):
         """Static buffers for graph replay at the given batch sizes (src/vui/model.py:814-881).
