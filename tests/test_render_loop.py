@@ -337,3 +337,43 @@ def test_stream_frames_equals_oracle(compile_rq):
     assert state.rewind() == int(om.seq_lens[0])
     with pytest.raises(NotImplementedError):
         next(stream_frames(state, chunks, top_p=0.9))
+
+
+@pytest.mark.gpu
+def test_render_audio_stream_schedule_and_samples():
+    """Audio emissions of inference.render_audio_stream: first after `first_chunk_frames`, then every `chunk_frames`,
+    flushed at a turn's end; concatenated they are the vocoder oracle's streaming decode of the frames that
+    stream_frames yields for the same arguments."""
+    import dataclasses
+
+    from oracle import codec_oracle as CO
+    from tests.util import make_model
+    from vui_amd.codec import CodecConfig, QwenCodecDecoder
+    from vui_amd.engine import Chunk
+    from vui_amd.inference import InferenceState, render_audio_stream, stream_frames
+
+    d, sd = _model()
+    ch = _chunks(d, 2)
+    cd = CO.CodecDims(n_codebooks=d.n_quantizers, codebook_size=d.codebook_size, codebook_dim=16, vq_dim=32, latent_dim=64,
+                      d_model=32, n_layers=2, n_heads=2, head_dim=16, mlp_dim=64, max_seq=130, up_ratios=(2, 2),
+                      decoder_dim=128, rates=(3, 2))
+    csd = CO.synthetic_codec_state_dict(cd, seed=4)
+    dec = QwenCodecDecoder(csd, CodecConfig(**dataclasses.asdict(cd)), device="cuda")
+    model = make_model(d, sd, torch.float32, max_seqlen=400)
+    state = InferenceState(model, dec, rq_top_k=1)
+    chunks = [Chunk(emb=e[None].cuda(), n_words=w) for e, w in ch]
+    kw = dict(top_k=1, eos_threshold=2.0, max_turn_secs=1.0)  # no end-of-turn inside the cap: 12 frames per turn
+    frames = [(f.cpu(), t) for f, t in stream_frames(state, chunks, **kw)]
+    per_turn = int(1.0 * 12.5)
+    assert len(frames) == 2 * per_turn
+    audio = [a.cpu() for a in render_audio_stream(state, chunks, chunk_frames=5, first_chunk_frames=2, **kw)]
+    # turn 1: 2, 5, then the flush of 5; turn 2: 5, 5, flush of 2
+    assert [a.shape[-1] // cd.hop for a in audio] == [2, 5, 5, 5, 5, 2]
+    ora = CO.CodecDecoderOracle(cd, csd)
+    ora.open_stream()
+    ref = torch.cat([ora.forward(f.view(1, -1, 1)) for f, _ in frames], dim=-1)
+    ora.close_stream()
+    got = torch.cat(audio, dim=-1)
+    assert got.shape == ref.shape and float((got - ref).abs().max()) < 2e-4
+    with pytest.raises(RuntimeError):
+        next(render_audio_stream(InferenceState(model, None, rq_top_k=1), chunks, **kw))

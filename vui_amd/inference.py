@@ -222,3 +222,34 @@ def render_codes_stream(state: InferenceState, chunks: "list[Chunk]", **kwargs):
         if turn_end is not None:
             yield torch.stack(pending), turn_end
             pending = []
+
+
+def render_audio_stream(state: InferenceState, chunks: "list[Chunk]", *, chunk_frames: int | None = None,
+                        ctx_frames: int | None = None, first_chunk_frames: int | None = None, **kwargs):
+    """Low-latency audio: consumes `stream_frames` and yields audio (1, 1, n * hop) every `chunk_frames` frames
+    (the first emission after `first_chunk_frames`), flushing at a turn's end (src/vui/inference.py:761-830).
+
+    The reference decodes each emission offline from its frames plus `ctx_frames` of context and cuts the context
+    off; the vocoder here streams (its convolution and attention state carries the whole history), so every frame
+    is decoded once, in order, and an emission is the concatenation of its frames' audio: the same schedule and the
+    same number of samples, without the seam the context window approximates.  `ctx_frames` is accepted for
+    callers that pass it."""
+    from .codec import CodecCtx
+
+    if state.codec is None:
+        raise RuntimeError("render_audio_stream() needs InferenceState(codec=...)")
+    chunk_size = chunk_frames if chunk_frames is not None else state.chunk_frames
+    first_size = first_chunk_frames if first_chunk_frames is not None else chunk_size
+    ctx = getattr(state, "_codec_ctx", None)
+    if ctx is None:
+        ctx = state._codec_ctx = CodecCtx(state.codec)
+    pending: list[Tensor] = []  # audio of the frames not yet emitted
+    have_emitted_first = False
+    for frame, turn_end in stream_frames(state, chunks, **kwargs):
+        pending.append(ctx.decode_frame(frame.view(1, -1, 1)).clone())
+        target = chunk_size if have_emitted_first else first_size
+        if turn_end is not None or len(pending) >= target:
+            yield torch.cat(pending, dim=-1)
+            pending = []
+            have_emitted_first = True  # the first-chunk size applies to the first emission of the call only
+
