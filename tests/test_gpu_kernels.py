@@ -54,9 +54,12 @@ def test_rmsnorm_gemv(lib, dt, B, N, K, norm):
         assert (got != ref).float().mean() < 0.05
 
 
-@pytest.mark.parametrize("B,N,K", [(1, 2304, 768), (16, 768, 2048), (4, 2048, 768)])
+@pytest.mark.parametrize("B,N,K", [(1, 2304, 768), (16, 768, 2048), (4, 2048, 768),
+                                   (3, 288, 288), (16, 56, 272), (2, 480, 352), (16, 16, 144), (5, 32, 56)])
 def test_gemv_int8(lib, B, N, K):
-    """Weight-only int8 against dequantise-then-matmul in fp32 on the same int8 weights."""
+    """Weight-only int8 against dequantise-then-matmul in fp32 on the same int8 weights.  The small shapes have a K that
+    is no multiple of 64: on the matrix-core form the last K step is then partly beyond the row (lanes with zero
+    weights), and K = 56 takes the one-wave-per-row-pair form."""
     from vui_amd import _lib
     from vui_amd.model import quantize_int8
 

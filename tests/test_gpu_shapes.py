@@ -71,3 +71,52 @@ def test_random_architecture_vs_oracle(seed):
                 assert float(top2[0] - top2[1]) <= 2 * TOL * float(logits[0, i].abs().max()), (d, fused, "depth head", i)
                 break  # later codebooks are conditioned on a different token
         m._native.status()
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_architecture_batch_vs_oracle(seed):
+    """2..16 rows over shuffled cache slots with ragged lengths, bf16 or weight-only int8: four decode steps (hidden
+    state, code-0 logits, positions) and the depth head of the batch against the oracle."""
+    rnd = random.Random(1000 + seed)
+    d = _dims(rnd)
+    sdkw = dict(TINY_SD)
+    sdkw["std"] = 0.15 * (64.0 / max(64, d.d_model)) ** 0.5
+    sd = O.synthetic_state_dict(d, **sdkw)
+    g = torch.Generator().manual_seed(seed)
+    int8 = rnd.random() < 0.4
+    B = rnd.choice([2, 3, 4, 5, 8, 9, 12, 16])
+    n_slots = B + rnd.randint(0, 3)
+    S = d.max_seqlen
+    m = make_model(d, sd, BF, int8=int8)
+    o = O.OracleModel(d, sd, BF, n_slots=n_slots, int8=int8)
+    m.decoder.allocate_flash_kv_cache(n_slots, m.device, BF)
+    lens = torch.randint(0, S - 12, (n_slots,), generator=g)
+    kc = O.rnd(0.5 * torch.randn(d.n_layers, n_slots, S, d.n_kv_heads, d.head_dim, generator=g), BF)
+    vc = O.rnd(0.5 * torch.randn(d.n_layers, n_slots, S, d.n_kv_heads, d.head_dim, generator=g), BF)
+    m.decoder._k.copy_(kc.to(BF))
+    m.decoder._v.copy_(vc.to(BF))
+    m.decoder.flash_kv_caches[0].seq_lens.copy_(lens.to(torch.int32))
+    o.k_cache.copy_(kc)
+    o.v_cache.copy_(vc)
+    o.seq_lens.copy_(lens)
+    slots = torch.randperm(n_slots, generator=g)[:B]
+    hid = torch.empty(B, d.d_model, dtype=BF, device="cuda")
+    cb0 = torch.empty(B, d.codebook_size, dtype=BF, device="cuda")
+    for i in range(4):
+        codes = torch.randint(0, d.codebook_size, (B, d.n_quantizers), generator=g)
+        h_ref, cb_ref, _ = o.decode_step(codes, slots)
+        m.decoder._step(codes=codes.cuda(), emb=None, slot_idx=slots.to(torch.int32).cuda(), seq_inc=None, B=B, hidden_out=hid,
+                        cb0_out=cb0, eos_out=None, n_splits=rnd.choice([1, 2, 4, 8]), stream=torch.cuda.current_stream().cuda_stream)
+        assert rel_err(hid, h_ref) <= TOL and rel_err(cb0, cb_ref) <= TOL, (d, B, int8, i)
+        assert m.decoder.flash_kv_caches[0].seq_lens.cpu().tolist() == o.seq_lens.tolist()
+    hidden = O.rnd(torch.randn(B, d.d_model, generator=g), BF)
+    c0 = torch.randint(0, d.codebook_size, (B,), generator=g)
+    want, logits = o.rq_generate(hidden, c0, 1.0, 1, return_logits=True)
+    got = m.rq_transformer.generate(hidden.to(BF).cuda(), c0.cuda(), temperature=1.0, top_k=1).cpu()
+    for b in range(B):
+        for i in range(d.n_quantizers - 1):
+            if got[b, i + 1] != want[b, i + 1]:
+                top2 = torch.topk(logits[b, i], 2).values
+                assert float(top2[0] - top2[1]) <= 2 * TOL * float(logits[b, i].abs().max()), (d, B, "depth head", b, i)
+                break
+    m._native.status()

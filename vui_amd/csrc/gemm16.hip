@@ -264,21 +264,22 @@ __global__ __launch_bounds__(G16_THREADS) void gemm16_kernel(const GemvArgs p) {
 #pragma unroll
   for (int i = 0; i < G16_MAXS; ++i) {
     const int step = wave + 4 * i;
-    if (step < nsteps) {
-      const int k = step * 64 + kg * 16;
-      if (k < K) {
-        const bf16_t* xp = xs + (size_t)f16 * KP + k;
-        const uint4 b_lo = *reinterpret_cast<const uint4*>(xp);
-        const uint4 b_hi = *reinterpret_cast<const uint4*>(xp + 8);
-        uint4 a_lo, a_hi;
-        W16<WT>::split(wr[i], a_lo, a_hi);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_lo), as_bf16x8(b_lo), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_hi), as_bf16x8(b_hi), acc, 0, 0, 0);
-        if (DUAL) {
-          W16<WT>::split(wr2[i], a_lo, a_hi);
-          acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_lo), as_bf16x8(b_lo), acc2, 0, 0, 0);
-          acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_hi), as_bf16x8(b_hi), acc2, 0, 0, 0);
-        }
+    if (step < nsteps) {  // uniform over the wave
+      // The matrix instructions run for all 64 lanes whatever the lanes' own conditions say, so nothing here may sit
+      // behind a per-lane branch: a lane whose 16 columns lie beyond K (the last step of a K that is no multiple of 64)
+      // holds zero weights (set when they were requested) and reads a staged chunk that exists.
+      const int k = min(step * 64 + kg * 16, K - 16);
+      const bf16_t* xp = xs + (size_t)f16 * KP + k;
+      const uint4 b_lo = *reinterpret_cast<const uint4*>(xp);
+      const uint4 b_hi = *reinterpret_cast<const uint4*>(xp + 8);
+      uint4 a_lo, a_hi;
+      W16<WT>::split(wr[i], a_lo, a_hi);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_lo), as_bf16x8(b_lo), acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_hi), as_bf16x8(b_hi), acc, 0, 0, 0);
+      if (DUAL) {
+        W16<WT>::split(wr2[i], a_lo, a_hi);
+        acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_lo), as_bf16x8(b_lo), acc2, 0, 0, 0);
+        acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a_hi), as_bf16x8(b_hi), acc2, 0, 0, 0);
       }
     }
   }
