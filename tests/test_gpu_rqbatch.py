@@ -39,11 +39,20 @@ def _wide_dims():
                   rq_n_layers=2, rq_n_heads=8, vocab_size=50, max_seqlen=64)
 
 
-@pytest.mark.parametrize("dims", ["small", "wide", "nano"])
+def _preset_b_dims():
+    # the 768-wide, 5-layer depth head: 144 QKV tiles, so the first 16 workgroups of a row group take a third one
+    return O.Dims(d_model=128, n_layers=1, n_heads=4, n_kv_heads=4, n_quantizers=16, codebook_size=2048, rq_d_model=768,
+                  rq_n_layers=5, rq_n_heads=8, vocab_size=50, max_seqlen=64)
+
+
+@pytest.mark.parametrize("dims", ["small", "wide", "preset_b", "nano"])
 def test_batched_depth_head_vs_oracle_and_sequence(dims):
-    if dims in ("small", "wide"):
-        d = _small_dims() if dims == "small" else _wide_dims()
-        sd = O.synthetic_state_dict(d, **TINY_SD)
+    if dims in ("small", "wide", "preset_b"):
+        d = {"small": _small_dims, "wide": _wide_dims, "preset_b": _preset_b_dims}[dims]()
+        sdkw = dict(TINY_SD)
+        if dims == "preset_b":
+            sdkw["std"] = 0.04  # keeps the logits of a 768-wide head in the range the tiny ones have
+        sd = O.synthetic_state_dict(d, **sdkw)
     else:
         d = O.Dims()
         sd = O.synthetic_state_dict(d, seed=0)

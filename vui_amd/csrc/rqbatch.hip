@@ -15,7 +15,8 @@
 //
 // Roles inside a row group (a workgroup holds several; every workgroup walks the same phases in order):
 //   all 64      keep the residual stream of the group's rows in LDS (fp32) and take two tiles (wl, wl + 64)
-//               of each matrix that follows an RMSNorm (QKV, W1/W3, logits head; projection of position 0)
+//               of each matrix that follows an RMSNorm (QKV, W1/W3, logits head; projection of position 0), and a
+//               third (wl + 128) of a QKV with more than 128 tiles (depth heads wider than 682)
 //   attention   workgroup 63 - task, task = local row * heads + head: that row's head, its keys/values of
 //               all layers and positions in LDS
 //   out tiles   workgroup 63 - tile - (R/16) * half: out_proj and W2 of tile < R/16 for one half of the group's rows
@@ -302,6 +303,9 @@ struct RqBatchArgs {
 
 struct RbLayer { const bf16_t *attn_norm, *wqkv, *wo, *mlp_norm, *w1, *w3, *w2; };
 
+// Q3: QKV has more than two tiles per workgroup of a row group (see the roles above); a compile-time switch, so that the
+// common form carries neither the third tile's registers nor its tests.
+template <bool Q3>
 __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   float* xres = (float*)smem;                             // [RB_RG][R]
@@ -441,10 +445,17 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
       uint64_t* qkvb = llp;
       llp += (size_t)B * (3 * R / 2);
       if (active) {
+        // QKV has three times the tiles of the other square matrices: a depth head wider than 2 * 64 * 16 / 3 features
+        // gives the first workgroups of a group a third tile (wl + 128)
         const Tile t0 = tile_of(0, nA, 3 * R, R), t1 = tile_of(1, nA, 3 * R, R);
-        TileW<8, false> w0, w1;
+        Tile t2 = {0, 3 * R, R, false};
+        TileW<8, false> w0, w1, w2;
         tile_prefetch<8, false>((const bf16_t*)Lw.wqkv, nullptr, t0, w0);
         tile_prefetch<8, false>((const bf16_t*)Lw.wqkv, nullptr, t1, w1);
+        if (Q3) {
+          t2 = tile_of(2, nA, 3 * R, R);
+          tile_prefetch<8, false>((const bf16_t*)Lw.wqkv, nullptr, t2, w2);
+        }
         const NormRegs nw = load_norm((const bf16_t*)Lw.attn_norm, R);
         if (ybuf) poll_add_norm_rows(ybuf + (size_t)b0 * (R / 2), c, xres, nw, a.rq_eps, R, Bg, xp, xs);
         else norm_rows(xres, nw, a.rq_eps, R, Bg, xp, xs);
@@ -455,6 +466,10 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
           ll_st(dst + 1, f2bf2(v[2], v[3]), ep);
         };
         tile_compute2<8, false>(xp, xs, t0, w0, t1, w1, red, Bg, epi);
+        if (Q3 && t2.on) {  // uniform over the workgroup
+          __syncthreads();  // the partial sums of the first two tiles have been read
+          tile_compute<8, false>(xp, xs, t2, w2, red, Bg, epi);
+        }
       }
       RB_TS();
       const bool kv_only = (t == 0 && l == a.rqL - 1);  // position 0 only feeds later keys/values
@@ -705,10 +720,9 @@ bool rq_batch_supported(const vui_config& c, int nwg, char* why, size_t why_len)
   else if (c.n_quantizers > 64) r = "too many codebooks";
   else if (rq_batch_lds_bytes(c) > 160 * 1024) r = "activations of 16 rows do not fit in LDS";
   else {
-    int nT = 3 * R / 16;
-    if (c.rq_ffn / 16 > nT) nT = c.rq_ffn / 16;
+    int nT = c.rq_ffn / 16;  // two tiles per workgroup of W1/W3 and of a codebook head, three of QKV
     if (c.codebook_size / 16 > nT) nT = c.codebook_size / 16;
-    if (nT > 2 * RB_NWL || R / 16 > RB_NWL || RB_RG * c.rq_heads > RB_NWL) r = "more tiles than a row group's workgroups take";
+    if (nT > 2 * RB_NWL || 3 * R / 16 > 3 * RB_NWL || R / 16 > RB_NWL || RB_RG * c.rq_heads > RB_NWL) r = "more tiles than a row group's workgroups take";
     if (nwg < RB_NWL * ((VUI_MAX_BATCH + RB_RG - 1) / RB_RG)) r = "too few workgroups for the row groups";
     if (c.codebook_size / 2 > RB_RG * (rb_xs(c))) r = "codebook longer than the staging area";
     if ((size_t)VUI_MAX_BATCH * (c.rq_ffn / 2) >= 65536) r = "exchange vector too long";
@@ -759,12 +773,14 @@ int rq_batch_max_resident(size_t lds_bytes) {
   HIP_TRY(hipGetDeviceProperties(&prop, dev));
   static size_t lds_attr = 0;
   if (lds_bytes > lds_attr) {
-    HIP_TRY(hipFuncSetAttribute((const void*)rq_batch_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    HIP_TRY(hipFuncSetAttribute((const void*)rq_batch_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    HIP_TRY(hipFuncSetAttribute((const void*)rq_batch_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
     lds_attr = lds_bytes;
   }
-  int occ = 0;
-  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, rq_batch_kernel, FR_THREADS, lds_bytes));
-  return occ * prop.multiProcessorCount;
+  int occ = 0, occ3 = 0;
+  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, rq_batch_kernel<false>, FR_THREADS, lds_bytes));
+  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ3, rq_batch_kernel<true>, FR_THREADS, lds_bytes));
+  return (occ < occ3 ? occ : occ3) * prop.multiProcessorCount;
 }
 
 #ifdef VUI_RB_CLOCK
@@ -790,7 +806,8 @@ int launch_rq_batch(const vui_config& c, const vui_weights* wdev, const void* hi
 #endif
   const RbLayout l = rb_layout(c);
   a.xs = rb_xs(c); a.off_xp = (int)l.xp; a.off_red = (int)l.red; a.off_misc = (int)l.misc; a.off_att = (int)l.att; a.off_kv = (int)l.kv;
-  hipLaunchKernelGGL(rq_batch_kernel, dim3(nwg), dim3(FR_THREADS), l.total, st, a);
+  if (3 * c.rq_dim / 16 > 2 * RB_NWL) hipLaunchKernelGGL(rq_batch_kernel<true>, dim3(nwg), dim3(FR_THREADS), l.total, st, a);
+  else hipLaunchKernelGGL(rq_batch_kernel<false>, dim3(nwg), dim3(FR_THREADS), l.total, st, a);
   HIP_TRY(hipGetLastError());
   return VUI_OK;
 }
