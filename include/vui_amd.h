@@ -14,9 +14,14 @@
  * kernel keep one workgroup resident on every compute unit and hand values to each other
  * while they run.  While such a launch is in flight NO other kernel may run on the device
  * (another stream, another context, another process): a workgroup kept off its compute unit
- * makes the others wait until a bounded spin gives up, the launch then commits nothing (no
- * position update, no repetition state, no codes), raises the context's error word, and
- * vui_ctx_status reports VUI_EHIP until the context is initialised again with vui_ctx_init.
+ * makes the others wait until a bounded spin gives up; the launch then raises the context's
+ * error word, and vui_ctx_status reports VUI_EHIP until the context is initialised again with
+ * vui_ctx_init.  The batch-1 frame kernel commits nothing in that case (no position update, no
+ * repetition state, no codes; its EOS probability reads -1).  The batched kernels (depth head and
+ * backbone step of 2..16 rows) and the vocoder's trunk kernel write their output buffers as they
+ * go: after a failed launch those hold unfinished values, which a caller must discard - so a caller
+ * checks vui_ctx_status before it uses what such launches wrote (the position update of a batched
+ * backbone step is withheld like the frame kernel's).
  *
  * Return value: 0 on success, a negative VUI_E* code on failure; vui_last_error() returns a
  * human-readable description of the last failure on the calling thread.
@@ -149,6 +154,11 @@ int vui_ctx_rq_batch(vui_ctx* ctx);
  * failing launch and the context stays unusable until vui_ctx_init is called again. */
 int vui_ctx_status(vui_ctx* ctx);
 
+/* Test aid: overwrites the context's launch-count word (waits for the device).  With 0xFFFFFFFF the next
+ * persistent launch finds its count wrapped, raises the error word (value 2) and ends without waiting for
+ * anything: the way to exercise the failure protocol without making a kernel wait.  No counterpart in the reference. */
+int vui_debug_set_epoch(vui_ctx* ctx, uint32_t value);
+
 /* Profiling aid: fused launches made after this call let four workgroups (`workgroup`, +1, +8, +131;
  * those beyond the grid do not exist) each write up to `cap` words (100 MHz clock << 8 | phase tag)
  * into their region of the device buffer buf: 4 regions of cap + 1 words, the last word of a region
@@ -188,7 +198,12 @@ typedef struct vui_sample_params {
                              (topk + scatter, engine.py:855-863; ties at the k-th place go to the lowest indices).
                              1: sampling.sample_top_k's rule used by inference.stream_frames, everything >= the
                              k-th largest kept (sampling.py:14-20).  The depth head always keeps ties (model.py:955-962). */
-  int32_t reserved;
+  float top_p;            /* vui_sample_cb0 / vui_sample_logits only, 0 = off.  > 0: the nucleus cut of
+                             sampling.sample_top_p (sampling.py:23-31) ahead of the top-k cut: in the order "largest
+                             probability first" an entry is kept while the probability strictly ahead of it is
+                             <= top_p.  With top_k > 0 this is sample_top_p_top_k (sampling.py:34-43): of the
+                             nucleus, everything >= its k-th largest entry.  Equal probabilities are ordered by
+                             index (torch.sort leaves that open).  The other entry points require 0. */
 } vui_sample_params;
 
 /* Device-side end-of-turn test of a streamed turn (Engine._stream_row's `step >= min_frames and sigmoid(eos) >

@@ -26,6 +26,10 @@ How each function is pinned (see tests/test_oracle_golden.py, tests/test_oracle_
   the analytic top-k softmax; the *random stream* itself has no counterpart in the reference
   (torch.multinomial's CUDA generator is third-party) -> "parity unpinned" for the
   drawn token under sampling, pinned for greedy.
+* top_p_probs / top_p_top_k_probs (nucleus cut, alone and with top-k): brute force over every ordering of small
+  probability vectors written out as exact binary fractions, including mass exactly at top_p, ties
+  across the boundary and top_p >= 1; parity of which of several EQUAL probabilities survives is
+  unpinned (torch.sort leaves it open), the lowest indices are kept.
 * rep_penalty: closed form + ring-buffer invariant (counts == histogram of the window).
 * int8 weight-only quantisation: closed form (scale = max|w|/127 per output row); the
   format is defined by the benchmark config, it has no reference implementation on this
@@ -302,6 +306,54 @@ def cb0_probs(logits: Tensor, temperature: float, top_k: int) -> np.ndarray:
         kept[order] = p[order]
         p = kept
     return p.numpy()
+
+
+def top_p_probs(probs: Tensor, p: float) -> Tensor:
+    """sampling.sample_top_p's kept weights, in index order (src/vui/sampling.py:23-31): probabilities sorted
+    largest first, an entry is dropped when the cumulative sum strictly ahead of it exceeds p
+    (`probs_sum - probs_sort > p`), the rest renormalised.  torch.sort leaves the order of equal probabilities
+    open; here (and on the device) equal ones go by index (stable sort)."""
+    ps, idx = torch.sort(probs.float(), dim=-1, descending=True, stable=True)
+    csum = torch.cumsum(ps, dim=-1)
+    ps = ps * (~(csum - ps > p)).float()
+    ps = ps / ps.sum(dim=-1, keepdim=True)
+    out = torch.zeros_like(ps)
+    out[idx] = ps
+    return out
+
+
+def top_p_top_k_probs(probs: Tensor, p: float, top_k: int) -> Tensor:
+    """sampling.sample_top_p_top_k's kept weights, in index order (src/vui/sampling.py:34-43): the nucleus as
+    above, then sample_top_k on the renormalised sorted vector (everything >= its k-th largest entry)."""
+    ps, idx = torch.sort(probs.float(), dim=-1, descending=True, stable=True)
+    csum = torch.cumsum(ps, dim=-1)
+    ps = ps * (~(csum - ps > p)).float()
+    ps = ps / ps.sum(dim=-1, keepdim=True)
+    kth = torch.topk(ps, min(top_k, ps.numel())).values[-1]
+    ps = ps * (ps >= kth).float()
+    out = torch.zeros_like(ps)
+    out[idx] = ps
+    return out
+
+
+def sample_codes_probs(logits: Tensor, temperature: float, top_k: "int | None", top_p: "float | None") -> np.ndarray:
+    """Kept, unnormalised weights (index order) of inference._sample_codes (src/vui/inference.py:491-504), which
+    picks among sampling.py's rules: sample_top_p_top_k (both given), sample_top_p (top_p alone and > 0),
+    sample_top_k (ties with the k-th largest kept), or the plain softmax."""
+    probs = torch.softmax(logits.float() / temperature, dim=-1)
+    if top_p is not None and top_k is not None:
+        return top_p_top_k_probs(probs, top_p, top_k).numpy()
+    if top_p is not None and top_p > 0:
+        return top_p_probs(probs, top_p).numpy()
+    if top_k is not None and top_k > 0:
+        kth = torch.topk(probs, min(top_k, probs.numel())).values[-1]
+        probs = probs * (probs >= kth).float()
+    return probs.numpy()
+
+
+def sample_codes(logits: Tensor, temperature: float, top_k: "int | None", top_p: "float | None", u: float) -> int:
+    """One draw of inference._sample_codes with the uniform `u` (inverse CDF in index order over the kept set)."""
+    return _inverse_cdf(sample_codes_probs(logits, temperature, top_k, top_p), u)
 
 
 def sample_cb0(logits: Tensor, counts: Tensor, penalty: float, temperature: float,

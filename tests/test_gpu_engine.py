@@ -335,3 +335,46 @@ def test_wide_depth_head_runs_in_the_one_launch_kernel():
         runs.append(frames.cpu())
     assert torch.equal(runs[0], runs[1])
     assert int(runs[0].min()) >= 0 and int(runs[0].max()) < d.codebook_size
+
+
+def test_failed_persistent_launch_commits_nothing_and_recovers():
+    """The failure protocol of the persistent kernels, without making any kernel wait: the host sets the context's
+    launch count to 0xFFFFFFFF, so the next launch finds it wrapped, raises the error word and ends at once (every
+    wait is skipped).  Nothing is committed by the frame kernel - position, frame counter, repetition state - the
+    EOS slot reads -1, vui_ctx_status reports the failure until vui_ctx_init has run, and after that the same
+    generation gives the frames of an undisturbed run."""
+    from vui_amd import _lib
+    from vui_amd.engine import GenConfig
+
+    d = tiny_dims(2)
+    sd = O.synthetic_state_dict(d, **TINY_SD)
+    cfg = GenConfig(temperature=0.9, top_k=10, rq_top_k=10, rep_penalty=1.2, rep_window=4, seed=5)
+    ids = torch.tensor([3, 11, 42, 7, 19])
+    m, eng = _engine(d, sd, BF)
+    nat = m._native
+    assert nat.fused(1)
+    row = eng.new_row()
+    h = row.prefill_emb(m.token_emb(ids.cuda()[None]))[:, -1]
+    good, _ = eng.generate([row], h, 6, cfg)
+    nat.status()
+    # the same generation again on a context whose launch count is about to wrap
+    row.reset()
+    h = row.prefill_emb(m.token_emb(ids.cuda()[None]))[:, -1]
+    _lib.check(nat.lib.vui_debug_set_epoch(nat.handle, 0xFFFFFFFF), "set_epoch")
+    with pytest.raises(RuntimeError, match="wrapped"):
+        eng.generate([row], h, 6, cfg)
+    torch.cuda.synchronize()
+    assert int(eng.seq_lens[0]) == 5          # no position was added by the five failed frame steps
+    assert int(eng._frame_ctr[0]) == 1        # the host set it to 1 after frame 0; no failed step advanced it
+    assert float(eng._rep_counts.sum()) == 1  # frame 0's stand-alone code-0 draw pushed one code, the failed steps none
+    g, frames, eos, _ = eng._frame_graph(1, cfg, None, 6)
+    assert float(eos[1, 0]) == -1.0           # a failed step marks its EOS slot
+    assert torch.equal(frames[1:6, :, : good.shape[-1]], good[1:])  # and logs no frame: the log still holds the first run's
+    with pytest.raises(RuntimeError):
+        nat.status()                          # sticky until the context is initialised again
+    nat.reinit()
+    nat.status()
+    row.reset()
+    h = row.prefill_emb(m.token_emb(ids.cuda()[None]))[:, -1]
+    again, _ = eng.generate([row], h, 6, cfg)
+    assert torch.equal(again, good)

@@ -206,6 +206,94 @@ def test_sampler_matches_oracle_draws(lib, CS, top_k):
     assert n_match >= 0.995 * n, (n_match, n)
 
 
+def _sample_cb0_rows(lib, logits_bf, temperature, top_k, top_p, seed, frame):
+    """vui_sample_cb0 over bf16 rows with the ties-kept rule (what inference.stream_frames calls)."""
+    from vui_amd import _lib
+
+    B, CS = logits_bf.shape
+    cfgc = _lib.VuiConfigC()
+    cfgc.dtype, cfgc.d_model, cfgc.n_layers, cfgc.n_heads, cfgc.n_kv_heads, cfgc.head_dim, cfgc.ffn = 0, 64, 1, 4, 4, 16, 64
+    cfgc.n_quantizers, cfgc.codebook_size, cfgc.rq_dim, cfgc.rq_layers, cfgc.rq_heads, cfgc.rq_ffn = 4, CS, 64, 0, 1, 8
+    cfgc.rope_dim, cfgc.max_seqlen, cfgc.n_slots, cfgc.norm_eps, cfgc.rq_norm_eps = 16, 16, 1, 1e-5, 1e-6
+    n = lib.vui_workspace_bytes(C.byref(cfgc), 16)
+    assert n > 0, _lib.last_error()
+    ws = torch.zeros(n + 256, dtype=torch.uint8, device="cuda")
+    dummy = torch.zeros(64, dtype=torch.float32, device="cuda")
+    w = _lib.WeightsC()
+    for f in ("audio_emb", "final_norm", "codec_head", "eos_w", "eos_b", "rope_table"):
+        setattr(w, f, dummy.data_ptr())
+    for f in ("attn_norm", "wqkv", "wo", "mlp_norm", "w1", "w3", "w2"):
+        setattr(w.layers[0], f, dummy.data_ptr())
+    h = C.c_void_p()
+    _lib.check(lib.vui_ctx_create(C.byref(cfgc), C.byref(w), (ws.data_ptr() + 255) & ~255, n, 16, C.byref(h)), "ctx")
+    ctr = torch.tensor([frame], dtype=torch.int32, device="cuda")
+    sp = _lib.SampleParamsC()
+    sp.temperature, sp.top_k, sp.seed, sp.frame_ctr, sp.keep_ties, sp.top_p = temperature, top_k, seed, ctr.data_ptr(), 1, top_p
+    out = torch.empty(B, dtype=torch.long, device="cuda")
+    ld = logits_bf.cuda()
+    _lib.check(lib.vui_sample_cb0(h, ld.data_ptr(), None, None, None, 1.0, 0, C.byref(sp), out.data_ptr(), B, stream()), "cb0")
+    torch.cuda.synchronize()
+    lib.vui_ctx_destroy(h)
+    return out.cpu()
+
+
+@pytest.mark.parametrize("CS,top_k,top_p", [(2048, 0, 0.9), (2048, 50, 0.8), (2048, 100, 0.3), (32, 0, 0.5), (32, 5, 0.7),
+                                            (4096, 0, 0.95), (100, 10, 1.0), (2048, 0, 0.05)])
+def test_sampler_nucleus_matches_oracle_draws(lib, CS, top_k, top_p):
+    """The nucleus cut of sampling.sample_top_p / sample_top_p_top_k on the device: fp32 logits through
+    vui_sample_logits (32-bit keys) and bf16 logits through vui_sample_cb0 (16-bit keys) give the oracle's pick on
+    the same uniform except where it falls within rounding of a CDF step or the budget within rounding of a
+    boundary; no pick lies outside a kept set widened by the boundary's own neighbours."""
+    from vui_amd import _lib
+
+    g = torch.Generator().manual_seed(CS * 3 + top_k + int(top_p * 100))
+    B = 16
+    lg = torch.randn(B, CS, generator=g) * 3
+    lg[5, : CS // 4] = lg[5, 0]  # a row whose boundary falls into a run of equal values
+    k_or = top_k if top_k > 0 else None
+    n_match = n = 0
+    for frame in range(12):
+        sp = _lib.SampleParamsC()
+        ctr = torch.tensor([frame], dtype=torch.int32, device="cuda")
+        sp.temperature, sp.top_k, sp.seed, sp.frame_ctr, sp.top_p = 0.8, top_k, 4321, ctr.data_ptr(), top_p
+        out = torch.empty(B, dtype=torch.long, device="cuda")
+        ld = lg.cuda()
+        _lib.check(lib.vui_sample_logits(ld.data_ptr(), None, CS, C.byref(sp), 2, out.data_ptr(), B, stream()), "sample")
+        got32 = out.cpu()
+        lgb = lg.to(BF)
+        got16 = _sample_cb0_rows(lib, lgb, 0.8, top_k, top_p, 4321, frame)
+        for b in range(B):
+            for got, src, cb in ((got32, lg[b], 2), (got16, lgb[b].float(), 0)):
+                u = O.uniform01(4321, frame, b, cb)
+                kept = O.sample_codes_probs(src, 0.8, k_or, top_p)
+                exp = O._inverse_cdf(kept, u)
+                n_match += int(got[b] == exp)
+                n += 1
+                # the pick is a kept entry, or (budget within rounding of a boundary) no smaller than the smallest kept one
+                pr = torch.softmax(src / 0.8, -1).numpy()
+                assert kept[int(got[b])] > 0 or pr[int(got[b])] >= pr[kept > 0].min() * (1 - 1e-5), (b, int(got[b]))
+    assert n_match >= 0.99 * n, (n_match, n)
+
+
+def test_sampler_nucleus_keeps_lowest_indices_of_a_tie(lib):
+    """Eight equal logits, temperature 1: probabilities of 1/8 each.  top_p = 0.3 keeps the entries with 0, 1/8 and
+    2/8 ahead of them - the three lowest indices - whatever the uniform."""
+    from vui_amd import _lib
+
+    lg = torch.full((16, 8), 0.5)
+    seen = set()
+    for frame in range(30):
+        sp = _lib.SampleParamsC()
+        ctr = torch.tensor([frame], dtype=torch.int32, device="cuda")
+        sp.temperature, sp.top_k, sp.seed, sp.frame_ctr, sp.top_p = 1.0, 0, 9, ctr.data_ptr(), 0.3
+        out = torch.empty(16, dtype=torch.long, device="cuda")
+        ld = lg.cuda()
+        _lib.check(lib.vui_sample_logits(ld.data_ptr(), None, 8, C.byref(sp), 1, out.data_ptr(), 16, stream()), "sample")
+        seen |= set(out.cpu().tolist())
+    assert seen == {0, 1, 2}
+    assert set(np.nonzero(O.sample_codes_probs(lg[0], 1.0, None, 0.3))[0]) == {0, 1, 2}
+
+
 def test_sampler_histogram(lib):
     """Chi-square of 20000 device draws against the analytic top-k softmax (benchmark configuration 3's
     distribution-level check)."""

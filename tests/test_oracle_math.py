@@ -224,3 +224,69 @@ def test_quantize_int8_round_trip_and_linear():
             acc = sum(int(q[n, kk]) * x[b, kk].item() for kk in range(33))
             assert abs(got[b, n].item() - acc * s[n].item()) <= 1e-5 * max(1.0, abs(acc * s[n].item()))
     assert torch.equal(O.linear_int8(x, q, s, BF), got.to(BF).float())
+
+
+# ---- nucleus cut (sampling.sample_top_p / sample_top_p_top_k) ----
+def _nucleus_by_hand(probs, p, top_k=None):
+    """The rule read off src/vui/sampling.py:23-43 as plain loops over exact fractions: walk the entries from
+    the largest down (equal ones by index), drop an entry when the mass strictly ahead of it exceeds p; with
+    top_k, of the survivors keep those not smaller than the k-th largest value of the masked vector."""
+    from fractions import Fraction
+
+    fr = [Fraction(x) for x in probs]
+    order = sorted(range(len(fr)), key=lambda i: (-fr[i], i))
+    ahead, kept = Fraction(0), []
+    for i in order:
+        if not ahead > Fraction(p):
+            kept.append(i)
+        ahead += fr[i]
+    if top_k is not None:
+        masked = sorted((fr[i] if i in kept else Fraction(0) for i in range(len(fr))), reverse=True)
+        kth = masked[min(top_k, len(fr)) - 1]
+        kept = [i for i in kept if fr[i] >= kth]
+    return set(kept)
+
+
+def test_nucleus_rule_against_brute_force():
+    """Every vector of 5 eighths summing to one (all orders, so ties and the index rule are met), every
+    p in eighths from 0 to 1 and beyond: sums of eighths are exact in fp32, so "mass exactly at p" is
+    decided the same way by the oracle's float arithmetic and by the fractions."""
+    n = 0
+    for parts in itertools.product(range(0, 9), repeat=5):
+        if sum(parts) != 8:
+            continue
+        probs = [c / 8 for c in parts]
+        t = torch.tensor(probs, dtype=F32)
+        for p16 in (0, 2, 4, 6, 8, 10, 12, 14, 16, 20):
+            want = _nucleus_by_hand(probs, p16 / 16)
+            got = O.top_p_probs(t, p16 / 16)
+            assert set(torch.nonzero(got).flatten().tolist()) == {i for i in want if probs[i] > 0}, (parts, p16)
+            # kept weights are the probabilities renormalised over the kept set
+            tot = sum(probs[i] for i in want)
+            for i in want:
+                assert abs(float(got[i]) - probs[i] / tot) < 1e-6
+            for k in (1, 2, 4, 5):
+                wantk = _nucleus_by_hand(probs, p16 / 16, k)
+                gotk = O.top_p_top_k_probs(t, p16 / 16, k)
+                assert set(torch.nonzero(gotk).flatten().tolist()) == {i for i in wantk if probs[i] > 0}, (parts, p16, k)
+            n += 1
+    assert n == 4950
+
+
+def test_nucleus_special_cases():
+    t = torch.tensor([0.125, 0.5, 0.125, 0.25], dtype=F32)
+    # the largest entry always survives (nothing lies ahead of it), also with p = 0
+    assert torch.nonzero(O.top_p_probs(t, 0.0)).flatten().tolist() == [1]
+    # mass exactly at p: 0.5 is not "> 0.5", so the second entry is kept; the third (0.75 ahead) is not
+    assert torch.nonzero(O.top_p_probs(t, 0.5)).flatten().tolist() == [1, 3]
+    # equal probabilities across the boundary: the lower index is the one kept
+    assert torch.nonzero(O.top_p_probs(t, 0.75)).flatten().tolist() == [0, 1, 3]
+    # p >= 1 keeps everything and changes nothing
+    assert torch.allclose(O.top_p_probs(t, 1.0), t)
+    # _sample_codes' dispatch (inference.py:491-504)
+    lg = torch.log(t)
+    assert np.count_nonzero(O.sample_codes_probs(lg, 1.0, None, None)) == 4
+    assert np.count_nonzero(O.sample_codes_probs(lg, 1.0, 2, None)) == 2
+    assert np.count_nonzero(O.sample_codes_probs(lg, 1.0, None, 0.0)) == 4    # top_p = 0 alone: no cut at all
+    assert np.count_nonzero(O.sample_codes_probs(lg, 1.0, 3, 0.0)) == 1       # beside a top_k: the nucleus of p = 0
+    assert np.count_nonzero(O.sample_codes_probs(lg, 1.0, 1, 0.9)) == 1

@@ -186,9 +186,9 @@ def test_engine_stream_sampled_and_cancel():
 @pytest.mark.gpu
 @pytest.mark.parametrize("graph", [False, True])
 def test_stream_audio_equals_vocoder_oracle_on_streamed_codes(graph):
-    """Row.stream_audio: every frame of Row.stream passed through the row's vocoder context.  Same turn, same
-    seed: the audio is the vocoder oracle's for the codes Row.stream yields; an early stop by the consumer
-    leaves the row and the vocoder context usable."""
+    """Row.stream (= stream_audio) on an engine with a vocoder: every frame of Row.stream_codes passed through the
+    row's vocoder context.  Same turn, same seed: the audio is the vocoder oracle's for the codes Row.stream_codes
+    yields; an early stop by the consumer leaves the row and the vocoder context usable."""
     import dataclasses
 
     from oracle import codec_oracle as CO
@@ -210,7 +210,7 @@ def test_stream_audio_equals_vocoder_oracle_on_streamed_codes(graph):
     cfg = GenConfig(eos_threshold=2.0, rep_window=4, top_k=5)
     eng = Engine(model=model, codec=dec, max_rows=1, max_seq=320)
     row = eng.new_row()
-    audio = [a.clone().cpu() for a in row.stream_audio(ch, cfg)]
+    audio = [a.clone().cpu() for a in row.stream(ch, cfg)]  # with a vocoder Row.stream hands out audio, as the reference's
     row.reset()
     row._codec_ctx.reset()
     it = row.stream_audio(ch, cfg)  # the consumer walks away after three frames
@@ -223,7 +223,7 @@ def test_stream_audio_equals_vocoder_oracle_on_streamed_codes(graph):
     assert len(again) == len(audio) and all(torch.equal(a, b) for a, b in zip(again, audio))
     row.reset()
     row._codec_ctx.reset()
-    codes = [f.cpu() for f in row.stream(ch, cfg)]
+    codes = [f.cpu() for f in row.stream_codes(ch, cfg)]
     n = 2 * cfg.max_turn_frames(3)
     assert len(audio) == len(codes) == n
     ora = CO.CodecDecoderOracle(cd, csd)

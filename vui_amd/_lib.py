@@ -48,7 +48,7 @@ class WeightsC(C.Structure):
 
 class SampleParamsC(C.Structure):
     _fields_ = [("temperature", C.c_float), ("top_k", C.c_int32), ("seed", C.c_uint64),
-                ("frame_ctr", C.c_void_p), ("state_rows", C.c_void_p), ("keep_ties", C.c_int32), ("reserved", C.c_int32)]
+                ("frame_ctr", C.c_void_p), ("state_rows", C.c_void_p), ("keep_ties", C.c_int32), ("top_p", C.c_float)]
 
 
 class EosStopC(C.Structure):
@@ -77,6 +77,7 @@ SIGNATURES = {
     "vui_ctx_init": (_I, [_P, _P]),
     "vui_ctx_fused": (_I, [_P, _I]),
     "vui_ctx_status": (_I, [_P]),
+    "vui_debug_set_epoch": (_I, [_P, C.c_uint32]),
     "vui_ctx_rq_batch": (_I, [_P]),
     "vui_debug_phase_clock": (_I, [_P, _P, _I, _I]),
     "vui_prefill_scratch_bytes": (_L, [C.POINTER(VuiConfigC), _I, _I]),

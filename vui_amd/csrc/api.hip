@@ -280,6 +280,13 @@ int vui_debug_phase_clock(vui_ctx* ctx, uint64_t* buf, int cap, int workgroup) {
   return VUI_OK;
 }
 
+int vui_debug_set_epoch(vui_ctx* ctx, uint32_t value) {
+  if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
+  HIP_TRY(hipDeviceSynchronize());
+  HIP_TRY(hipMemcpy(ctx->ctl, &value, sizeof(value), hipMemcpyHostToDevice));
+  return VUI_OK;
+}
+
 int vui_ctx_status(vui_ctx* ctx) {
   if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
   uint32_t h[4] = {0, 0, 0, 0};
@@ -410,7 +417,7 @@ static SampleArgs sample_base(const vui_sample_params* sp) {
   SampleArgs s;
   memset(&s, 0, sizeof(s));
   s.temperature = sp->temperature; s.top_k = sp->top_k; s.seed = sp->seed; s.frame_ctr = sp->frame_ctr;
-  s.state_rows = sp->state_rows;
+  s.state_rows = sp->state_rows; s.top_p = sp->top_p;
   return s;
 }
 
@@ -476,6 +483,7 @@ int vui_rq_generate(vui_ctx* ctx, const void* hidden, const int64_t* code0, cons
   if (c.rq_layers < 1) { vui_set_error("context has no depth head"); return VUI_EINVAL; }
   if (!hidden || !code0 || !sp || !codes_out) { vui_set_error("NULL argument"); return VUI_EINVAL; }
   if (n_q < 2 || n_q > c.n_quantizers || codes_stride < n_q) { vui_set_error("n_q=%d outside [2,%d] or stride %d too small", n_q, c.n_quantizers, codes_stride); return VUI_EINVAL; }
+  if (sp->top_p > 0.f) { vui_set_error("the depth head draws with temperature and top-k only (model.py:955-962): top_p must be 0"); return VUI_EINVAL; }
   hipStream_t st = (hipStream_t)stream;
   if (use_fused(ctx, B)) {
     FrameArgs a;
@@ -547,6 +555,7 @@ int vui_frame_step(vui_ctx* ctx, int64_t* codes_io, const int32_t* slot_idx, int
   void* cb0 = cb0_out ? cb0_out : ctx->cb0;
   if (window > 0 && rep_counts && penalty > 1.0f && (!rep_hist || !rep_pos)) { vui_set_error("a repetition window needs rep_hist and rep_pos"); return VUI_EINVAL; }
   if (n_q < 2 || n_q > c.n_quantizers) { vui_set_error("n_q=%d outside [2,%d]", n_q, c.n_quantizers); return VUI_EINVAL; }
+  if (sp_cb0->top_p > 0.f || sp_rq->top_p > 0.f) { vui_set_error("vui_frame_step is Engine's step, whose samplers have no nucleus cut: top_p must be 0 (vui_sample_cb0 takes it)"); return VUI_EINVAL; }
   if (use_fused(ctx, B)) {
     if (!seq_lens || !k_cache || !v_cache) { vui_set_error("seq_lens and the KV caches are required"); return VUI_EINVAL; }
     FrameArgs a;

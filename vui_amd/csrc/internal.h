@@ -107,6 +107,7 @@ struct SampleArgs {
   int window;
   float temperature;
   int top_k;
+  float top_p;         // > 0: nucleus cut ahead of the top-k cut (stand-alone sampling kernel only)
   uint64_t seed;
   const int32_t* frame_ctr;
   const int32_t* state_rows;  // (B) or nullptr: repetition state / random-stream row of row b

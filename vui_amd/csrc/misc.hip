@@ -92,6 +92,7 @@ template <typename T, int EMAX>
 __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const SampleArgs p) {
   __shared__ SampleShared sh;
   __shared__ __align__(16) int hist[HIST_WORDS];
+  __shared__ NucleusShared nuc;
   const int b = blockIdx.x, tid = threadIdx.x;
   const int CS = p.CS;
   const int E = (CS + SAMP_THREADS - 1) / SAMP_THREADS;  // contiguous elements per thread
@@ -118,6 +119,7 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const SampleArgs p
   }
   const uint32_t frame = p.frame_ctr ? (uint32_t)p.frame_ctr[0] : 0u;
   const uint32_t rnd = philox_u32(p.seed, frame, (uint32_t)sb, (uint32_t)p.codebook, 0u);
+  if (p.top_p > 0.f && !greedy) nucleus_cut<EMAX>(l, key, raw_keys ? 16 : 0, CS, E, p.top_p, nuc);  // uniform over the block
   const int pick = block_sample<EMAX>(l, key, raw_keys ? 16 : 0, CS, E, greedy, p.top_k, rnd, (uint32_t)p.codebook, sh, hist, p.exact_k != 0);
 
   if (tid == 0) {

@@ -423,7 +423,8 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
       if (t == 1) {
         if (tid < Bg) { int64_t cc = a.code0[b0 + tid]; codes_s[tid] = (int)(cc < 0 ? 0 : (cc >= CS ? CS - 1 : cc)); }
       } else {
-        ll_poll_auto(codebuf + b0, Bg, c, [&](int i, uint32_t v) { codes_s[i] = (int)v; });
+        // (clamped: after a wait that was given up the word may hold anything, and the code indexes the embedding table)
+        ll_poll_auto(codebuf + b0, Bg, c, [&](int i, uint32_t v) { codes_s[i] = (int)min(v, (uint32_t)(CS - 1)); });
       }
       __syncthreads();
       for (int i = tid; i < Bg * (R / 8); i += FR_THREADS) {

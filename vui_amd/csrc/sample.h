@@ -125,6 +125,10 @@ __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32
     if (sh.sred[w] > M) { M = sh.sred[w]; Mi = sh.ired[w]; }
     else if (sh.sred[w] == M) Mi = min(Mi, sh.ired[w]);
   }
+  // Logits that hold no ordinary number (all NaN or all -inf: only a launch that has given up its waits and runs on
+  // with unfinished words can produce them) leave no candidate; the pick must still be an index of the codebook,
+  // because callers gather embedding rows with it.
+  if (Mi < 0 || Mi >= CS) Mi = 0;
   if (greedy) { __syncthreads(); return Mi; }
   SAMP_TS(1);
 
@@ -264,6 +268,134 @@ __device__ __forceinline__ int block_sample(const float (&l)[EMAX], const uint32
   // no barrier here: the next draw of this workgroup (codebook + 1) uses the other slot, and every other word of the
   // shared state is next written behind a barrier of that draw which this read precedes
   return pick;
+}
+
+// ---- nucleus cut (sampling.sample_top_p / sample_top_p_top_k, src/vui/sampling.py:23-43) ----
+// In the order "largest probability first, equal ones by index" an element is kept while the probability mass
+// strictly ahead of it is <= top_p; everything behind is dropped (l = -inf) before the top-k cut and the draw of
+// block_sample.  The masses are summed as integers (weight exp(l - max) in units of 2^-32, 64-bit totals), so the
+// kept set does not depend on the order in which threads add: the same logits always give the same set.
+// The boundary key is found one byte per round from the top, as the k-th key is in block_sample: per round a
+// 256-bin histogram of MASS among the keys that share the bytes chosen so far, and the lowest digit whose mass
+// above it still fits the remaining budget.  Of the keys equal to the boundary key (equal probabilities) the
+// lowest indices are kept, one more than fit entirely into what is left of the budget.
+// mass: 256 words of LDS; ties: one int per wave.  Every thread of the 256 calls this.
+struct NucleusShared {
+  unsigned long long mass[256];
+  unsigned long long tot[SAMP_THREADS / WAVE];
+  float mx[SAMP_THREADS / WAVE];
+  int ties[SAMP_THREADS / WAVE];
+};
+__device__ __forceinline__ unsigned long long shfl_down_u64(unsigned long long v, int off) {
+  const uint32_t lo = (uint32_t)__shfl_down((int)(uint32_t)v, off), hi = (uint32_t)__shfl_down((int)(uint32_t)(v >> 32), off);
+  return ((unsigned long long)hi << 32) | lo;
+}
+template <int EMAX>
+__device__ __forceinline__ void nucleus_cut(float (&l)[EMAX], uint32_t (&key)[EMAX], int low_bit, int CS, int E, float top_p,
+                                            NucleusShared& ns) {
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  // maximum, then the integer weights and their total
+  float m = -INFINITY;
+#pragma unroll
+  for (int e = 0; e < EMAX; ++e) if (e < E) m = fmaxf(m, l[e]);
+  m = rows_max(group16_max(m));
+  if (lane == 0) ns.mx[wave] = m;
+  ns.mass[tid] = 0ull;
+  __syncthreads();
+  float M = ns.mx[0];
+#pragma unroll
+  for (int w = 1; w < SAMP_THREADS / WAVE; ++w) M = fmaxf(M, ns.mx[w]);
+  unsigned long long q[EMAX], mine = 0ull;
+#pragma unroll
+  for (int e = 0; e < EMAX; ++e) {
+    q[e] = 0ull;
+    if (e < E && tid * E + e < CS) q[e] = (unsigned long long)(__expf(l[e] - M) * 4294967296.0f);
+    mine += q[e];
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) mine += shfl_down_u64(mine, off);
+  if (lane == 0) ns.tot[wave] = mine;
+  __syncthreads();
+  unsigned long long Z = 0ull;
+#pragma unroll
+  for (int w = 0; w < SAMP_THREADS / WAVE; ++w) Z += ns.tot[w];
+  unsigned long long rem = (unsigned long long)((double)top_p * (double)Z);  // the budget: mass allowed strictly ahead
+  uint32_t thr = 0u;
+  const int rounds = (32 - low_bit) / 8;
+  for (int round = 0; round < rounds; ++round) {
+    const int shift = 24 - 8 * round;
+#pragma unroll
+    for (int e = 0; e < EMAX; ++e)
+      if (e < E && tid * E + e < CS && q[e] && (round == 0 || (key[e] >> (shift + 8)) == (thr >> (shift + 8))))
+        atomicAdd(&ns.mass[(key[e] >> shift) & 255], q[e]);
+    __syncthreads();
+    // every wave for itself: lane holds bins 4 lane .. 4 lane + 3; mass above each of them inside the round
+    const unsigned long long b0 = ns.mass[4 * lane], b1 = ns.mass[4 * lane + 1], b2 = ns.mass[4 * lane + 2], b3 = ns.mass[4 * lane + 3];
+    unsigned long long above = b0 + b1 + b2 + b3;  // becomes: mass in the bins of higher lanes
+    {
+      unsigned long long v = above;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const unsigned long long t = shfl_down_u64(v, off);
+        if (lane + off < 64) v += t;
+      }
+      above = v - above;
+    }
+    // the lowest digit whose mass above still fits: the lanes' candidates, lowest lane wins
+    int digit = -1;
+    unsigned long long ab = 0ull;
+    if (above + b3 + b2 + b1 <= rem) { digit = 4 * lane; ab = above + b3 + b2 + b1; }
+    else if (above + b3 + b2 <= rem) { digit = 4 * lane + 1; ab = above + b3 + b2; }
+    else if (above + b3 <= rem) { digit = 4 * lane + 2; ab = above + b3; }
+    else if (above <= rem) { digit = 4 * lane + 3; ab = above; }
+    const unsigned long long found = __ballot(digit >= 0);  // never empty: nothing lies above digit 255
+    const int src = (int)__builtin_ctzll(found);
+    digit = __builtin_amdgcn_readlane(digit, src);
+    const uint32_t ab_lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)ab, src), ab_hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(ab >> 32), src);
+    rem -= ((unsigned long long)ab_hi << 32) | ab_lo;
+    thr |= (uint32_t)digit << shift;
+    __syncthreads();  // every wave has read the bins
+    ns.mass[tid] = 0ull;
+    __syncthreads();
+  }
+  // the boundary class: keys equal to thr (above low_bit); their common weight; ranks in index order
+  const uint32_t tt = thr >> low_bit;
+  int eq = 0;
+  unsigned long long qc = 0ull;
+#pragma unroll
+  for (int e = 0; e < EMAX; ++e)
+    if (e < E && tid * E + e < CS && (key[e] >> low_bit) == tt) { ++eq; qc = q[e]; }
+  int incl = eq;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int t = __shfl_up(incl, off);
+    if (lane >= off) incl += t;
+  }
+  if (lane == WAVE - 1) ns.ties[wave] = incl;
+  // any member's weight will do (equal keys carry equal values): the largest seen in the wave, then in the block
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) { const unsigned long long t = shfl_down_u64(qc, off); qc = t > qc ? t : qc; }
+  if (lane == 0) ns.tot[wave] = qc;
+  __syncthreads();
+  int before = incl - eq;
+  unsigned long long qcl = 0ull;
+#pragma unroll
+  for (int w = 0; w < SAMP_THREADS / WAVE; ++w) { if (w < wave) before += ns.ties[w]; qcl = ns.tot[w] > qcl ? ns.tot[w] : qcl; }
+  // member number r (from 0) has r * qcl ahead of it inside the class
+  const unsigned long long fit = qcl ? rem / qcl : 0xffffffffull;
+  const unsigned long long n_keep = fit + 1ull;
+  int seen = 0;
+  const uint32_t dropped = float_key(-INFINITY);
+#pragma unroll
+  for (int e = 0; e < EMAX; ++e) {
+    if (e < E && tid * E + e < CS) {
+      const uint32_t k = key[e] >> low_bit;
+      bool keep = k > tt;
+      if (k == tt) { keep = (unsigned long long)(before + seen) < n_keep; ++seen; }
+      if (!keep) { l[e] = -INFINITY; key[e] = dropped; }
+    }
+  }
+  __syncthreads();
 }
 
 // penalised, biased, temperature-scaled value of one logit

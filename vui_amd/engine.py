@@ -172,26 +172,35 @@ class Row:
         codes = self._engine._render_row(self, chunks, cfg)
         return codes, self._engine._decode_full(codes)
 
-    def stream(self, chunks: "list[Chunk]", cfg: GenConfig = GenConfig(), cancel=None, *, reset_rep: bool = True,
-               final_turn: bool = False) -> Iterator[Tensor]:
-        """Streams the code frames of one assistant turn, chunk by chunk (Row.stream,
-        src/vui/engine.py:204-244; frames of codes instead of audio, the vocoder is not part of this
-        package).  cancel: object with is_set(), polled per frame."""
+    def stream_codes(self, chunks: "list[Chunk]", cfg: GenConfig = GenConfig(), cancel=None, *, reset_rep: bool = True,
+                     final_turn: bool = False) -> Iterator[Tensor]:
+        """The code frames (Q',) int64 of one assistant turn, chunk by chunk: Engine._stream_row's frames before
+        the vocoder (src/vui/engine.py:1308-1521).  No counterpart of its own in the reference, whose Row.stream
+        hands out audio only.  cancel: object with is_set(), polled per frame."""
         if self._engine.max_rows != 1:
             raise RuntimeError(f"stream() requires Engine(max_rows=1), got {self._engine.max_rows}")
         yield from self._engine._stream_row(self, chunks, cfg, cancel, reset_rep=reset_rep, final_turn=final_turn)
 
-    def stream_audio(self, chunks: "list[Chunk]", cfg: GenConfig = GenConfig(), cancel=None, *, reset_rep: bool = True,
-                     final_turn: bool = False) -> Iterator[Tensor]:
-        """`stream` with every frame passed through the row's vocoder context: yields audio (1, 1, 1920)
-        per frame, as Row.stream of the reference does (src/vui/engine.py:204-244, 1349-1356, 1537-1546).
-        The vocoder stream is seeded once per session from the row's buffered codes."""
+    def stream(self, chunks: "list[Chunk]", cfg: GenConfig = GenConfig(), cancel=None, *, reset_rep: bool = True,
+               final_turn: bool = False) -> Iterator[Tensor]:
+        """Streams one assistant turn as audio, (1, 1, 1920) float per frame, as Row.stream of the reference
+        does (src/vui/engine.py:211-244, 1349-1356, 1537-1546): every frame of `stream_codes` goes through the
+        row's vocoder context, which is seeded once per session from the row's buffered codes.  An engine built
+        without a vocoder has no audio to give: there `stream` yields the code frames themselves."""
         if self._codec_ctx is None:
-            raise RuntimeError("stream_audio() needs Engine(codec=...)")
+            yield from self.stream_codes(chunks, cfg, cancel, reset_rep=reset_rep, final_turn=final_turn)
+            return
         if self._codec_ctx._stack is None:
             self._codec_ctx.prefill(n_codebooks=cfg.n_codebooks)
-        for codes in self.stream(chunks, cfg, cancel, reset_rep=reset_rep, final_turn=final_turn):
+        for codes in self.stream_codes(chunks, cfg, cancel, reset_rep=reset_rep, final_turn=final_turn):
             yield self._engine._stream_decode_frame(self, codes, cfg.n_codebooks)
+
+    def stream_audio(self, chunks: "list[Chunk]", cfg: GenConfig = GenConfig(), cancel=None, *, reset_rep: bool = True,
+                     final_turn: bool = False) -> Iterator[Tensor]:
+        """`stream` on an engine that must have a vocoder (raises otherwise)."""
+        if self._codec_ctx is None:
+            raise RuntimeError("stream_audio() needs Engine(codec=...)")
+        yield from self.stream(chunks, cfg, cancel, reset_rep=reset_rep, final_turn=final_turn)
 
     def mark_prompt(self) -> int:
         self._prompt_offset = self.offset
@@ -784,6 +793,10 @@ class Engine:
                 row_turn_count[r.idx] += 1
             for r in hit:
                 next_chunk(r)
+        # the batched depth head of the last step (or of a chunk start behind it) has not been checked yet: a
+        # persistent launch that gave up a wait raised the error word, and its codes must not be returned as results
+        stream.synchronize()
+        nat.status()
         result: dict[int, Tensor] = {}
         for r in rows:
             n = row_frame_count[r.idx]
@@ -961,6 +974,8 @@ class Engine:
             for slot in to_remove:
                 active.pop(slot).row.close()
             backfill()
+        stream.synchronize()
+        nat.status()  # the last step's depth head and the chunk starts behind it
         return [torch.stack(b) if b else torch.zeros(0, nq, dtype=torch.long, device=self.device) for b in frame_bufs]
 
     # ------------------------------------------------------------------ streaming single-row turn

@@ -6,7 +6,8 @@ that `render_codes_stream`, `render_audio_stream` and the TTS worker consume (sr
 It differs from `Engine._stream_row` exactly where the reference's two drivers differ: code 0 is drawn with
 `sampling.sample_top_k` (everything >= the k-th largest probability kept) on EVERY frame, the first of a chunk
 included; the depth head runs before the end-of-turn test, so a turn's last frame is drawn and then dropped;
-the step is `Vui.decode_step(codes, pos)`; a chunk is capped by max_turn_secs alone.
+the step is `Vui.decode_step(codes, pos)`; a chunk is capped by max_turn_secs alone; `top_p` adds the nucleus
+cut of `sampling.sample_top_p` / `sample_top_p_top_k` to the code-0 draw.
 
 Text handling (cleaning, chunking, tokenising) is outside this package: chunks arrive as `Chunk`s whose `emb`
 holds the embeddings of `[spk] text` (+ `[SC]` where the next chunk changes speaker, + cond_bias), as the
@@ -143,8 +144,6 @@ def stream_frames(state: InferenceState, chunks: "list[Chunk]", *, temperature: 
 
     resume=False starts from position 0 (a prompt is written by the caller through state.prefill_prompt and
     resume=True, as the reference's low-latency path does)."""
-    if top_p is not None:
-        raise NotImplementedError("top_p sampling is not part of the native sampler")
     if not chunks:
         return
     model, nat = state.model, state.model._native
@@ -163,7 +162,15 @@ def stream_frames(state: InferenceState, chunks: "list[Chunk]", *, temperature: 
     code0 = torch.zeros(1, dtype=torch.long, device=dev)
     win = rep_window if (use_rep and rep_window > 0) else 0
     k = 1 if top_k == 1 else (top_k if (top_k is not None and top_k > 0) else 0)
-    sp0 = make_sample_params(temperature, k, seed, frame_ctr, keep_ties=True)
+    # _sample_codes (inference.py:491-504): both given -> sample_top_p_top_k, top_p alone (> 0) -> sample_top_p,
+    # else top-k or the plain softmax.  A nucleus of top_p <= 0 beside a top_k holds the largest probability alone.
+    p = 0.0
+    if top_p is not None and (top_k is not None or top_p > 0):
+        if top_p <= 0:
+            k = 1
+        else:
+            p = float(top_p)
+    sp0 = make_sample_params(temperature, k, seed, frame_ctr, keep_ties=True, top_p=p)
     rq.seed = seed
 
     def rq_sample(cb0_logits: Tensor, hidden: Tensor) -> Tensor:

@@ -184,6 +184,10 @@ class _Native:
     def status(self) -> None:
         _lib.check(self.lib.vui_ctx_status(self.handle), "vui_ctx_status")
 
+    def reinit(self) -> None:
+        """vui_ctx_init again: clears a raised error word (and rewrites the workspace's derived weight copies)."""
+        _lib.check(self.lib.vui_ctx_init(self.handle, torch.cuda.current_stream().cuda_stream), "vui_ctx_init")
+
     def __del__(self):
         try:
             if getattr(self, "handle", None):
@@ -228,8 +232,9 @@ class Graph:
 
 
 def make_sample_params(temperature: float, top_k: int | None, seed: int, frame_ctr: Tensor | None,
-                       state_rows: Tensor | None = None, keep_ties: bool = False):
+                       state_rows: Tensor | None = None, keep_ties: bool = False, top_p: float = 0.0):
     sp = _lib.SampleParamsC()
+    sp.top_p = float(top_p)
     sp.keep_ties = 1 if keep_ties else 0
     sp.state_rows = state_rows.data_ptr() if state_rows is not None else None
     sp.temperature = float(temperature)
