@@ -52,7 +52,7 @@ def gpu_bench(args):
     max_seq = 64 * ((n_prefix + n_text + K + W + n_lat + 2 + 63) // 64)
     t0 = time.time()
     sd = synthetic_state_dict(d, seed=0)
-    model = Vui(nano_for_cache(args.preset, max_seq), sd, device="cuda", dtype=torch.bfloat16)
+    model = Vui(nano_for_cache(args.preset, max_seq), sd, device="cuda", dtype=torch.bfloat16, int8=args.int8)
     eng = Engine(model=model, max_rows=1, max_seq=max_seq)
     row = eng.new_row()
     g = torch.Generator().manual_seed(0)
@@ -97,6 +97,12 @@ def gpu_bench(args):
     torch.cuda.synchronize()
     lat = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(n_lat))
     fb = frame_bytes(model.config.model, (L_start + L_end) / 2.0)
+    if args.int8:  # the backbone's matrices are one byte per weight plus a bf16 scale per row
+        mm = model.config.model
+        w16 = mm.n_layers * ((mm.n_heads + 2 * mm.kv_heads) * mm.head_dim * mm.d_model + mm.d_model * mm.d_model + 3 * mm.ffn * mm.d_model) * 2
+        rows_ = mm.n_layers * ((mm.n_heads + 2 * mm.kv_heads) * mm.head_dim + 2 * mm.d_model + 2 * mm.ffn)
+        fb["backbone"] += -w16 // 2 + rows_ * 2
+        fb["frame"] = fb["backbone"] + fb["rq_unique"]
     out = {
         "metric": "codec frames/sec at batch 1 (Vui Nano bf16)", "value": round(fps, 2), "unit": "frames/s",
         "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(ms_per, 4), "higher_is_better": True,
@@ -104,7 +110,8 @@ def gpu_bench(args):
         "rtf": round(fps / 12.5, 2), "p50_ms": round(lat[len(lat) // 2], 4), "p99_ms": round(lat[int(len(lat) * 0.99)], 4),
         "config": {"workload": "e2e_b1: 512-frame voice prefix + 64 text tokens prefilled, then one HIP-graph "
                                "replay per codec frame (backbone step + code-0 sampling + depth head, 16 codebooks)",
-                   "preset": args.preset, "kv_len": [L_start, L_end], "sampling": "T=0.9 top-k=100 rep=1.1/24",
+                   "preset": args.preset, "backbone_weights": "int8 (weight-only, per-row bf16 scales)" if args.int8 else "bf16",
+                   "kv_len": [L_start, L_end], "sampling": "T=0.9 top-k=100 rep=1.1/24",
                    "latency_sample": f"p50/p99 over the {n_lat} frames after the timed region, one event per frame",
                    "setup_s": round(setup_s, 1)},
         "frame_bytes": {k: int(v) for k, v in fb.items()},
@@ -245,6 +252,52 @@ def b16_line(sd, preset="A", n=100):
     return {"config": "e2e_b16_int8_ragged", "us_per_frame_step": round(us, 1), "aggregate_frames_per_s": round(16e6 / us, 1),
             "rtf": round(16e6 / us / 12.5, 1), "steps": n, "kv_bytes": int(kv_bytes), "int8_weight_bytes": int(wbytes),
             "achieved_GBs": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "mfma_busy_frac": MEASURED_B16_MFMA_BUSY}
+
+
+def batch_sweep(sd, preset="A", n=40, batches=(1, 2, 4, 8, 16)):
+    """The frame step (backbone step + code-0 draw + depth head, one captured graph per batch size) for 1..16
+    concurrent streams, with bf16 and with int8 backbone weights: ragged caches as in benchmark configuration 5
+    (lengths U[128, 2048] from seed 5, the first B of them; filled N(0, 1)), n replays each after 3 warm-ups."""
+    import torch
+
+    from vui_amd.engine import Engine, GenConfig
+    from vui_amd.model import Vui
+    from vui_amd.synthetic import nano_for_cache
+
+    S = 2048 + 256
+    g = torch.Generator().manual_seed(5)
+    lens = torch.randint(128, 2049, (16,), generator=g).to(torch.int32)
+    out = []
+    for int8 in (False, True):
+        model = Vui(nano_for_cache(preset, S), sd, device="cuda", dtype=torch.bfloat16, int8=int8)
+        m = model.config.model
+        eng = Engine(model=model, max_rows=16, max_seq=S)
+        model.decoder._k.normal_()
+        model.decoder._v.normal_()
+        rows = [eng.new_row() for _ in range(16)]
+        hid = torch.randn(16, m.d_model, generator=g).to(torch.bfloat16).cuda()
+        for B in batches:
+            eng.seq_lens.zero_()
+            eng.seq_lens[:B] = lens[:B].cuda()
+            eng.generate(rows[:B], hid[:B], 1, GenConfig())
+            gr, _, _, _ = eng._frame_graph(B, GenConfig(), None, n + 4)
+            eng.seq_lens[:B] = lens[:B].cuda()
+            for _ in range(3):
+                gr.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(n):
+                gr.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            model._native.status()
+            us = e0.elapsed_time(e1) * 1e3 / n
+            out.append({"B": B, "weights": "int8" if int8 else "bf16", "us_per_step": round(us, 1),
+                        "aggregate_frames_per_s": round(B * 1e6 / us, 1)})
+        del eng, model, rows
+        torch.cuda.empty_cache()
+    return out
 
 
 def serve_line(sd, preset="A", n_requests=32, max_rows=16):
@@ -453,6 +506,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--preset", default="A", choices=["A", "B"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--int8", action="store_true", help="batch 1 with the backbone's matrices as weight-only int8")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the batch sweep of the default line")
+    ap.add_argument("--sweep-only", action="store_true", help="print only the batch sweep (B = 1..16, bf16 and int8 weights)")
     ap.add_argument("--no-roofline", action="store_true")
     ap.add_argument("--no-b16", action="store_true", help="skip the 16-stream int8 leg of the default line")
     ap.add_argument("--suite", action="store_true", help="also print one JSON line per further benchmark config")
@@ -491,6 +547,11 @@ def main():
 
         print(json.dumps(serve_line(synthetic_state_dict(nano_for_cache(args.preset, 64).model, seed=0), args.preset)))
         return
+    if args.sweep_only:
+        from vui_amd.synthetic import nano_for_cache, synthetic_state_dict
+
+        print(json.dumps({"batch_sweep": batch_sweep(synthetic_state_dict(nano_for_cache(args.preset, 64).model, seed=0), args.preset)}))
+        return
     if args.b16_only:
         from vui_amd.synthetic import nano_for_cache, synthetic_state_dict
 
@@ -504,6 +565,9 @@ def main():
         # batch 16 (benchmark configuration 5) beside the batch-1 figure, after its timed region: 16 int8 streams
         # with ragged caches, a bounded number of replays of the captured step
         out["b16"] = b16_line(sd, args.preset, n=60)
+    if not args.no_sweep and not args.suite:
+        del model, eng
+        out["batch_sweep"] = batch_sweep(sd, args.preset)
     extra = suite(model, eng, d, sd, args.preset) if args.suite else []
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.preset)

@@ -188,11 +188,12 @@ def test_config1_greedy_grid_fp32():
 BF16_TOL = 2.0 ** -5  # stated bf16 tolerance: 8 bf16 ulps of the largest logit
 
 
-@pytest.mark.parametrize("fused", [0, 1])
-def test_nano_backbone_bf16_vs_oracle(fused):
+@pytest.mark.parametrize("fused,int8", [(0, False), (1, False), (0, True), (1, True)])
+def test_nano_backbone_bf16_vs_oracle(fused, int8):
     """One decode step at Vui Nano dims in bf16 at cache lengths 0, 255, 1023 and 4095, as a sequence of
     kernels (fused=0) and as the one persistent kernel (fused=1, whose attention split and merge phases are
-    code of their own).
+    code of their own); with bf16 weights and with the backbone's matrices as weight-only int8 (the oracle
+    evaluates the same int8 weights and scales: the quantisation itself is not part of the difference).
 
     With an empty cache the native step equals the oracle's bf16 regime bit for bit (same
     roundings, same per-row summation).  With a filled cache the attention sums run in another
@@ -202,8 +203,10 @@ def test_nano_backbone_bf16_vs_oracle(fused):
     regime, (b) no further from the fp32 evaluation than the oracle's bf16 regime is (x1.3),
     (c) same argmax wherever the oracle's top-2 margin exceeds the tolerance."""
     S = 4608  # cache lengths up to the longest of the benchmark's backbone configurations (4096 keys)
-    d, sd, m, o = _nano_models(BF, S=S)
-    of = O.OracleModel(d, {k: O.rnd(v, BF) for k, v in sd.items()}, F32, max_seqlen=S)
+    d, sd, m, o = _nano_models(BF, int8=int8, S=S)
+    of = O.OracleModel(d, {k: O.rnd(v, BF) for k, v in sd.items()}, F32, max_seqlen=S, int8=int8)
+    if int8:  # the fp32 evaluation takes the very int8 weights of the two bf16 sides
+        of.q8 = o.q8
     m.decoder.allocate_flash_kv_cache(1, m.device, BF, max_seqlen=S)
     assert m._native.fused(fused) == bool(fused), "the fused kernel must be available on an MI355X"
     g = torch.Generator().manual_seed(3)
@@ -227,7 +230,7 @@ def test_nano_backbone_bf16_vs_oracle(fused):
         m.decoder._step(codes=codes.cuda(), emb=None, slot_idx=None, seq_inc=None, B=1, hidden_out=hid,
                         cb0_out=cb0, eos_out=eos, n_splits=32, stream=torch.cuda.current_stream().cuda_stream)
         assert int(m.decoder.flash_kv_caches[0].seq_lens[0]) == L + 1
-        if L == 0 and not fused:
+        if L == 0 and not fused and not int8:
             # no attention sums to reorder: the step follows the oracle's roundings closely (on this input bit for
             # bit when last measured; a rounding tie that falls the other way in one GEMV sum moves a few ulps)
             assert rel_err(cb0, cb_ref) <= 2.0 ** -7 and rel_err(hid, h_ref) <= 2.0 ** -7

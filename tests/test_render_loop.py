@@ -341,8 +341,17 @@ def test_stream_frames_equals_oracle(compile_rq):
     turns = list(render_codes_stream(state, chunks[:1], resume=True, eos_threshold=thr, **kw))
     assert len(turns) == 1 and turns[0][0].shape[1] == d.n_quantizers
     assert state.rewind() == int(om.seq_lens[0])
-    with pytest.raises(NotImplementedError):
-        next(stream_frames(state, chunks, top_p=0.9))
+    # the nucleus cut of _sample_codes (inference.py:491-504): a nucleus too small for a second entry holds the
+    # largest probability alone, so the turn equals the greedy one frame for frame; a wide one runs, stays inside
+    # the codebooks and repeats with the same seed
+    kw_p = dict(kw, top_k=None, top_p=1e-6)
+    tiny = [(f.cpu(), t) for f, t in stream_frames(state, chunks, eos_threshold=thr, **kw_p)]
+    assert len(tiny) == len(got) and all(torch.equal(a, b) for (a, _), (b, _) in zip(tiny, got))
+    kw_w = dict(kw, top_k=20, top_p=0.9, temperature=0.9, seed=3)
+    wide = [f.cpu() for f, _ in stream_frames(state, chunks, eos_threshold=2.0, **kw_w)]
+    again = [f.cpu() for f, _ in stream_frames(state, chunks, eos_threshold=2.0, **kw_w)]
+    assert len(wide) == len(again) > 10 and all(torch.equal(a, b) for a, b in zip(wide, again))
+    assert all(int(f.min()) >= 0 and int(f.max()) < d.codebook_size for f in wide)
 
 
 @pytest.mark.gpu

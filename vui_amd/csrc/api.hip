@@ -307,7 +307,7 @@ static void fused_base(vui_ctx* ctx, FrameArgs& a) {
   a.ll = ctx->ll; a.epoch = ctx->ctl; a.arrive = ctx->ctl + 1; a.err = ctx->ctl + 2;
   a.prof = ctx->prof; a.prof_cap = ctx->prof_cap; a.prof_wg = ctx->prof_wg;
   a.ns = ctx->ns; a.lds_kv_off = (int)(ctx->lds_bytes - frame_rq_lds_cache_bytes(c));
-  a.rq_kg = frame_rq_keys_global(c); a.rq_kscratch = (uint16_t*)ctx->rq_ks;
+  a.rq_kg = frame_rq_keys_global(c); a.rq_kscratch = (uint16_t*)ctx->rq_ks; a.w_int8 = c.int8_backbone;
 }
 static bool use_fused(vui_ctx* ctx, int B) { return ctx->fused_ok && ctx->fused_on && B == 1; }
 

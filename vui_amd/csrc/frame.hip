@@ -64,10 +64,16 @@ __device__ __forceinline__ Plan make_plan(int npairs, int K, int wg, int nwg, in
   return plan_of(pairs_of(npairs, wg, nwg), K, wg, nwg, wave);
 }
 
-template <int MAXC, bool DUAL>
+// I8: the matrix is int8 with one bf16 scale per row (weight-only quantisation): a chunk of eight weights is eight
+// bytes, widened to packed bf16 pairs in registers at the point of use (exact: every int8 is a bf16), and the row's
+// scale multiplies the finished sum.
+template <bool I8> struct WVec { typedef uint4 T; };
+template <> struct WVec<true> { typedef uint2 T; };
+template <int MAXC, bool DUAL, bool I8 = false>
 struct WRegs {
-  uint4 a[2][2][MAXC];
-  uint4 b[DUAL ? 2 : 1][DUAL ? 2 : 1][DUAL ? MAXC : 1];
+  typename WVec<I8>::T a[2][2][MAXC];
+  typename WVec<I8>::T b[DUAL ? 2 : 1][DUAL ? 2 : 1][DUAL ? MAXC : 1];
+  uint32_t sa[I8 ? 2 : 1], sb[(I8 && DUAL) ? 2 : 1];  // int8: the bf16 scales of a slot's two rows, packed
 };
 
 __device__ __forceinline__ void cvt8(const uint4& r, float* o) {
@@ -76,31 +82,65 @@ __device__ __forceinline__ void cvt8(const uint4& r, float* o) {
   o[4] = __uint_as_float(r.z << 16); o[5] = __uint_as_float(r.z & 0xffff0000u);
   o[6] = __uint_as_float(r.w << 16); o[7] = __uint_as_float(r.w & 0xffff0000u);
 }
+// eight int8 -> four packed bf16 pairs (a sign-extending byte conversion per weight, a packing conversion per pair)
+__device__ __forceinline__ uint4 widen8(const uint2& w) {
+  uint4 r;
+  r.x = f2bf2((float)(int8_t)(w.x & 0xff), (float)(int8_t)((w.x >> 8) & 0xff));
+  r.y = f2bf2((float)(int8_t)((w.x >> 16) & 0xff), (float)(int8_t)(w.x >> 24));
+  r.z = f2bf2((float)(int8_t)(w.y & 0xff), (float)(int8_t)((w.y >> 8) & 0xff));
+  r.w = f2bf2((float)(int8_t)((w.y >> 16) & 0xff), (float)(int8_t)(w.y >> 24));
+  return r;
+}
 
-template <int MAXC, bool DUAL>
-__device__ __forceinline__ void gemv_prefetch(const bf16_t* W, const bf16_t* W2, int K, const Plan& p,
-                                              WRegs<MAXC, DUAL>& r) {
+// W, W2: (N, K) row-major bf16, or int8 with the per-row bf16 scales S, S2
+template <int MAXC, bool DUAL, bool I8>
+__device__ __forceinline__ void gemv_prefetch(const void* Wv, const void* W2v, int K, const Plan& p,
+                                              WRegs<MAXC, DUAL, I8>& r, const bf16_t* S = nullptr, const bf16_t* S2 = nullptr) {
   const int lane = threadIdx.x & 63;
+  if constexpr (!I8) {
+    const bf16_t* W = (const bf16_t*)Wv;
+    const bf16_t* W2 = (const bf16_t*)W2v;
 #pragma unroll
-  for (int s = 0; s < 2; ++s)
+    for (int s = 0; s < 2; ++s)
 #pragma unroll
-    for (int rr = 0; rr < 2; ++rr)
+      for (int rr = 0; rr < 2; ++rr)
 #pragma unroll
-      for (int i = 0; i < MAXC; ++i) {
-        const int c = p.c0 + lane + WAVE * i;
-        const bool on = s < p.nslots && c < p.c1;
-        const size_t off = ((size_t)(2 * p.gp[s] + rr)) * K + (size_t)c * 8;
-        r.a[s][rr][i] = on ? *reinterpret_cast<const uint4*>(W + off) : make_uint4(0, 0, 0, 0);
-        if (DUAL) r.b[s][rr][i] = on ? *reinterpret_cast<const uint4*>(W2 + off) : make_uint4(0, 0, 0, 0);
-      }
+        for (int i = 0; i < MAXC; ++i) {
+          const int c = p.c0 + lane + WAVE * i;
+          const bool on = s < p.nslots && c < p.c1;
+          const size_t off = ((size_t)(2 * p.gp[s] + rr)) * K + (size_t)c * 8;
+          r.a[s][rr][i] = on ? *reinterpret_cast<const uint4*>(W + off) : make_uint4(0, 0, 0, 0);
+          if (DUAL) r.b[s][rr][i] = on ? *reinterpret_cast<const uint4*>(W2 + off) : make_uint4(0, 0, 0, 0);
+        }
+  } else {
+    const int8_t* W = (const int8_t*)Wv;
+    const int8_t* W2 = (const int8_t*)W2v;
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int rr = 0; rr < 2; ++rr)
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i) {
+          const int c = p.c0 + lane + WAVE * i;
+          const bool on = s < p.nslots && c < p.c1;
+          const size_t off = ((size_t)(2 * p.gp[s] + rr)) * K + (size_t)c * 8;
+          r.a[s][rr][i] = on ? *reinterpret_cast<const uint2*>(W + off) : make_uint2(0, 0);
+          if (DUAL) r.b[s][rr][i] = on ? *reinterpret_cast<const uint2*>(W2 + off) : make_uint2(0, 0);
+        }
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      r.sa[s] = s < p.nslots ? *reinterpret_cast<const uint32_t*>(S + 2 * p.gp[s]) : 0u;
+      if (DUAL) r.sb[s] = s < p.nslots ? *reinterpret_cast<const uint32_t*>(S2 + 2 * p.gp[s]) : 0u;
+    }
+  }
 }
 
 // xp: K staged activations in LDS as packed bf16 pairs (K/2 words; every activation this kernel
 // multiplies is a bf16 value, so nothing is lost).  red: 4 x 4 floats of LDS.  epi(gp, v0, v1, u0, u1)
 // is called by every lane of the finishing wave (same arguments in all lanes) with the fp32 dot products of
-// rows 2gp, 2gp+1 (u*: second matrix).
-template <int MAXC, bool DUAL, typename Epi>
-__device__ __forceinline__ void gemv_compute(const uint32_t* xp, const Plan& p, const WRegs<MAXC, DUAL>& r, float* red,
+// rows 2gp, 2gp+1 (u*: second matrix), times the rows' scales for int8 weights.
+template <int MAXC, bool DUAL, bool I8, typename Epi>
+__device__ __forceinline__ void gemv_compute(const uint32_t* xp, const Plan& p, const WRegs<MAXC, DUAL, I8>& r, float* red,
                                              Epi&& epi) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;  // the wave index as a scalar
   float res[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
@@ -118,8 +158,13 @@ __device__ __forceinline__ void gemv_compute(const uint32_t* xp, const Plan& p, 
       for (int i = 0; i < MAXC; ++i) {
 #pragma unroll
         for (int rr = 0; rr < 2; ++rr) {
-          acc[s][rr] = dot8_bf(r.a[s][rr][i], x[i], acc[s][rr]);
-          if (DUAL) acc[s][2 + rr] = dot8_bf(r.b[s][rr][i], x[i], acc[s][2 + rr]);
+          if constexpr (I8) {
+            acc[s][rr] = dot8_bf(widen8(r.a[s][rr][i]), x[i], acc[s][rr]);
+            if (DUAL) acc[s][2 + rr] = dot8_bf(widen8(r.b[s][rr][i]), x[i], acc[s][2 + rr]);
+          } else {
+            acc[s][rr] = dot8_bf(r.a[s][rr][i], x[i], acc[s][rr]);
+            if (DUAL) acc[s][2 + rr] = dot8_bf(r.b[s][rr][i], x[i], acc[s][2 + rr]);
+          }
         }
       }
     }
@@ -139,6 +184,14 @@ __device__ __forceinline__ void gemv_compute(const uint32_t* xp, const Plan& p, 
     const float z = wave_sum2(acc[0][0], acc[0][1]);
     res[0][0] = dpp_f<0x00>(z); res[0][1] = dpp_f<0x55>(z);
   }
+  // int8: y[n] = scale[n] * sum_k q[n, k] x[k], the scale applied once to the finished sum
+#define FR_SCALED(s, v0, v1, u0, u1)                                      \
+  do {                                                                    \
+    if constexpr (I8) {                                                   \
+      v0 *= bf_lo(r.sa[s]); v1 *= bf_hi(r.sa[s]);                         \
+      if (DUAL) { u0 *= bf_lo(r.sb[s]); u1 *= bf_hi(r.sb[s]); }           \
+    }                                                                     \
+  } while (0)
   if (p.KS > 1) {  // uniform over the workgroup
     if (lane == 0) { red[wave * 4 + 0] = res[0][0]; red[wave * 4 + 1] = res[0][1]; red[wave * 4 + 2] = res[0][2]; red[wave * 4 + 3] = res[0][3]; }
     __syncthreads();
@@ -147,12 +200,14 @@ __device__ __forceinline__ void gemv_compute(const uint32_t* xp, const Plan& p, 
       for (int k = 0; k < p.KS; ++k)
 #pragma unroll
         for (int j = 0; j < 4; ++j) t[j] += red[(wave + k) * 4 + j];
+      FR_SCALED(0, t[0], t[1], t[2], t[3]);
       epi(p.gp[0], t[0], t[1], t[2], t[3]);
     }
   } else {
-    if (p.nslots > 0) epi(p.gp[0], res[0][0], res[0][1], res[0][2], res[0][3]);
-    if (p.nslots > 1) epi(p.gp[1], res[1][0], res[1][1], res[1][2], res[1][3]);
+    if (p.nslots > 0) { FR_SCALED(0, res[0][0], res[0][1], res[0][2], res[0][3]); epi(p.gp[0], res[0][0], res[0][1], res[0][2], res[0][3]); }
+    if (p.nslots > 1) { FR_SCALED(1, res[1][0], res[1][1], res[1][2], res[1][3]); epi(p.gp[1], res[1][0], res[1][1], res[1][2], res[1][3]); }
   }
+#undef FR_SCALED
 }
 
 // norm weights of a thread's feature pairs (pairs tid and tid + 256), fetched ahead of the wait
@@ -267,11 +322,20 @@ __device__ __forceinline__ void load_logits8(const uint32_t* lgw, int E, int CS,
   }
 }
 
-struct LayerP { const bf16_t *attn_norm, *wqkv, *wo, *mlp_norm, *w1, *w3, *w2; };
+struct LayerP { const bf16_t *attn_norm, *wqkv, *wo, *mlp_norm, *w1, *w3, *w2; };  // the backbone's matrices: bf16 or int8
+// row scales of a backbone layer's int8 matrices: fetched from the weight table one layer ahead (uniform addresses,
+// so the scalar unit does it) and kept in registers - the LDS pointer table has no room to spare
+struct LayerS { const bf16_t *s_qkv, *s_o, *s_1, *s_3, *s_2; };
+__device__ __forceinline__ LayerS load_scales(const vui_weights& W, int l) {
+  const vui_layer_weights& g = W.layers[l];
+  LayerS r = {(const bf16_t*)g.s_qkv, (const bf16_t*)g.s_o, (const bf16_t*)g.s_1, (const bf16_t*)g.s_3, (const bf16_t*)g.s_2};
+  return r;
+}
 
 // KG: the depth head's keys live in a per-workgroup global scratch area instead of LDS (see below); a compile-time
 // switch, so that the common form pays nothing for it.
-template <bool KG>
+// I8: the backbone's five matrices per layer are int8 with per-row scales (the heads and the depth head stay bf16).
+template <bool KG, bool I8>
 __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   float* xres = (float*)(smem + LDS_XRES);
@@ -419,8 +483,14 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
     const int cpd = (hd + 15) / 16;
     const bool mrg_on = wg < a.H * cpd;
 
+    LayerS Ls = {nullptr, nullptr, nullptr, nullptr, nullptr}, Ls_next = Ls;
+    if constexpr (I8) Ls_next = load_scales(W, 0);
     for (int l = 0; l < a.L; ++l) {
       const LayerP Lw = lp[l];
+      if constexpr (I8) {
+        Ls = Ls_next;
+        if (l + 1 < a.L) Ls_next = load_scales(W, l + 1);
+      }
       bf16_t* kcl = a.kc + slab * l;
       bf16_t* vcl = a.vc + slab * l;
       // this layer's window and rotation (src/vui/model.py:406-418, 504-509): a global layer sees the whole cache
@@ -450,9 +520,9 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       const bool att_on = att_s < ns_eff && wg < a.H * NS;
       const int att_lo = start + att_s * chunk, att_hi = min(att_lo + chunk, len);
       // ---- QKV + RoPE + cache append ----
-      WRegs<2, false> wr;
+      WRegs<2, false, I8> wr;
       const Plan P_qkv = plan_of(n_qkv, d, wg, nwg, wave);
-      gemv_prefetch<2, false>(Lw.wqkv, nullptr, d, P_qkv, wr);
+      gemv_prefetch<2, false, I8>(Lw.wqkv, nullptr, d, P_qkv, wr, Ls.s_qkv);
       const NormW nw1 = load_normw(Lw.attn_norm, d);
       TS(1);
       if (ybuf) poll_add(xres, ybuf, d / 2, c);
@@ -462,7 +532,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       TS(3);
       uint64_t* qkvbuf = llp;
       llp += np_qkv;
-      gemv_compute<2, false>(xp, P_qkv, wr, red, [&](int gp, float v0, float v1, float, float) {
+      gemv_compute<2, false, I8>(xp, P_qkv, wr, red, [&](int gp, float v0, float v1, float, float) {
         const bool s0 = (gp == P_qkv.gp[0]);
         float o0 = bf2f(f2bf(v0)), o1 = bf2f(f2bf(v1));
         const int rg = s0 ? l_region[0] : l_region[1];
@@ -641,28 +711,28 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       // ---- out_proj ----
       const RepBuf obuf = rep_alloc(llp, d / 2);
       {
-        WRegs<2, false> w2;
+        WRegs<2, false, I8> w2;
         const Plan P_o = plan_of(n_o, d, wg, nwg, wave);
-        gemv_prefetch<2, false>(Lw.wo, nullptr, d, P_o, w2);
+        gemv_prefetch<2, false, I8>(Lw.wo, nullptr, d, P_o, w2, Ls.s_o);
         poll_words(xp, rep_rd(attbuf), d / 2, c);
         TS(7);
-        gemv_compute<2, false>(xp, P_o, w2, red, [&](int gp, float v0, float v1, float, float) {
+        gemv_compute<2, false, I8>(xp, P_o, w2, red, [&](int gp, float v0, float v1, float, float) {
           rep_st(obuf, gp, pack2(v0, v1), ep); });
       }
       TS(8);
       // ---- SwiGLU ----
       const RepBuf hbuf = rep_alloc(llp, a.F / 2);
       {
-        WRegs<2, true> w3;
+        WRegs<2, true, I8> w3;
         const Plan P_sw = plan_of(n_sw, d, wg, nwg, wave);
-        gemv_prefetch<2, true>(Lw.w1, Lw.w3, d, P_sw, w3);
+        gemv_prefetch<2, true, I8>(Lw.w1, Lw.w3, d, P_sw, w3, Ls.s_1, Ls.s_3);
         const NormW nw2 = load_normw(Lw.mlp_norm, d);
         poll_add(xres, rep_rd(obuf), d / 2, c);
         TS(9);
         stage_norm(xres, nw2, a.eps, d, xp);
         __syncthreads();
         TS(10);
-        gemv_compute<2, true>(xp, P_sw, w3, red, [&](int gp, float v0, float v1, float u0, float u1) {
+        gemv_compute<2, true, I8>(xp, P_sw, w3, red, [&](int gp, float v0, float v1, float u0, float u1) {
           const float a0 = bf2f(f2bf(v0)), a1 = bf2f(f2bf(v1)), c0 = bf2f(f2bf(u0)), c1 = bf2f(f2bf(u1));
           const float s0 = bf2f(f2bf(a0 * __builtin_amdgcn_rcpf(1.0f + __expf(-a0)))), s1 = bf2f(f2bf(a1 * __builtin_amdgcn_rcpf(1.0f + __expf(-a1))));
           rep_st(hbuf, gp, pack2(s0 * c0, s1 * c1), ep);
@@ -672,12 +742,12 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       // ---- W2 ----
       const RepBuf yb = rep_alloc(llp, d / 2);
       {
-        WRegs<4, false> w4;
+        WRegs<4, false, I8> w4;
         const Plan P_w2 = plan_of(n_o, a.F, wg, nwg, wave);
-        gemv_prefetch<4, false>(Lw.w2, nullptr, a.F, P_w2, w4);
+        gemv_prefetch<4, false, I8>(Lw.w2, nullptr, a.F, P_w2, w4, Ls.s_2);
         poll_words(xp, rep_rd(hbuf), a.F / 2, c);
         TS(12);
-        gemv_compute<4, false>(xp, P_w2, w4, red, [&](int gp, float v0, float v1, float, float) {
+        gemv_compute<4, false, I8>(xp, P_w2, w4, red, [&](int gp, float v0, float v1, float, float) {
           rep_st(yb, gp, pack2(v0, v1), ep); });
       }
       ybuf = rep_rd(yb);
@@ -687,7 +757,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
     {
       const Plan p = make_plan(a.CS / 2, d, wg, nwg, wave);
       WRegs<2, false> wr;
-      gemv_prefetch<2, false>(g_codec_head, nullptr, d, p, wr);
+      gemv_prefetch<2, false, false>(g_codec_head, nullptr, d, p, wr);
       const NormW nwf = load_normw(g_final_norm, d);
       uint32_t eosw[8];  // this lane's eos-head weight pairs (pair = lane, lane+64, ...), d <= 1024
 #pragma unroll
@@ -697,7 +767,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       stage_norm(xres, nwf, a.eps, d, xp);
       __syncthreads();
       const RepBuf lgbuf = rep_alloc(llp, a.CS / 2);
-      gemv_compute<2, false>(xp, p, wr, red, [&](int gp, float v0, float v1, float, float) {
+      gemv_compute<2, false, false>(xp, p, wr, red, [&](int gp, float v0, float v1, float, float) {
         const uint32_t pk = pack2(v0, v1);
         rep_st(lgbuf, gp, pk, ep);
         if (a.cb0_out && lane == 0) *reinterpret_cast<uint32_t*>(a.cb0_out + 2 * gp) = pk;
@@ -794,12 +864,12 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
     if (g_rq_proj) {
       const Plan p = make_plan(R / 2, d, wg, nwg, wave);
       WRegs<2, false> wr;
-      gemv_prefetch<2, false>(g_rq_proj, nullptr, d, p, wr);
+      gemv_prefetch<2, false, false>(g_rq_proj, nullptr, d, p, wr);
       // only pairs this wave really owns are inside pos_emb[0, R)
       const uint32_t pe0 = p.nslots > 0 ? *reinterpret_cast<const uint32_t*>(pos_emb + 2 * p.gp[0]) : 0u;
       const uint32_t pe1 = p.nslots > 1 ? *reinterpret_cast<const uint32_t*>(pos_emb + 2 * p.gp[1]) : 0u;
       const RepBuf tb = rep_alloc(llp, R / 2);
-      gemv_compute<2, false>(xp, p, wr, red, [&](int gp, float v0, float v1, float, float) {
+      gemv_compute<2, false, false>(xp, p, wr, red, [&](int gp, float v0, float v1, float, float) {
         const uint32_t pe = (gp == p.gp[0]) ? pe0 : pe1;
         const float o0 = bf2f(f2bf(v0)) + __uint_as_float(pe << 16), o1 = bf2f(f2bf(v1)) + __uint_as_float(pe & 0xffff0000u);
         rep_st(tb, gp, pack2(o0, o1), ep);
@@ -838,13 +908,13 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           TS(30);
           WRegs<2, false> wr;
           const Plan R_qkv = plan_of(m_qkv, R, wg, nwg, wave);
-          gemv_prefetch<2, false>(Lw.wqkv, nullptr, R, R_qkv, wr);
+          gemv_prefetch<2, false, false>(Lw.wqkv, nullptr, R, R_qkv, wr);
           const NormW nw1 = load_normw(Lw.attn_norm, R);
           if (ybuf) poll_add(xres, ybuf, R / 2, c);
           TS(31);
           stage_norm(xres, nw1, a.rq_eps, R, xp);
           __syncthreads();
-          gemv_compute<2, false>(xp, R_qkv, wr, red, [&](int gp, float v0, float v1, float, float) {
+          gemv_compute<2, false, false>(xp, R_qkv, wr, red, [&](int gp, float v0, float v1, float, float) {
             rep_st(qkvb, gp, pack2(v0, v1), ep); });
         }
         const bool kv_only = (t == 0 && l == a.rqL - 1);  // position 0 only feeds later keys/values
@@ -854,7 +924,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
         {
           WRegs<2, false> wr;
           const Plan R_o = plan_of(m_o, R, wg, nwg, wave);
-          if (!kv_only) gemv_prefetch<2, false>(Lw.wo, nullptr, R, R_o, wr);
+          if (!kv_only) gemv_prefetch<2, false, false>(Lw.wo, nullptr, R, R_o, wr);
           __syncthreads();  // xn (A's input) fully consumed before q overwrites it
           ll_poll_auto(rep_rd(qkvb), 3 * R / 2, c, [&](int i, uint32_t v) {
             const int n = 2 * i;
@@ -968,7 +1038,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           }
           __syncthreads();
           TS(33);
-          gemv_compute<2, false>(xp + R / 2, R_o, wr, red, [&](int gp, float v0, float v1, float, float) {
+          gemv_compute<2, false, false>(xp + R / 2, R_o, wr, red, [&](int gp, float v0, float v1, float, float) {
             rep_st(ob, gp, pack2(v0, v1), ep); });
         }
         TS(34);
@@ -977,13 +1047,13 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
         {
           WRegs<2, true> wr;
           const Plan R_sw = plan_of(m_sw, R, wg, nwg, wave);
-          gemv_prefetch<2, true>(Lw.w1, Lw.w3, R, R_sw, wr);
+          gemv_prefetch<2, true, false>(Lw.w1, Lw.w3, R, R_sw, wr);
           const NormW nw2 = load_normw(Lw.mlp_norm, R);
           poll_add(xres, rep_rd(ob), R / 2, c);
           TS(35);
           stage_norm(xres, nw2, a.rq_eps, R, xp);
           __syncthreads();
-          gemv_compute<2, true>(xp, R_sw, wr, red, [&](int gp, float v0, float v1, float u0, float u1) {
+          gemv_compute<2, true, false>(xp, R_sw, wr, red, [&](int gp, float v0, float v1, float u0, float u1) {
             const float a0 = bf2f(f2bf(v0)), a1 = bf2f(f2bf(v1)), c0 = bf2f(f2bf(u0)), c1 = bf2f(f2bf(u1));
             const float s0 = bf2f(f2bf(a0 * __builtin_amdgcn_rcpf(1.0f + __expf(-a0)))), s1 = bf2f(f2bf(a1 * __builtin_amdgcn_rcpf(1.0f + __expf(-a1))));
             rep_st(hb, gp, pack2(s0 * c0, s1 * c1), ep);
@@ -995,10 +1065,10 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
         {
           WRegs<4, false> wr;
           const Plan R_w2 = plan_of(m_o, a.rqF, wg, nwg, wave);
-          gemv_prefetch<4, false>(Lw.w2, nullptr, a.rqF, R_w2, wr);
+          gemv_prefetch<4, false, false>(Lw.w2, nullptr, a.rqF, R_w2, wr);
           poll_words(xp, rep_rd(hb), a.rqF / 2, c);
           TS(37);
-          gemv_compute<4, false>(xp, R_w2, wr, red, [&](int gp, float v0, float v1, float, float) {
+          gemv_compute<4, false, false>(xp, R_w2, wr, red, [&](int gp, float v0, float v1, float, float) {
             rep_st(yb, gp, pack2(v0, v1), ep); });
         }
         ybuf = rep_rd(yb);
@@ -1007,14 +1077,14 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
         // ---- head t-1: logits of codebook t, then the draw in every workgroup ----
         WRegs<2, false> wr;
         const Plan R_hd = plan_of(m_hd, R, wg, nwg, wave);
-        gemv_prefetch<2, false>(g_rq_head + (size_t)(t - 1) * CS * R, nullptr, R, R_hd, wr);
+        gemv_prefetch<2, false, false>(g_rq_head + (size_t)(t - 1) * CS * R, nullptr, R, R_hd, wr);
         TS(40);
         poll_add(xres, ybuf, R / 2, c);
         TS(41);
         stage_norm(xres, nw_rq, a.rq_eps, R, xp);
         __syncthreads();
         const RepBuf lgbuf = rep_alloc(llp, CS / 2);
-        gemv_compute<2, false>(xp, R_hd, wr, red, [&](int gp, float v0, float v1, float, float) {
+        gemv_compute<2, false, false>(xp, R_hd, wr, red, [&](int gp, float v0, float v1, float, float) {
           rep_st(lgbuf, gp, pack2(v0, v1), ep); });
         TS(42);
         const uint32_t rnd = philox_u32(a.seed1, frame1, 0u, (uint32_t)t, 0u);  // ahead of the wait
@@ -1165,7 +1235,6 @@ size_t frame_lds_bytes_backbone(const vui_config& c) { return (size_t)LDS_FIXED 
 bool frame_supported(const vui_config& c, int nwg, int ns, bool with_rq, char* why, size_t why_len) {
   const char* r = nullptr;
   if (c.dtype != VUI_DTYPE_BF16) r = "bf16 only";
-  else if (c.int8_backbone) r = "int8 weights use the per-kernel path";
   else if (c.d_model > 1024 || c.ffn > 2048 || c.rq_dim > 1024 || c.rq_ffn > 2048) r = "vector longer than the LDS staging area";
   else if (c.codebook_size > 2048 || (c.codebook_size & 1)) r = "codebook_size > 2048";
   else if (c.n_quantizers > 64) r = "too many codebooks";
@@ -1201,12 +1270,16 @@ int frame_max_resident(size_t lds_bytes, int* n_cu) {
   if (lds_bytes > lds_attr) {
     // room for the optional phase-clock buffer where it fits
     const size_t want = lds_bytes + frame_prof_lds_bytes() <= 160 * 1024 ? lds_bytes + frame_prof_lds_bytes() : lds_bytes;
-    HIP_TRY(hipFuncSetAttribute((const void*)frame_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)want));
-    HIP_TRY(hipFuncSetAttribute((const void*)frame_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)want));
+    HIP_TRY(hipFuncSetAttribute((const void*)frame_kernel<false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)want));
+    HIP_TRY(hipFuncSetAttribute((const void*)frame_kernel<true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)want));
+    HIP_TRY(hipFuncSetAttribute((const void*)frame_kernel<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)want));
+    HIP_TRY(hipFuncSetAttribute((const void*)frame_kernel<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)want));
     lds_attr = lds_bytes;
   }
-  int occ = 0;
-  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, frame_kernel<true>, FR_THREADS, lds_bytes));
+  int occ = 0, occ8 = 0;
+  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, frame_kernel<true, false>, FR_THREADS, lds_bytes));
+  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ8, frame_kernel<true, true>, FR_THREADS, lds_bytes));
+  if (occ8 < occ) occ = occ8;
   if (n_cu) *n_cu = prop.multiProcessorCount;
   return occ * prop.multiProcessorCount;
 }
@@ -1218,8 +1291,13 @@ int launch_frame(const FrameArgs& a_in, int nwg, size_t lds_bytes, hipStream_t s
     if (lds_bytes + frame_prof_lds_bytes() > 160 * 1024) { vui_set_error("no LDS left for the phase clock"); return VUI_EINVAL; }
     lds_bytes += frame_prof_lds_bytes();
   }
-  if (a.rq_kg) hipLaunchKernelGGL(frame_kernel<true>, dim3(nwg), dim3(FR_THREADS), lds_bytes, st, a);
-  else hipLaunchKernelGGL(frame_kernel<false>, dim3(nwg), dim3(FR_THREADS), lds_bytes, st, a);
+  if (a.w_int8) {
+    if (a.rq_kg) hipLaunchKernelGGL((frame_kernel<true, true>), dim3(nwg), dim3(FR_THREADS), lds_bytes, st, a);
+    else hipLaunchKernelGGL((frame_kernel<false, true>), dim3(nwg), dim3(FR_THREADS), lds_bytes, st, a);
+  } else {
+    if (a.rq_kg) hipLaunchKernelGGL((frame_kernel<true, false>), dim3(nwg), dim3(FR_THREADS), lds_bytes, st, a);
+    else hipLaunchKernelGGL((frame_kernel<false, false>), dim3(nwg), dim3(FR_THREADS), lds_bytes, st, a);
+  }
   HIP_TRY(hipGetLastError());
   return VUI_OK;
 }

@@ -193,6 +193,7 @@ struct FrameArgs {
   int ns;    // attention key splits per head
   int mode;  // FR_* bits
   int lds_kv_off;  // byte offset of the depth-head K/V store in LDS
+  int w_int8;      // 1: the backbone's matrices are int8 with per-row scales
   int rq_kg;       // 1: depth-head keys in rq_kscratch (a region per workgroup), values in LDS
   uint16_t* rq_kscratch;
   uint64_t* prof;  // optional (prof_cap + 1) words: (clock << 8 | tag) per phase point, count in the last word

@@ -138,11 +138,12 @@ __device__ __forceinline__ void ll_poll_n(const uint64_t* buf, int n, Ctl& c, F&
     if (idx < n) sink(idx, (uint32_t)v[i]);
   }
 }
-// picks the round count from the vector length (uniform over the workgroup); an empty vector is no wait at all
-// (the clamped addresses of ll_poll_n would otherwise point in front of the buffer)
+// picks the round count from the vector length (uniform over the workgroup).  Precondition: n >= 1 - the clamped
+// addresses of ll_poll_n would point in front of an empty vector.  Every caller waits for a vector whose length is a
+// model dimension (or a row count that it has tested to be positive), and the host refuses configurations with a
+// zero dimension (check_cfg, rq_batch_supported, the codec's init), so the waits carry no test of their own.
 template <typename F>
 __device__ __forceinline__ void ll_poll_auto(const uint64_t* buf, int n, Ctl& c, F&& sink) {
-  if (n <= 0) return;
   if (n <= FR_THREADS) ll_poll_n<1>(buf, n, c, sink);
   else if (n <= 2 * FR_THREADS) ll_poll_n<2>(buf, n, c, sink);
   else if (n <= 3 * FR_THREADS) ll_poll_n<3>(buf, n, c, sink);
