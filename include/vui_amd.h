@@ -116,7 +116,8 @@ int vui_version(void);
 /* Bytes of device workspace a context needs for up to max_batch rows.  For a configuration that has the one-pass
  * prompt ingestion (vui_prefill) this includes a second copy of the layers' projection weights in the operand
  * layout of its GEMMs (Vui Nano: 311 MB), and for one that has the batched depth-head kernel a copy of the depth
- * head's matrices in that kernel's layout (58 MB); both are written by vui_ctx_init. */
+ * head's matrices in that kernel's layout (58 MB); for a configuration that has the batched backbone kernel a copy of the codec head in its layout
+ * and, with int8 weights, of the layers' int8 matrices (Vui Nano: 3 + 156 MB).  All are written by vui_ctx_init. */
 int64_t vui_workspace_bytes(const vui_config* cfg, int max_batch);
 /* Bytes of ONE of the two (K or V) backbone caches: layers * slots * S * KV * hd elements.
  * Layout (layers, slots, S, KV, hd); layer l's (slots, S, KV, hd) slab is what the reference
@@ -148,6 +149,11 @@ int vui_ctx_fused(vui_ctx* ctx, int enable);
 /* 1 when the depth head of 2..16 rows runs as one persistent kernel (bf16, enough resident workgroups, the
  * fused form switched on), else 0 and vui_last_error() says why.  No counterpart in the reference. */
 int vui_ctx_rq_batch(vui_ctx* ctx);
+/* 1 when the backbone step of 2..16 rows (vui_backbone_step, and through it vui_frame_step) runs as one persistent
+ * kernel (bf16 activations, bf16 or int8 weights, dimensions in multiples of 64, enough resident workgroups, the fused
+ * form switched on), else 0 and vui_last_error() says why; the kernel sequence runs then.  n_splits is not used by the
+ * persistent form: it deals its workgroups to key ranges by the rows' cache lengths.  No counterpart in the reference. */
+int vui_ctx_bb_batch(vui_ctx* ctx);
 /* Synchronous health check (a blocking 16-byte device-to-host copy): VUI_EHIP if a persistent launch gave up
  * waiting for another workgroup, or if the 32-bit launch count of the context has wrapped (after 2^32 - 1
  * persistent launches; the launch that would wrap does nothing).  Either way nothing was committed by the

@@ -9,7 +9,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libvui_amd.so")
-SOURCES = ["gemv.hip", "gemm16.hip", "attn.hip", "misc.hip", "frame.hip", "rqbatch.hip", "prefill.hip", "codec.hip", "api.hip"]
+SOURCES = ["gemv.hip", "gemm16.hip", "attn.hip", "misc.hip", "frame.hip", "rqbatch.hip", "bbatch.hip", "prefill.hip", "codec.hip", "api.hip"]
 FLAGS = [
     "-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
     # packed-fp32 instructions are kept out of every code object of this library
@@ -43,7 +43,7 @@ def build(verbose: bool = True) -> str:
                 print("\n".join(lines), file=sys.stderr)
         return obj
 
-    with ThreadPoolExecutor(max_workers=min(9, len(SOURCES))) as ex:
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
         objs = list(ex.map(one, SOURCES))
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)

@@ -76,6 +76,11 @@ struct vui_ctx {
   // persistent depth head for 2..16 rows
   int rqb_ok;
   char rqb_why[96];
+  // persistent backbone step for 2..16 rows
+  int bb_ok;
+  char bb_why[96];
+  void* bb_w8;    // the layers' int8 matrices in the kernel's operand layout (int8 contexts)
+  void* bb_head;  // the codec head in that layout
 };
 
 #define FUSED_NWG 256
@@ -84,7 +89,9 @@ struct vui_ctx {
 // the batch-1 frame kernel and the batched depth head never run at the same time: one exchange area
 static size_t ll_words_needed(const vui_config& c) {
   const size_t a = frame_ll_words(c, FUSED_NS), b = (c.dtype == VUI_DTYPE_BF16 && c.rq_layers > 0) ? rq_batch_ll_words(c) : 0;
-  return a > b ? a : b;
+  const size_t e = bb_batch_supported(c, FUSED_NWG, nullptr, 0) ? bb_batch_ll_words(c, FUSED_NWG) : 0;
+  const size_t m = a > b ? a : b;
+  return m > e ? m : e;
 }
 
 struct Carve {
@@ -150,6 +157,8 @@ static size_t carve(const vui_config* c, int Bm, vui_ctx* x) {
   TAKE(rq_tw, void*, rq_batch_weight_bytes(*c, FUSED_NWG));  // empty when the batched depth-head kernel is unavailable
   TAKE(wdev_t, vui_weights*, sizeof(vui_weights));
   TAKE(rq_ks, void*, frame_rq_key_scratch_bytes(*c, FUSED_NWG));
+  TAKE(bb_w8, void*, bb_batch_weight8_bytes(*c, FUSED_NWG));  // empty for bf16 weights (the prefill copy serves) or when the kernel is unavailable
+  TAKE(bb_head, void*, bb_batch_head_bytes(*c, FUSED_NWG));
 #undef TAKE
   return cv.off;
 }
@@ -250,6 +259,20 @@ int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream) {
     if (cap < 0) return cap;
     if (cap >= ctx->nwg) ctx->fused_bb_ok = 1;
   }
+  ctx->bb_ok = 0;
+  ctx->bb_why[0] = 0;
+  if (bb_batch_supported(ctx->cfg, ctx->nwg, ctx->bb_why, sizeof(ctx->bb_why))) {
+    const bool i8 = ctx->cfg.int8_backbone != 0;
+    if (!i8 && !prefill_weight_bytes(ctx->cfg)) snprintf(ctx->bb_why, sizeof(ctx->bb_why), "no tiled copy of the bf16 matrices (the prompt-ingestion pass is unavailable)");
+    else {
+      if ((rc = bb_batch_tile_weights(ctx->cfg, ctx->w, i8 ? ctx->bb_w8 : nullptr, ctx->bb_head, st))) return rc;
+      HIP_TRY(hipStreamSynchronize(st));
+      const int cap = bb_batch_max_resident(ctx->cfg);
+      if (cap < 0) return cap;
+      if (cap >= ctx->nwg) ctx->bb_ok = 1;
+      else snprintf(ctx->bb_why, sizeof(ctx->bb_why), "only %d workgroups can be resident, %d needed", cap, ctx->nwg);
+    }
+  }
   ctx->rqb_ok = 0;
   ctx->rqb_why[0] = 0;
   if (rq_batch_supported(ctx->cfg, ctx->nwg, ctx->rqb_why, sizeof(ctx->rqb_why))) {
@@ -278,6 +301,12 @@ int vui_debug_phase_clock(vui_ctx* ctx, uint64_t* buf, int cap, int workgroup) {
   if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
   ctx->prof = buf; ctx->prof_cap = buf ? cap : 0; ctx->prof_wg = workgroup;
   return VUI_OK;
+}
+
+int vui_ctx_bb_batch(vui_ctx* ctx) {
+  if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
+  if (!ctx->bb_ok && ctx->bb_why[0]) vui_set_error("batched backbone kernel unavailable: %s", ctx->bb_why);
+  return (ctx->bb_ok && ctx->fused_on) ? 1 : 0;
 }
 
 int vui_debug_set_epoch(vui_ctx* ctx, uint32_t value) {
@@ -355,6 +384,10 @@ int vui_backbone_step(vui_ctx* ctx, const int64_t* codes_in, const void* emb_in,
     if (!ctx->fused_ok) a.lds_kv_off = (int)ctx->lds_bb;  // no depth-head cache in this launch
     return launch_frame(a, ctx->nwg, ctx->fused_ok ? ctx->lds_bytes : ctx->lds_bb, st);
   }
+  if (ctx->bb_ok && ctx->fused_on && B > 1)
+    return launch_bb_batch(c, ctx->wdev, c.int8_backbone ? ctx->bb_w8 : ctx->pf_w, ctx->bb_head, codes_in, emb_in, slot_idx, seq_lens, seq_inc, B,
+                           k_cache, v_cache, hidden_out ? hidden_out : ctx->hidden, cb0_out ? cb0_out : ctx->cb0,
+                           eos_out ? eos_out : ctx->eos, ctx->ll, ctx->ctl, ctx->nwg, st);
   const int d = c.d_model, H = c.n_heads, KV = c.n_kv_heads, hd = c.head_dim;
   if (codes_in) rc = launch_embed(c.dtype, codes_in, ctx->w.audio_emb, ctx->x, B, c.n_quantizers, c.codebook_size, d, st);
   else rc = launch_copy_rows(c.dtype, emb_in, ctx->x, (int64_t)B * d, st);

@@ -181,6 +181,10 @@ class _Native:
         """True when the depth head of 2..16 rows runs as one persistent kernel."""
         return bool(self.lib.vui_ctx_rq_batch(self.handle))
 
+    def bb_batch(self) -> bool:
+        """True when the backbone step of 2..16 rows runs as one persistent kernel."""
+        return bool(self.lib.vui_ctx_bb_batch(self.handle))
+
     def status(self) -> None:
         _lib.check(self.lib.vui_ctx_status(self.handle), "vui_ctx_status")
 
