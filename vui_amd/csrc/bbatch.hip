@@ -15,9 +15,10 @@
 // Per layer and group:
 //   A  RMSNorm + QKV tiles, rotation of q and k in the epilogue; k and v of the new position go to the cache and,
 //      like q, into the exchange
-//   B  attention over the ragged rows: the group's workgroups are dealt to (row, head, key range) pieces, long
-//      rows getting more pieces; keys and values stream from the cache with 16 loads per lane in flight, the new
-//      position's come from the exchange
+//   B  attention over the ragged rows: the group's workgroups are dealt to (row, set of HG heads, key range) pieces,
+//      long rows getting more key ranges (HG = 2 for 13-16 rows: twice as fine a division as one head set per
+//      workgroup of a 64-workgroup group allows); keys and values stream from the cache with 16 loads per lane in
+//      flight, the new position's come from the exchange
 //   C  merge of a (row, head)'s pieces
 //   D  out_proj tiles
 //   E  residual + RMSNorm + W1/W3 tiles + SwiGLU
@@ -45,7 +46,7 @@ __device__ __forceinline__ void cvt8(const uint4& r, float* o) {
 }
 
 #define BB_RG 4        // rows per row group
-#define BB_MAXSPL 16   // key-range pieces per (row, head) at most
+#define BB_MAXSPL 16   // key ranges per row at most (a merge waits for that many partial results)
 #define BB_U 8         // keys per lane group in flight per attention step
 
 struct BbTile { int n0; bool on; };
@@ -57,16 +58,17 @@ struct BbTile { int n0; bool on; };
 // the lane's 16 bytes (k % 16 = 0..15) at lane * 16.  A wave's fragment load is then 1 KiB contiguous.
 template <bool I8, int MAXS> struct BbW { uint4 a[I8 ? MAXS : 2 * MAXS]; };
 
-template <bool I8, int MAXS>
+// EXACT: K is MAXS * 256, every wave has exactly MAXS steps and nothing is conditional
+template <bool I8, int MAXS, bool EXACT>
 __device__ __forceinline__ void bb_prefetch(const void* Wt, int K, const BbTile& t, BbW<I8, MAXS>& r) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (!t.on) return;  // uniform over the workgroup
-  const int nsteps = K >> 6;
+  const int nsteps = EXACT ? 4 * MAXS : (K >> 6);
   const size_t band = (size_t)(t.n0 >> 4) * nsteps;
 #pragma unroll
   for (int i = 0; i < MAXS; ++i) {
     const int s = wave + 4 * i;
-    if (s < nsteps) {  // uniform over the wave; a step past the end is never used
+    if (EXACT || s < nsteps) {  // uniform over the wave; a step past the end is never used
       if (I8) {
         r.a[i] = *reinterpret_cast<const uint4*>((const uint8_t*)Wt + (band + s) * 1024 + lane * 16);
       } else {
@@ -97,12 +99,12 @@ __device__ __forceinline__ void bb_split(const BbW<I8, MAXS>& w, int i, uint4& a
 // xp: activations as packed bf16 pairs, row stride xs words, row BB_RG all zero (it stands for the columns of the
 // matrix-core tile that have no row).  red: NT x 4 x 64 x (4 | 8) floats.  epi(j, n, lr, v[4], u[4]) is called by the
 // lanes of wave j for tile j: features n .. n+3 of local row lr (u: second matrix).
-template <bool I8, int MAXS, int NT, bool DUAL, typename Epi>
+template <bool I8, int MAXS, int NT, bool DUAL, bool EXACT, typename Epi>
 __device__ __forceinline__ void bb_compute(const uint32_t* xp, int xs, int K, const BbTile (&t)[NT], const BbW<I8, MAXS> (&w)[NT],
                                            const BbW<I8, MAXS> (&w2)[DUAL ? NT : 1], float* red, int nrows, Epi&& epi) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, l16 = lane & 15, kg = lane >> 4;
   if (!t[0].on) return;  // uniform over the workgroup; a later tile is never on without the first
-  const int nsteps = K >> 6;
+  const int nsteps = EXACT ? 4 * MAXS : (K >> 6);
   bb_floatx4 acc[NT], acc2[NT];
 #pragma unroll
   for (int j = 0; j < NT; ++j) { acc[j] = bb_floatx4{0.f, 0.f, 0.f, 0.f}; acc2[j] = acc[j]; }
@@ -110,7 +112,7 @@ __device__ __forceinline__ void bb_compute(const uint32_t* xp, int xs, int K, co
 #pragma unroll
   for (int i = 0; i < MAXS; ++i) {
     const int s = wave + 4 * i;
-    if (s < nsteps) {  // uniform over the wave: the matrix instructions below run for all 64 lanes
+    if (EXACT || s < nsteps) {  // uniform over the wave: the matrix instructions below run for all 64 lanes
       const uint4 x0 = *reinterpret_cast<const uint4*>(xrow + 32 * s);
       const uint4 x1 = *reinterpret_cast<const uint4*>(xrow + 32 * s + 4);
 #pragma unroll
@@ -269,28 +271,31 @@ __device__ __forceinline__ void bb_poll_add_norm_rows(const uint64_t* buf, const
 // i / n for 0 <= i < 65536 with inv = ceil(2^32 / n)
 __device__ __forceinline__ int bb_div(int i, uint32_t inv) { return (int)__umulhi((uint32_t)i, inv); }
 
-// Wait for `nrows` rows of `len` words each (row b at buf + rowoff[r0 + b]) and put them into xp rows 0.. as they are.
-__device__ __forceinline__ void bb_poll_rows(const uint64_t* buf, const int* rowoff, int r0, int nrows, int len, uint32_t inv_len, Ctl& c,
-                                             uint32_t* xp, int xs) {
+// Wait for `nrows` rows of `len` words each (row b at buf + rowbase(r0 + b), words) and put them into xp rows 0.. as
+// they are.  Every thread has NW words in flight per round (one trip to memory for 256 * NW words when the data
+// is there).
+template <int NW, typename RowBase>
+__device__ __forceinline__ void bb_poll_rows_n(const uint64_t* buf, RowBase&& rowbase, int r0, int nrows, int len, uint32_t inv_len, Ctl& c,
+                                               uint32_t* xp, int xs) {
   const int n = nrows * len;
-  for (int base = 0; base < n; base += FR_THREADS * 4) {
-    const uint64_t* p[4];
-    int lr[4], j[4];
+  for (int base = 0; base < n; base += FR_THREADS * NW) {
+    const uint64_t* p[NW];
+    int dst[NW];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < NW; ++i) {
       const int idx = min(base + (int)threadIdx.x + FR_THREADS * i, n - 1);
-      lr[i] = bb_div(idx, inv_len);
-      j[i] = idx - lr[i] * len;
-      p[i] = buf + rowoff[r0 + lr[i]] + j[i];
+      const int lr = bb_div(idx, inv_len), j = idx - lr * len;
+      p[i] = buf + rowbase(r0 + lr) + j;
+      dst[i] = lr * xs + j;
     }
-    uint64_t v[4];
+    uint64_t v[NW];
     int spins = 0;
     while (true) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = ll_ld(p[i]);
+      for (int i = 0; i < NW; ++i) v[i] = ll_ld(p[i]);
       uint32_t bad = 0;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) bad |= (uint32_t)(v[i] >> 32) ^ c.epoch;
+      for (int i = 0; i < NW; ++i) bad |= (uint32_t)(v[i] >> 32) ^ c.epoch;
       if (bad == 0u || c.dead) break;
       if (++spins > SPIN_LIMIT) {
         c.dead = 1;
@@ -298,9 +303,19 @@ __device__ __forceinline__ void bb_poll_rows(const uint64_t* buf, const int* row
       }
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (base + (int)threadIdx.x + FR_THREADS * i < n) xp[(size_t)lr[i] * xs + j[i]] = (uint32_t)v[i];
+    for (int i = 0; i < NW; ++i)
+      if (base + (int)threadIdx.x + FR_THREADS * i < n) xp[dst[i]] = (uint32_t)v[i];
   }
+}
+// picks the words in flight from the vector length (uniform over the workgroup)
+template <typename RowBase>
+__device__ __forceinline__ void bb_poll_rows(const uint64_t* buf, RowBase&& rowbase, int r0, int nrows, int len, uint32_t inv_len, Ctl& c,
+                                             uint32_t* xp, int xs) {
+  const int n = nrows * len;
+  if (n <= 2 * FR_THREADS) bb_poll_rows_n<2>(buf, rowbase, r0, nrows, len, inv_len, c, xp, xs);
+  else if (n <= 4 * FR_THREADS) bb_poll_rows_n<4>(buf, rowbase, r0, nrows, len, inv_len, c, xp, xs);
+  else if (n <= 8 * FR_THREADS) bb_poll_rows_n<8>(buf, rowbase, r0, nrows, len, inv_len, c, xp, xs);
+  else bb_poll_rows_n<16>(buf, rowbase, r0, nrows, len, inv_len, c, xp, xs);
 }
 
 struct BbArgs {
@@ -319,7 +334,11 @@ struct BbArgs {
   uint64_t* ll;
   uint32_t *epoch, *arrive, *err;
   int xs;
+  int hg;                                  // heads per attention piece (1, 2, 4 or 8; divides H)
+  int min_keys;                            // no key range shorter than this is made by splitting
   int off_xp, off_red, off_att, off_misc;  // LDS offsets, bytes (xres at 0)
+  unsigned long long* dbg;                 // profiling builds: 256 words for the phase stamps of workgroup dbg_wg
+  int dbg_wg;
 };
 
 // small per-workgroup state in LDS
@@ -327,12 +346,14 @@ struct BbMisc {
   int lens[VUI_MAX_BATCH], slots[VUI_MAX_BATCH], order[VUI_MAX_BATCH];
   int grow[BB_RG], gslot[BB_RG], gpos[BB_RG];  // batch row, cache slot and position of the group's rows
   int off_q[BB_RG], off_d[BB_RG], off_f[BB_RG];  // word offsets of the rows in exchange vectors of nqkv/2, d/2, F/2 words
-  int spl[2][BB_RG], poff[2][BB_RG + 1];        // attention plan (0: windowed layers, 1: global layers): pieces per head, first piece
+  int spl[2][BB_RG], poff[2][BB_RG + 1];        // attention plan (0: windowed layers, 1: global layers): key ranges per row, first piece
   int Bg;
   int erow[BB_RG][64];                          // embedding table rows of the group's input codes
 };
 
-template <bool I8, int NTQ>
+// SD, SF: K steps (of 64) per wave for K = d_model (and heads x head_dim) and K = ffn.  EXACT: d_model = heads x
+// head_dim = SD * 256 and ffn = SF * 256, so no step is conditional (the Vui Nano form).
+template <bool I8, int NTQ, int SD, int SF, bool EXACT>
 __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   float* xres = (float*)smem;                             // [BB_RG][d] residual stream of the group's rows
@@ -388,8 +409,8 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
     }
     for (int lr = Bg; lr < BB_RG; ++lr) { ms.grow[lr] = 0; ms.gslot[lr] = 0; ms.gpos[lr] = 0; ms.off_q[lr] = 0; ms.off_d[lr] = 0; ms.off_f[lr] = 0; }
     ms.Bg = Bg;
-    // attention plans: one piece per (row, head) to start with; the spare workgroups go, one set of heads at a time,
-    // to the row whose pieces are longest (no piece below 64 keys)
+    // attention plans: one key range per row to start with (H / HG pieces); the spare workgroups go, one set of
+    // pieces at a time, to the row whose ranges are longest (no range below 32 keys)
     for (int v = 0; v < 2; ++v) {
       int nk[BB_RG], sp[BB_RG];
       for (int lr = 0; lr < BB_RG; ++lr) {
@@ -398,19 +419,19 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
         nk[lr] = len - start;
         sp[lr] = lr < Bg ? 1 : 0;
       }
-      int spare = NWL / H - Bg;
+      int spare = NWL / (H / a.hg) - Bg;
       while (spare > 0) {
-        int best = -1, bestv = 64;
-        for (int lr = 0; lr < Bg; ++lr) {
+        int best = -1, bestv = 0;
+        for (int lr = 0; lr < Bg; ++lr) {  // the row with the longest ranges that one more range leaves at min_keys or above
           const int per = (nk[lr] + sp[lr] - 1) / sp[lr];
-          if (sp[lr] < BB_MAXSPL && per > bestv) { bestv = per; best = lr; }
+          if (sp[lr] < BB_MAXSPL && nk[lr] >= (sp[lr] + 1) * a.min_keys && per > bestv) { bestv = per; best = lr; }
         }
         if (best < 0) break;
         ++sp[best];
         --spare;
       }
       int off = 0;
-      for (int lr = 0; lr < BB_RG; ++lr) { ms.spl[v][lr] = sp[lr]; ms.poff[v][lr] = off; off += sp[lr] * H; }
+      for (int lr = 0; lr < BB_RG; ++lr) { ms.spl[v][lr] = sp[lr]; ms.poff[v][lr] = off; off += sp[lr] * (H / a.hg); }
       ms.poff[v][BB_RG] = off;
     }
   }
@@ -473,9 +494,15 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
   const size_t wsz = I8 ? 1 : 2;
   const size_t layer_elems = (size_t)nqkv * d + (size_t)d * nq + 3 * (size_t)F * d;
   const size_t slab = (size_t)a.n_slots * S * nkv;
-  constexpr int SD = 4;   // K steps per wave for K = d (d <= 1024)
-  constexpr int SF = 8;   // for K = ffn (ffn <= 2048)
 
+#ifdef VUI_BB_CLOCK
+  __shared__ unsigned long long dbg_ts[256];
+  int dbg_n = 0;
+#define BB_TS() do { if (a.dbg && wg == a.dbg_wg && tid == 0 && dbg_n < 255) dbg_ts[dbg_n++] = wall_clock64(); } while (0)
+#else
+#define BB_TS() do { } while (0)
+#endif
+  BB_TS();
   uint64_t* llp = a.ll;
   const uint64_t* ybuf = nullptr;  // previous layer's W2 output, still to be added
   for (int l = 0; l < a.L; ++l) {
@@ -495,6 +522,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
     const int rope_dim_l = (glob && W.rope_table_global) ? a.global_rope_dim : a.rope_dim;
 
     // ---- A: RMSNorm + QKV, rotation, cache append ----
+    BB_TS();
     uint64_t* qkvb = llp;
     llp += (size_t)B * (nqkv / 2);
     if (active) {
@@ -502,7 +530,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
       BbW<I8, SD> w[NTQ];
       const BbW<I8, SD> nodual[1] = {};
 #pragma unroll
-      for (int j = 0; j < NTQ; ++j) { t[j] = tile_of(j, nA); bb_prefetch<I8, SD>(t_qkv, d, t[j], w[j]); }
+      for (int j = 0; j < NTQ; ++j) { t[j] = tile_of(j, nA); bb_prefetch<I8, SD, EXACT>(t_qkv, d, t[j], w[j]); }
       const BbNorm nw = bb_load_norm((const bf16_t*)Lw.attn_norm, d);
       // what the epilogue of this lane will need (wave j < NTQ: tile j, local row l16, features n .. n + 3): scales,
       // the row's position and its rotation factors, requested now
@@ -526,7 +554,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
       if (ybuf) bb_poll_add_norm_rows(ybuf, ms.off_d, c, xres, nw, a.eps, d, Bg, xp, xs);
       else bb_norm_rows(xres, nw, a.eps, d, Bg, xp, xs);
       __syncthreads();
-      bb_compute<I8, SD, NTQ, false>(xp, xs, d, t, w, nodual, red, Bg, [&](int, int n, int lr, const float* v, const float*) {
+      bb_compute<I8, SD, NTQ, false, EXACT>(xp, xs, d, t, w, nodual, red, Bg, [&](int, int n, int lr, const float* v, const float*) {
         float o[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) o[r] = v[r];
@@ -548,16 +576,22 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
     }
 
     // ---- B: attention pieces ----
-    uint64_t* part = llp;  // piece p of group g at (g * NWL + p) * (hd + 2)
-    llp += (size_t)nwg * (hd + 2);
+    BB_TS();
+    const int pw_ = hd + 2;                 // words of one head's partial result: max, sum, acc[hd]
+    const int HG = a.hg, NHQ = H / HG;      // heads per piece, head sets per row
+    uint64_t* part = llp;                   // piece p of group g at (g * NWL + p) * HG * pw_, its head hs at + hs * pw_
+    llp += (size_t)nwg * HG * pw_;
     if (active) {
       const int npieces = ms.poff[plan][BB_RG];
+      // lane groups of 16: head slot hs = group % HG, key slot ks = group / HG
+      const int KP = 16 / HG;  // keys a workgroup takes per step and load round
+      const int G = H / a.KV;
       for (int p = wl; p < npieces; p += NWL) {  // uniform over the workgroup; one piece per workgroup as a rule
         int lr = 0;
 #pragma unroll
         for (int r = 1; r < BB_RG; ++r) if (p >= ms.poff[plan][r]) lr = r;
         const int rel = p - ms.poff[plan][lr];
-        const int sp = rel / H, h = rel - sp * H;
+        const int sp = rel / NHQ, hq = rel - sp * NHQ;
         const int nsp = ms.spl[plan][lr];
         const int pos = ms.gpos[lr], slot = ms.gslot[lr], len = pos + 1;
         const int start = win_l > 0 ? max(0, len - 1 - win_l) : 0;
@@ -565,8 +599,10 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
         chunk = (chunk + 15) & ~15;
         const int lo = start + sp * chunk, hi = min(lo + chunk, len);
         const bool has_new = pos >= lo && pos < hi;
-        const int kvh = h / (H / a.KV);
         const int g = wave * 4 + (lane >> 4);
+        const int hs = g & (HG - 1), ks = g / HG;
+        const int h = hq * HG + hs;
+        const int kvh = h / G, kvh0 = (hq * HG) / G, nkvh = (hq * HG + HG - 1) / G - kvh0 + 1;
         const bool act = l16 * 8 < hd;
         const size_t rowstride = (size_t)nkv;
         const bf16_t* kbase = kcl + ((size_t)slot * S) * rowstride + kvh * hd + (act ? l16 * 8 : 0);
@@ -576,63 +612,82 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
         uint4 kr[BB_U], vr[BB_U];
 #pragma unroll
         for (int u = 0; u < BB_U; ++u) {
-          const int j = min(lo + g + 16 * u, hi - 1);  // hi >= 1
+          const int j = min(lo + ks + KP * u, hi - 1);  // hi >= 1
           kr[u] = *reinterpret_cast<const uint4*>(kbase + (size_t)j * rowstride);
           vr[u] = *reinterpret_cast<const uint4*>(vbase + (size_t)j * rowstride);
         }
-        float* qh = att;                 // q | new k | new v, 128 floats each
-        float* gm = att + 384;           // 16 maxima, 16 sums, 16 weights
-        float* gacc = att + 448;         // 16 x 128
-        float* fin = att + 448 + 2048;   // max, sum, acc[hd]
-        const int hw = hd / 2;
+        uint32_t* qw = (uint32_t*)att;   // q of the piece's heads | new k | new v of their KV heads, packed pairs (<= 1536 words)
+        float* gm = att + 1536;          // 16 maxima, 16 sums, 16 weights, 16 head maxima
+        float* gacc = att + 1536 + 64;   // 16 x 128
+        const int nqw = HG * hd / 2, nkw = nkvh * hd / 2;
         __syncthreads();
         {
+          // one wait for everything the piece needs of the row: q of its heads and, where the new position is in the
+          // piece, the key and value of their KV heads
           const uint64_t* row = qkvb + ms.off_q[lr];
-          const uint64_t* p0 = tid < hw ? row + (h * hd) / 2 + tid : nullptr;
-          const uint64_t* p1 = (has_new && tid < hw) ? row + (nq + kvh * hd) / 2 + tid : nullptr;
-          const uint64_t* p2 = (has_new && tid < hw) ? row + (nq + nkv + kvh * hd) / 2 + tid : nullptr;
-          uint32_t r0, r1, r2;
-          poll3(p0, p1, p2, c, r0, r1, r2);
-          if (tid < hw) {
-            qh[2 * tid] = bf_lo(r0); qh[2 * tid + 1] = bf_hi(r0);
-            qh[128 + 2 * tid] = bf_lo(r1); qh[128 + 2 * tid + 1] = bf_hi(r1);
-            qh[256 + 2 * tid] = bf_lo(r2); qh[256 + 2 * tid + 1] = bf_hi(r2);
+          const uint64_t* rq_ = row + (hq * HG * hd) / 2;
+          const uint64_t* rk_ = row + (nq + kvh0 * hd) / 2 - nqw;
+          const uint64_t* rv_ = row + (nq + nkv + kvh0 * hd) / 2 - nqw - nkw;
+          const int n = nqw + (has_new ? 2 * nkw : 0);
+          for (int base = 0; base < n; base += FR_THREADS * 2) {
+            const uint64_t* pp[2];
+            int idx[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+              idx[i] = min(base + tid + FR_THREADS * i, n - 1);
+              pp[i] = (idx[i] < nqw ? rq_ : (idx[i] < nqw + nkw ? rk_ : rv_)) + idx[i];
+            }
+            uint64_t v[2];
+            int spins = 0;
+            while (true) {
+#pragma unroll
+              for (int i = 0; i < 2; ++i) v[i] = ll_ld(pp[i]);
+              const uint32_t bad = ((uint32_t)(v[0] >> 32) ^ ep) | ((uint32_t)(v[1] >> 32) ^ ep);
+              if (bad == 0u || c.dead) break;
+              if (++spins > SPIN_LIMIT) { c.dead = 1; __hip_atomic_store(c.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+              if (base + tid + FR_THREADS * i < n) qw[idx[i]] = (uint32_t)v[i];
           }
         }
         __syncthreads();
         const float scale = 1.0f / sqrtf((float)hd);
         float q8[8], kn8[8], vn8[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          q8[e] = act ? qh[l16 * 8 + e] : 0.f;
-          kn8[e] = act ? qh[128 + l16 * 8 + e] : 0.f;
-          vn8[e] = act ? qh[256 + l16 * 8 + e] : 0.f;
+        {
+          const uint4 z4 = make_uint4(0, 0, 0, 0);
+          const uint4 qv = act ? *reinterpret_cast<const uint4*>(qw + (hs * hd + l16 * 8) / 2) : z4;
+          cvt8(qv, q8);
+          const uint4 kv_ = (act && has_new) ? *reinterpret_cast<const uint4*>(qw + nqw + ((kvh - kvh0) * hd + l16 * 8) / 2) : z4;
+          cvt8(kv_, kn8);
+          const uint4 vv_ = (act && has_new) ? *reinterpret_cast<const uint4*>(qw + nqw + nkw + ((kvh - kvh0) * hd + l16 * 8) / 2) : z4;
+          cvt8(vv_, vn8);
         }
         float m = -INFINITY, lsum = 0.f, acc[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-        for (int j0 = lo + g; j0 < hi; j0 += 16 * BB_U) {
+        for (int j0 = lo + ks; j0 < hi; j0 += KP * BB_U) {
           // the next step's keys and values go out before this step's arithmetic
           uint4 kn[BB_U], vn[BB_U];
 #pragma unroll
           for (int u = 0; u < BB_U; ++u) {
-            const int j = min(j0 + 16 * BB_U + 16 * u, hi - 1);  // past the piece: its last key again, never used
+            const int j = min(j0 + KP * BB_U + KP * u, hi - 1);  // past the piece: its last key again, never used
             kn[u] = *reinterpret_cast<const uint4*>(kbase + (size_t)j * rowstride);
             vn[u] = *reinterpret_cast<const uint4*>(vbase + (size_t)j * rowstride);
           }
-          float s[BB_U];
+          float sc_[BB_U];
           float mn = m;
 #pragma unroll
           for (int u = 0; u < BB_U; ++u) {
-            const int j = j0 + 16 * u;
+            const int j = j0 + KP * u;
             float k8[8];
             cvt8(kr[u], k8);
             float dsum = 0.f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) dsum = fmaf(q8[e], (j == pos) ? kn8[e] : k8[e], dsum);
             dsum = group16_sum(act ? dsum : 0.f) * scale;
-            s[u] = j < hi ? dsum : -INFINITY;
-            mn = fmaxf(mn, s[u]);
+            sc_[u] = j < hi ? dsum : -INFINITY;
+            mn = fmaxf(mn, sc_[u]);
           }
           const float r = expf(m - mn);  // 0 on the first step (m = -inf); mn is finite: j0 < hi
           lsum *= r;
@@ -640,8 +695,8 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
           for (int e = 0; e < 8; ++e) acc[e] *= r;
 #pragma unroll
           for (int u = 0; u < BB_U; ++u) {
-            const int j = j0 + 16 * u;
-            const float pw = expf(s[u] - mn);  // 0 for a key beyond the piece
+            const int j = j0 + KP * u;
+            const float pw = expf(sc_[u] - mn);  // 0 for a key beyond the piece
             lsum += pw;
             float v8[8];
             cvt8(vr[u], v8);
@@ -652,46 +707,45 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
 #pragma unroll
           for (int u = 0; u < BB_U; ++u) { kr[u] = kn[u]; vr[u] = vn[u]; }
         }
-        // the 16 lane groups -> the piece
+        // the key slots of a head -> the head's partial result
         if (l16 == 0) { gm[g] = m; gm[16 + g] = lsum; }
         if (act) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) gacc[g * 128 + l16 * 8 + e] = acc[e];
         }
         __syncthreads();
-        if (tid < 16) {
+        if (tid < 16) {  // weight of lane group tid inside its head: exp(m - max over the head's key slots)
+          const int hs_ = tid & (HG - 1);
           float M = -INFINITY;
-#pragma unroll
-          for (int i = 0; i < 16; ++i) M = fmaxf(M, gm[i]);
+          for (int k2 = 0; k2 < KP; ++k2) M = fmaxf(M, gm[hs_ + HG * k2]);
           gm[32 + tid] = (gm[tid] == -INFINITY) ? 0.f : expf(gm[tid] - M);
-          if (tid == 0) fin[0] = M;
+          gm[48 + tid] = M;
         }
         __syncthreads();
-        uint64_t* po = part + ((size_t)grp * NWL + p) * (hd + 2);
-        if (tid < hd) {
-          float o = 0.f;
-#pragma unroll
-          for (int i = 0; i < 16; ++i) o = fmaf(gm[32 + i], gacc[i * 128 + tid], o);
-          ll_st(po + 2 + tid, __float_as_uint(o), ep);
-        }
-        if (tid == 128) {
-          float Lt = 0.f;
-#pragma unroll
-          for (int i = 0; i < 16; ++i) Lt = fmaf(gm[32 + i], gm[16 + i], Lt);
-          ll_st(po, __float_as_uint(fin[0]), ep);
-          ll_st(po + 1, __float_as_uint(Lt), ep);
+        uint64_t* po = part + ((size_t)grp * NWL + p) * HG * pw_;
+        for (int i = tid; i < HG * pw_; i += FR_THREADS) {
+          const int hh = i / pw_, j = i - hh * pw_;
+          float o;
+          if (j == 0) o = gm[48 + hh];
+          else if (j == 1) { o = 0.f; for (int k2 = 0; k2 < KP; ++k2) o = fmaf(gm[32 + hh + HG * k2], gm[16 + hh + HG * k2], o); }
+          else { o = 0.f; for (int k2 = 0; k2 < KP; ++k2) o = fmaf(gm[32 + hh + HG * k2], gacc[(hh + HG * k2) * 128 + j - 2], o); }
+          ll_st(po + i, __float_as_uint(o), ep);
         }
       }
     }
 
     // ---- C: merge the pieces of (row, head) ----
+    BB_TS();
     uint64_t* attb = llp;
     llp += (size_t)B * (nq / 2);
     if (mrg_on) {
       const int nsp = ms.spl[plan][mrg_lr];
-      const uint64_t* pb = part + ((size_t)grp * NWL + ms.poff[plan][mrg_lr] + mrg_h) * (hd + 2);  // piece sp at + sp * H * (hd + 2)
-      float* pieces = red;  // nsp x (hd + 2)
-      const int pw_ = hd + 2, n = nsp * pw_;
+      const int mhq = mrg_h / HG, mhs = mrg_h - mhq * HG;
+      // key range sp of the head's set is piece poff + sp * NHQ + mhq
+      const uint64_t* pb = part + (((size_t)grp * NWL + ms.poff[plan][mrg_lr] + mhq) * HG + mhs) * pw_;
+      const size_t pstride = (size_t)NHQ * HG * pw_;
+      float* pieces = red;  // nsp x pw_
+      const int n = nsp * pw_;
       __syncthreads();
       for (int base = 0; base < n; base += FR_THREADS * 4) {
         const uint64_t* pp[4];
@@ -700,7 +754,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
         for (int i = 0; i < 4; ++i) {
           idx[i] = min(base + tid + FR_THREADS * i, n - 1);
           const int sp = idx[i] / pw_, j = idx[i] - sp * pw_;
-          pp[i] = pb + (size_t)sp * H * pw_ + j;
+          pp[i] = pb + (size_t)sp * pstride + j;
         }
         uint64_t v[4];
         int spins = 0;
@@ -735,48 +789,21 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
     }
 
     // ---- D: out_proj ----
+    BB_TS();
     uint64_t* ob = llp;
     llp += (size_t)B * (d / 2);
     if (out_on) {
       BbTile t[1] = {{16 * out_tile, true}};
       BbW<I8, SD> w[1];
       const BbW<I8, SD> nodual[1] = {};
-      bb_prefetch<I8, SD>(t_o, nq, t[0], w[0]);
+      bb_prefetch<I8, SD, EXACT>(t_o, nq, t[0], w[0]);
       const int en = t[0].n0 + 4 * kg;
       uint2 esc = make_uint2(0, 0);
       if (I8) esc = *reinterpret_cast<const uint2*>((const bf16_t*)Lw.s_o + en);
       __syncthreads();
-      // rows of attb are nq/2 words at row * (nq / 2): the d/2 offsets apply only when nq == d, so use explicit ones
-      {
-        const int len = nq / 2, n = out_nr * len;
-        for (int base = 0; base < n; base += FR_THREADS * 4) {
-          const uint64_t* pp[4];
-          int lr_[4], j_[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int idx = min(base + tid + FR_THREADS * i, n - 1);
-            lr_[i] = bb_div(idx, inv_q2);
-            j_[i] = idx - lr_[i] * len;
-            pp[i] = attb + (size_t)ms.grow[out_r0 + lr_[i]] * len + j_[i];
-          }
-          uint64_t v[4];
-          int spins = 0;
-          while (true) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) v[i] = ll_ld(pp[i]);
-            uint32_t bad = 0;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) bad |= (uint32_t)(v[i] >> 32) ^ ep;
-            if (bad == 0u || c.dead) break;
-            if (++spins > SPIN_LIMIT) { c.dead = 1; __hip_atomic_store(c.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-          }
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            if (base + tid + FR_THREADS * i < n) xp[(size_t)lr_[i] * xs + j_[i]] = (uint32_t)v[i];
-        }
-      }
+      bb_poll_rows(attb, [&](int r) { return (size_t)ms.grow[r] * (nq / 2); }, out_r0, out_nr, nq / 2, inv_q2, c, xp, xs);
       __syncthreads();
-      bb_compute<I8, SD, 1, false>(xp, xs, nq, t, w, nodual, red, out_nr, [&](int, int n, int lr, const float* v, const float*) {
+      bb_compute<I8, SD, 1, false, EXACT>(xp, xs, nq, t, w, nodual, red, out_nr, [&](int, int n, int lr, const float* v, const float*) {
         float o[4] = {v[0], v[1], v[2], v[3]};
         if (I8) { o[0] *= bf_lo(esc.x); o[1] *= bf_hi(esc.x); o[2] *= bf_lo(esc.y); o[3] *= bf_hi(esc.y); }
         uint64_t* dst = ob + ms.off_d[out_r0 + lr] + n / 2;
@@ -786,13 +813,14 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
     }
 
     // ---- E: residual, RMSNorm, W1/W3, SwiGLU ----
+    BB_TS();
     uint64_t* hb = llp;
     llp += (size_t)B * (F / 2);
     if (active) {
       BbTile t[2] = {tile_of(0, nS), tile_of(1, nS)};
       BbW<I8, SD> w[2], w3[2];
 #pragma unroll
-      for (int j = 0; j < 2; ++j) { bb_prefetch<I8, SD>(t_1, d, t[j], w[j]); bb_prefetch<I8, SD>(t_3, d, t[j], w3[j]); }
+      for (int j = 0; j < 2; ++j) { bb_prefetch<I8, SD, EXACT>(t_1, d, t[j], w[j]); bb_prefetch<I8, SD, EXACT>(t_3, d, t[j], w3[j]); }
       const BbNorm nw = bb_load_norm((const bf16_t*)Lw.mlp_norm, d);
       int en = 0;
 #pragma unroll
@@ -802,7 +830,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
       if (I8) { esc = *reinterpret_cast<const uint2*>((const bf16_t*)Lw.s_1 + en); esc3 = *reinterpret_cast<const uint2*>((const bf16_t*)Lw.s_3 + en); }
       bb_poll_add_norm_rows(ob, ms.off_d, c, xres, nw, a.eps, d, Bg, xp, xs);
       __syncthreads();
-      bb_compute<I8, SD, 2, true>(xp, xs, d, t, w, w3, red, Bg, [&](int, int n, int lr, const float* v, const float* u) {
+      bb_compute<I8, SD, 2, true, EXACT>(xp, xs, d, t, w, w3, red, Bg, [&](int, int n, int lr, const float* v, const float* u) {
         float g1[4] = {v[0], v[1], v[2], v[3]}, g3[4] = {u[0], u[1], u[2], u[3]};
         if (I8) {
           g1[0] *= bf_lo(esc.x); g1[1] *= bf_hi(esc.x); g1[2] *= bf_lo(esc.y); g1[3] *= bf_hi(esc.y);
@@ -821,20 +849,21 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
     }
 
     // ---- F: W2 ----
+    BB_TS();
     uint64_t* yb = llp;
     llp += (size_t)B * (d / 2);
     if (out_on) {
       BbTile t[1] = {{16 * out_tile, true}};
       BbW<I8, SF> w[1];
       const BbW<I8, SF> nodual[1] = {};
-      bb_prefetch<I8, SF>(t_2, F, t[0], w[0]);
+      bb_prefetch<I8, SF, EXACT>(t_2, F, t[0], w[0]);
       const int en = t[0].n0 + 4 * kg;
       uint2 esc = make_uint2(0, 0);
       if (I8) esc = *reinterpret_cast<const uint2*>((const bf16_t*)Lw.s_2 + en);
       __syncthreads();
-      bb_poll_rows(hb, ms.off_f, out_r0, out_nr, F / 2, inv_f2, c, xp, xs);
+      bb_poll_rows(hb, [&](int r) { return (size_t)ms.off_f[r]; }, out_r0, out_nr, F / 2, inv_f2, c, xp, xs);
       __syncthreads();
-      bb_compute<I8, SF, 1, false>(xp, xs, F, t, w, nodual, red, out_nr, [&](int, int n, int lr, const float* v, const float*) {
+      bb_compute<I8, SF, 1, false, EXACT>(xp, xs, F, t, w, nodual, red, out_nr, [&](int, int n, int lr, const float* v, const float*) {
         float o[4] = {v[0], v[1], v[2], v[3]};
         if (I8) { o[0] *= bf_lo(esc.x); o[1] *= bf_hi(esc.x); o[2] *= bf_lo(esc.y); o[3] *= bf_hi(esc.y); }
         uint64_t* dst = yb + ms.off_d[out_r0 + lr] + n / 2;
@@ -846,12 +875,13 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
   }
 
   // ---- final norm, codec head, eos head, hidden output ----
+  BB_TS();
   if (active) {
     BbTile t[2] = {tile_of(0, nH), tile_of(1, nH)};
     BbW<false, SD> w[2];
     const BbW<false, SD> nodual[1] = {};
 #pragma unroll
-    for (int j = 0; j < 2; ++j) bb_prefetch<false, SD>(a.thead, d, t[j], w[j]);
+    for (int j = 0; j < 2; ++j) bb_prefetch<false, SD, EXACT>(a.thead, d, t[j], w[j]);
     const BbNorm nw = bb_load_norm((const bf16_t*)W.final_norm, d);
     // eos head weights of this lane's pairs (wl < Bg computes row wl's)
     uint32_t eosw[8];
@@ -872,7 +902,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
         if (lane == 0) a.eos_out[b] = f2bf(tsum + eosb);
       }
     }
-    bb_compute<false, SD, 2, false>(xp, xs, d, t, w, nodual, red, Bg, [&](int, int n, int lr, const float* v, const float*) {
+    bb_compute<false, SD, 2, false, EXACT>(xp, xs, d, t, w, nodual, red, Bg, [&](int, int n, int lr, const float* v, const float*) {
       if (a.cb0_out)
         *reinterpret_cast<uint2*>(a.cb0_out + (size_t)ms.grow[lr] * a.CS + n) = make_uint2(f2bf2(v[0], v[1]), f2bf2(v[2], v[3]));
     });
@@ -880,6 +910,10 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
 
   // ---- position update and launch handshake by workgroup 0 ----
   __syncthreads();
+  BB_TS();
+#ifdef VUI_BB_CLOCK
+  if (a.dbg && wg == a.dbg_wg && tid == 0) { for (int i = 0; i < dbg_n; ++i) a.dbg[i] = dbg_ts[i]; a.dbg[255] = dbg_n; }
+#endif
   if (wg == 0 && tid == 0) {
     // every workgroup has read the positions before it reported its arrival
     int spins = 0;
@@ -908,7 +942,7 @@ BbLayout bb_layout(const vui_config& c) {
   size_t off = (size_t)BB_RG * c.d_model * 4;
   l.xp = off; off += (size_t)(BB_RG + 1) * bb_xs(c) * 4;
   l.red = off; off += 3 * 4 * 64 * 8 * 4;  // three single or two double tiles' partial sums (also: 16 pieces of 130 floats)
-  l.att = off; off += (size_t)(448 + 2048 + 136) * 4;
+  l.att = off; off += (size_t)(1536 + 64 + 2048) * 4;  // the row's q/k/v words, the lane groups' maxima/sums/weights, their accumulators
   l.misc = off; off += (sizeof(BbMisc) + 15) & ~(size_t)15;
   l.total = (off + 15) & ~(size_t)15;
   return l;
@@ -951,7 +985,8 @@ bool bb_batch_supported(const vui_config& c, int nwg, char* why, size_t why_len)
   else if (nwg != 256) r = "needs 256 resident workgroups";
   else {
     const int NWL = 64;  // the smallest group
-    if ((nq + 2 * nkv) / 16 > 3 * NWL || c.ffn / 16 > 2 * NWL || c.d_model / 16 > NWL || BB_RG * c.n_heads > NWL) r = "more tiles or heads than a row group's workgroups take";
+    if ((nq + 2 * nkv) / 16 > 3 * NWL || c.ffn / 16 > 2 * NWL || c.d_model / 16 > NWL || BB_RG * c.n_heads > NWL || c.n_heads > 16) r = "more tiles or heads than a row group's workgroups take";
+    if (nq + 2 * nkv > 3072) r = "q, k and v of a row longer than the attention staging area";
     if ((size_t)c.ffn / 2 * BB_RG >= 65536) r = "exchange vector too long";
     if (bb_layout(c).total > 160 * 1024) r = "activations do not fit in LDS";
   }
@@ -961,7 +996,7 @@ bool bb_batch_supported(const vui_config& c, int nwg, char* why, size_t why_len)
 
 size_t bb_batch_ll_words(const vui_config& c, int nwg) {
   const size_t B = VUI_MAX_BATCH, nq = (size_t)c.n_heads * c.head_dim, nkv = (size_t)c.n_kv_heads * c.head_dim;
-  const size_t layer = B * ((nq + 2 * nkv) / 2 + nq / 2 + c.d_model / 2 + c.ffn / 2 + c.d_model / 2) + (size_t)nwg * (c.head_dim + 2);
+  const size_t layer = B * ((nq + 2 * nkv) / 2 + nq / 2 + c.d_model / 2 + c.ffn / 2 + c.d_model / 2) + (size_t)nwg * 8 * (c.head_dim + 2);  // a piece holds at most 8 heads' partial results
   return layer * c.n_layers + 64;
 }
 size_t bb_batch_lds_bytes(const vui_config& c) { return bb_layout(c).total; }
@@ -1003,23 +1038,33 @@ int bb_batch_tile_weights(const vui_config& c, const vui_weights& w, void* dst8,
   return VUI_OK;
 }
 
+// the kernel's instantiations: Vui Nano's shape (768 wide, ffn 2048) with nothing conditional, and the general one
+static bool bb_exact(const vui_config& c) { return c.d_model == 768 && c.n_heads * c.head_dim == 768 && c.ffn == 2048; }
+typedef void (*bb_kernel_t)(const BbArgs);
+static bb_kernel_t bb_pick(const vui_config& c) {
+  if (bb_exact(c)) return c.int8_backbone ? bb_batch_kernel<true, 3, 3, 8, true> : bb_batch_kernel<false, 3, 3, 8, true>;
+  return c.int8_backbone ? bb_batch_kernel<true, 3, 4, 8, false> : bb_batch_kernel<false, 3, 4, 8, false>;
+}
+
 int bb_batch_max_resident(const vui_config& c) {
   int dev = 0;
   HIP_TRY(hipGetDevice(&dev));
   hipDeviceProp_t prop;
   HIP_TRY(hipGetDeviceProperties(&prop, dev));
   const size_t lds = bb_layout(c).total;
-  static size_t lds_attr = 0;
-  if (lds > lds_attr) {
-    HIP_TRY(hipFuncSetAttribute((const void*)bb_batch_kernel<false, 3>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    HIP_TRY(hipFuncSetAttribute((const void*)bb_batch_kernel<true, 3>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    lds_attr = lds;
-  }
-  int occ = 0, occ8 = 0;
-  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, bb_batch_kernel<false, 3>, FR_THREADS, lds));
-  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ8, bb_batch_kernel<true, 3>, FR_THREADS, lds));
-  return (occ < occ8 ? occ : occ8) * prop.multiProcessorCount;
+  const bb_kernel_t k = bb_pick(c);
+  HIP_TRY(hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  int occ = 0;
+  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, k, FR_THREADS, lds));
+  return occ * prop.multiProcessorCount;
 }
+
+#ifdef VUI_BB_CLOCK
+// profiling builds only: where the next launches drop the phase stamps of workgroup wg
+static unsigned long long* g_bb_dbg = nullptr;
+static int g_bb_dbg_wg = 0;
+extern "C" void vui_debug_bb_batch_clock(unsigned long long* buf, int wg) { g_bb_dbg = buf; g_bb_dbg_wg = wg; }
+#endif
 
 int launch_bb_batch(const vui_config& c, const vui_weights* wdev, const void* tiled_layers, const void* tiled_head, const int64_t* codes_in,
                     const void* emb_in, const int32_t* slot_idx, int32_t* seq_lens, const int32_t* seq_inc, int B, void* k_cache,
@@ -1035,9 +1080,17 @@ int launch_bb_batch(const vui_config& c, const vui_weights* wdev, const void* ti
   a.kc = (uint16_t*)k_cache; a.vc = (uint16_t*)v_cache; a.hidden_out = (uint16_t*)hidden_out; a.cb0_out = (uint16_t*)cb0_out;
   a.eos_out = (uint16_t*)eos_out; a.ll = ll; a.epoch = ctl; a.arrive = ctl + 1; a.err = ctl + 2;
   const BbLayout l = bb_layout(c);
+#ifdef VUI_BB_CLOCK
+  a.dbg = g_bb_dbg; a.dbg_wg = g_bb_dbg_wg;
+#endif
+  // heads per attention piece: two from five rows on (a group then has 128 or 64 workgroups, and pairs of heads
+  // divide its rows' keys twice as finely as whole head sets per key range would; measured 727 against 774 us for
+  // 16 rows, 596 against 610 for 8, no difference for 4); a key range is not split below 64 keys (32..128 measure
+  // the same)
+  a.hg = (B > BB_RG && c.n_heads % 2 == 0) ? 2 : 1;
+  a.min_keys = 64;
   a.xs = bb_xs(c); a.off_xp = (int)l.xp; a.off_red = (int)l.red; a.off_att = (int)l.att; a.off_misc = (int)l.misc;
-  if (c.int8_backbone) hipLaunchKernelGGL((bb_batch_kernel<true, 3>), dim3(nwg), dim3(FR_THREADS), l.total, st, a);
-  else hipLaunchKernelGGL((bb_batch_kernel<false, 3>), dim3(nwg), dim3(FR_THREADS), l.total, st, a);
+  hipLaunchKernelGGL(bb_pick(c), dim3(nwg), dim3(FR_THREADS), l.total, st, a);
   HIP_TRY(hipGetLastError());
   return VUI_OK;
 }
