@@ -120,3 +120,83 @@ def test_random_architecture_batch_vs_oracle(seed):
                 assert float(top2[0] - top2[1]) <= 2 * TOL * float(logits[b, i].abs().max()), (d, B, "depth head", b, i)
                 break
     m._native.status()
+
+
+def _dims64(rnd: random.Random) -> O.Dims:
+    """Architectures the persistent batched backbone kernel takes: widths in multiples of 64 (heads x head_dim equal to
+    d_model), a codebook in multiples of 16, rotated widths in fours; grouped KV heads, windows and global layers drawn."""
+    hd = rnd.choice([16, 32, 64, 96, 128])
+    H = rnd.choice([h for h in (2, 4, 6, 8, 12, 16) if (h * hd) % 64 == 0 and h * hd <= 1024])
+    kv = rnd.choice([k for k in (1, 2, 3, 4, 6, 8, 16) if H % k == 0 and (k * hd) % 16 == 0])
+    kw = dict(d_model=hd * H, n_layers=rnd.randint(1, 3), n_heads=H, n_kv_heads=kv, n_quantizers=rnd.choice([2, 4, 8, 16]),
+              codebook_size=rnd.choice([16, 64, 256, 2048]), rq_d_model=64, rq_n_layers=1, rq_n_heads=2, vocab_size=50,
+              max_seqlen=rnd.choice([96, 300]), intermediate_size=64 * rnd.randint(1, 12))
+    if rnd.random() < 0.5:
+        kw["rope_dim"] = rnd.choice([x for x in (4, 8, 16, 32) if x <= hd])
+    if rnd.random() < 0.5:
+        kw["window_size"] = rnd.choice([3, 17, 70])
+        kw["global_every"] = rnd.choice([None, 2, 3])
+        if rnd.random() < 0.5:
+            kw["global_rope_dim"] = rnd.choice([x for x in (4, 8, 16) if x <= hd])
+    return O.Dims(**kw)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_persistent_batched_backbone_vs_oracle(seed):
+    """The backbone step of 2..16 rows as one persistent kernel (row groups by cache length, key ranges dealt by
+    length, the general instantiation with conditional steps): hidden state, code-0 logits, end-of-turn logit, cache
+    rows and positions of three steps against the oracle, bf16 and int8 weights, shuffled slots, ragged caches; and
+    within the tolerance of the kernel sequence on the same inputs."""
+    rnd = random.Random(7000 + seed)
+    d = _dims64(rnd)
+    sdkw = dict(TINY_SD)
+    sdkw["std"] = 0.15 * (64.0 / max(64, d.d_model)) ** 0.5
+    sd = O.synthetic_state_dict(d, **sdkw)
+    g = torch.Generator().manual_seed(seed)
+    int8 = seed % 2 == 1
+    B = [2, 3, 4, 5, 8, 9, 12, 13, 16, 16, 7, 2][seed]
+    n_slots = B + rnd.randint(0, 2)
+    S = d.max_seqlen
+    lens = torch.randint(0, S - 8, (n_slots,), generator=g)
+    lens[0] = 0  # an empty cache among them
+    kc = O.rnd(0.5 * torch.randn(d.n_layers, n_slots, S, d.n_kv_heads, d.head_dim, generator=g), BF)
+    vc = O.rnd(0.5 * torch.randn(d.n_layers, n_slots, S, d.n_kv_heads, d.head_dim, generator=g), BF)
+    slots = torch.randperm(n_slots, generator=g)[:B]
+    codes_all = torch.randint(0, d.codebook_size, (3, B, d.n_quantizers), generator=g)
+    o = O.OracleModel(d, sd, BF, n_slots=n_slots, int8=int8)
+    o.k_cache.copy_(kc)
+    o.v_cache.copy_(vc)
+    o.seq_lens.copy_(lens)
+    refs = [o.decode_step(codes_all[i], slots) for i in range(3)]
+    outs = {}
+    for fused in (1, 0):
+        m = make_model(d, sd, BF, int8=int8)
+        m.decoder.allocate_flash_kv_cache(n_slots, m.device, BF)
+        m._native.fused(fused)
+        if fused:
+            assert m._native.bb_batch(), (d, "the persistent batched backbone kernel must take this architecture")
+        m.decoder._k.copy_(kc.to(BF))
+        m.decoder._v.copy_(vc.to(BF))
+        m.decoder.flash_kv_caches[0].seq_lens.copy_(lens.to(torch.int32))
+        hid = torch.empty(B, d.d_model, dtype=BF, device="cuda")
+        cb0 = torch.empty(B, d.codebook_size, dtype=BF, device="cuda")
+        eos = torch.empty(B, 1, dtype=BF, device="cuda")
+        for i in range(3):
+            m.decoder._step(codes=codes_all[i].cuda(), emb=None, slot_idx=slots.to(torch.int32).cuda(), seq_inc=None, B=B,
+                            hidden_out=hid, cb0_out=cb0, eos_out=eos, n_splits=4, stream=torch.cuda.current_stream().cuda_stream)
+            h_ref, cb_ref, eos_ref = refs[i]
+            assert rel_err(hid, h_ref) <= TOL and rel_err(cb0, cb_ref) <= TOL, (d, B, int8, fused, i, rel_err(hid, h_ref), rel_err(cb0, cb_ref))
+            assert float((eos.float().cpu() - eos_ref).abs().max()) <= TOL * max(1.0, float(cb_ref.abs().max())), (d, B, fused, i)
+            outs[(fused, i)] = (hid.clone(), cb0.clone())
+        m._native.status()
+        assert m.decoder.flash_kv_caches[0].seq_lens.cpu().tolist() == o.seq_lens.tolist()
+        # the three appended positions of every row, layer 0 and the last layer
+        for b in range(B):
+            s = int(slots[b])
+            for l in (0, d.n_layers - 1):
+                got = m.decoder._k[l, s, int(lens[s]):int(lens[s]) + 3].float().cpu()
+                assert rel_err(got, o.k_cache[l, s, int(lens[s]):int(lens[s]) + 3]) <= TOL, (d, b, l)
+                got = m.decoder._v[l, s, int(lens[s]):int(lens[s]) + 3].float().cpu()
+                assert rel_err(got, o.v_cache[l, s, int(lens[s]):int(lens[s]) + 3]) <= TOL, (d, b, l)
+    for i in range(3):
+        assert rel_err(outs[(1, i)][0], outs[(0, i)][0]) <= TOL and rel_err(outs[(1, i)][1], outs[(0, i)][1]) <= TOL

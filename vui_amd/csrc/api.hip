@@ -79,7 +79,8 @@ struct vui_ctx {
   // persistent backbone step for 2..16 rows
   int bb_ok;
   char bb_why[96];
-  void* bb_w8;    // the layers' int8 matrices in the kernel's operand layout (int8 contexts)
+  void* bb_w8;    // the layers' matrices in the kernel's operand layout where it keeps a copy of its own (int8; bf16 without the prefill copy)
+  size_t bb_w8_bytes;
   void* bb_head;  // the codec head in that layout
 };
 
@@ -157,7 +158,7 @@ static size_t carve(const vui_config* c, int Bm, vui_ctx* x) {
   TAKE(rq_tw, void*, rq_batch_weight_bytes(*c, FUSED_NWG));  // empty when the batched depth-head kernel is unavailable
   TAKE(wdev_t, vui_weights*, sizeof(vui_weights));
   TAKE(rq_ks, void*, frame_rq_key_scratch_bytes(*c, FUSED_NWG));
-  TAKE(bb_w8, void*, bb_batch_weight8_bytes(*c, FUSED_NWG));  // empty for bf16 weights (the prefill copy serves) or when the kernel is unavailable
+  TAKE(bb_w8, void*, bb_batch_weight_bytes(*c, FUSED_NWG));  // empty for bf16 weights with a prefill copy (that one serves) or when the kernel is unavailable
   TAKE(bb_head, void*, bb_batch_head_bytes(*c, FUSED_NWG));
 #undef TAKE
   return cv.off;
@@ -262,16 +263,13 @@ int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream) {
   ctx->bb_ok = 0;
   ctx->bb_why[0] = 0;
   if (bb_batch_supported(ctx->cfg, ctx->nwg, ctx->bb_why, sizeof(ctx->bb_why))) {
-    const bool i8 = ctx->cfg.int8_backbone != 0;
-    if (!i8 && !prefill_weight_bytes(ctx->cfg)) snprintf(ctx->bb_why, sizeof(ctx->bb_why), "no tiled copy of the bf16 matrices (the prompt-ingestion pass is unavailable)");
-    else {
-      if ((rc = bb_batch_tile_weights(ctx->cfg, ctx->w, i8 ? ctx->bb_w8 : nullptr, ctx->bb_head, st))) return rc;
-      HIP_TRY(hipStreamSynchronize(st));
-      const int cap = bb_batch_max_resident(ctx->cfg);
-      if (cap < 0) return cap;
-      if (cap >= ctx->nwg) ctx->bb_ok = 1;
-      else snprintf(ctx->bb_why, sizeof(ctx->bb_why), "only %d workgroups can be resident, %d needed", cap, ctx->nwg);
-    }
+    ctx->bb_w8_bytes = bb_batch_weight_bytes(ctx->cfg, ctx->nwg);
+    if ((rc = bb_batch_tile_weights(ctx->cfg, ctx->w, ctx->bb_w8_bytes ? ctx->bb_w8 : nullptr, ctx->bb_head, st))) return rc;
+    HIP_TRY(hipStreamSynchronize(st));
+    const int cap = bb_batch_max_resident(ctx->cfg);
+    if (cap < 0) return cap;
+    if (cap >= ctx->nwg) ctx->bb_ok = 1;
+    else snprintf(ctx->bb_why, sizeof(ctx->bb_why), "only %d workgroups can be resident, %d needed", cap, ctx->nwg);
   }
   ctx->rqb_ok = 0;
   ctx->rqb_why[0] = 0;
@@ -385,7 +383,7 @@ int vui_backbone_step(vui_ctx* ctx, const int64_t* codes_in, const void* emb_in,
     return launch_frame(a, ctx->nwg, ctx->fused_ok ? ctx->lds_bytes : ctx->lds_bb, st);
   }
   if (ctx->bb_ok && ctx->fused_on && B > 1)
-    return launch_bb_batch(c, ctx->wdev, c.int8_backbone ? ctx->bb_w8 : ctx->pf_w, ctx->bb_head, codes_in, emb_in, slot_idx, seq_lens, seq_inc, B,
+    return launch_bb_batch(c, ctx->wdev, ctx->bb_w8_bytes ? ctx->bb_w8 : ctx->pf_w, ctx->bb_head, codes_in, emb_in, slot_idx, seq_lens, seq_inc, B,
                            k_cache, v_cache, hidden_out ? hidden_out : ctx->hidden, cb0_out ? cb0_out : ctx->cb0,
                            eos_out ? eos_out : ctx->eos, ctx->ll, ctx->ctl, ctx->nwg, st);
   const int d = c.d_model, H = c.n_heads, KV = c.n_kv_heads, hd = c.head_dim;

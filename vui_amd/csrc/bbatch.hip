@@ -1001,24 +1001,33 @@ size_t bb_batch_ll_words(const vui_config& c, int nwg) {
 }
 size_t bb_batch_lds_bytes(const vui_config& c) { return bb_layout(c).total; }
 
-// bytes of the tiled int8 copy of the layers' matrices (int8 contexts) and of the tiled codec head
-size_t bb_batch_weight8_bytes(const vui_config& c, int nwg) {
-  if (!c.int8_backbone || !bb_batch_supported(c, nwg, nullptr, 0)) return 0;
+// bytes of this kernel's own tiled copy of the layers' matrices: the int8 matrices of an int8 context, the bf16
+// matrices where the prompt-ingestion pass (whose copy is used otherwise) does not take the configuration; and of the
+// tiled codec head
+size_t bb_batch_weight_bytes(const vui_config& c, int nwg) {
+  if (!bb_batch_supported(c, nwg, nullptr, 0)) return 0;
+  if (!c.int8_backbone && prefill_weight_bytes(c)) return 0;
   const size_t nq = (size_t)c.n_heads * c.head_dim, nkv = (size_t)c.n_kv_heads * c.head_dim, d = c.d_model, F = c.ffn;
-  return ((nq + 2 * nkv) * d + d * nq + 3 * F * d) * c.n_layers;
+  return ((nq + 2 * nkv) * d + d * nq + 3 * F * d) * c.n_layers * (c.int8_backbone ? 1 : 2);
 }
 size_t bb_batch_head_bytes(const vui_config& c, int nwg) {
   return bb_batch_supported(c, nwg, nullptr, 0) ? (size_t)c.codebook_size * c.d_model * 2 : 0;
 }
 
-int bb_batch_tile_weights(const vui_config& c, const vui_weights& w, void* dst8, void* dst_head, hipStream_t st) {
+int bb_batch_tile_weights(const vui_config& c, const vui_weights& w, void* dst_layers, void* dst_head, hipStream_t st) {
   const size_t nq = (size_t)c.n_heads * c.head_dim, nkv = (size_t)c.n_kv_heads * c.head_dim, d = c.d_model, F = c.ffn;
-  if (dst8) {
-    uint8_t* o = (uint8_t*)dst8;
+  if (dst_layers) {
+    const bool i8 = c.int8_backbone != 0;
+    char* o = (char*)dst_layers;
     auto tile = [&](const void* src, size_t N, size_t K) {
-      const size_t pieces = N * (K / 16);
-      hipLaunchKernelGGL(bb_tile8_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, st, (const uint8_t*)src, o, N, (int)K);
-      o += N * K;
+      if (i8) {
+        const size_t pieces = N * (K / 16);
+        hipLaunchKernelGGL(bb_tile8_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, st, (const uint8_t*)src, (uint8_t*)o, N, (int)K);
+      } else {
+        const size_t pieces = N * (K / 8);
+        hipLaunchKernelGGL(bb_tile16_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, st, (const bf16_t*)src, (bf16_t*)o, N, (int)K);
+      }
+      o += N * K * (i8 ? 1 : 2);
     };
     for (int l = 0; l < c.n_layers; ++l) {
       const vui_layer_weights& L = w.layers[l];

@@ -229,9 +229,9 @@ int launch_rq_batch(const vui_config& c, const vui_weights* wdev, const void* hi
 bool bb_batch_supported(const vui_config& c, int nwg, char* why, size_t why_len);
 size_t bb_batch_ll_words(const vui_config& c, int nwg);
 size_t bb_batch_lds_bytes(const vui_config& c);
-size_t bb_batch_weight8_bytes(const vui_config& c, int nwg);  // tiled int8 copy of the layers' matrices (int8 contexts), else 0
+size_t bb_batch_weight_bytes(const vui_config& c, int nwg);   // own tiled copy of the layers' matrices (int8 contexts; bf16 ones without the prefill copy), else 0
 size_t bb_batch_head_bytes(const vui_config& c, int nwg);     // tiled copy of the codec head
-int bb_batch_tile_weights(const vui_config& c, const vui_weights& w, void* dst8, void* dst_head, hipStream_t st);
+int bb_batch_tile_weights(const vui_config& c, const vui_weights& w, void* dst_layers, void* dst_head, hipStream_t st);
 int bb_batch_max_resident(const vui_config& c);
 int launch_bb_batch(const vui_config& c, const vui_weights* wdev, const void* tiled_layers, const void* tiled_head, const int64_t* codes_in,
                     const void* emb_in, const int32_t* slot_idx, int32_t* seq_lens, const int32_t* seq_inc, int B, void* k_cache,
