@@ -192,6 +192,16 @@ int vui_backbone_step(vui_ctx* ctx, const int64_t* codes_in, const void* emb_in,
 /* Sampling parameters shared by the two samplers.  The uniform for (row b, codebook c) of
  * frame f is Philox4x32-10(key = seed, counter = (f, b, c, 0)); *frame_ctr is read on the
  * device, so a captured graph can be replayed with a new frame number. */
+/* Sampling settings kept in DEVICE memory (16 bytes), read by the kernels when they run: a step recorded into a HIP
+ * graph with vui_sample_params.dev set serves every temperature, top-k and seed - the host rewrites the block
+ * (an ordinary stream-ordered copy) instead of capturing a graph per setting.  The reference keeps its temperature
+ * in a 0-d device tensor filled before each replay for the same reason (model.py:1011). */
+typedef struct vui_sample_dev {
+  float temperature;
+  int32_t top_k;
+  uint64_t seed;
+} vui_sample_dev;
+
 typedef struct vui_sample_params {
   float temperature;      /* <= 0 means greedy */
   int32_t top_k;          /* 1 = greedy (lowest index of the maximum), <= 0 = no truncation */
@@ -210,6 +220,8 @@ typedef struct vui_sample_params {
                              <= top_p.  With top_k > 0 this is sample_top_p_top_k (sampling.py:34-43): of the
                              nucleus, everything >= its k-th largest entry.  Equal probabilities are ordered by
                              index (torch.sort leaves that open).  The other entry points require 0. */
+  const vui_sample_dev* dev; /* device pointer or NULL.  Set: temperature, top_k and seed are read from there on
+                                the device at run time and the three fields above are ignored. */
 } vui_sample_params;
 
 /* Device-side end-of-turn test of a streamed turn (Engine._stream_row's `step >= min_frames and sigmoid(eos) >

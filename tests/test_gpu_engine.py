@@ -378,3 +378,47 @@ def test_failed_persistent_launch_commits_nothing_and_recovers():
     h = row.prefill_emb(m.token_emb(ids.cuda()[None]))[:, -1]
     again, _ = eng.generate([row], h, 6, cfg)
     assert torch.equal(again, good)
+
+
+def test_one_frame_graph_serves_every_sampling_setting():
+    """Temperature, top-k and seed are read by the captured frame step from device memory: requests that differ in
+    them (and in length) replay ONE graph, and each gives exactly the frames of an engine that never saw the others."""
+    from vui_amd.engine import GenConfig
+
+    d = tiny_dims(2)
+    sd = O.synthetic_state_dict(d, **TINY_SD)
+    ids = torch.tensor([3, 11, 42, 7, 19])
+    cfgs = [GenConfig(temperature=0.9, top_k=10, rq_top_k=10, rep_penalty=1.2, rep_window=4, seed=s) for s in (1, 2, 3)]
+    cfgs += [GenConfig(temperature=0.6, top_k=5, rq_top_k=7, rep_penalty=1.2, rep_window=4, seed=2),
+             GenConfig(temperature=1.0, top_k=1, rep_penalty=1.2, rep_window=4, seed=9)]
+    lengths = [8, 12, 8, 20, 6]
+
+    def run(eng, m, cfg, n):
+        row = eng.new_row()
+        h = row.prefill_emb(m.token_emb(ids.cuda()[None]))[:, -1]
+        frames, _ = eng.generate([row], h, n, cfg)
+        row.close()
+        return frames.cpu()
+
+    m, eng = _engine(d, sd, BF)
+    shared = [run(eng, m, c, n) for c, n in zip(cfgs, lengths)]
+    assert len(eng._frame_graphs) == 1
+    shared_again = run(eng, m, cfgs[0], lengths[0])
+    assert torch.equal(shared_again, shared[0]) and len(eng._frame_graphs) == 1
+    for c, n, got in zip(cfgs, lengths, shared):
+        m2, eng2 = _engine(d, sd, BF)
+        assert torch.equal(run(eng2, m2, c, n), got), (c, n)
+    assert not torch.equal(shared[0][:8], shared[1][:8])  # another seed, other frames
+    # the depth head's own captured graphs likewise: one per (rows, codebooks)
+    rq = m.rq_transformer
+    hid = torch.randn(1, d.d_model, device="cuda").to(BF)
+    c0 = torch.zeros(1, dtype=torch.long, device="cuda")
+    outs = []
+    for t, s in ((0.7, 0), (0.9, 0), (0.7, 5)):
+        rq.seed = s
+        rq._ctr.zero_()
+        outs.append(rq.generate_cuda_graph_kv(hid, c0, t).clone())
+    assert len(rq._gkv_graphs) == 1
+    rq.seed = 0
+    rq._ctr.zero_()
+    assert torch.equal(rq.generate_cuda_graph_kv(hid, c0, 0.7), outs[0])

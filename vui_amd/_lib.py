@@ -48,7 +48,7 @@ class WeightsC(C.Structure):
 
 class SampleParamsC(C.Structure):
     _fields_ = [("temperature", C.c_float), ("top_k", C.c_int32), ("seed", C.c_uint64),
-                ("frame_ctr", C.c_void_p), ("state_rows", C.c_void_p), ("keep_ties", C.c_int32), ("top_p", C.c_float)]
+                ("frame_ctr", C.c_void_p), ("state_rows", C.c_void_p), ("keep_ties", C.c_int32), ("top_p", C.c_float), ("dev", C.c_void_p)]
 
 
 class EosStopC(C.Structure):

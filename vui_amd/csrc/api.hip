@@ -448,7 +448,7 @@ static SampleArgs sample_base(const vui_sample_params* sp) {
   SampleArgs s;
   memset(&s, 0, sizeof(s));
   s.temperature = sp->temperature; s.top_k = sp->top_k; s.seed = sp->seed; s.frame_ctr = sp->frame_ctr;
-  s.state_rows = sp->state_rows; s.top_p = sp->top_p;
+  s.state_rows = sp->state_rows; s.top_p = sp->top_p; s.dev = sp->dev;
   return s;
 }
 
@@ -521,12 +521,12 @@ int vui_rq_generate(vui_ctx* ctx, const void* hidden, const int64_t* code0, cons
     fused_base(ctx, a);
     a.mode = FR_RQ;
     a.rq_hidden = (const uint16_t*)hidden; a.rq_code0 = code0; a.logit_bias = logit_bias; a.n_q = n_q;
-    a.temp1 = sp->temperature; a.topk1 = sp->top_k; a.seed1 = sp->seed; a.frame_ctr1 = sp->frame_ctr;
+    a.temp1 = sp->temperature; a.topk1 = sp->top_k; a.seed1 = sp->seed; a.frame_ctr1 = sp->frame_ctr; a.sdev1 = sp->dev;
     a.codes_out = codes_out; a.codes_stride = codes_stride; a.zero_pad = zero_pad;
     return launch_frame(a, ctx->nwg, ctx->lds_bytes, st);
   }
   if (ctx->rqb_ok && ctx->fused_on && B > 1)
-    return launch_rq_batch(c, ctx->wdev_t, hidden, code0, logit_bias, n_q, sp->temperature, sp->top_k, sp->seed, sp->frame_ctr,
+    return launch_rq_batch(c, ctx->wdev_t, hidden, code0, logit_bias, n_q, sp->temperature, sp->top_k, sp->seed, sp->dev, sp->frame_ctr,
                            codes_out, codes_stride, zero_pad, B, ctx->ll, ctx->ctl, ctx->nwg, st);
   const int R = c.rq_dim, CS = c.codebook_size;
   const char* pos_emb = (const char*)ctx->w.rq_pos_emb;
@@ -598,6 +598,7 @@ int vui_frame_step(vui_ctx* ctx, int64_t* codes_io, const int32_t* slot_idx, int
     a.rep_counts = rep_counts; a.rep_hist = rep_hist; a.rep_pos = rep_pos; a.penalty = penalty; a.rep_window = window;
     a.temp0 = sp_cb0->temperature; a.topk0 = sp_cb0->top_k; a.seed0 = sp_cb0->seed; a.frame_ctr0 = sp_cb0->frame_ctr;
     a.temp1 = sp_rq->temperature; a.topk1 = sp_rq->top_k; a.seed1 = sp_rq->seed; a.frame_ctr1 = sp_rq->frame_ctr;
+    a.sdev0 = sp_cb0->dev; a.sdev1 = sp_rq->dev;
     a.code0_out = ctx->code0; a.logit_bias = logit_bias; a.n_q = n_q;
     a.codes_out = codes_io; a.codes_stride = c.n_quantizers; a.zero_pad = 1;
     a.frames_out = frames_out; a.eos_prob_out = eos_prob_out; a.max_frames = max_frames; a.frame_ctr = frame_ctr;

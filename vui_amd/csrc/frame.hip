@@ -786,8 +786,13 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       }
       if (a.mode & FR_CB0) {
         const int E = (a.CS + FR_THREADS - 1) / FR_THREADS;
-        const bool greedy = (a.topk0 == 1) || !(a.temp0 > 0.f);
-        const float div = greedy ? 1.0f : a.temp0;
+        // sampling settings: from the launch arguments, or from the device block a captured step reads anew at each
+        // replay (fetched where they are used: kept live from the top of the kernel they cost scalar registers)
+        const float temp0 = a.sdev0 ? a.sdev0->temperature : a.temp0;
+        const int topk0 = a.sdev0 ? a.sdev0->top_k : a.topk0;
+        const uint64_t seed0 = a.sdev0 ? a.sdev0->seed : a.seed0;
+        const bool greedy = (topk0 == 1) || !(temp0 > 0.f);
+        const float div = greedy ? 1.0f : temp0;
         const float* counts = (a.rep_counts && a.penalty > 1.0f) ? a.rep_counts : nullptr;
         // this thread's repetition counts, fetched ahead of the wait for the logits
         float cn[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -802,7 +807,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
             for (int e = 0; e < 8; ++e) { const int j = tid * E + e; if (e < E && j < a.CS) cn[e] = counts[j]; }
           }
         }
-        const uint32_t rnd0 = philox_u32(a.seed0, frame0, 0u, 0u, 0u);  // ahead of the wait
+        const uint32_t rnd0 = philox_u32(seed0, frame0, 0u, 0u, 0u);  // ahead of the wait
         poll_words((uint32_t*)lg, rep_rd(lgbuf), a.CS / 2, c);
         float lv[8], raw[8];
         uint32_t key[8];
@@ -823,7 +828,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
           }
         }
         TS(20);
-        code0 = block_sample<8>(lv, key, counts ? 0 : 16, a.CS, E, greedy, a.topk0, rnd0, 0u, ssh, (int*)sc, a.exact0 != 0);
+        code0 = block_sample<8>(lv, key, counts ? 0 : 16, a.CS, E, greedy, topk0, rnd0, 0u, ssh, (int*)sc, a.exact0 != 0);
         TS(21);
       }
     }
@@ -1087,12 +1092,15 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
         gemv_compute<2, false, false>(xp, R_hd, wr, red, [&](int gp, float v0, float v1, float, float) {
           rep_st(lgbuf, gp, pack2(v0, v1), ep); });
         TS(42);
-        const uint32_t rnd = philox_u32(a.seed1, frame1, 0u, (uint32_t)t, 0u);  // ahead of the wait
+        const float temp1 = a.sdev1 ? a.sdev1->temperature : a.temp1;
+        const int topk1 = a.sdev1 ? a.sdev1->top_k : a.topk1;
+        const uint64_t seed1 = a.sdev1 ? a.sdev1->seed : a.seed1;
+        const uint32_t rnd = philox_u32(seed1, frame1, 0u, (uint32_t)t, 0u);  // ahead of the wait
         poll_words((uint32_t*)lg, rep_rd(lgbuf), CS / 2, c);
         TS(43);
         const int E = (CS + FR_THREADS - 1) / FR_THREADS;
-        const bool greedy = (a.topk1 == 1) || !(a.temp1 > 0.f);
-        const float div = greedy ? 1.0f : a.temp1;
+        const bool greedy = (topk1 == 1) || !(temp1 > 0.f);
+        const float div = greedy ? 1.0f : temp1;
         const float* bias = a.logit_bias ? a.logit_bias + (size_t)(t - 1) * CS : nullptr;
         float lv[8], raw[8];
         uint32_t key[8];
@@ -1107,7 +1115,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
             key[e] = float_key(bias ? lv[e] : raw[e]);
           }
         }
-        prev_code = block_sample<8>(lv, key, bias ? 0 : 16, CS, E, greedy, a.topk1, rnd, (uint32_t)t, ssh, (int*)sc);
+        prev_code = block_sample<8>(lv, key, bias ? 0 : 16, CS, E, greedy, topk1, rnd, (uint32_t)t, ssh, (int*)sc);
         TS(44);
 #ifdef VUI_SAMPLE_CLOCK
         if (prof_on && tid == 0) {

@@ -108,6 +108,7 @@ struct SampleArgs {
   float temperature;
   int top_k;
   float top_p;         // > 0: nucleus cut ahead of the top-k cut (stand-alone sampling kernel only)
+  const vui_sample_dev* dev;  // if set: temperature, top_k, seed come from this device block
   uint64_t seed;
   const int32_t* frame_ctr;
   const int32_t* state_rows;  // (B) or nullptr: repetition state / random-stream row of row b
@@ -166,6 +167,7 @@ struct FrameArgs {
   float temp0; int topk0;
   float temp1; int topk1;
   uint64_t seed0, seed1;
+  const vui_sample_dev *sdev0, *sdev1;  // if set: the settings of the code-0 draw / the depth head's draws, read on the device
   const int32_t* frame_ctr0;
   const int32_t* frame_ctr1;
   int64_t* code0_out;
@@ -222,8 +224,8 @@ size_t rq_batch_weight_bytes(const vui_config& c, int nwg);  // tiled copies of 
 int rq_batch_tile_weights(const vui_config& c, const vui_weights& w, void* dst, vui_weights* tiled, hipStream_t st);
 int rq_batch_max_resident(size_t lds_bytes);
 int launch_rq_batch(const vui_config& c, const vui_weights* wdev, const void* hidden, const int64_t* code0, const float* logit_bias,
-                    int n_q, float temp, int topk, uint64_t seed, const int32_t* frame_ctr, int64_t* codes_out, int codes_stride,
-                    int zero_pad, int B, uint64_t* ll, uint32_t* ctl, int nwg, hipStream_t st);
+                    int n_q, float temp, int topk, uint64_t seed, const vui_sample_dev* sdev, const int32_t* frame_ctr, int64_t* codes_out,
+                    int codes_stride, int zero_pad, int B, uint64_t* ll, uint32_t* ctl, int nwg, hipStream_t st);
 
 // bbatch.hip: the backbone step of 2..16 rows as one persistent kernel
 bool bb_batch_supported(const vui_config& c, int nwg, char* why, size_t why_len);

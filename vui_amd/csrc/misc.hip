@@ -97,8 +97,11 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const SampleArgs p
   const int CS = p.CS;
   const int E = (CS + SAMP_THREADS - 1) / SAMP_THREADS;  // contiguous elements per thread
   const T* lg = (const T*)p.logits + (size_t)b * CS;
-  const bool greedy = (p.top_k == 1) || !(p.temperature > 0.f);
-  const float div = greedy ? 1.0f : p.temperature;
+  const float s_temp = p.dev ? p.dev->temperature : p.temperature;
+  const int s_topk = p.dev ? p.dev->top_k : p.top_k;
+  const uint64_t s_seed = p.dev ? p.dev->seed : p.seed;
+  const bool greedy = (s_topk == 1) || !(s_temp > 0.f);
+  const float div = greedy ? 1.0f : s_temp;
   const int sb = p.state_rows ? p.state_rows[b] : b;  // row of the repetition state and of the random stream
   const float* counts = (p.rep_counts && p.penalty > 1.0f) ? p.rep_counts + (size_t)sb * CS : nullptr;
 
@@ -118,9 +121,9 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const SampleArgs p
     }
   }
   const uint32_t frame = p.frame_ctr ? (uint32_t)p.frame_ctr[0] : 0u;
-  const uint32_t rnd = philox_u32(p.seed, frame, (uint32_t)sb, (uint32_t)p.codebook, 0u);
+  const uint32_t rnd = philox_u32(s_seed, frame, (uint32_t)sb, (uint32_t)p.codebook, 0u);
   if (p.top_p > 0.f && !greedy) nucleus_cut<EMAX>(l, key, raw_keys ? 16 : 0, CS, E, p.top_p, nuc);  // uniform over the block
-  const int pick = block_sample<EMAX>(l, key, raw_keys ? 16 : 0, CS, E, greedy, p.top_k, rnd, (uint32_t)p.codebook, sh, hist, p.exact_k != 0);
+  const int pick = block_sample<EMAX>(l, key, raw_keys ? 16 : 0, CS, E, greedy, s_topk, rnd, (uint32_t)p.codebook, sh, hist, p.exact_k != 0);
 
   if (tid == 0) {
     p.out[(size_t)b * p.out_stride + p.out_col] = (int64_t)pick;

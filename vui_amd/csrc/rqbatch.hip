@@ -292,6 +292,7 @@ struct RqBatchArgs {
   float temp;
   int topk;
   uint64_t seed;
+  const vui_sample_dev* sdev;  // if set: the three above are read from here
   const int32_t* frame_ctr;
   uint64_t* ll;
   uint32_t *epoch, *arrive, *err;
@@ -331,6 +332,9 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
   const bf16_t* g_head = (const bf16_t*)W.rq_head_w;
   const bf16_t* g_norm = (const bf16_t*)W.rq_norm;
   const uint32_t frame = a.frame_ctr ? (uint32_t)a.frame_ctr[0] : 0u;
+  const float s_temp = a.sdev ? a.sdev->temperature : a.temp;
+  const int s_topk = a.sdev ? a.sdev->top_k : a.topk;
+  const uint64_t s_seed = a.sdev ? a.sdev->seed : a.seed;
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
   if (tid == 0) __hip_atomic_fetch_add(a.arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
@@ -638,13 +642,13 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
         const int b = b0 + wl;
         // the row's logits pass through the first words of the staging area
         uint32_t* lgw = xp;
-        const uint32_t rnd = philox_u32(a.seed, frame, (uint32_t)b, (uint32_t)t, 0u);  // ahead of the wait
+        const uint32_t rnd = philox_u32(s_seed, frame, (uint32_t)b, (uint32_t)t, 0u);  // ahead of the wait
         __syncthreads();
         ll_poll_auto(lgb + (size_t)b * (CS / 2), CS / 2, c, [&](int i, uint32_t v) { lgw[i] = v; });
         __syncthreads();
         const int E = (CS + FR_THREADS - 1) / FR_THREADS;
-        const bool greedy = (a.topk == 1) || !(a.temp > 0.f);
-        const float div = greedy ? 1.0f : a.temp;
+        const bool greedy = (s_topk == 1) || !(s_temp > 0.f);
+        const float div = greedy ? 1.0f : s_temp;
         const float* bias = a.logit_bias ? a.logit_bias + (size_t)(t - 1) * CS : nullptr;
         float lv[8];
         uint32_t key[8];
@@ -661,7 +665,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
         }
         __syncthreads();  // every thread holds its logits: the staging words go back to zero (the spare row must
         for (int i = tid; i < CS / 2; i += FR_THREADS) lgw[i] = 0u;  // read as zero, the others are rewritten by the next norm)
-        const int code = block_sample<8>(lv, key, bias ? 0 : 16, CS, E, greedy, a.topk, rnd, (uint32_t)t, ssh, (int*)red);
+        const int code = block_sample<8>(lv, key, bias ? 0 : 16, CS, E, greedy, s_topk, rnd, (uint32_t)t, ssh, (int*)red);
         if (tid == 0) {
           ll_st(cb + b, (uint32_t)code, ep);
           a.codes_out[(size_t)b * a.codes_stride + t] = code;
@@ -792,14 +796,14 @@ extern "C" void vui_debug_rq_batch_clock(unsigned long long* buf, int wg) { g_rb
 #endif
 
 int launch_rq_batch(const vui_config& c, const vui_weights* wdev, const void* hidden, const int64_t* code0, const float* logit_bias,
-                    int n_q, float temp, int topk, uint64_t seed, const int32_t* frame_ctr, int64_t* codes_out, int codes_stride,
-                    int zero_pad, int B, uint64_t* ll, uint32_t* ctl, int nwg, hipStream_t st) {
+                    int n_q, float temp, int topk, uint64_t seed, const vui_sample_dev* sdev, const int32_t* frame_ctr, int64_t* codes_out,
+                    int codes_stride, int zero_pad, int B, uint64_t* ll, uint32_t* ctl, int nwg, hipStream_t st) {
   RqBatchArgs a;
   memset(&a, 0, sizeof(a));
   a.B = B; a.d = c.d_model; a.R = c.rq_dim; a.rqH = c.rq_heads; a.rqF = c.rq_ffn; a.rqL = c.rq_layers; a.Q = c.n_quantizers;
   a.CS = c.codebook_size; a.n_q = n_q; a.rq_eps = c.rq_norm_eps; a.w = wdev; a.hidden = (const uint16_t*)hidden; a.code0 = code0;
   a.codes_out = codes_out; a.codes_stride = codes_stride; a.zero_pad = zero_pad; a.logit_bias = logit_bias; a.temp = temp;
-  a.topk = topk; a.seed = seed; a.frame_ctr = frame_ctr; a.ll = ll; a.epoch = ctl; a.arrive = ctl + 1; a.err = ctl + 2;
+  a.topk = topk; a.seed = seed; a.sdev = sdev; a.frame_ctr = frame_ctr; a.ll = ll; a.epoch = ctl; a.arrive = ctl + 1; a.err = ctl + 2;
 #ifdef VUI_RB_CLOCK
   a.dbg = g_rb_dbg; a.dbg_wg = g_rb_dbg_wg;
 #else

@@ -16,7 +16,7 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from .model import MAX_BATCH, Graph, Vui, make_sample_params
+from .model import MAX_BATCH, Graph, SampleDev, Vui, make_sample_params
 
 FRAME_RATE = 12.5  # codec frames per second (src/vui/qwen_codec.py:27-30)
 DEFAULT_WPS = 3.0  # words per second when the prompt gives none (src/vui/engine.py:41)
@@ -292,6 +292,8 @@ class Engine:
         self._stop_state = torch.zeros(2, dtype=torch.int32, device=dev)
         self._stop_init = torch.tensor([0, 1], dtype=torch.int32, device=dev)
         self._stop_host = [torch.zeros(1, dtype=torch.int32).pin_memory() for _ in range(2)]
+        # sampling settings of the captured frame step (code-0 draw, depth-head draws), read on the device
+        self._sdev0, self._sdev1 = SampleDev(dev), SampleDev(dev)
 
     def _splits(self, B: int) -> int:
         return self.model.decoder.default_splits(B)
@@ -483,8 +485,13 @@ class Engine:
         sampling with repetition penalty, the depth head, frame log, counters.  stop = (eos_threshold,
         min_frames): the step also runs the end-of-turn test on the device (self._stop_state)."""
         nq = cfg.n_codebooks if cfg.n_codebooks > 0 else self.Q
-        key = (B, nq, cfg.temperature, cfg.top_k, cfg.rq_top_k, cfg.rep_penalty, cfg.rep_window, cfg.seed,
-               None if slot_idx is None else tuple(slot_idx.tolist()), max_frames, stop)
+        # temperature, top-k values and seed live in two device blocks the step reads when it runs, so that a
+        # request with another seed or temperature replays the same graph (the reference captures once, too)
+        self._sdev0.set(cfg.temperature, cfg.top_k, cfg.seed)
+        self._sdev1.set(cfg.temperature, cfg.rq_top_k if cfg.top_k != 1 else 1, cfg.seed)
+        # the frame log is sized in powers of two from 256 frames, so that runs of different lengths share a graph
+        max_frames = 0 if max_frames <= 0 else max(256, 1 << (max_frames - 1).bit_length())
+        key = (B, nq, cfg.rep_penalty, cfg.rep_window, None if slot_idx is None else tuple(slot_idx.tolist()), max_frames, stop)
         hit = self._frame_graphs.get(key)
         if hit is not None:
             self._frame_graphs[key] = self._frame_graphs.pop(key)  # most recently used last
@@ -494,8 +501,8 @@ class Engine:
         # max_frames == 0: no frame log, eos holds the (B) probabilities of the latest step
         frames = torch.zeros(max_frames, B, self.Q, dtype=torch.long, device=self.device) if max_frames else None
         eos = torch.zeros(max(max_frames, 1), B, dtype=torch.float32, device=self.device)
-        sp0 = make_sample_params(cfg.temperature, cfg.top_k, cfg.seed, self._frame_ctr)
-        sp1 = make_sample_params(cfg.temperature, cfg.rq_top_k if cfg.top_k != 1 else 1, cfg.seed, self._frame_ctr)
+        sp0 = make_sample_params(cfg.temperature, cfg.top_k, cfg.seed, self._frame_ctr, dev=self._sdev0)
+        sp1 = make_sample_params(cfg.temperature, cfg.rq_top_k if cfg.top_k != 1 else 1, cfg.seed, self._frame_ctr, dev=self._sdev1)
         use_rep = cfg.rep_penalty > 1.0
         win = cfg.rep_window if (use_rep and self._rep_history is not None) else 0
         codes_io = self._gc_codes_in if slot_idx is not None else self._g_codes_in
@@ -517,7 +524,7 @@ class Engine:
         # captured without a warm-up run: the step mutates seq_lens, the rep state and the counter
         g = Graph(self.model, body, warmup=0)
         entry = (g, frames, eos, (sp0, sp1, slot_idx, stop_c))
-        if len(self._frame_graphs) >= self.max_frame_graphs:  # a serving loop with ever new seeds must not grow without bound
+        if len(self._frame_graphs) >= self.max_frame_graphs:  # shapes, not settings, key a graph; still bounded
             self._frame_graphs.pop(next(iter(self._frame_graphs)))
         self._frame_graphs[key] = entry
         return entry

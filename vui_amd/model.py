@@ -235,10 +235,33 @@ class Graph:
             pass
 
 
+class SampleDev:
+    """vui_sample_dev: temperature, top-k and seed in 16 bytes of device memory that captured steps read when they
+    run.  `set` is a stream-ordered copy (it waits for the copy on the host), skipped when nothing changed."""
+
+    def __init__(self, device):
+        self.buf = torch.zeros(16, dtype=torch.uint8, device=device)
+        self._cur = None
+
+    def set(self, temperature: float, top_k: "int | None", seed: int) -> "SampleDev":
+        import struct
+
+        val = (float(temperature), int(top_k) if top_k is not None else 0, int(seed) & 0xFFFFFFFFFFFFFFFF)
+        if val != self._cur:
+            self.buf.copy_(torch.frombuffer(bytearray(struct.pack("<fiQ", *val)), dtype=torch.uint8))
+            self._cur = val
+        return self
+
+    def data_ptr(self) -> int:
+        return self.buf.data_ptr()
+
+
 def make_sample_params(temperature: float, top_k: int | None, seed: int, frame_ctr: Tensor | None,
-                       state_rows: Tensor | None = None, keep_ties: bool = False, top_p: float = 0.0):
+                       state_rows: Tensor | None = None, keep_ties: bool = False, top_p: float = 0.0,
+                       dev: "SampleDev | None" = None):
     sp = _lib.SampleParamsC()
     sp.top_p = float(top_p)
+    sp.dev = dev.data_ptr() if dev is not None else None
     sp.keep_ties = 1 if keep_ties else 0
     sp.state_rows = state_rows.data_ptr() if state_rows is not None else None
     sp.temperature = float(temperature)
@@ -413,6 +436,7 @@ class RQTransformer:
         self._gkv_graphs: dict = {}
         self._gkv_batch_sizes: tuple[int, ...] = ()
         self._ctr = torch.zeros(1, dtype=torch.int32, device=model.device)
+        self._gkv_dev = None
 
     def _call(self, hidden, code0, bias, n_q, sp, codes_out, B, stream):
         nat = self._model._native
@@ -479,10 +503,15 @@ class RQTransformer:
         self._gkv_logit_bias.zero_()
         if logit_bias is not None:
             self._gkv_logit_bias[: logit_bias.size(0)].copy_(logit_bias)
-        key = (B, Q, float(temperature), int(self.seed), self._gkv_top_k)  # everything a captured launch bakes in
+        # temperature, top-k and seed sit in a device block that the captured launch reads at each replay (the
+        # reference fills a 0-d temperature tensor before its replay, model.py:1011): one graph per (B, Q')
+        if self._gkv_dev is None:
+            self._gkv_dev = SampleDev(self._gkv_codes_out.device)
+        self._gkv_dev.set(temperature, self._gkv_top_k, self.seed)
+        key = (B, Q)
         g = self._gkv_graphs.get(key)
         if g is None:
-            sp = make_sample_params(temperature, self._gkv_top_k, self.seed, self._ctr)
+            sp = make_sample_params(temperature, self._gkv_top_k, self.seed, self._ctr, dev=self._gkv_dev)
             g = Graph(self._model, lambda st: self._call(self._gkv_backbone, self._gkv_code0, self._gkv_logit_bias,
                                                          Q, sp, self._gkv_codes_out, B, st))
             g._sp = sp
