@@ -176,7 +176,7 @@ def vocoder_line():
                  "hbm_frac": round(cb / us / 1e3 / HBM_PEAK_GBS, 4)}
 
 
-def prefill_line(model2, eng2, g, loop_too=True, reps=5):
+def prefill_line(model2, eng2, g, loop_too=True, reps=5, name="prefill_b1"):
     """Prompt ingestion: 576 positions (512 audio frames + 64 text tokens) in one pass per layer against the
     position-by-position path; flops = 2 x positions x backbone weights (attention is a few % more)."""
     import torch
@@ -209,7 +209,7 @@ def prefill_line(model2, eng2, g, loop_too=True, reps=5):
         dec.PREFILL_MIN = 4
     wparams = (frame_bytes(m, 0)["backbone"] - 67584 - m.n_quantizers * m.d_model * 2 - 3145728) / 2
     fl = 2.0 * 576 * wparams
-    return {"config": "prefill_b1", "positions": 576, "ms_one_pass": round(us_pass / 1e3, 3), "ms_position_by_position": round(us_loop / 1e3, 2),
+    return {"config": name, "positions": 576, "ms_one_pass": round(us_pass / 1e3, 3), "ms_position_by_position": round(us_loop / 1e3, 2),
             "achieved_TFLOPs": round(fl / us_pass / 1e6, 1), "mfma_frac": round(fl / us_pass / 1e6 / 2500.0, 4)}
 
 
@@ -300,7 +300,7 @@ def batch_sweep(sd, preset="A", n=40, batches=(1, 2, 4, 8, 16)):
     return out
 
 
-def serve_line(sd, preset="A", n_requests=32, max_rows=16):
+def serve_line(sd, preset="A", n_requests=32, max_rows=16, int8=False):
     """Continuous batching as a served workload (Engine.render_continuous): n_requests requests, each a
     256-position prompt and two text chunks of 16 positions / 5 words, through max_rows rows (bf16); EOS off,
     so every chunk runs to its 40-frame cap.  Wall clock includes prompt ingestion, the host loop, the
@@ -312,7 +312,7 @@ def serve_line(sd, preset="A", n_requests=32, max_rows=16):
     from vui_amd.synthetic import nano_for_cache
 
     S = 512
-    model = Vui(nano_for_cache(preset, S), sd, device="cuda", dtype=torch.bfloat16)
+    model = Vui(nano_for_cache(preset, S), sd, device="cuda", dtype=torch.bfloat16, int8=int8)
     m = model.config.model
     eng = Engine(model=model, max_rows=max_rows, max_seq=S)
     g = torch.Generator().manual_seed(9)
@@ -329,7 +329,7 @@ def serve_line(sd, preset="A", n_requests=32, max_rows=16):
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     n_frames = sum(len(o) for o in out)
-    return {"config": "continuous_batching_b16", "requests": n_requests, "rows": max_rows, "frames": n_frames,
+    return {"config": "continuous_batching_b16" + ("_int8" if int8 else ""), "requests": n_requests, "rows": max_rows, "frames": n_frames,
             "wall_s": round(dt, 3), "aggregate_frames_per_s": round(n_frames / dt, 1), "rtf_aggregate": round(n_frames / dt / 12.5, 1)}
 
 
@@ -401,6 +401,10 @@ def suite(model, eng, d, sd, preset="A"):
     lines.append({"config": "rq_head_b1", "frames": 1000, "us_per_frame": round(us, 2), "unique_bytes": int(b),
                   "achieved_GBs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4)})
     lines.append(prefill_line(model2, eng2, g))
+    model8 = Vui(nano_for_cache(preset, 1024), sd, device="cuda", dtype=torch.bfloat16, int8=True)
+    eng8 = Engine(model=model8, max_rows=1, max_seq=1024)
+    lines.append(prefill_line(model8, eng8, g, name="prefill_b1_int8"))
+    del model8, eng8
     emb = (torch.randn(1, 576, m.d_model, generator=g) * 0.08).to(torch.bfloat16).cuda()
     # a streamed turn: one graph replay per frame plus the host's per-frame EOS read (Row.stream)
     from vui_amd.engine import Chunk
@@ -440,6 +444,7 @@ def suite(model, eng, d, sd, preset="A"):
     del eng2, model2, voc
     lines.append(b16_line(sd, preset))
     lines.append(serve_line(sd, preset))
+    lines.append(serve_line(sd, preset, int8=True))
     lines.append(copy_line())
     return lines
 
@@ -538,14 +543,15 @@ def main():
         from vui_amd.synthetic import nano_for_cache, synthetic_state_dict
 
         sd = synthetic_state_dict(nano_for_cache(args.preset, 64).model, seed=0)
-        model2 = Vui(nano_for_cache(args.preset, 1024), sd, device="cuda", dtype=torch.bfloat16)
+        model2 = Vui(nano_for_cache(args.preset, 1024), sd, device="cuda", dtype=torch.bfloat16, int8=args.int8)
         eng2 = Engine(model=model2, max_rows=1, max_seq=1024)
-        print(json.dumps(prefill_line(model2, eng2, torch.Generator().manual_seed(0), loop_too=False, reps=20)))
+        print(json.dumps(prefill_line(model2, eng2, torch.Generator().manual_seed(0), loop_too=False, reps=20,
+                                      name="prefill_b1_int8" if args.int8 else "prefill_b1")))
         return
     if args.serve_only:
         from vui_amd.synthetic import nano_for_cache, synthetic_state_dict
 
-        print(json.dumps(serve_line(synthetic_state_dict(nano_for_cache(args.preset, 64).model, seed=0), args.preset)))
+        print(json.dumps(serve_line(synthetic_state_dict(nano_for_cache(args.preset, 64).model, seed=0), args.preset, int8=args.int8)))
         return
     if args.sweep_only:
         from vui_amd.synthetic import nano_for_cache, synthetic_state_dict

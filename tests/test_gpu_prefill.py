@@ -94,15 +94,23 @@ def test_prefill_window_and_errors():
         m.decoder.forward_flash(torch.zeros(1, 300, d.d_model, dtype=BF, device="cuda"), None)
 
 
-def test_prefill_nano_576_positions():
-    """The benchmark's prompt (512 audio frames + 64 text tokens) at Vui Nano dims: last hidden state of
-    the pass against the position-by-position path, and the decode step after it."""
+@pytest.mark.parametrize("int8", [False, True])
+def test_prefill_nano_576_positions(int8):
+    """The benchmark's prompt (512 audio frames + 64 text tokens) at Vui Nano dims, with bf16 and with weight-only
+    int8 matrices: the pass against the oracle (which evaluates the same int8 weights) on the first 96 positions,
+    its last hidden state and the cache it leaves against the position-by-position path."""
     d = O.Dims()
     sd = O.synthetic_state_dict(d, seed=0)
-    m = make_model(d, sd, BF, max_seqlen=1408)
+    m = make_model(d, sd, BF, int8=int8, max_seqlen=1408)
     m.decoder.allocate_flash_kv_cache(1, m.device, BF, max_seqlen=1408)
+    assert m.decoder._prefill_available()
     g = torch.Generator().manual_seed(0)
     emb = O.rnd(torch.randn(1, 576, d.d_model, generator=g) * 0.02 * 4, BF).to(BF).cuda()
+    o = O.OracleModel(d, sd, BF, n_slots=1, max_seqlen=128, int8=int8)
+    ref96 = o.prefill(emb[0, :96].float().cpu(), slot=0)
+    got96 = m.decoder.forward_flash(emb[:, :96].contiguous(), None)[0]
+    assert rel_err(got96, ref96) <= BF16_TOL, rel_err(got96, ref96)
+    m.decoder.flash_kv_caches[0].seq_lens.zero_()
     a = m.decoder.forward_flash(emb, None)
     ka = m.decoder._k[:, 0, :576].clone()
     m.decoder.flash_kv_caches[0].seq_lens.zero_()

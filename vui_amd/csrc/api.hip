@@ -357,7 +357,8 @@ int vui_prefill(vui_ctx* ctx, const void* emb_in, int T, int slot, int pos0, int
   if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
   if (!emb_in || !seq_lens || !k_cache || !v_cache || !hidden_out || !scratch) { vui_set_error("vui_prefill: NULL argument"); return VUI_EINVAL; }
   if (((uintptr_t)scratch & 255) || scratch_bytes < 0) { vui_set_error("vui_prefill: scratch must be 256-byte aligned"); return VUI_EINVAL; }
-  return launch_prefill(ctx->cfg, ctx->w, prefill_weight_bytes(ctx->cfg) ? ctx->pf_w : nullptr, emb_in, T, slot, pos0, seq_lens, k_cache,
+  const void* tiled = prefill_weight_bytes(ctx->cfg) ? ctx->pf_w : ((ctx->cfg.int8_backbone && ctx->bb_w8_bytes) ? ctx->bb_w8 : nullptr);
+  return launch_prefill(ctx->cfg, ctx->w, tiled, emb_in, T, slot, pos0, seq_lens, k_cache,
                         v_cache, hidden_out, scratch, (size_t)scratch_bytes, (hipStream_t)stream);
 }
 

@@ -2,7 +2,8 @@
 //
 //   Decoder.forward_flash / Engine._prefill_emb with T > 1  (src/vui/model.py:534-549, engine.py:674-694)
 //
-// bf16 only.  Per layer: row RMSNorm, QKV GEMM, one kernel that rotates the new keys, appends keys and values to the
+// bf16 activations; the layers' matrices bf16, or int8 with per-row scales (widened in registers inside the GEMMs,
+// the scale on the finished sum).  Per layer: row RMSNorm, QKV GEMM, one kernel that rotates the new keys, appends keys and values to the
 // cache and stages the slot's keys / transposed values in operand layout, causal attention of the new positions
 // against them (the same kernel rotates the queries in place; scores never leave the registers; probabilities
 // rounded to bf16 before they meet the values), out_proj GEMM with the residual add in its epilogue, row RMSNorm, one GEMM over
@@ -37,7 +38,10 @@ __host__ __device__ __forceinline__ size_t pf_toff(int r, int k, int K) {
 
 struct PfGemm {
   const bf16_t* X;   // activations (M x K), tiled
-  const bf16_t* W;   // weights (N x K), tiled
+  const void* W;     // weights (N x K), tiled: bf16, or int8 (the byte form of the layout: block (r / 16, k / 64) at
+                     // ((r / 16) * (K / 64) + k / 64) * 1024 bytes, the 16 bytes k % 16 = 0..15 of lane (r % 16) + 16 * ((k % 64) / 16)
+                     // at 16 * lane) with the per-row scales sc (and sc2 for the second matrix of a SwiGLU pair)
+  const bf16_t *sc, *sc2;
   void* C;           // output (M x N) bf16: row-major with row stride ldc (PF_RESID: in place on the residual), or tiled
   int M, N, K, ldc;
 };
@@ -58,8 +62,18 @@ __global__ __launch_bounds__(256) void pf_tile_kernel(const bf16_t* __restrict__
 // results do not depend on timing).
 // DUAL: two weight matrices against the same activations, h = rnd(rnd(silu(rnd(a))) * rnd(c)) written once
 // (SwiGLU, src/vui/model.py:282) instead of two products and a pass over both.
-template <int EPI, bool DUAL>
-__global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf16_t* __restrict__ W2, int c_tiled) {
+// eight int8 -> four packed bf16 pairs, exact
+__device__ __forceinline__ uint4 pf_widen8(uint32_t lo, uint32_t hi) {
+  uint4 r;
+  r.x = f2bf2((float)(int8_t)(lo & 0xff), (float)(int8_t)((lo >> 8) & 0xff));
+  r.y = f2bf2((float)(int8_t)((lo >> 16) & 0xff), (float)(int8_t)(lo >> 24));
+  r.z = f2bf2((float)(int8_t)(hi & 0xff), (float)(int8_t)((hi >> 8) & 0xff));
+  r.w = f2bf2((float)(int8_t)((hi >> 16) & 0xff), (float)(int8_t)(hi >> 24));
+  return r;
+}
+
+template <int EPI, bool DUAL, bool I8>
+__global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const void* __restrict__ W2, int c_tiled) {
   constexpr int TILE = 1024;  // floats of one partial tile
   constexpr int PW = (DUAL ? 2 : 1) * TILE;
   __shared__ float part[4 * PW];
@@ -75,14 +89,15 @@ __global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf1
   const int s0 = nsteps * wave / 4, s1 = nsteps * (wave + 1) / 4;
   const int MB = (p.M + 15) >> 4, NB = (p.N + 15) >> 4;  // 16-row blocks; a tile past the end reads the last block again
   const bf16_t* xr[2];
-  const bf16_t* wr[2];
-  const bf16_t* vr[2];
+  const char* wr[2];  // byte addresses: a block is 2048 bytes of bf16 (two 16-byte pieces per lane) or 1024 of int8 (one)
+  const char* vr[2];
+  constexpr int WB = I8 ? 1024 : 2048, WL = 16;
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     xr[j] = p.X + (size_t)min((m0 >> 4) + j, MB - 1) * nsteps * 1024 + lane * 8;
-    const size_t wo = (size_t)min((n0 >> 4) + j, NB - 1) * nsteps * 1024 + lane * 8;
-    wr[j] = p.W + wo;
-    vr[j] = DUAL ? W2 + wo : p.W + wo;
+    const size_t wo = (size_t)min((n0 >> 4) + j, NB - 1) * nsteps * WB + lane * WL;
+    wr[j] = (const char*)p.W + wo;
+    vr[j] = DUAL ? (const char*)W2 + wo : (const char*)p.W + wo;
   }
   pf_floatx4 acc[2][2], acc2[2][2];
 #pragma unroll
@@ -102,11 +117,26 @@ __global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf1
 #pragma unroll
     for (int h = 0; h < 2; ++h)
 #pragma unroll
+      for (int j = 0; j < 2; ++j) xa[j][h] = *reinterpret_cast<const uint4*>(xr[j] + k + 512 * h);
+    if (I8) {
+#pragma unroll
       for (int j = 0; j < 2; ++j) {
-        xa[j][h] = *reinterpret_cast<const uint4*>(xr[j] + k + 512 * h);
-        wa[j][h] = *reinterpret_cast<const uint4*>(wr[j] + k + 512 * h);
-        if (DUAL) va[j][h] = *reinterpret_cast<const uint4*>(vr[j] + k + 512 * h);
+        const uint4 w8 = *reinterpret_cast<const uint4*>(wr[j] + (size_t)s * WB);
+        wa[j][0] = pf_widen8(w8.x, w8.y); wa[j][1] = pf_widen8(w8.z, w8.w);
+        if (DUAL) {
+          const uint4 v8 = *reinterpret_cast<const uint4*>(vr[j] + (size_t)s * WB);
+          va[j][0] = pf_widen8(v8.x, v8.y); va[j][1] = pf_widen8(v8.z, v8.w);
+        }
       }
+    } else {
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          wa[j][h] = *reinterpret_cast<const uint4*>(wr[j] + (size_t)s * WB + 1024 * h);
+          if (DUAL) va[j][h] = *reinterpret_cast<const uint4*>(vr[j] + (size_t)s * WB + 1024 * h);
+        }
+    }
 #pragma unroll
     for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -137,6 +167,10 @@ __global__ __launch_bounds__(256) void pf_gemm4_kernel(const PfGemm p, const bf1
     if (DUAL) u[r] = ((part[TILE + e] + part[PW + TILE + e]) + part[2 * PW + TILE + e]) + part[3 * PW + TILE + e];
   }
   if (m >= p.M || n >= p.N) return;
+  if (I8) {  // y[n] = scale[n] * sum_k q[n, k] x[k]
+    for (int r = 0; r < 4; ++r)
+      if (n + r < p.N) { v[r] *= bf2f(p.sc[n + r]); if (DUAL) u[r] *= bf2f(p.sc2[n + r]); }
+  }
   bf16_t* c = (bf16_t*)p.C + (c_tiled ? pf_toff(m, n, p.N) : (size_t)m * p.ldc + n);  // n % 4 == 0: inside one piece
   if (DUAL) {
 #pragma unroll
@@ -378,13 +412,19 @@ __global__ __launch_bounds__(256) void pf_stage_kv_kernel(bf16_t* __restrict__ q
 
 __global__ void pf_set_len_kernel(int32_t* seq_lens, int slot, int v) { seq_lens[slot] = v; }
 
-// bf16 out, K split over the waves of a workgroup; W2 != nullptr: the SwiGLU pair
-static int pf_gemm4(int epi, const PfGemm& g, const bf16_t* W2, int c_tiled, hipStream_t st) {
+// bf16 out, K split over the waves of a workgroup; W2 != nullptr: the SwiGLU pair; i8: int8 matrices with g.sc / g.sc2
+static int pf_gemm4(int epi, const PfGemm& g, const void* W2, int c_tiled, bool i8, hipStream_t st) {
   if (g.K % 64 || g.N % 16 || g.M < 1 || g.N < 1 || (c_tiled && g.N % 64)) { vui_set_error("prefill GEMM: bad shape N=%d K=%d", g.N, g.K); return VUI_EINVAL; }
   const dim3 grid((unsigned)(((g.M + 31) / 32) * ((g.N + 31) / 32)));
-  if (W2) hipLaunchKernelGGL((pf_gemm4_kernel<PF_BF16, true>), grid, dim3(256), 0, st, g, W2, c_tiled);
-  else if (epi == PF_RESID) hipLaunchKernelGGL((pf_gemm4_kernel<PF_RESID, false>), grid, dim3(256), 0, st, g, W2, c_tiled);
-  else hipLaunchKernelGGL((pf_gemm4_kernel<PF_BF16, false>), grid, dim3(256), 0, st, g, W2, c_tiled);
+  if (i8) {
+    if (W2) hipLaunchKernelGGL((pf_gemm4_kernel<PF_BF16, true, true>), grid, dim3(256), 0, st, g, W2, c_tiled);
+    else if (epi == PF_RESID) hipLaunchKernelGGL((pf_gemm4_kernel<PF_RESID, false, true>), grid, dim3(256), 0, st, g, W2, c_tiled);
+    else hipLaunchKernelGGL((pf_gemm4_kernel<PF_BF16, false, true>), grid, dim3(256), 0, st, g, W2, c_tiled);
+  } else {
+    if (W2) hipLaunchKernelGGL((pf_gemm4_kernel<PF_BF16, true, false>), grid, dim3(256), 0, st, g, W2, c_tiled);
+    else if (epi == PF_RESID) hipLaunchKernelGGL((pf_gemm4_kernel<PF_RESID, false, false>), grid, dim3(256), 0, st, g, W2, c_tiled);
+    else hipLaunchKernelGGL((pf_gemm4_kernel<PF_BF16, false, false>), grid, dim3(256), 0, st, g, W2, c_tiled);
+  }
   HIP_TRY(hipGetLastError());
   return VUI_OK;
 }
@@ -410,9 +450,10 @@ static size_t pf_layer_elems(const vui_config& c) {
   const size_t d = c.d_model, nq = (size_t)c.n_heads * c.head_dim, nkv = (size_t)c.n_kv_heads * c.head_dim, F = c.ffn;
   return (nq + 2 * nkv) * d + d * nq + 2 * F * d + d * F;
 }
+// the pass's own tiled copy: bf16 matrices only (an int8 context reads the batched backbone kernel's tiled int8 copy)
 size_t prefill_weight_bytes(const vui_config& c) {
   char why[96];
-  return prefill_supported(c, why, sizeof(why)) ? pf_layer_elems(c) * c.n_layers * 2 : 0;
+  return (!c.int8_backbone && prefill_supported(c, why, sizeof(why))) ? pf_layer_elems(c) * c.n_layers * 2 : 0;
 }
 
 // one-time: the layers' projection weights in the GEMMs' operand layout
@@ -439,7 +480,8 @@ int prefill_tile_weights(const vui_config& c, const vui_weights& w, void* dst, h
 bool prefill_supported(const vui_config& c, char* why, size_t why_len) {
   const char* r = nullptr;
   const int nkv = c.n_kv_heads * c.head_dim;
-  if (c.dtype != VUI_DTYPE_BF16 || c.int8_backbone) r = "bf16 weights only";
+  if (c.dtype != VUI_DTYPE_BF16) r = "bf16 activations only";
+  else if (c.int8_backbone && !bb_batch_weight_bytes(c, 256)) r = "int8 weights: no tiled int8 copy (it belongs to the batched backbone kernel, which does not take this configuration)";
   else if ((c.d_model % 64) || (c.ffn % 64) || ((c.n_heads * c.head_dim) % 64) || (c.head_dim % 32) || c.head_dim > 128 || (nkv % 8) || (c.rope_dim & 1))
     r = "d_model, heads x head_dim and ffn must be multiples of 64, head_dim a multiple of 32 up to 128";
   else if (c.n_kv_heads < 1 || c.n_heads % c.n_kv_heads) r = "heads must be a multiple of KV heads";
@@ -473,17 +515,19 @@ int launch_prefill(const vui_config& c, const vui_weights& w, const void* tiled_
   int rc;
   for (int l = 0; l < c.n_layers; ++l) {
     const vui_layer_weights& lw = w.layers[l];
-    const bf16_t* t_qkv = (const bf16_t*)tiled_w + pf_layer_elems(c) * l;
-    const bf16_t* t_o = t_qkv + (size_t)(nq + 2 * nkv) * d;
-    const bf16_t* t_1 = t_o + (size_t)d * nq;
-    const bf16_t* t_3 = t_1 + (size_t)F * d;
-    const bf16_t* t_2 = t_3 + (size_t)F * d;
+    const bool i8 = c.int8_backbone != 0;
+    const size_t wsz = i8 ? 1 : 2;
+    const char* t_qkv = (const char*)tiled_w + pf_layer_elems(c) * wsz * l;
+    const char* t_o = t_qkv + (size_t)(nq + 2 * nkv) * d * wsz;
+    const char* t_1 = t_o + (size_t)d * nq * wsz;
+    const char* t_3 = t_1 + (size_t)F * d * wsz;
+    const char* t_2 = t_3 + (size_t)F * d * wsz;
     bf16_t* kc = (bf16_t*)k_cache + slab * l;
     bf16_t* vc = (bf16_t*)v_cache + slab * l;
     hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)lw.attn_norm, xn, T, d, c.norm_eps, 1);
     PfGemm g{};
-    g.X = xn; g.W = t_qkv; g.C = qkv; g.M = T; g.N = nq + 2 * nkv; g.K = d; g.ldc = nq + 2 * nkv;
-    if ((rc = pf_gemm4(PF_BF16, g, nullptr, 0, st))) return rc;
+    g.X = xn; g.W = t_qkv; g.C = qkv; g.M = T; g.N = nq + 2 * nkv; g.K = d; g.ldc = nq + 2 * nkv; g.sc = (const bf16_t*)lw.s_qkv;
+    if ((rc = pf_gemm4(PF_BF16, g, nullptr, 0, i8, st))) return rc;
     // attention over the L cached positions of this slot
     bf16_t* krow = kc + (size_t)slot * S * nkv;
     bf16_t* vrow = vc + (size_t)slot * S * nkv;
@@ -502,15 +546,15 @@ int launch_prefill(const vui_config& c, const vui_weights& w, const void* tiled_
       }
     }
     PfGemm wo{};
-    wo.X = att; wo.W = t_o; wo.C = x; wo.ldc = d; wo.M = T; wo.N = d; wo.K = nq;
-    if ((rc = pf_gemm4(PF_RESID, wo, nullptr, 0, st))) return rc;
+    wo.X = att; wo.W = t_o; wo.C = x; wo.ldc = d; wo.M = T; wo.N = d; wo.K = nq; wo.sc = (const bf16_t*)lw.s_o;
+    if ((rc = pf_gemm4(PF_RESID, wo, nullptr, 0, i8, st))) return rc;
     hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)lw.mlp_norm, xn, T, d, c.norm_eps, 1);
     PfGemm f1{};
-    f1.X = xn; f1.W = t_1; f1.C = fa; f1.ldc = F; f1.M = T; f1.N = F; f1.K = d;
-    if ((rc = pf_gemm4(PF_BF16, f1, t_3, 1, st))) return rc;  // written tiled: operand of W2
+    f1.X = xn; f1.W = t_1; f1.C = fa; f1.ldc = F; f1.M = T; f1.N = F; f1.K = d; f1.sc = (const bf16_t*)lw.s_1; f1.sc2 = (const bf16_t*)lw.s_3;
+    if ((rc = pf_gemm4(PF_BF16, f1, t_3, 1, i8, st))) return rc;  // written tiled: operand of W2
     PfGemm f2{};
-    f2.X = fa; f2.W = t_2; f2.C = x; f2.ldc = d; f2.M = T; f2.N = d; f2.K = F;
-    if ((rc = pf_gemm4(PF_RESID, f2, nullptr, 0, st))) return rc;
+    f2.X = fa; f2.W = t_2; f2.C = x; f2.ldc = d; f2.M = T; f2.N = d; f2.K = F; f2.sc = (const bf16_t*)lw.s_2;
+    if ((rc = pf_gemm4(PF_RESID, f2, nullptr, 0, i8, st))) return rc;
   }
   hipLaunchKernelGGL(pf_rownorm_kernel, dim3((T + 3) / 4), dim3(256), 0, st, x, (const bf16_t*)w.final_norm, (bf16_t*)out, T, d, c.norm_eps, 0);
   hipLaunchKernelGGL(pf_set_len_kernel, dim3(1), dim3(1), 0, st, seq_lens, slot, L);
