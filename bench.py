@@ -441,7 +441,23 @@ def suite(model, eng, d, sd, preset="A"):
     dt = time.perf_counter() - t0
     lines.append({"config": "stream_b1_audio", "frames": n_out, "chunks": 4, "ms_per_frame_wall": round(dt * 1e3 / n_out, 4),
                   "frames_per_s": round(n_out / dt, 1), "rtf": round(n_out / dt / 12.5, 2)})
-    del eng2, model2, voc
+    # the same turn with the GPU divided: decode step on 160 compute units, vocoder of the previous frame beside it
+    # on the other 96 (Engine(split_cus=160))
+    del eng2, row2, row3
+    eng3 = Engine(model=model2, codec=voc, max_rows=1, max_seq=1024, split_cus=160)
+    row4 = eng3.new_row()
+    n_out = sum(1 for _ in row4.stream_audio(chunks[:1], cfg_s))
+    row4.reset()
+    row4._codec_ctx.reset()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    n_out = sum(1 for _ in row4.stream_audio(chunks, cfg_s))
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    model2._native.status()
+    lines.append({"config": "stream_b1_audio_split160", "frames": n_out, "chunks": 4, "ms_per_frame_wall": round(dt * 1e3 / n_out, 4),
+                  "frames_per_s": round(n_out / dt, 1), "rtf": round(n_out / dt / 12.5, 2)})
+    del eng3, row4, model2, voc
     lines.append(b16_line(sd, preset))
     lines.append(serve_line(sd, preset))
     lines.append(serve_line(sd, preset, int8=True))

@@ -146,6 +146,17 @@ int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream);
  * local memory keeps its keys in the workspace and is still fused; when even its values alone do not fit,
  * vui_backbone_step alone still takes the fused form, under the same switch.  No counterpart in the reference. */
 int vui_ctx_fused(vui_ctx* ctx, int enable);
+/* A stream whose kernels run on compute units [first_cu, first_cu + n_cus) only (hipExtStreamCreateWithCUMask),
+ * and a context whose batch-1 one-launch kernel uses `nwg` workgroups instead of one per compute unit of the whole
+ * GPU (160, 192, 224 or all of them): together they leave the other compute units to other work of the same process while a frame step runs
+ * (a persistent kernel needs every one of its workgroups resident: on a stream of its own with n_cus >= nwg it
+ * has them).  vui_ctx_workgroups is called after vui_ctx_init (which restores the full width); with nwg below
+ * the full width the batched persistent kernels (2..16 rows) are switched off for the context.  The stream is
+ * kept for the life of the process: there is no destroy call (on this ROCm release creating a masked stream after
+ * one had been destroyed crashed, and so did a mask that is not one contiguous range).  No counterpart in the reference. */
+int vui_cu_stream_create(int first_cu, int n_cus, vui_stream_t* out);
+int vui_ctx_workgroups(vui_ctx* ctx, int nwg);
+
 /* 1 when the depth head of 2..16 rows runs as one persistent kernel (bf16, enough resident workgroups, the
  * fused form switched on), else 0 and vui_last_error() says why.  No counterpart in the reference. */
 int vui_ctx_rq_batch(vui_ctx* ctx);

@@ -188,12 +188,14 @@ def test_config1_greedy_grid_fp32():
 BF16_TOL = 2.0 ** -5  # stated bf16 tolerance: 8 bf16 ulps of the largest logit
 
 
-@pytest.mark.parametrize("fused,int8", [(0, False), (1, False), (0, True), (1, True)])
-def test_nano_backbone_bf16_vs_oracle(fused, int8):
+@pytest.mark.parametrize("fused,int8,nwg", [(0, False, 0), (1, False, 0), (0, True, 0), (1, True, 0), (1, False, 160), (1, True, 192)])
+def test_nano_backbone_bf16_vs_oracle(fused, int8, nwg):
     """One decode step at Vui Nano dims in bf16 at cache lengths 0, 255, 1023 and 4095, as a sequence of
     kernels (fused=0) and as the one persistent kernel (fused=1, whose attention split and merge phases are
     code of their own); with bf16 weights and with the backbone's matrices as weight-only int8 (the oracle
-    evaluates the same int8 weights and scales: the quantisation itself is not part of the difference).
+    evaluates the same int8 weights and scales: the quantisation itself is not part of the difference); nwg: the
+    persistent kernel on that many workgroups instead of one per compute unit (vui_ctx_workgroups: other rows per
+    workgroup, another attention split).
 
     With an empty cache the native step equals the oracle's bf16 regime bit for bit (same
     roundings, same per-row summation).  With a filled cache the attention sums run in another
@@ -209,6 +211,8 @@ def test_nano_backbone_bf16_vs_oracle(fused, int8):
         of.q8 = o.q8
     m.decoder.allocate_flash_kv_cache(1, m.device, BF, max_seqlen=S)
     assert m._native.fused(fused) == bool(fused), "the fused kernel must be available on an MI355X"
+    if nwg:
+        m._native.workgroups(nwg)
     g = torch.Generator().manual_seed(3)
     for L in (0, 255, 1023, 4095):
         Sf = 1100 if L < 1100 else S  # positions filled with noise (everything a step at this length can read)
@@ -229,6 +233,7 @@ def test_nano_backbone_bf16_vs_oracle(fused, int8):
         eos = torch.empty(1, 1, dtype=BF, device="cuda")
         m.decoder._step(codes=codes.cuda(), emb=None, slot_idx=None, seq_inc=None, B=1, hidden_out=hid,
                         cb0_out=cb0, eos_out=eos, n_splits=32, stream=torch.cuda.current_stream().cuda_stream)
+        m._native.status()
         assert int(m.decoder.flash_kv_caches[0].seq_lens[0]) == L + 1
         if L == 0 and not fused and not int8:
             # no attention sums to reorder: the step follows the oracle's roundings closely (on this input bit for
@@ -243,12 +248,14 @@ def test_nano_backbone_bf16_vs_oracle(fused, int8):
             assert int(cb0[0].float().argmax()) == int(cb_ref[0].argmax())
 
 
-@pytest.mark.parametrize("fused", [0, 1])
+@pytest.mark.parametrize("fused", [0, 1, 160])
 def test_nano_rq_bf16_vs_oracle(fused):
     """Depth head at Vui Nano dims in bf16: greedy tokens equal wherever the oracle's top-2 margin
     exceeds the tolerance (batch of 4 through the kernel sequence; row by row through the fused kernel)."""
     d, sd, m, o = _nano_models(BF)
-    assert m._native.fused(fused) == bool(fused)
+    assert m._native.fused(min(fused, 1)) == bool(fused)
+    if fused > 1:  # the fused kernel on that many workgroups
+        m._native.workgroups(fused)
     g = torch.Generator().manual_seed(4)
     hidden = O.rnd(torch.randn(4, d.d_model, generator=g), BF)
     code0 = torch.randint(0, d.codebook_size, (4,), generator=g)

@@ -184,11 +184,13 @@ def test_engine_stream_sampled_and_cancel():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("graph", [False, True])
+@pytest.mark.parametrize("graph", [False, True, "split"])
 def test_stream_audio_equals_vocoder_oracle_on_streamed_codes(graph):
     """Row.stream (= stream_audio) on an engine with a vocoder: every frame of Row.stream_codes passed through the
     row's vocoder context.  Same turn, same seed: the audio is the vocoder oracle's for the codes Row.stream_codes
-    yields; an early stop by the consumer leaves the row and the vocoder context usable."""
+    yields; an early stop by the consumer leaves the row and the vocoder context usable.  "split": the engine
+    with the GPU divided between the decode step (160 compute units) and the vocoder (the rest), the vocoder of
+    one frame running beside the decode step of the next."""
     import dataclasses
 
     from oracle import codec_oracle as CO
@@ -203,12 +205,12 @@ def test_stream_audio_equals_vocoder_oracle_on_streamed_codes(graph):
                       decoder_dim=128, rates=(3, 2))
     csd = CO.synthetic_codec_state_dict(cd, seed=4)
     dec = QwenCodecDecoder(csd, CodecConfig(**dataclasses.asdict(cd)), device="cuda")
-    if graph:
+    if graph is True:
         dec.setup_streaming_graph(1)
     model = make_model(d, sd, torch.bfloat16, max_seqlen=320)
     ch = [Chunk(emb=e[None].cuda().to(torch.bfloat16), n_words=w) for e, w in _chunks(d, 2, words=3)]
     cfg = GenConfig(eos_threshold=2.0, rep_window=4, top_k=5)
-    eng = Engine(model=model, codec=dec, max_rows=1, max_seq=320)
+    eng = Engine(model=model, codec=dec, max_rows=1, max_seq=320, split_cus=160 if graph == "split" else None)
     row = eng.new_row()
     audio = [a.clone().cpu() for a in row.stream(ch, cfg)]  # with a vocoder Row.stream hands out audio, as the reference's
     row.reset()

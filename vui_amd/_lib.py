@@ -80,6 +80,8 @@ SIGNATURES = {
     "vui_debug_set_epoch": (_I, [_P, C.c_uint32]),
     "vui_ctx_rq_batch": (_I, [_P]),
     "vui_ctx_bb_batch": (_I, [_P]),
+    "vui_cu_stream_create": (_I, [_I, _I, C.POINTER(_P)]),
+    "vui_ctx_workgroups": (_I, [_P, _I]),
     "vui_debug_phase_clock": (_I, [_P, _P, _I, _I]),
     "vui_prefill_scratch_bytes": (_L, [C.POINTER(VuiConfigC), _I, _I]),
     "vui_prefill": (_I, [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _L, _P]),

@@ -7,6 +7,7 @@
 #include <new>
 
 #include "internal.h"
+#include <hip/hip_ext.h>
 
 static thread_local char g_err[512] = "";
 
@@ -279,6 +280,39 @@ int vui_ctx_init(vui_ctx* ctx, vui_stream_t stream) {
     if (cap >= ctx->nwg) ctx->rqb_ok = 1;
     else snprintf(ctx->rqb_why, sizeof(ctx->rqb_why), "only %d workgroups can be resident, %d needed", cap, ctx->nwg);
   }
+  return VUI_OK;
+}
+
+// ---- a share of the GPU for the one-launch kernel ----
+int vui_cu_stream_create(int first_cu, int n_cus, vui_stream_t* out) {
+  if (!out) { vui_set_error("NULL argument"); return VUI_EINVAL; }
+  int dev = 0, cus = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  if (first_cu < 0 || n_cus < 1 || first_cu + n_cus > cus || cus > 1024) { vui_set_error("compute units [%d, %d) outside [0, %d)", first_cu, first_cu + n_cus, cus); return VUI_EINVAL; }
+  uint32_t mask[32];
+  memset(mask, 0, sizeof(mask));
+  for (int b = first_cu; b < first_cu + n_cus; ++b) mask[b >> 5] |= 1u << (b & 31);
+  hipStream_t st = nullptr;
+  HIP_TRY(hipExtStreamCreateWithCUMask(&st, (uint32_t)((cus + 31) / 32), mask));
+  *out = (vui_stream_t)st;
+  return VUI_OK;
+}
+
+int vui_ctx_workgroups(vui_ctx* ctx, int nwg) {
+  if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
+  const vui_config& c = ctx->cfg;
+  if (!ctx->fused_ok) { vui_set_error("the one-launch kernel is not available: %s", ctx->fused_why); return VUI_EINVAL; }
+  // widths that were run against the oracle; at 144 (the fewest the widest matrix of Vui Nano allows) a launch ended
+  // in its bounded wait, cause not found, so narrower widths are refused rather than tried
+  if (nwg < 160 || nwg > FUSED_NWG || nwg % 32) { vui_set_error("workgroups %d: 160, 192, 224 or %d", nwg, FUSED_NWG); return VUI_EINVAL; }
+  int ns = nwg / (c.n_heads > 0 ? c.n_heads : 1);
+  if (ns > FUSED_NS) ns = FUSED_NS;
+  char why[96] = "";
+  if (ns < 1 || !frame_supported(c, nwg, ns, true, why, sizeof(why))) { vui_set_error("the one-launch kernel does not run on %d workgroups: %s", nwg, why[0] ? why : "too few for the heads"); return VUI_EINVAL; }
+  ctx->nwg = nwg;
+  ctx->ns = ns;
+  if (nwg != FUSED_NWG) { ctx->rqb_ok = 0; ctx->bb_ok = 0; snprintf(ctx->rqb_why, sizeof(ctx->rqb_why), "the context was limited to %d workgroups", nwg); snprintf(ctx->bb_why, sizeof(ctx->bb_why), "the context was limited to %d workgroups", nwg); }
   return VUI_OK;
 }
 

@@ -190,10 +190,46 @@ class Row:
         if self._codec_ctx is None:
             yield from self.stream_codes(chunks, cfg, cancel, reset_rep=reset_rep, final_turn=final_turn)
             return
-        if self._codec_ctx._stack is None:
-            self._codec_ctx.prefill(n_codebooks=cfg.n_codebooks)
-        for codes in self.stream_codes(chunks, cfg, cancel, reset_rep=reset_rep, final_turn=final_turn):
-            yield self._engine._stream_decode_frame(self, codes, cfg.n_codebooks)
+        eng = self._engine
+        if eng._split is None:
+            if self._codec_ctx._stack is None:
+                self._codec_ctx.prefill(n_codebooks=cfg.n_codebooks)
+            for codes in self.stream_codes(chunks, cfg, cancel, reset_rep=reset_rep, final_turn=final_turn):
+                yield eng._stream_decode_frame(self, codes, cfg.n_codebooks)
+            return
+        # divided GPU: a frame's codes are complete when stream_codes hands them out (it has waited for the step's
+        # event), so the vocoder of frame f is enqueued on its own share at once and runs while the decode step of
+        # frame f + 1, already in flight, finishes on the other; its audio is handed out one iteration later.  The
+        # audio tensor is the vocoder's static buffer: it is overwritten when the generator is resumed.
+        s_dec, s_voc = eng._split
+        cur = torch.cuda.current_stream()
+        s_dec.wait_stream(cur)
+        s_voc.wait_stream(cur)
+        with torch.cuda.stream(s_voc):
+            if self._codec_ctx._stack is None:
+                self._codec_ctx.prefill(n_codebooks=cfg.n_codebooks)
+        it = self.stream_codes(chunks, cfg, cancel, reset_rep=reset_rep, final_turn=final_turn)
+        pending = None  # (audio, event) of the vocoder step in flight
+        try:
+            while True:
+                with torch.cuda.stream(s_dec):
+                    codes = next(it, None)
+                if pending is not None:
+                    audio, ev = pending
+                    pending = None
+                    ev.synchronize()
+                    yield audio
+                if codes is None:
+                    break
+                with torch.cuda.stream(s_voc):
+                    audio = eng._stream_decode_frame(self, codes, cfg.n_codebooks)
+                    ev = torch.cuda.Event()
+                    ev.record(s_voc)
+                pending = (audio, ev)
+        finally:
+            it.close()
+            cur.wait_stream(s_dec)
+            cur.wait_stream(s_voc)
 
     def stream_audio(self, chunks: "list[Chunk]", cfg: GenConfig = GenConfig(), cancel=None, *, reset_rep: bool = True,
                      final_turn: bool = False) -> Iterator[Tensor]:
@@ -228,7 +264,7 @@ class Engine:
     """Streaming (B=1) and batched (B=N) decode over one flash-style KV cache."""
 
     def __init__(self, name: str | None = None, *, model: Vui | None = None, codec=None, max_rows: int = 1,
-                 max_seq: int | None = None, sc_token_id: int | None = None):
+                 max_seq: int | None = None, sc_token_id: int | None = None, split_cus: int | None = None):
         if model is None:
             if name is None:
                 raise ValueError("pass model= or a local checkpoint path")
@@ -258,8 +294,38 @@ class Engine:
         self._rows: dict[int, Row] = {}
         self._frame_graphs: dict = {}
         self._lane_streams: list = []
+        self._split = None
+        if split_cus:
+            self._setup_split(int(split_cus))
 
     # ------------------------------------------------------------------ setup
+    def _setup_split(self, n: int) -> None:
+        """Audio streaming on a divided GPU: the decode step's one-launch kernel runs on compute units [0, n) and
+        the vocoder on the rest, each on a stream that is bound to its share (vui_cu_stream_create), so that the
+        vocoder of frame f runs beside the decode step of frame f + 1 (Row.stream).  The context is limited to n
+        workgroups for good, and the vocoder runs as separate launches: a persistent kernel sized for the whole
+        GPU would wait for workgroups that its share has no room for.  No counterpart in the reference, which
+        runs the two one after the other (src/vui/engine.py:1537-1546)."""
+        if self.codec is None or self.max_rows != 1:
+            raise ValueError("split_cus needs Engine(codec=..., max_rows=1)")
+        cus = torch.cuda.get_device_properties(self.device).multi_processor_count
+        if not 0 < n < cus:
+            raise ValueError(f"split_cus={n} outside (0, {cus})")
+        nat = self.model._native
+        streams = []
+        for first, count in ((0, n), (n, cus - n)):
+            h = C.c_void_p()
+            _lib.check(nat.lib.vui_cu_stream_create(first, count, C.byref(h)), "vui_cu_stream_create")
+            streams.append(torch.cuda.ExternalStream(h.value, device=self.device))
+        nat.workgroups(n)
+        self._frame_graphs.clear()  # captured steps hold the width they were captured with
+        self.codec.persistent(0)
+        self.codec._graphs.clear()
+        with torch.cuda.stream(streams[1]):
+            self.codec.setup_streaming_graph(1)
+        torch.cuda.synchronize()
+        self._split = tuple(streams)
+
     def _setup_graphs(self) -> None:
         """src/vui/engine.py:375-432.  KV cache of max_rows + 1 slots (the last one is the write-only
         target of bucket padding rows), static in/out buffers, batched and bucketed step graphs."""
@@ -1070,6 +1136,8 @@ class Engine:
                            "vui_rq_generate")
                 self._frame_ctr += 1
                 frame = codes_io[0, :nq].clone()
+                if self._split is not None:
+                    stream.synchronize()  # the vocoder reads this frame on another stream
                 if use_gate:
                     held.append(frame)
                 else:
@@ -1112,9 +1180,10 @@ class Engine:
                                 top1s.append(p1)
                             flag_t = self._stop_host[step & 1]
                             flag_t.copy_(self._stop_state[:1], non_blocking=True)
+                            frame_t = codes_io[0, :nq].clone()  # before the event: a frame handed out is complete
                             ev = torch.cuda.Event()
                             ev.record(stream)
-                            launched = (codes_io[0, :nq].clone(), ev, flag_t, gathering)
+                            launched = (frame_t, ev, flag_t, gathering)
                             step += 1
                     if pending is not None:
                         frame, ev, flag_t, was_gathering = pending

@@ -185,6 +185,10 @@ class _Native:
         """True when the backbone step of 2..16 rows runs as one persistent kernel."""
         return bool(self.lib.vui_ctx_bb_batch(self.handle))
 
+    def workgroups(self, n: int) -> None:
+        """The batch-1 one-launch kernel on n workgroups instead of one per compute unit (vui_ctx_workgroups)."""
+        _lib.check(self.lib.vui_ctx_workgroups(self.handle, int(n)), "vui_ctx_workgroups")
+
     def status(self) -> None:
         _lib.check(self.lib.vui_ctx_status(self.handle), "vui_ctx_status")
 
