@@ -120,13 +120,16 @@ def gpu_bench(args):
     return out, (model, eng, d, sd)
 
 
-# HBM traffic of one frame_kernel launch on the default workload, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (KiB per dispatch) scaled by what the same counters read for a plain copy of known size;
-# see profiles/frame_kernel_e2e_b1.txt.  None until measured.
-# MFMA busy cycles / busy cycles of the 16-stream step's matrix-core kernels, from rocprofv3 --pmc
-# SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CYCLES; see profiles/e2e_b16_int8_step_kernels.txt.
-MEASURED_B16_MFMA_BUSY = {"gemm16_kernel": [0.08, 0.16], "rq_batch_kernel": 0.49}
-MEASURED_TRAFFIC_BYTES = 522_142_720  # at cache length 577..682 (algorithmic 413.7 MB there): 1.26 x
+# Figures that rocprofv3 counters gave in runs of their own (a counter run serialises every dispatch, so they cannot be
+# taken inside this program's timed region); every line that carries one names the file it comes from.
+# HBM traffic of one frame_kernel launch (whole frame, bf16): FETCH_SIZE and WRITE_SIZE, KiB per dispatch, each scaled
+# by what the same counter reads for a plain 512 MiB device copy (bench.py --calib): 2.000 and 1.000.
+MEASURED_TRAFFIC = {"bytes": 522_218_957, "source": "profiles/frame_kernel_e2e_b1.txt", "cache_length": [577, 681],
+                    "algorithmic_bytes_there": 415289344,
+                    "command": "rocprofv3 --pmc FETCH_SIZE (then WRITE_SIZE) -- python3 bench.py --steps 50 --warmup 5 --no-cpu --no-b16 --no-sweep --calib"}
+# MFMA busy cycles / busy cycles of the two persistent kernels of the 16-stream step.
+MEASURED_B16_MFMA_BUSY = {"bb_batch_kernel": 0.35, "rq_batch_kernel": 0.49, "source": "profiles/e2e_b16_int8_step_kernels.txt",
+                          "command": "rocprofv3 --pmc SQ_BUSY_CYCLES SQ_VALU_MFMA_BUSY_CYCLES -- python3 bench.py --b16-only --steps 2"}
 
 
 def kernel_roofline(out, fb):
@@ -137,7 +140,8 @@ def kernel_roofline(out, fb):
     ach = fb["frame"] / (us * 1e-6) / 1e9
     return {"bound": "hbm", "kernel": "frame_kernel (backbone step + code-0 sampling + depth head, one launch per frame)",
             "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES, "us_per_launch": round(us, 2), "algorithmic_bytes": int(fb["frame"])}
+            "traffic": MEASURED_TRAFFIC["bytes"], "traffic_measured_at": {k: v for k, v in MEASURED_TRAFFIC.items() if k != "bytes"},
+            "us_per_launch": round(us, 2), "algorithmic_bytes": int(fb["frame"])}
 
 
 def vocoder_line():
@@ -252,6 +256,102 @@ def b16_line(sd, preset="A", n=100):
     return {"config": "e2e_b16_int8_ragged", "us_per_frame_step": round(us, 1), "aggregate_frames_per_s": round(16e6 / us, 1),
             "rtf": round(16e6 / us / 12.5, 1), "steps": n, "kv_bytes": int(kv_bytes), "int8_weight_bytes": int(wbytes),
             "achieved_GBs": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "mfma_busy_frac": MEASURED_B16_MFMA_BUSY}
+
+
+def phase_clock(args):
+    """Wall-clock stamps that one workgroup of frame_kernel takes at its phase boundaries (vui_debug_phase_clock),
+    of one frame at cache length ~630: mean and total microseconds per pair of consecutive stamp ids.  The ids
+    are the TS(n) marks of frame.hip (1-6: a backbone layer; 30-: a depth-head layer pass)."""
+    import collections
+
+    import torch
+
+    from vui_amd.engine import Engine, GenConfig
+    from vui_amd.model import Vui
+    from vui_amd.synthetic import nano_for_cache, synthetic_state_dict
+
+    d = nano_for_cache(args.preset, 64).model
+    S = 2304
+    model = Vui(nano_for_cache(args.preset, S), synthetic_state_dict(d, seed=0), device="cuda", dtype=torch.bfloat16, int8=args.int8)
+    eng = Engine(model=model, max_rows=1, max_seq=S)
+    row = eng.new_row()
+    model.decoder._k.normal_()
+    model.decoder._v.normal_()
+    eng.seq_lens[0] = 600
+    g = torch.Generator().manual_seed(0)
+    h = torch.randn(1, d.d_model, generator=g).to(torch.bfloat16).cuda()
+    cfg = GenConfig()
+    eng.generate([row], h, 30, cfg)
+    cap = 1000  # stamps the kernel keeps per launch
+    buf = torch.zeros(4 * (cap + 1), dtype=torch.int64, device="cuda")
+    nat = model._native
+    nat.lib.vui_debug_phase_clock(nat.handle, buf.data_ptr(), cap, args.phase_clock_wg)
+    eng._frame_graphs = {}
+    eng.generate([row], h, 4, cfg)
+    torch.cuda.synchronize()
+    nat.status()
+    b = buf.cpu().tolist()
+    n = b[cap] & 0xFFFFFFFF
+    ev = [(x >> 8, x & 255) for x in b[:n]]
+    seg = collections.defaultdict(list)
+    for (t0, i0), (t1, i1) in zip(ev, ev[1:]):
+        seg[(i0, i1)].append((t1 - t0) / 100.0)  # the clock counts 100 MHz
+    print(json.dumps({"config": "frame_kernel_phase_clock", "int8": bool(args.int8), "workgroup": args.phase_clock_wg, "stamps": n,
+                      "segments": [{"from": k[0], "to": k[1], "n": len(v), "mean_us": round(sum(v) / len(v), 3),
+                                    "total_us": round(sum(v), 1)} for k, v in sorted(seg.items())]}))
+
+
+def bb_phase_clock(args):
+    """Phase stamps of one workgroup of bb_batch_kernel (a library built with -DVUI_BB_CLOCK, e.g.
+    VUI_EXTRA_HIPCC_FLAGS=-DVUI_BB_CLOCK python -m vui_amd.build): B rows of benchmark configuration 5, five
+    steps, the stamps of the last.  Per layer: QKV, attention pieces, merge, out_proj, W1/W3 + SwiGLU, W2."""
+    import ctypes as C
+
+    import torch
+
+    from vui_amd.engine import Engine
+    from vui_amd.model import Vui
+    from vui_amd.synthetic import nano_for_cache, synthetic_state_dict
+
+    B = args.bb_phase_clock
+    d = nano_for_cache(args.preset, 64).model
+    S = 2304
+    model = Vui(nano_for_cache(args.preset, S), synthetic_state_dict(d, seed=0), device="cuda", dtype=torch.bfloat16, int8=args.int8)
+    lib = model._native.lib
+    if not hasattr(lib, "vui_debug_bb_batch_clock"):
+        sys.exit("this library was built without -DVUI_BB_CLOCK")
+    eng = Engine(model=model, max_rows=16, max_seq=S)
+    model.decoder._k.normal_()
+    model.decoder._v.normal_()
+    g = torch.Generator().manual_seed(5)
+    lens = torch.randint(128, 2049, (16,), generator=g).to(torch.int32)
+    codes = torch.randint(0, d.codebook_size, (16, d.n_quantizers), generator=g).cuda()
+    buf = torch.zeros(256, dtype=torch.int64, device="cuda")
+    lib.vui_debug_bb_batch_clock.argtypes = [C.c_void_p, C.c_int]
+    lib.vui_debug_bb_batch_clock(buf.data_ptr(), args.phase_clock_wg)
+    st = torch.cuda.current_stream().cuda_stream
+    hid = torch.empty(B, d.d_model, dtype=torch.bfloat16, device="cuda")
+    cb0 = torch.empty(B, d.codebook_size, dtype=torch.bfloat16, device="cuda")
+    eos = torch.empty(B, 1, dtype=torch.bfloat16, device="cuda")
+    for _ in range(5):
+        eng.seq_lens.zero_()
+        eng.seq_lens[:B] = lens[:B].cuda()
+        model.decoder._step(codes=codes[:B], emb=None, slot_idx=None, seq_inc=None, B=B, hidden_out=hid, cb0_out=cb0,
+                            eos_out=eos, n_splits=8, stream=st)
+    torch.cuda.synchronize()
+    model._native.status()
+    b = buf.cpu().tolist()
+    ts = b[:b[255]]
+    names = ["qkv", "attention_pieces", "merge", "out_proj", "swiglu", "w2"]  # stamps: start, six per layer, final, end
+    L = d.n_layers
+    per = {k: [] for k in names}
+    for l in range(L):
+        for k in range(6):
+            per[names[k]].append((ts[1 + 6 * l + k + 1] - ts[1 + 6 * l + k]) / 100.0)
+    print(json.dumps({"config": "bb_batch_kernel_phase_clock", "rows": B, "int8": bool(args.int8), "workgroup": args.phase_clock_wg,
+                      "total_us": (ts[-1] - ts[0]) / 100.0, "setup_us": (ts[1] - ts[0]) / 100.0,
+                      "final_us": (ts[-1] - ts[1 + 6 * L]) / 100.0,
+                      "per_layer_mean_us": {k: round(sum(v) / L, 2) for k, v in per.items()}}))
 
 
 def batch_sweep(sd, preset="A", n=40, batches=(1, 2, 4, 8, 16)):
@@ -543,11 +643,20 @@ def main():
                     help="print only the continuous-batching line (32 requests through 16 rows, wall clock)")
     ap.add_argument("--vocoder-only", action="store_true",
                     help="print only the vocoder line (the run rocprofv3 summaries of the vocoder kernels come from)")
+    ap.add_argument("--phase-clock", action="store_true",
+                    help="print the phase stamps of one workgroup of the batch-1 frame kernel (with --int8: int8 weights)")
+    ap.add_argument("--bb-phase-clock", type=int, default=0, metavar="ROWS",
+                    help="print the phase stamps of the batched backbone kernel for ROWS rows (needs a -DVUI_BB_CLOCK build)")
+    ap.add_argument("--phase-clock-wg", type=int, default=0, help="the workgroup whose stamps are taken")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (streams are independent); "
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.phase_clock:
+        return phase_clock(args)
+    if args.bb_phase_clock:
+        return bb_phase_clock(args)
     if args.vocoder_only:
         print(json.dumps(vocoder_line()[1]))
         return
@@ -583,6 +692,9 @@ def main():
     out, (model, eng, d, sd) = gpu_bench(args)
     if not args.no_roofline:
         out["roofline"] = kernel_roofline(out, out["frame_bytes"])
+        if args.int8 or args.preset != "A":  # the counters were read for preset A with bf16 weights only
+            out["roofline"]["traffic"] = None
+            out["roofline"].pop("traffic_measured_at", None)
     if not args.no_b16 and not args.suite:
         # batch 16 (benchmark configuration 5) beside the batch-1 figure, after its timed region: 16 int8 streams
         # with ragged caches, a bounded number of replays of the captured step
