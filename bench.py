@@ -543,6 +543,7 @@ def suite(model, eng, d, sd, preset="A"):
                   "frames_per_s": round(n_out / dt, 1), "rtf": round(n_out / dt / 12.5, 2)})
     # the same turn with the GPU divided: decode step on 160 compute units, vocoder of the previous frame beside it
     # on the other 96 (Engine(split_cus=160))
+    row3._codec_ctx.reset()  # closes the vocoder's open stream
     del eng2, row2, row3
     eng3 = Engine(model=model2, codec=voc, max_rows=1, max_seq=1024, split_cus=160)
     row4 = eng3.new_row()
