@@ -555,7 +555,8 @@ def suite(model, eng, d, sd, preset="A"):
     n_out = sum(1 for _ in row4.stream_audio(chunks, cfg_s))
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    model2._native.status()
+    model2._native.status()  # raises if a persistent launch gave up a wait
+    voc.frames_since_reset()  # raises if the vocoder flagged a bad code or a frame beyond its window
     lines.append({"config": "stream_b1_audio_split160", "frames": n_out, "chunks": 4, "ms_per_frame_wall": round(dt * 1e3 / n_out, 4),
                   "frames_per_s": round(n_out / dt, 1), "rtf": round(n_out / dt / 12.5, 2)})
     del eng3, row4, model2, voc
