@@ -84,6 +84,14 @@ int vui_codec_decode_frame(vui_codec* c, const int64_t* codes, int32_t n_q, floa
  * needs all its workgroups resident. */
 int vui_codec_persistent(vui_codec* c, int enable);
 
+/* The persistent form on `nwg` workgroups instead of one per compute unit of the whole GPU, for a caller that runs
+ * the vocoder on a stream bound to part of the GPU (vui_cu_stream_create of vui_amd.h) beside other work: the
+ * kernel needs all its workgroups resident on the compute units its stream may use.  With fewer workgroups each
+ * owns more rows of every matrix; below about 96 (at the reference's dims) the rows no longer fit the registers a
+ * wave keeps them in and the call fails with VUI_EINVAL (vui_codec_persistent(c, 0) then runs the launches).
+ * Steps captured earlier keep the width they were captured with.  No counterpart in the reference. */
+int vui_codec_workgroups(vui_codec* c, int nwg);
+
 /* Synchronous: frames decoded since the last reset (reads a device counter on `stream`), or a negative
  * code; VUI_EINVAL after a code outside [0, codebook_size) or a frame beyond max_seq was seen. */
 int64_t vui_codec_status(vui_codec* c, vui_stream_t stream);

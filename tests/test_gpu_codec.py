@@ -121,6 +121,35 @@ def test_persistent_trunk_equals_kernel_sequence(small):
         assert dec.persistent(1)
 
 
+@pytest.mark.parametrize("nwg", [96, 128, 40])
+def test_persistent_trunk_on_fewer_workgroups(small, full, nwg):
+    """vui_codec_workgroups: the persistent kernel on part of the GPU (more rows of every matrix per workgroup, the
+    row plan of its second instantiation) against the oracle at reduced dims and against the reference's own vectors
+    at the real dims; 40 workgroups cannot hold the real model's rows and are refused there."""
+    d, ora, dec = small
+    g = torch.Generator().manual_seed(9)
+    codes = torch.randint(0, d.codebook_size, (1, d.n_codebooks, 12), generator=g).cuda()
+    try:
+        dec.workgroups(nwg)
+        assert dec.persistent()
+        assert err(dec(codes), ora.forward(codes.cpu())) < TOL
+    finally:
+        dec.workgroups(256)
+    df, sdf, decf, fx = full
+    try:
+        if nwg < 96:
+            with pytest.raises(RuntimeError, match="rows per wave"):
+                decf.workgroups(nwg)
+            return
+        decf.workgroups(nwg)
+        codes = fx["codes"].cuda()
+        with decf.streaming(1):
+            st = torch.cat([decf(codes[:, :, t:t + 1]).clone() for t in range(codes.shape[2])], dim=-1)
+        assert err(st, fx["stream"]) < TOL, err(st, fx["stream"])
+    finally:
+        decf.workgroups(256)
+
+
 def test_errors_are_reported(small):
     d, ora, dec = small
     bad = torch.full((1, d.n_codebooks, 1), d.codebook_size, dtype=torch.long).cuda()

@@ -94,6 +94,7 @@ SIGNATURES = {
     "vui_codec_decode_frame": (_I, [_P, _P, C.c_int32, _P, _P]),
     "vui_codec_status": (_L, [_P, _P]),
     "vui_codec_persistent": (_I, [_P, _I]),
+    "vui_codec_workgroups": (_I, [_P, _I]),
     "vui_backbone_step": (_I, [_P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _P]),
     "vui_sample_cb0": (_I, [_P, _P, _P, _P, _P, _F, _I, C.POINTER(SampleParamsC), _P, _I, _P]),
     "vui_rq_generate": (_I, [_P, _P, _P, _P, _I, C.POINTER(SampleParamsC), _P, _I, _I, _I, _P]),

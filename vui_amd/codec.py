@@ -286,6 +286,12 @@ class QwenCodecDecoder:
         (captured graphs keep the form they were captured with)."""
         return bool(self.lib.vui_codec_persistent(self.handle, int(enable)))
 
+    def workgroups(self, n: int) -> None:
+        """The persistent form of the one-column steps on n workgroups (vui_codec_workgroups): for a vocoder that
+        runs on a stream bound to part of the GPU.  Captured graphs are dropped: they hold the old width."""
+        _lib.check(self.lib.vui_codec_workgroups(self.handle, int(n)), "vui_codec_workgroups")
+        self._graphs.clear()
+
     def setup_streaming_graph(self, batch_size: int = 1, n_q: int | None = None, **_) -> None:
         """Captures the one-frame step as a HIP graph over static in/out buffers
         (setup_streaming_graph, qwen_codec.py:1138-1189).  The capture itself advances nothing."""

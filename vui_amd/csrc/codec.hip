@@ -445,14 +445,23 @@ struct CvTrunk {
   float eps;
 };
 
-#define TR_MAXR 4  // rows per wave and phase
-#define TR_MAXC 6  // float4 chunks per lane and row: K <= 1536
+#define TR_MAXC 6   // float4 chunks per lane and row: K <= 1536
+#define TR_REGS 24  // float4 registers of a wave's rows of one phase: rows per wave x chunks per row
 
-struct TrRows { float4 w[TR_MAXR][TR_MAXC]; };
+// Rows per wave, phase by phase.  The kernel is built for a whole GPU (256 workgroups) and for the share of one that a
+// caller leaves to the vocoder beside other work (NARROW: 96 workgroups and more): a workgroup then owns 256 / 96
+// times the rows, and every phase keeps its rows x chunks within TR_REGS registers.
+template <bool NARROW> struct TrPlan {
+  static constexpr int VQ = NARROW ? 2 : 1, PRE = NARROW ? 3 : 1, IN = NARROW ? 2 : 1, QKV = NARROW ? 10 : 4, O = NARROW ? 2 : 1,
+                       GU = NARROW ? 6 : 4, DN = NARROW ? 2 : 1, OUT = NARROW ? 3 : 1, UP = NARROW ? 6 : 4;
+};
+
+struct TrRows { float4 w[TR_REGS]; };
 
 // rows r_lo + wave, r_lo + wave + 4, ... below r_hi of W (M x K): request them
 template <int MAXR, int MAXC>
 __device__ __forceinline__ void tr_prefetch(const float* W, int K, int r_lo, int r_hi, TrRows& rr) {
+  static_assert(MAXR * MAXC <= TR_REGS, "rows x chunks of a phase exceed the wave's registers");
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
 #pragma unroll
   for (int i = 0; i < MAXR; ++i) {
@@ -461,7 +470,7 @@ __device__ __forceinline__ void tr_prefetch(const float* W, int K, int r_lo, int
     for (int c = 0; c < MAXC; ++c) {
       const int k = (lane + 64 * c) * 4;
       const bool on = row < r_hi && k < K;
-      rr.w[i][c] = on ? *reinterpret_cast<const float4*>(W + (size_t)row * K + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+      rr.w[i * MAXC + c] = on ? *reinterpret_cast<const float4*>(W + (size_t)row * K + k) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
   }
 }
@@ -479,8 +488,9 @@ __device__ __forceinline__ void tr_compute(const float* xs, int K, int r_lo, int
         const int k = (lane + 64 * c) * 4;
         if (k < K) {
           const float4 x = *reinterpret_cast<const float4*>(xs + k);
-          s = fmaf(rr.w[i][c].x, x.x, s); s = fmaf(rr.w[i][c].y, x.y, s);
-          s = fmaf(rr.w[i][c].z, x.z, s); s = fmaf(rr.w[i][c].w, x.w, s);
+          const float4 w = rr.w[i * MAXC + c];
+          s = fmaf(w.x, x.x, s); s = fmaf(w.y, x.y, s);
+          s = fmaf(w.z, x.z, s); s = fmaf(w.w, x.w, s);
         }
       }
       s = wave_sum(s);
@@ -517,7 +527,9 @@ __device__ __forceinline__ float tr_rstd(const float* x, int n, float eps, float
   return 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)n + eps);
 }
 
+template <bool NARROW>
 __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
+  typedef TrPlan<NARROW> P;
   extern __shared__ __align__(16) float tsm[];
   // xs: current input vector (<= 1536) | x: residual stream (D) | q (hd) | sc (max_seq) | part (4*hd) | red (16)
   float* xs = tsm;
@@ -550,7 +562,7 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
 
   // ---- quantizer projection: rows of [W_sem | W_ac] against [sum of semantic rows | sum of acoustic rows] ----
   tr_rows(V, wg, nwg, lo, hi);
-  tr_prefetch<1, 2>(a.Wvq, 2 * cd, lo, hi, rr);
+  tr_prefetch<P::VQ, 2>(a.Wvq, 2 * cd, lo, hi, rr);
   for (int ch = tid; ch < cd; ch += FR_THREADS) {  // every workgroup sums the codebook rows itself
     float s0 = 0.f, s1 = 0.f;
     for (int i0 = 0; i0 < a.n_q; i0 += 16) {
@@ -572,19 +584,20 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
   __syncthreads();
   uint64_t* b_y1 = take(V);
   const int pbase = ring_base(a.pre_in, f);
-  tr_compute<1, 2>(xs, 2 * cd, lo, hi, rr, [&](int row, float s) {
+  tr_compute<P::VQ, 2>(xs, 2 * cd, lo, hi, rr, [&](int row, float s) {
     if (lane == 0) { put(b_y1, row, s); *ring_ptr(a.pre_in, pbase, row, a.pre_in.pad) = s; }
   });
   // ---- pre_conv: three taps = the two previous frames' columns and this one ----
   tr_rows(L, wg, nwg, lo, hi);
-  {
-    const int wave_row = lo + wave;  // one row per wave: (3, L, V) tap-major
+#pragma unroll
+  for (int i = 0; i < P::PRE; ++i) {
+    const int wave_row = lo + wave + 4 * i;  // (3, L, V) tap-major
 #pragma unroll
     for (int cc = 0; cc < TR_MAXC; ++cc) {
       const int k = (lane + 64 * cc) * 4;  // index into [tap][ci]
       const int tap = k / V, ci = k - tap * V;
       const bool on = wave_row < hi && k < 3 * V;
-      rr.w[0][cc] = on ? *reinterpret_cast<const float4*>(a.Wpre + ((size_t)tap * L + wave_row) * V + ci) : make_float4(0.f, 0.f, 0.f, 0.f);
+      rr.w[i * TR_MAXC + cc] = on ? *reinterpret_cast<const float4*>(a.Wpre + ((size_t)tap * L + wave_row) * V + ci) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
   }
   __syncthreads();  // xs is free again
@@ -592,18 +605,18 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
   ll_poll_auto(b_y1, V, c, [&](int i, uint32_t v) { xs[2 * V + i] = __uint_as_float(v); });
   __syncthreads();
   uint64_t* b_pre = take(L);
-  tr_compute<1, TR_MAXC>(xs, 3 * V, lo, hi, rr, [&](int row, float s) { if (lane == 0) put(b_pre, row, s + a.bpre[row]); });
+  tr_compute<P::PRE, TR_MAXC>(xs, 3 * V, lo, hi, rr, [&](int row, float s) { if (lane == 0) put(b_pre, row, s + a.bpre[row]); });
   // ---- input_proj ----
   tr_rows(D, wg, nwg, lo, hi);
-  tr_prefetch<1, 4>(a.Win, L, lo, hi, rr);
+  tr_prefetch<P::IN, 4>(a.Win, L, lo, hi, rr);
   __syncthreads();
   get(b_pre, L, xs);
   uint64_t* b_x = take(D);
-  tr_compute<1, 4>(xs, L, lo, hi, rr, [&](int row, float s) { if (lane == 0) put(b_x, row, s + a.bin[row]); });
+  tr_compute<P::IN, 4>(xs, L, lo, hi, rr, [&](int row, float s) { if (lane == 0) put(b_x, row, s + a.bin[row]); });
   {
     int qlo, qhi;
     tr_rows_qkv(3 * A, wg, nwg, a.H, qlo, qhi);
-    tr_prefetch<TR_MAXR, 2>(a.layers[0].Wqkv, D, qlo, qhi, rr);
+    tr_prefetch<P::QKV, 2>(a.layers[0].Wqkv, D, qlo, qhi, rr);
   }
   get(b_x, D, x);
 
@@ -644,11 +657,11 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
     const float r1 = tr_rstd(x, D, a.eps, red);
     tr_rows_qkv(3 * A, wg, nwg, a.H, lo, hi);
     uint64_t* b_qkv = take(3 * A);
-    tr_compute<TR_MAXR, 2>(x, D, lo, hi, rr, [&](int row, float s) { if (lane == 0) put(b_qkv, row, s * r1); });
+    tr_compute<P::QKV, 2>(x, D, lo, hi, rr, [&](int row, float s) { if (lane == 0) put(b_qkv, row, s * r1); });
     uint64_t* b_att = take(A);
     int olo, ohi;
     tr_rows(D, wg, nwg, olo, ohi);
-    tr_prefetch<1, 4>(W.Wo, A, olo, ohi, rr);
+    tr_prefetch<P::O, 4>(W.Wo, A, olo, ohi, rr);
     // ---- attention: workgroup h owns head h ----
     if (wg < a.H) {
       const int h = wg, half = hd >> 1, pos = f;
@@ -745,11 +758,11 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
     }
     get(b_att, A, xs);
     uint64_t* b_o = take(D);
-    tr_compute<1, 4>(xs, A, olo, ohi, rr, [&](int row, float s) { if (lane == 0) put(b_o, row, s); });
+    tr_compute<P::O, 4>(xs, A, olo, ohi, rr, [&](int row, float s) { if (lane == 0) put(b_o, row, s); });
     int glo, ghi;
     tr_rows(mlp, wg, nwg, glo, ghi);  // channels; rows 2i, 2i + 1 are gate_i, up_i
     glo *= 2; ghi *= 2;
-    tr_prefetch<TR_MAXR, 2>(W.Wgu, D, glo, ghi, rr);
+    tr_prefetch<P::GU, 2>(W.Wgu, D, glo, ghi, rr);
     ll_poll_auto(b_o, D, c, [&](int i, uint32_t v) { x[i] += asc_r[i / FR_THREADS] * __uint_as_float(v); });
     // ---- gate / up rows interleaved: channel i = silu(gate_i) * up_i ----
     const float r2 = tr_rstd(x, D, a.eps, red);
@@ -757,7 +770,7 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
     {
       // a wave's rows glo + wave + 4 i alternate between gate and up of different channels: pair through LDS
       float* pair = part;
-      tr_compute<TR_MAXR, 2>(x, D, glo, ghi, rr, [&](int row, float s) { if (lane == 0) pair[row - glo] = s * r2; });
+      tr_compute<P::GU, 2>(x, D, glo, ghi, rr, [&](int row, float s) { if (lane == 0) pair[row - glo] = s * r2; });
       __syncthreads();
       for (int i = tid; 2 * i + 1 < ghi - glo; i += FR_THREADS) {
         const float ga = pair[2 * i], up = pair[2 * i + 1];
@@ -766,18 +779,18 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
     }
     int dlo, dhi;
     tr_rows(D, wg, nwg, dlo, dhi);
-    tr_prefetch<1, 4>(W.Wd, mlp, dlo, dhi, rr);
+    tr_prefetch<P::DN, 4>(W.Wd, mlp, dlo, dhi, rr);
     get(b_h, mlp, xs);
     uint64_t* b_d = take(D);
-    tr_compute<1, 4>(xs, mlp, dlo, dhi, rr, [&](int row, float s) { if (lane == 0) put(b_d, row, s); });
+    tr_compute<P::DN, 4>(xs, mlp, dlo, dhi, rr, [&](int row, float s) { if (lane == 0) put(b_d, row, s); });
     if (l + 1 < a.n_layers) {
       int qlo, qhi;
       tr_rows_qkv(3 * A, wg, nwg, a.H, qlo, qhi);
-      tr_prefetch<TR_MAXR, 2>(a.layers[l + 1].Wqkv, D, qlo, qhi, rr);
+      tr_prefetch<P::QKV, 2>(a.layers[l + 1].Wqkv, D, qlo, qhi, rr);
     } else {
       int plo, phi;
       tr_rows(L, wg, nwg, plo, phi);
-      tr_prefetch<1, 2>(a.Wout, D, plo, phi, rr);
+      tr_prefetch<P::OUT, 2>(a.Wout, D, plo, phi, rr);
     }
     ll_poll_auto(b_d, D, c, [&](int i, uint32_t v) { x[i] += msc_r[i / FR_THREADS] * __uint_as_float(v); });
   }
@@ -786,18 +799,18 @@ __global__ __launch_bounds__(FR_THREADS) void cv_trunk_kernel(const CvTrunk a) {
   tr_rows(L, wg, nwg, lo, hi);
   const int obase = ring_base(a.out, f);
   if (a.Wt0 == nullptr) {
-    tr_compute<1, 2>(x, D, lo, hi, rr, [&](int row, float s) {
+    tr_compute<P::OUT, 2>(x, D, lo, hi, rr, [&](int row, float s) {
       if (lane == 0) *ring_ptr(a.out, obase, row, a.out.pad) = s * r3 + a.bout[row];
     });
   } else {
     uint64_t* b_lat = take(L);
-    tr_compute<1, 2>(x, D, lo, hi, rr, [&](int row, float s) { if (lane == 0) put(b_lat, row, s * r3 + a.bout[row]); });
+    tr_compute<P::OUT, 2>(x, D, lo, hi, rr, [&](int row, float s) { if (lane == 0) put(b_lat, row, s * r3 + a.bout[row]); });
     // ---- first upsampling stage: transposed conv with kernel = stride: row m -> channel m / r0, column m % r0 ----
     tr_rows(L * a.r0, wg, nwg, lo, hi);
-    tr_prefetch<TR_MAXR, 4>(a.Wt0, L, lo, hi, rr);
+    tr_prefetch<P::UP, 4>(a.Wt0, L, lo, hi, rr);
     __syncthreads();
     get(b_lat, L, xs);
-    tr_compute<TR_MAXR, 4>(xs, L, lo, hi, rr, [&](int row, float s) {
+    tr_compute<P::UP, 4>(xs, L, lo, hi, rr, [&](int row, float s) {
       if (lane == 0) *ring_ptr(a.out, obase, row / a.r0, a.out.pad + row % a.r0) = s + a.bt0[row / a.r0];
     });
   }
@@ -977,11 +990,31 @@ struct vui_codec {
   CvTrunk trunk;
   int trunk_steps = 0;  // leading entries of `steps` the trunk kernel replaces (the codebook kernel as well)
   int trunk_wgs = 0;
+  int trunk_narrow = 0;  // the row plan of the kernel instantiation that trunk_wgs workgroups take
+  int trunk_cap = 0;     // workgroups that can be resident at once on the whole GPU (at most 256 are used)
   size_t trunk_lds = 0;
   int use_trunk = 1;
 };
 
 static int ipow2(int n) { int r = 1; while (r < n) r <<= 1; return r; }
+
+// Whether nwg workgroups can take the one-column steps with the row plan TrPlan<narrow>: every phase's rows per wave
+// within the plan, every vector within the kernel's LDS areas.
+template <bool NARROW> static bool trunk_fits_t(const vui_codec_config& k, int nwg) {
+  typedef TrPlan<NARROW> P;
+  const int A = k.n_heads * k.head_dim;
+  auto fits = [&](int M, int K, int maxr, int maxc, int n) { return n > 0 && ((M + n - 1) / n + 3) / 4 <= maxr && K <= 256 * maxc && K % 4 == 0; };
+  const int nq = nwg >= 4 * k.n_heads ? nwg - k.n_heads : nwg;  // the head-owning workgroups stay out of the q/k/v rows
+  return nwg >= k.n_heads && fits(k.vq_dim, 2 * k.codebook_dim, P::VQ, 2, nwg) && fits(k.latent_dim, 3 * k.vq_dim, P::PRE, TR_MAXC, nwg) &&
+         fits(k.d_model, k.latent_dim, P::IN, 4, nwg) && fits(3 * A, k.d_model, P::QKV, 2, nq) && fits(k.d_model, A, P::O, 4, nwg) &&
+         2 * ((k.mlp_dim + nwg - 1) / nwg) <= 4 * P::GU && fits(k.d_model, k.mlp_dim, P::DN, 4, nwg) &&
+         fits(k.latent_dim, k.d_model, P::OUT, 2, nwg) && (k.n_up == 0 || fits(k.latent_dim * k.up_ratios[0], k.latent_dim, P::UP, 4, nwg)) &&
+         k.head_dim <= 64 && k.max_seq <= 256 && k.d_model <= 1536 && A <= 1536 && k.mlp_dim <= 1536 && k.latent_dim <= 1536 &&
+         3 * k.vq_dim <= 1536;
+}
+static bool trunk_fits(const vui_codec_config& k, int nwg, bool narrow) {
+  return narrow ? trunk_fits_t<true>(k, nwg) : trunk_fits_t<false>(k, nwg);
+}
 
 static int cv_check(const vui_codec_config* c) {
   if (!c) { vui_set_error("NULL codec config"); return VUI_EINVAL; }
@@ -1405,21 +1438,15 @@ int vui_codec_init(const vui_codec_config* cfg, const void* const* tensors, int3
   // the persistent trunk needs all its workgroups resident at once and the per-wave row counts it was built for
   {
     const vui_codec_config& k = c->cfg;
-    const int A = k.n_heads * k.head_dim;
     c->trunk_lds = (size_t)(1536 + k.d_model + 64 + k.max_seq + 192 + 256 + 16) * 4;
     int dev = 0, cus = 0, per_cu = 0;
     HIP_TRY(hipGetDevice(&dev));
     HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)cv_trunk_kernel, FR_THREADS, c->trunk_lds));
-    int nwg = cus * per_cu < 256 ? cus * per_cu : 256;
-    auto fits_n = [&](int M, int K, int maxr, int maxc, int n) { return n > 0 && ((M + n - 1) / n + 3) / 4 <= maxr && K <= 256 * maxc && K % 4 == 0; };
-    auto fits = [&](int M, int K, int maxr, int maxc) { return nwg > 0 && ((M + nwg - 1) / nwg + 3) / 4 <= maxr && K <= 256 * maxc && K % 4 == 0; };
-    const bool ok = nwg >= k.n_heads && fits(k.vq_dim, 2 * k.codebook_dim, 1, 2) && fits(k.latent_dim, 3 * k.vq_dim, 1, TR_MAXC) &&
-                    fits(k.d_model, k.latent_dim, 1, 4) && fits_n(3 * A, k.d_model, TR_MAXR, 2, nwg >= 4 * k.n_heads ? nwg - k.n_heads : nwg) && fits(k.d_model, A, 1, 4) &&
-                    2 * ((k.mlp_dim + nwg - 1) / nwg) <= 4 * TR_MAXR && fits(k.d_model, k.mlp_dim, 1, 4) && fits(k.latent_dim, k.d_model, 1, 2) &&
-                    (k.n_up == 0 || fits(k.latent_dim * k.up_ratios[0], k.latent_dim, TR_MAXR, 4)) && k.head_dim <= 64 && k.max_seq <= 256 &&
-                    k.d_model <= 1536 && A <= 1536 && k.mlp_dim <= 1536 && k.latent_dim <= 1536 && 3 * k.vq_dim <= 1536;
-    c->trunk_wgs = ok ? nwg : 0;
+    HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)cv_trunk_kernel<true>, FR_THREADS, c->trunk_lds));
+    c->trunk_cap = cus * per_cu < 256 ? cus * per_cu : 256;
+    c->trunk_wgs = 0;
+    for (int narrow = 0; narrow < 2 && !c->trunk_wgs; ++narrow)
+      if (trunk_fits(k, c->trunk_cap, narrow != 0)) { c->trunk_wgs = c->trunk_cap; c->trunk_narrow = narrow; }
     c->use_trunk = 1;
   }
   *out = c;
@@ -1427,6 +1454,15 @@ int vui_codec_init(const vui_codec_config* cfg, const void* const* tensors, int3
 }
 
 void vui_codec_destroy(vui_codec* c) { delete c; }
+
+int vui_codec_workgroups(vui_codec* c, int nwg) {
+  if (!c) { vui_set_error("NULL codec"); return VUI_EINVAL; }
+  if (nwg < 1 || nwg > c->trunk_cap) { vui_set_error("codec: %d workgroups outside [1, %d]", nwg, c->trunk_cap); return VUI_EINVAL; }
+  for (int narrow = 0; narrow < 2; ++narrow)
+    if (trunk_fits(c->cfg, nwg, narrow != 0)) { c->trunk_wgs = nwg; c->trunk_narrow = narrow; return VUI_OK; }
+  vui_set_error("codec: the persistent form of the one-column steps does not run on %d workgroups (too many rows per wave)", nwg);
+  return VUI_EINVAL;
+}
 
 int vui_codec_persistent(vui_codec* c, int enable) {
   if (!c) { vui_set_error("NULL codec"); return 0; }
@@ -1462,7 +1498,8 @@ int vui_codec_decode_frame(vui_codec* c, const int64_t* codes, int32_t n_q, floa
   if (c->use_trunk && c->trunk_wgs > 0) {
     CvTrunk tk = c->trunk;
     tk.codes = codes; tk.n_q = n_q;
-    hipLaunchKernelGGL(cv_trunk_kernel, dim3(c->trunk_wgs), dim3(FR_THREADS), c->trunk_lds, st, tk);
+    if (c->trunk_narrow) hipLaunchKernelGGL(cv_trunk_kernel<true>, dim3(c->trunk_wgs), dim3(FR_THREADS), c->trunk_lds, st, tk);
+    else hipLaunchKernelGGL(cv_trunk_kernel<false>, dim3(c->trunk_wgs), dim3(FR_THREADS), c->trunk_lds, st, tk);
     first = (size_t)c->trunk_steps;
   } else {
     CvVq vq = c->vq;

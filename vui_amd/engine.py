@@ -303,8 +303,9 @@ class Engine:
         """Audio streaming on a divided GPU: the decode step's one-launch kernel runs on compute units [0, n) and
         the vocoder on the rest, each on a stream that is bound to its share (vui_cu_stream_create), so that the
         vocoder of frame f runs beside the decode step of frame f + 1 (Row.stream).  The context is limited to n
-        workgroups for good, and the vocoder runs as separate launches: a persistent kernel sized for the whole
-        GPU would wait for workgroups that its share has no room for.  No counterpart in the reference, which
+        workgroups for good and the vocoder's persistent kernel to as many as its share has compute units (a
+        persistent kernel sized for the whole GPU would wait for workgroups that its share has no room for; where
+        the vocoder's rows do not fit that few workgroups it runs as separate launches).  No counterpart in the reference, which
         runs the two one after the other (src/vui/engine.py:1537-1546)."""
         if self.codec is None or self.max_rows != 1:
             raise ValueError("split_cus needs Engine(codec=..., max_rows=1)")
@@ -319,7 +320,11 @@ class Engine:
             streams.append(torch.cuda.ExternalStream(h.value, device=self.device))
         nat.workgroups(n)
         self._frame_graphs.clear()  # captured steps hold the width they were captured with
-        self.codec.persistent(0)
+        try:  # the vocoder's persistent kernel on its share, where its rows fit that few workgroups
+            self.codec.workgroups(cus - n)
+            self.codec.persistent(1)
+        except RuntimeError:
+            self.codec.persistent(0)
         self.codec._graphs.clear()
         with torch.cuda.stream(streams[1]):
             self.codec.setup_streaming_graph(1)
