@@ -422,3 +422,58 @@ def test_one_frame_graph_serves_every_sampling_setting():
     rq.seed = 0
     rq._ctr.zero_()
     assert torch.equal(rq.generate_cuda_graph_kv(hid, c0, 0.7), outs[0])
+
+
+def test_compute_unit_ranges_and_context_widths():
+    """vui_cu_stream_create takes one contiguous range inside the GPU; vui_ctx_workgroups takes the widths the
+    one-launch kernel was run against the oracle with, switches the batched kernels off below the full width and is
+    undone by vui_ctx_init.  Frames on 192 workgroups of a bound stream are well-formed and repeatable."""
+    import ctypes as C
+
+    from vui_amd import _lib
+    from vui_amd.engine import GenConfig
+
+    lib = _lib.load()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    h = C.c_void_p()
+    for first, n in ((-1, 8), (0, 0), (cus - 8, 16), (0, cus + 1)):
+        assert lib.vui_cu_stream_create(first, n, C.byref(h)) != 0
+        assert "compute units" in _lib.last_error()
+    assert lib.vui_cu_stream_create(0, 1, None) != 0
+    d = tiny_dims(2)
+    sd = O.synthetic_state_dict(d, **TINY_SD)
+    m, eng = _engine(d, sd, BF)
+    nat = m._native
+    assert nat.fused(-1)
+    batched = (nat.rq_batch(), nat.bb_batch())
+    for bad in (0, 144, 152, 200, 257):
+        with pytest.raises(RuntimeError, match="workgroups"):
+            nat.workgroups(bad)
+    nat.workgroups(192)
+    assert nat.fused(-1) and not nat.rq_batch() and not nat.bb_batch()
+    _lib.check(lib.vui_cu_stream_create(0, 192, C.byref(h)), "vui_cu_stream_create")
+    stream = torch.cuda.ExternalStream(h.value)
+    cfg = GenConfig(temperature=0.9, top_k=10, rq_top_k=10, seed=2)
+    ids = torch.tensor([4, 9, 2, 7])
+    runs = []
+    for _ in range(2):
+        torch.cuda.synchronize()
+        with torch.cuda.stream(stream):
+            row = eng.new_row()
+            hid = row.prefill_emb(m.token_emb(ids.cuda()[None]))[:, -1]
+            frames, _ = eng.generate([row], hid, 6, cfg)
+            row.close()
+        stream.synchronize()
+        nat.status()
+        runs.append(frames.cpu())
+    assert torch.equal(runs[0], runs[1])
+    assert int(runs[0].min()) >= 0 and int(runs[0].max()) < d.codebook_size
+    nat.reinit()  # the full width again
+    assert (nat.rq_batch(), nat.bb_batch()) == batched
+    torch.cuda.synchronize()
+    row = eng.new_row()
+    hid = row.prefill_emb(m.token_emb(ids.cuda()[None]))[:, -1]
+    eng._frame_graphs.clear()
+    full, _ = eng.generate([row], hid, 6, cfg)
+    nat.status()
+    assert full.shape == runs[0].shape
