@@ -9,9 +9,11 @@
 // head do, with the matrix cores inside: a workgroup owns tiles of 16 output features of each weight matrix and
 // multiplies them with the activations of its rows (v_mfma_f32_16x16x32_bf16, int8 weights widened in registers).
 //
-// Rows are dealt to row groups of up to four, sorted by cache length and dealt in serpentine order so that the
-// groups carry about the same number of keys; a group is served by NWL = 256 / groups workgroups (64 for 13-16
-// rows, 256 for 2-4), because what a phase costs is the number of exchanged words one workgroup has to wait for.
+// Rows are dealt to min(rows, 4) row groups, sorted by cache length and dealt in serpentine order so that the
+// groups carry about the same number of keys; a group is served by NWL = 256 / groups workgroups (128 for 2 rows,
+// 64 from 3 rows on), because what a phase costs is the number of exchanged words one workgroup has to wait for:
+// four groups of one or two rows beat one or two groups of four (measured: 4 rows 1434 -> 1371 us per frame step,
+// 8 rows 1603 -> 1557), although a lone row's keys are then streamed by 64 workgroups instead of 256.
 // Per layer and group:
 //   A  RMSNorm + QKV tiles, rotation of q and k in the epilogue; k and v of the new position go to the cache and,
 //      like q, into the exchange
@@ -372,7 +374,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
   const vui_weights& W = *a.w;
 
   // ---- rows -> groups, roles ----
-  const int ngroups = (B + BB_RG - 1) / BB_RG;
+  const int ngroups = min(B, BB_RG);
   const int NWL = nwg >> (ngroups <= 1 ? 0 : (ngroups <= 2 ? 1 : 2));  // workgroups per group
   const int grp = wg / NWL, wl = wg % NWL;
   if (tid < B) {

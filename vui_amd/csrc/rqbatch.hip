@@ -8,7 +8,8 @@
 // matrix cores inside: a workgroup owns tiles of 16 output features of a weight matrix and multiplies
 // them with the activations of its rows in one v_mfma_f32_16x16x32_bf16 per 32 k.
 //
-// The rows are split into row groups of 4, each served by 64 workgroups: reading an exchanged vector is
+// The rows are split into row groups of 4 (up to 4 rows: one row per group), each served by 64 workgroups:
+// reading an exchanged vector is
 // bound by the number of 8-byte words one CU has to poll (about one per two clocks), so four groups that
 // each poll a quarter of the rows beat one group polling all sixteen by ~2x (measured), although the
 // weights are then read four times (from L2) and the matrix-core tile is a quarter full.
@@ -340,7 +341,11 @@ __global__ __launch_bounds__(FR_THREADS, 1) void rq_batch_kernel(const RqBatchAr
 
   // row group of this workgroup and its roles inside the group
   const int grp = wg / RB_NWL, wl = wg % RB_NWL;
-  const int b0 = grp * RB_RG, Bg = min(max(B - b0, 0), RB_RG);
+  // rows per group: up to four rows take a group each (a phase costs what a workgroup waits for: the exchanged
+  // words of its group's rows; measured 3-5 % of the step at 2-4 rows).  Eight rows as four groups of two were
+  // slower than as two groups of four (all 256 workgroups then stream every weight), so more rows keep groups of four.
+  const int rg = B <= RB_RG ? 1 : RB_RG;
+  const int b0 = grp * rg, Bg = min(max(B - b0, 0), rg);
   const bool active = Bg > 0;
   const int nA = 3 * R / 16, nS = a.rqF / 16, nH = CS / 16, nO = R / 16;
   const int back = RB_NWL - 1 - wl;
