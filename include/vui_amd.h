@@ -153,7 +153,10 @@ int vui_ctx_fused(vui_ctx* ctx, int enable);
  * has them).  vui_ctx_workgroups is called after vui_ctx_init (which restores the full width); with nwg below
  * the full width the batched persistent kernels (2..16 rows) are switched off for the context.  The stream is
  * kept for the life of the process: there is no destroy call (on this ROCm release creating a masked stream after
- * one had been destroyed crashed, and so did a mask that is not one contiguous range).  No counterpart in the reference. */
+ * one had been destroyed crashed, and so did a mask that is not one contiguous range).  A persistent kernel needs a
+ * range whose size is a multiple of 32, so that every shader engine of every XCD keeps the same number of compute units
+ * (workgroups are dealt evenly over the engines; with an uneven share one engine cannot hold its part of the grid).
+ * No counterpart in the reference. */
 int vui_cu_stream_create(int first_cu, int n_cus, vui_stream_t* out);
 int vui_ctx_workgroups(vui_ctx* ctx, int nwg);
 

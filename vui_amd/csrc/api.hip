@@ -303,8 +303,11 @@ int vui_ctx_workgroups(vui_ctx* ctx, int nwg) {
   if (!ctx) { vui_set_error("NULL context"); return VUI_EINVAL; }
   const vui_config& c = ctx->cfg;
   if (!ctx->fused_ok) { vui_set_error("the one-launch kernel is not available: %s", ctx->fused_why); return VUI_EINVAL; }
-  // widths that were run against the oracle; at 144 and 152 (144 is the fewest the widest matrix of Vui Nano allows) the
-  // first launch ended in its bounded wait, cause not found, so other widths are refused rather than tried
+  // A persistent kernel on a stream bound to part of the GPU needs every workgroup resident on the compute units of its
+  // range.  The dispatcher deals workgroups evenly over the shader engines of every XCD, so the range must leave every
+  // engine the same number of compute units: multiples of 32 (8 XCDs x 4 engines).  On 144 and 152 units (18 and 19 per
+  // XCD) the launch ended in its bounded wait, while the same 152 workgroups on the whole GPU ran: one engine was asked
+  // for more resident workgroups than it had units.  160 is the fewest the widest matrix of Vui Nano allows.
   if (nwg < 160 || nwg > FUSED_NWG || nwg % 32) { vui_set_error("workgroups %d: 160, 192, 224 or %d", nwg, FUSED_NWG); return VUI_EINVAL; }
   int ns = nwg / (c.n_heads > 0 ? c.n_heads : 1);
   if (ns > FUSED_NS) ns = FUSED_NS;
