@@ -488,6 +488,35 @@ def suite(model, eng, d, sd, preset="A"):
         b = frame_bytes(m, L)["backbone"]
         lines.append({"config": "backbone_step_b1", "kv_len": L, "us_per_step": round(us, 2), "us_per_layer": round(us / m.n_layers, 2),
                       "algorithmic_bytes": int(b), "achieved_GBs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4)})
+    # the same step with cold caches: three copies of the weights (3 x 311 MB, more than the 256 MB memory-side cache)
+    # with a cache each, taken in turn, so that no step finds its weights or keys where the previous step left them
+    cold = [(model2, eng2)]
+    for _ in range(2):
+        sdc = {k: v.clone() for k, v in sd.items()}
+        mc = Vui(nano_for_cache(preset, 4608), sdc, device="cuda", dtype=torch.bfloat16)
+        ec = Engine(model=mc, max_rows=1, max_seq=4608)
+        mc.decoder._k.normal_()
+        mc.decoder._v.normal_()
+        ec._decode_step()
+        cold.append((mc, ec))
+    for L in (256, 1024, 4096):
+        n = 198
+        for _, e in cold:
+            e.seq_lens[0] = L - n // 6
+        k = [0]
+
+        def step():
+            cold[k[0] % 3][1]._decode_graph.replay()
+            k[0] += 1
+
+        us = timed(step, n)
+        b = frame_bytes(m, L)["backbone"]
+        lines.append({"config": "backbone_step_b1_cold", "kv_len": L, "weight_copies": 3, "us_per_step": round(us, 2),
+                      "us_per_layer": round(us / m.n_layers, 2), "algorithmic_bytes": int(b), "achieved_GBs": round(b / us / 1e3, 1),
+                      "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBS, 4)})
+    for mc, ec in cold[1:]:
+        mc._native.status()
+    del cold, mc, ec, sdc
     # config 3: depth head alone, 1000 frames, T=0.8 top-k 50
     rq = model2.rq_transformer
     rq.setup_cuda_graph_kv(model2.device, torch.bfloat16, top_k=50, batch_sizes=(1,))
