@@ -260,6 +260,9 @@ class Row:
         self.close()
 
 
+_CU_STREAMS: dict = {}  # (device, first compute unit, count) -> stream bound to that range (never destroyed)
+
+
 class Engine:
     """Streaming (B=1) and batched (B=N) decode over one flash-style KV cache."""
 
@@ -315,9 +318,12 @@ class Engine:
         nat = self.model._native
         streams = []
         for first, count in ((0, n), (n, cus - n)):
-            h = C.c_void_p()
-            _lib.check(nat.lib.vui_cu_stream_create(first, count, C.byref(h)), "vui_cu_stream_create")
-            streams.append(torch.cuda.ExternalStream(h.value, device=self.device))
+            key = (torch.device(self.device).index or 0, first, count)
+            if key not in _CU_STREAMS:  # bound streams are kept for the life of the process: one per range
+                h = C.c_void_p()
+                _lib.check(nat.lib.vui_cu_stream_create(first, count, C.byref(h)), "vui_cu_stream_create")
+                _CU_STREAMS[key] = torch.cuda.ExternalStream(h.value, device=self.device)
+            streams.append(_CU_STREAMS[key])
         nat.workgroups(n)
         self._frame_graphs.clear()  # captured steps hold the width they were captured with
         try:  # the vocoder's persistent kernel on its share, where its rows fit that few workgroups
