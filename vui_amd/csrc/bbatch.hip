@@ -18,7 +18,7 @@
 //   A  RMSNorm + QKV tiles, rotation of q and k in the epilogue; k and v of the new position go to the cache and,
 //      like q, into the exchange
 //   B  attention over the ragged rows: the group's workgroups are dealt to (row, set of HG heads, key range) pieces,
-//      long rows getting more key ranges (HG = 2 for 13-16 rows: twice as fine a division as one head set per
+//      long rows getting more key ranges (HG = 2 from 5 rows on: twice as fine a division as one head set per
 //      workgroup of a 64-workgroup group allows); keys and values stream from the cache with 16 loads per lane in
 //      flight, the new position's come from the exchange
 //   C  merge of a (row, head)'s pieces
