@@ -354,6 +354,40 @@ def bb_phase_clock(args):
                       "per_layer_mean_us": {k: round(sum(v) / L, 2) for k, v in per.items()}}))
 
 
+def split_audio_line(sd, preset="A", split_cus=160):
+    """A streamed turn with audio out on a divided GPU (Engine(split_cus=...)): decode step on split_cus compute
+    units, vocoder of the previous frame beside it on the rest; 4 chunks, wall clock."""
+    import torch
+
+    from vui_amd.codec import CodecConfig, QwenCodecDecoder
+    from vui_amd.engine import Chunk, Engine, GenConfig
+    from vui_amd.model import Vui
+    from vui_amd.synthetic import nano_for_cache, synthetic_codec_state_dict
+
+    model = Vui(nano_for_cache(preset, 1024), sd, device="cuda", dtype=torch.bfloat16)
+    ccfg = CodecConfig()
+    voc = QwenCodecDecoder(synthetic_codec_state_dict(ccfg, 0), ccfg)
+    eng = Engine(model=model, codec=voc, max_rows=1, max_seq=1024, split_cus=split_cus)
+    g = torch.Generator().manual_seed(0)
+    emb = (torch.randn(1, 16, model.config.model.d_model, generator=g) * 0.08).to(torch.bfloat16).cuda()
+    chunks = [Chunk(emb=emb, n_words=40) for _ in range(4)]
+    cfg_s = GenConfig(eos_threshold=2.0, max_secs=60.0)
+    row = eng.new_row()
+    n_out = sum(1 for _ in row.stream(chunks[:1], cfg_s))  # warm: graph captures
+    row.reset()
+    row._codec_ctx.reset()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    n_out = sum(1 for _ in row.stream(chunks, cfg_s))
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    model._native.status()  # raises if a persistent launch gave up a wait
+    voc.frames_since_reset()  # raises if the vocoder flagged a bad code or a frame beyond its window
+    return {"config": f"stream_b1_audio_split{split_cus}", "frames": n_out, "chunks": 4, "ms_per_frame_wall": round(dt * 1e3 / n_out, 4),
+            "frames_per_s": round(n_out / dt, 1), "rtf": round(n_out / dt / 12.5, 2),
+            "vocoder_persistent_workgroups": torch.cuda.get_device_properties(0).multi_processor_count - split_cus if voc.persistent() else 0}
+
+
 def batch_sweep(sd, preset="A", n=40, batches=(1, 2, 4, 8, 16)):
     """The frame step (backbone step + code-0 draw + depth head, one captured graph per batch size) for 1..16
     concurrent streams, with bf16 and with int8 backbone weights: ragged caches as in benchmark configuration 5
@@ -573,22 +607,8 @@ def suite(model, eng, d, sd, preset="A"):
     # the same turn with the GPU divided: decode step on 160 compute units, vocoder of the previous frame beside it
     # on the other 96 (Engine(split_cus=160))
     row3._codec_ctx.reset()  # closes the vocoder's open stream
-    del eng2, row2, row3
-    eng3 = Engine(model=model2, codec=voc, max_rows=1, max_seq=1024, split_cus=160)
-    row4 = eng3.new_row()
-    n_out = sum(1 for _ in row4.stream_audio(chunks[:1], cfg_s))
-    row4.reset()
-    row4._codec_ctx.reset()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    n_out = sum(1 for _ in row4.stream_audio(chunks, cfg_s))
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    model2._native.status()  # raises if a persistent launch gave up a wait
-    voc.frames_since_reset()  # raises if the vocoder flagged a bad code or a frame beyond its window
-    lines.append({"config": "stream_b1_audio_split160", "frames": n_out, "chunks": 4, "ms_per_frame_wall": round(dt * 1e3 / n_out, 4),
-                  "frames_per_s": round(n_out / dt, 1), "rtf": round(n_out / dt / 12.5, 2)})
-    del eng3, row4, model2, voc
+    del eng2, row2, row3, model2, voc
+    lines.append(split_audio_line(sd, preset))
     lines.append(b16_line(sd, preset))
     lines.append(serve_line(sd, preset))
     lines.append(serve_line(sd, preset, int8=True))
@@ -674,6 +694,8 @@ def main():
                     help="print only the continuous-batching line (32 requests through 16 rows, wall clock)")
     ap.add_argument("--vocoder-only", action="store_true",
                     help="print only the vocoder line (the run rocprofv3 summaries of the vocoder kernels come from)")
+    ap.add_argument("--split-audio-only", action="store_true",
+                    help="print only the streamed turn with audio on a divided GPU (the run its rocprofv3 summary comes from)")
     ap.add_argument("--phase-clock", action="store_true",
                     help="print the phase stamps of one workgroup of the batch-1 frame kernel (with --int8: int8 weights)")
     ap.add_argument("--bb-phase-clock", type=int, default=0, metavar="ROWS",
@@ -690,6 +712,11 @@ def main():
         return bb_phase_clock(args)
     if args.vocoder_only:
         print(json.dumps(vocoder_line()[1]))
+        return
+    if args.split_audio_only:
+        from vui_amd.synthetic import nano_for_cache, synthetic_state_dict
+
+        print(json.dumps(split_audio_line(synthetic_state_dict(nano_for_cache(args.preset, 64).model, seed=0), args.preset)))
         return
     if args.prefill_only:
         import torch
