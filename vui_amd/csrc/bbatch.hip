@@ -18,7 +18,7 @@
 //   A  RMSNorm + QKV tiles, rotation of q and k in the epilogue; k and v of the new position go to the cache and,
 //      like q, into the exchange
 //   B  attention over the ragged rows: the group's workgroups are dealt to (row, set of HG heads, key range) pieces,
-//      long rows getting more key ranges (HG = 2 from 5 rows on: twice as fine a division as one head set per
+//      long rows getting more key ranges (HG = 2 from 9 rows on: twice as fine a division as one head set per
 //      workgroup of a 64-workgroup group allows); keys and values stream from the cache with 16 loads per lane in
 //      flight, the new position's come from the exchange
 //   C  merge of a (row, head)'s pieces
@@ -1094,11 +1094,11 @@ int launch_bb_batch(const vui_config& c, const vui_weights* wdev, const void* ti
 #ifdef VUI_BB_CLOCK
   a.dbg = g_bb_dbg; a.dbg_wg = g_bb_dbg_wg;
 #endif
-  // heads per attention piece: two from five rows on (a group then has 128 or 64 workgroups, and pairs of heads
-  // divide its rows' keys twice as finely as whole head sets per key range would; measured 727 against 774 us for
-  // 16 rows, 596 against 610 for 8, no difference for 4); a key range is not split below 64 keys (32..128 measure
-  // the same)
-  a.hg = (B > BB_RG && c.n_heads % 2 == 0) ? 2 : 1;
+  // heads per attention piece: two from nine rows on (a group of 64 workgroups then holds three or four rows, and
+  // pairs of heads divide their keys twice as finely as whole head sets per key range would; measured for the frame
+  // step of 16 rows 1716 against 1728 us, of 8 rows - two rows per group - 1554 against 1548, four heads per piece
+  // 1765 / 1588); a key range is not split below 64 keys (32..128 measure the same)
+  a.hg = (B > 2 * BB_RG && c.n_heads % 2 == 0) ? 2 : 1;
   a.min_keys = 64;
   a.xs = bb_xs(c); a.off_xp = (int)l.xp; a.off_red = (int)l.red; a.off_att = (int)l.att; a.off_misc = (int)l.misc;
   hipLaunchKernelGGL(bb_pick(c), dim3(nwg), dim3(FR_THREADS), l.total, st, a);
