@@ -210,6 +210,7 @@ class Row:
                 self._codec_ctx.prefill(n_codebooks=cfg.n_codebooks)
         it = self.stream_codes(chunks, cfg, cancel, reset_rep=reset_rep, final_turn=final_turn)
         pending = None  # (audio, event) of the vocoder step in flight
+        first = True    # the first frame's audio is handed out as soon as it is done (time to the first sound)
         try:
             while True:
                 with torch.cuda.stream(s_dec):
@@ -225,7 +226,12 @@ class Row:
                     audio = eng._stream_decode_frame(self, codes, cfg.n_codebooks)
                     ev = torch.cuda.Event()
                     ev.record(s_voc)
-                pending = (audio, ev)
+                if first:
+                    first = False
+                    ev.synchronize()
+                    yield audio
+                else:
+                    pending = (audio, ev)
         finally:
             it.close()
             cur.wait_stream(s_dec)
