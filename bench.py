@@ -393,6 +393,48 @@ def split_audio_line(sd, preset="A", split_cus=160):
             "vocoder_persistent_workgroups": torch.cuda.get_device_properties(0).multi_processor_count - split_cus if voc.persistent() else 0}
 
 
+def rq_phase_clock(args):
+    """Phase stamps of one workgroup of rq_batch_kernel at codebook 8 (a library built with -DVUI_RB_CLOCK): the
+    depth head of ROWS rows, three calls, the stamps of the last.  Per layer: norm + QKV tiles, attention,
+    out_proj, norm + W1/W3 + SwiGLU, W2; then the logits head and the draw."""
+    import ctypes as C
+
+    import torch
+
+    from vui_amd.model import Vui
+    from vui_amd.synthetic import nano_for_cache, synthetic_state_dict
+
+    B = args.rq_phase_clock
+    d = nano_for_cache(args.preset, 64).model
+    model = Vui(nano_for_cache(args.preset, 256), synthetic_state_dict(d, seed=0), device="cuda", dtype=torch.bfloat16)
+    model.decoder.allocate_flash_kv_cache(1, model.device, torch.bfloat16, max_seqlen=256)
+    lib = model._native.lib
+    if not hasattr(lib, "vui_debug_rq_batch_clock"):
+        sys.exit("this library was built without -DVUI_RB_CLOCK")
+    buf = torch.zeros(64, dtype=torch.int64, device="cuda")
+    lib.vui_debug_rq_batch_clock.argtypes = [C.c_void_p, C.c_int]
+    lib.vui_debug_rq_batch_clock(buf.data_ptr(), args.phase_clock_wg)
+    g = torch.Generator().manual_seed(0)
+    hid = torch.randn(B, d.d_model, generator=g).to(torch.bfloat16).cuda()
+    c0 = torch.randint(0, d.codebook_size, (B,), generator=g).cuda()
+    for _ in range(3):
+        model.rq_transformer.generate(hid, c0, temperature=0.8, top_k=50)
+    torch.cuda.synchronize()
+    model._native.status()
+    b = buf.cpu().tolist()
+    ts = b[:b[63]]
+    L = d.rq_n_layers
+    names = ["qkv", "attention", "out_proj", "swiglu", "w2"]
+    per = {k: [] for k in names}
+    for l in range(L):
+        for k in range(5):
+            nxt = ts[5 * l + k + 1]
+            per[names[k]].append((nxt - ts[5 * l + k]) / 100.0)
+    print(json.dumps({"config": "rq_batch_kernel_phase_clock", "rows": B, "workgroup": args.phase_clock_wg, "codebook": 8,
+                      "per_layer_mean_us": {k: round(sum(v) / L, 2) for k, v in per.items()},
+                      "layers_us": round((ts[5 * L] - ts[0]) / 100.0, 2), "logits_and_draw_us": round((ts[-1] - ts[5 * L]) / 100.0, 2)}))
+
+
 def batch_sweep(sd, preset="A", n=40, batches=(1, 2, 4, 8, 16)):
     """The frame step (backbone step + code-0 draw + depth head, one captured graph per batch size) for 1..16
     concurrent streams, with bf16 and with int8 backbone weights: ragged caches as in benchmark configuration 5
@@ -710,6 +752,8 @@ def main():
                     help="print the phase stamps of one workgroup of the batch-1 frame kernel (with --int8: int8 weights)")
     ap.add_argument("--bb-phase-clock", type=int, default=0, metavar="ROWS",
                     help="print the phase stamps of the batched backbone kernel for ROWS rows (needs a -DVUI_BB_CLOCK build)")
+    ap.add_argument("--rq-phase-clock", type=int, default=0, metavar="ROWS",
+                    help="print the phase stamps of the batched depth-head kernel for ROWS rows (needs a -DVUI_RB_CLOCK build)")
     ap.add_argument("--phase-clock-wg", type=int, default=0, help="the workgroup whose stamps are taken")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -720,6 +764,8 @@ def main():
         return phase_clock(args)
     if args.bb_phase_clock:
         return bb_phase_clock(args)
+    if args.rq_phase_clock:
+        return rq_phase_clock(args)
     if args.vocoder_only:
         print(json.dumps(vocoder_line()[1]))
         return
