@@ -93,7 +93,22 @@ __device__ __forceinline__ uint4 widen8(const uint2& w) {
 }
 
 // W, W2: (N, K) row-major bf16, or int8 with the per-row bf16 scales S, S2
-template <int MAXC, bool DUAL, bool I8>
+// NT: the matrix is read once per launch (the backbone's matrices, the codec head, the depth head's projection and
+// per-codebook heads): its loads carry the non-temporal hint, so that 311 MB of such reads per frame do not push out of
+// the caches what is read again and again (the depth head's layer matrices, 16 passes per frame; the keys and values,
+// every frame).  Measured: 1.033 -> 0.992 ms per frame (int8 weights 1.023 -> 1.005); the same hint on the key / value
+// loads made it slower (0.997 / 1.019): they are what the caches should keep from frame to frame.
+typedef unsigned int fr_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int fr_u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint4 ld_nt16(const void* p) {
+  const fr_u32x4 v = __builtin_nontemporal_load((const __attribute__((address_space(1))) fr_u32x4*)p);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint2 ld_nt8(const void* p) {
+  const fr_u32x2 v = __builtin_nontemporal_load((const __attribute__((address_space(1))) fr_u32x2*)p);
+  return make_uint2(v.x, v.y);
+}
+template <int MAXC, bool DUAL, bool I8, bool NT = false>
 __device__ __forceinline__ void gemv_prefetch(const void* Wv, const void* W2v, int K, const Plan& p,
                                               WRegs<MAXC, DUAL, I8>& r, const bf16_t* S = nullptr, const bf16_t* S2 = nullptr) {
   const int lane = threadIdx.x & 63;
@@ -109,8 +124,13 @@ __device__ __forceinline__ void gemv_prefetch(const void* Wv, const void* W2v, i
           const int c = p.c0 + lane + WAVE * i;
           const bool on = s < p.nslots && c < p.c1;
           const size_t off = ((size_t)(2 * p.gp[s] + rr)) * K + (size_t)c * 8;
-          r.a[s][rr][i] = on ? *reinterpret_cast<const uint4*>(W + off) : make_uint4(0, 0, 0, 0);
-          if (DUAL) r.b[s][rr][i] = on ? *reinterpret_cast<const uint4*>(W2 + off) : make_uint4(0, 0, 0, 0);
+          if constexpr (NT) {
+            r.a[s][rr][i] = on ? ld_nt16(W + off) : make_uint4(0, 0, 0, 0);
+            if (DUAL) r.b[s][rr][i] = on ? ld_nt16(W2 + off) : make_uint4(0, 0, 0, 0);
+          } else {
+            r.a[s][rr][i] = on ? *reinterpret_cast<const uint4*>(W + off) : make_uint4(0, 0, 0, 0);
+            if (DUAL) r.b[s][rr][i] = on ? *reinterpret_cast<const uint4*>(W2 + off) : make_uint4(0, 0, 0, 0);
+          }
         }
   } else {
     const int8_t* W = (const int8_t*)Wv;
@@ -124,8 +144,13 @@ __device__ __forceinline__ void gemv_prefetch(const void* Wv, const void* W2v, i
           const int c = p.c0 + lane + WAVE * i;
           const bool on = s < p.nslots && c < p.c1;
           const size_t off = ((size_t)(2 * p.gp[s] + rr)) * K + (size_t)c * 8;
-          r.a[s][rr][i] = on ? *reinterpret_cast<const uint2*>(W + off) : make_uint2(0, 0);
-          if (DUAL) r.b[s][rr][i] = on ? *reinterpret_cast<const uint2*>(W2 + off) : make_uint2(0, 0);
+          if constexpr (NT) {
+            r.a[s][rr][i] = on ? ld_nt8(W + off) : make_uint2(0, 0);
+            if (DUAL) r.b[s][rr][i] = on ? ld_nt8(W2 + off) : make_uint2(0, 0);
+          } else {
+            r.a[s][rr][i] = on ? *reinterpret_cast<const uint2*>(W + off) : make_uint2(0, 0);
+            if (DUAL) r.b[s][rr][i] = on ? *reinterpret_cast<const uint2*>(W2 + off) : make_uint2(0, 0);
+          }
         }
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
@@ -522,7 +547,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       // ---- QKV + RoPE + cache append ----
       WRegs<2, false, I8> wr;
       const Plan P_qkv = plan_of(n_qkv, d, wg, nwg, wave);
-      gemv_prefetch<2, false, I8>(Lw.wqkv, nullptr, d, P_qkv, wr, Ls.s_qkv);
+      gemv_prefetch<2, false, I8, true>(Lw.wqkv, nullptr, d, P_qkv, wr, Ls.s_qkv);
       const NormW nw1 = load_normw(Lw.attn_norm, d);
       TS(1);
       if (ybuf) poll_add(xres, ybuf, d / 2, c);
@@ -713,7 +738,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       {
         WRegs<2, false, I8> w2;
         const Plan P_o = plan_of(n_o, d, wg, nwg, wave);
-        gemv_prefetch<2, false, I8>(Lw.wo, nullptr, d, P_o, w2, Ls.s_o);
+        gemv_prefetch<2, false, I8, true>(Lw.wo, nullptr, d, P_o, w2, Ls.s_o);
         poll_words(xp, rep_rd(attbuf), d / 2, c);
         TS(7);
         gemv_compute<2, false, I8>(xp, P_o, w2, red, [&](int gp, float v0, float v1, float, float) {
@@ -725,7 +750,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       {
         WRegs<2, true, I8> w3;
         const Plan P_sw = plan_of(n_sw, d, wg, nwg, wave);
-        gemv_prefetch<2, true, I8>(Lw.w1, Lw.w3, d, P_sw, w3, Ls.s_1, Ls.s_3);
+        gemv_prefetch<2, true, I8, true>(Lw.w1, Lw.w3, d, P_sw, w3, Ls.s_1, Ls.s_3);
         const NormW nw2 = load_normw(Lw.mlp_norm, d);
         poll_add(xres, rep_rd(obuf), d / 2, c);
         TS(9);
@@ -744,7 +769,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
       {
         WRegs<4, false, I8> w4;
         const Plan P_w2 = plan_of(n_o, a.F, wg, nwg, wave);
-        gemv_prefetch<4, false, I8>(Lw.w2, nullptr, a.F, P_w2, w4, Ls.s_2);
+        gemv_prefetch<4, false, I8, true>(Lw.w2, nullptr, a.F, P_w2, w4, Ls.s_2);
         poll_words(xp, rep_rd(hbuf), a.F / 2, c);
         TS(12);
         gemv_compute<4, false, I8>(xp, P_w2, w4, red, [&](int gp, float v0, float v1, float, float) {
@@ -757,7 +782,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
     {
       const Plan p = make_plan(a.CS / 2, d, wg, nwg, wave);
       WRegs<2, false> wr;
-      gemv_prefetch<2, false, false>(g_codec_head, nullptr, d, p, wr);
+      gemv_prefetch<2, false, false, true>(g_codec_head, nullptr, d, p, wr);
       const NormW nwf = load_normw(g_final_norm, d);
       uint32_t eosw[8];  // this lane's eos-head weight pairs (pair = lane, lane+64, ...), d <= 1024
 #pragma unroll
@@ -869,7 +894,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
     if (g_rq_proj) {
       const Plan p = make_plan(R / 2, d, wg, nwg, wave);
       WRegs<2, false> wr;
-      gemv_prefetch<2, false, false>(g_rq_proj, nullptr, d, p, wr);
+      gemv_prefetch<2, false, false, true>(g_rq_proj, nullptr, d, p, wr);
       // only pairs this wave really owns are inside pos_emb[0, R)
       const uint32_t pe0 = p.nslots > 0 ? *reinterpret_cast<const uint32_t*>(pos_emb + 2 * p.gp[0]) : 0u;
       const uint32_t pe1 = p.nslots > 1 ? *reinterpret_cast<const uint32_t*>(pos_emb + 2 * p.gp[1]) : 0u;
@@ -1082,7 +1107,7 @@ __global__ __launch_bounds__(FR_THREADS, 1) void frame_kernel(const FrameArgs a)
         // ---- head t-1: logits of codebook t, then the draw in every workgroup ----
         WRegs<2, false> wr;
         const Plan R_hd = plan_of(m_hd, R, wg, nwg, wave);
-        gemv_prefetch<2, false, false>(g_rq_head + (size_t)(t - 1) * CS * R, nullptr, R, R_hd, wr);
+        gemv_prefetch<2, false, false, true>(g_rq_head + (size_t)(t - 1) * CS * R, nullptr, R, R_hd, wr);
         TS(40);
         poll_add(xres, ybuf, R / 2, c);
         TS(41);
