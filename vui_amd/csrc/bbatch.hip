@@ -47,6 +47,21 @@ __device__ __forceinline__ void cvt8(const uint4& r, float* o) {
   o[6] = __uint_as_float(r.w << 16); o[7] = __uint_as_float(r.w & 0xffff0000u);
 }
 
+// Keys and values are read once per launch and a batch's caches (1.2 GB for 16 ragged rows) are far larger than the
+// memory-side cache, so their loads carry the non-temporal hint and leave the cache to what the step reads again:
+// the depth head's matrices of the next launch (16 int8 rows 1726 -> 1650 us per frame step, 8 rows 1546 -> 1507).
+// The same hint on the weight tiles - each read by one workgroup of every row group - helped two rows and cost four,
+// and is not used.
+typedef unsigned int bb_u32x4 __attribute__((ext_vector_type(4)));
+template <bool NT> __device__ __forceinline__ uint4 bb_ld16(const void* p) {
+  if constexpr (NT) {
+    const bb_u32x4 v = __builtin_nontemporal_load((const __attribute__((address_space(1))) bb_u32x4*)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+  } else {
+    return *reinterpret_cast<const uint4*>(p);
+  }
+}
+
 #define BB_RG 4        // rows per row group
 #define BB_MAXSPL 16   // key ranges per row at most (a merge waits for that many partial results)
 #define BB_U 8         // keys per lane group in flight per attention step
@@ -72,11 +87,11 @@ __device__ __forceinline__ void bb_prefetch(const void* Wt, int K, const BbTile&
     const int s = wave + 4 * i;
     if (EXACT || s < nsteps) {  // uniform over the wave; a step past the end is never used
       if (I8) {
-        r.a[i] = *reinterpret_cast<const uint4*>((const uint8_t*)Wt + (band + s) * 1024 + lane * 16);
+        r.a[i] = bb_ld16<false>((const uint8_t*)Wt + (band + s) * 1024 + lane * 16);
       } else {
         const bf16_t* p = (const bf16_t*)Wt + (band + s) * 1024 + lane * 8;
-        r.a[2 * i] = *reinterpret_cast<const uint4*>(p);
-        r.a[2 * i + 1] = *reinterpret_cast<const uint4*>(p + 512);
+        r.a[2 * i] = bb_ld16<false>(p);
+        r.a[2 * i + 1] = bb_ld16<false>(p + 512);
       }
     }
   }
@@ -615,8 +630,8 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
 #pragma unroll
         for (int u = 0; u < BB_U; ++u) {
           const int j = min(lo + ks + KP * u, hi - 1);  // hi >= 1
-          kr[u] = *reinterpret_cast<const uint4*>(kbase + (size_t)j * rowstride);
-          vr[u] = *reinterpret_cast<const uint4*>(vbase + (size_t)j * rowstride);
+          kr[u] = bb_ld16<true>(kbase + (size_t)j * rowstride);
+          vr[u] = bb_ld16<true>(vbase + (size_t)j * rowstride);
         }
         uint32_t* qw = (uint32_t*)att;   // q of the piece's heads | new k | new v of their KV heads, packed pairs (<= 1536 words)
         float* gm = att + 1536;          // 16 maxima, 16 sums, 16 weights, 16 head maxima
@@ -674,8 +689,8 @@ __global__ __launch_bounds__(FR_THREADS, 1) void bb_batch_kernel(const BbArgs a)
 #pragma unroll
           for (int u = 0; u < BB_U; ++u) {
             const int j = min(j0 + KP * BB_U + KP * u, hi - 1);  // past the piece: its last key again, never used
-            kn[u] = *reinterpret_cast<const uint4*>(kbase + (size_t)j * rowstride);
-            vn[u] = *reinterpret_cast<const uint4*>(vbase + (size_t)j * rowstride);
+            kn[u] = bb_ld16<true>(kbase + (size_t)j * rowstride);
+            vn[u] = bb_ld16<true>(vbase + (size_t)j * rowstride);
           }
           float sc_[BB_U];
           float mn = m;
