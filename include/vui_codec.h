@@ -89,6 +89,9 @@ int vui_codec_persistent(vui_codec* c, int enable);
  * kernel needs all its workgroups resident on the compute units its stream may use.  With fewer workgroups each
  * owns more rows of every matrix; below about 96 (at the reference's dims) the rows no longer fit the registers a
  * wave keeps them in and the call fails with VUI_EINVAL (vui_codec_persistent(c, 0) then runs the launches).
+ * A vocoder limited this way reads its weights (each byte once per frame) with non-temporal loads, which leaves the
+ * caches to the kernels it runs beside (measured: the decode step beside it 4 % faster; the vocoder alone would be
+ * 4 % slower with them, so at the full width they are not used).
  * Steps captured earlier keep the width they were captured with.  No counterpart in the reference. */
 int vui_codec_workgroups(vui_codec* c, int nwg);
 
