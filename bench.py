@@ -124,11 +124,11 @@ def gpu_bench(args):
 # taken inside this program's timed region); every line that carries one names the file it comes from.
 # HBM traffic of one frame_kernel launch (whole frame, bf16): FETCH_SIZE and WRITE_SIZE, KiB per dispatch, each scaled
 # by what the same counter reads for a plain 512 MiB device copy (bench.py --calib): 2.000 and 1.000.
-MEASURED_TRAFFIC = {"bytes": 522_218_957, "source": "profiles/frame_kernel_e2e_b1.txt", "cache_length": [577, 681],
+MEASURED_TRAFFIC = {"bytes": 488_214_606, "source": "profiles/frame_kernel_e2e_b1.txt", "cache_length": [577, 681],
                     "algorithmic_bytes_there": 415289344,
                     "command": "rocprofv3 --pmc FETCH_SIZE (then WRITE_SIZE) -- python3 bench.py --steps 50 --warmup 5 --no-cpu --no-b16 --no-sweep --calib"}
 # MFMA busy cycles / busy cycles of the two persistent kernels of the 16-stream step.
-MEASURED_B16_MFMA_BUSY = {"bb_batch_kernel": 0.35, "rq_batch_kernel": 0.49, "source": "profiles/e2e_b16_int8_step_kernels.txt",
+MEASURED_B16_MFMA_BUSY = {"bb_batch_kernel": 0.37, "rq_batch_kernel": 0.50, "source": "profiles/e2e_b16_int8_step_kernels.txt",
                           "command": "rocprofv3 --pmc SQ_BUSY_CYCLES SQ_VALU_MFMA_BUSY_CYCLES -- python3 bench.py --b16-only --steps 2"}
 
 
